@@ -1,0 +1,180 @@
+"""numpy front end of the CPU oracle (oracle/insc_oracle.c).
+
+TEST INFRASTRUCTURE ONLY: imported by tests/, by the smoke check and by the cpu_baseline
+leg of the benchmark, never by the shipped package.  Each function is a thin ctypes call
+into the C restatement; the reference source each one follows is cited in the C file.
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB = None
+
+_i32p = ctypes.POINTER(ctypes.c_int32)
+_f32p = ctypes.POINTER(ctypes.c_float)
+
+
+def build(force=False):
+    so = os.path.join(_HERE, "liborc.so")
+    if force or not os.path.exists(so):
+        subprocess.check_call(["make", "-C", _HERE, "-B", "liborc.so"], stdout=subprocess.DEVNULL)
+    return so
+
+
+def lib():
+    global _LIB
+    if _LIB is None:
+        L = ctypes.CDLL(build())
+        L.orc_grid_build.restype = ctypes.c_int64
+        L.orc_ssc_rules.restype = ctypes.c_int64
+        L.orc_down2_rules.restype = ctypes.c_int64
+        L.orc_conv_forward.restype = ctypes.c_double
+        L.orc_nin_forward.restype = ctypes.c_double
+        L.orc_num_threads.restype = ctypes.c_int
+        _LIB = L
+    return _LIB
+
+
+def _ip(a):
+    return a.ctypes.data_as(_i32p) if a is not None else None
+
+
+def _fp(a):
+    return a.ctypes.data_as(_f32p) if a is not None else None
+
+
+def _c4(coords):
+    c = np.ascontiguousarray(coords, dtype=np.int32)
+    if c.ndim != 2 or c.shape[1] not in (3, 4):
+        raise ValueError("coords must be [P,3] or [P,4]")
+    if c.shape[1] == 3:
+        c = np.concatenate([c, np.zeros((len(c), 1), np.int32)], 1)
+    return np.ascontiguousarray(c)
+
+
+def _f(a):
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+def num_threads():
+    return lib().orc_num_threads()
+
+
+def grid_build(coords):
+    """-> (site_of_point[P], site_coords[N,4], count[N]); sites numbered by first appearance."""
+    c = _c4(coords)
+    P = len(c)
+    sop = np.empty(P, np.int32)
+    sc = np.empty((max(P, 1), 4), np.int32)
+    cnt = np.empty(max(P, 1), np.int32)
+    n = lib().orc_grid_build(_ip(c), ctypes.c_int64(P), _ip(sop), _ip(sc), _ip(cnt))
+    return sop, sc[:n].copy(), cnt[:n].copy()
+
+
+def grid_query(site_coords, q):
+    sc, q = _c4(site_coords), _c4(q)
+    out = np.empty(len(q), np.int32)
+    lib().orc_grid_query(_ip(sc), ctypes.c_int64(len(sc)), _ip(q), ctypes.c_int64(len(q)), _ip(out))
+    return out
+
+
+def input_forward(feats, site_of_point, count, mode=4):
+    f = _f(feats)
+    P, C = f.shape
+    N = len(count)
+    out = np.empty((N, C), np.float32)
+    lib().orc_input_forward(_fp(f), ctypes.c_int64(P), C, _ip(np.ascontiguousarray(site_of_point, np.int32)),
+                            _ip(np.ascontiguousarray(count, np.int32)), ctypes.c_int64(N), int(mode == 4), _fp(out))
+    return out
+
+
+def output_forward(feats, site_of_point):
+    f = _f(feats)
+    sop = np.ascontiguousarray(site_of_point, np.int32)
+    out = np.empty((len(sop), f.shape[1]), np.float32)
+    lib().orc_output_forward(_fp(f), f.shape[1], _ip(sop), ctypes.c_int64(len(sop)), _fp(out))
+    return out
+
+
+def ssc_rules(site_coords, zmajor=False):
+    """-> (nbr[N,27], counts[27], pairs[R,2]) ; pairs are the 27 lists back to back."""
+    sc = _c4(site_coords)
+    N = len(sc)
+    nbr = np.empty((N, 27), np.int32)
+    counts = np.zeros(27, np.int32)
+    pairs = np.empty((max(27 * N, 1), 2), np.int32)
+    r = lib().orc_ssc_rules(_ip(sc), ctypes.c_int64(N), int(zmajor), _ip(nbr), _ip(counts), _ip(pairs))
+    return nbr, counts, pairs[:r].copy()
+
+
+def down2_rules(fine_coords):
+    """-> (parent[Nf], offset[Nf], coarse_coords[Nc,4])."""
+    fc = _c4(fine_coords)
+    Nf = len(fc)
+    parent = np.empty(Nf, np.int32)
+    off = np.empty(Nf, np.int32)
+    cc = np.empty((max(Nf, 1), 4), np.int32)
+    n = lib().orc_down2_rules(_ip(fc), ctypes.c_int64(Nf), _ip(parent), _ip(off), _ip(cc))
+    return parent, off, cc[:n].copy()
+
+
+def down2_pairs(parent, offset):
+    """Rulebook form of a size-2 stride-2 layer: 8 lists of (fine, coarse), back to back."""
+    counts = np.bincount(offset, minlength=8).astype(np.int32)
+    order = np.argsort(offset, kind="stable")
+    pairs = np.stack([order.astype(np.int32), parent[order]], 1)
+    return counts, np.ascontiguousarray(pairs, np.int32)
+
+
+def conv_forward(feats, W, bias, pairs, counts, n_out, swap=False):
+    f, W = _f(feats), _f(W)
+    K, Cin, Cout = W.shape
+    assert f.shape[1] == Cin and len(counts) == K
+    out = np.empty((n_out, Cout), np.float32)
+    b = _f(bias) if bias is not None else None
+    p = np.ascontiguousarray(pairs, np.int32)
+    c = np.ascontiguousarray(counts, np.int32)
+    flops = lib().orc_conv_forward(_fp(f), _fp(out), ctypes.c_int64(n_out), _fp(W), _fp(b), _ip(p), _ip(c), K, Cin,
+                                   Cout, int(swap))
+    return out, flops
+
+
+def bn_forward(feats, mean, var, gamma, beta, eps=1e-4, leakiness=0.0):
+    f = _f(feats)
+    out = np.empty_like(f)
+    g = _f(gamma) if gamma is not None else None
+    b = _f(beta) if beta is not None else None
+    lib().orc_bn_forward(_fp(f), _fp(out), ctypes.c_int64(f.shape[0]), f.shape[1], _fp(_f(mean)), _fp(_f(var)),
+                         _fp(g), _fp(b), ctypes.c_float(eps), ctypes.c_float(leakiness))
+    return out
+
+
+def nin_forward(feats, W, bias=None):
+    f, W = _f(feats), _f(W)
+    out = np.empty((f.shape[0], W.shape[1]), np.float32)
+    b = _f(bias) if bias is not None else None
+    lib().orc_nin_forward(_fp(f), _fp(out), ctypes.c_int64(f.shape[0]), _fp(W), _fp(b), W.shape[0], W.shape[1])
+    return out
+
+
+# --------------------------------------------------------------------------------------
+# canonical forms used to compare integer structures bit-exactly
+# --------------------------------------------------------------------------------------
+def canonical_sites(site_coords):
+    """Rows sorted by (b, z, y, x): the key order of the reference's GPU grid."""
+    sc = _c4(site_coords)
+    o = np.lexsort((sc[:, 0], sc[:, 1], sc[:, 2], sc[:, 3]))
+    return sc[o]
+
+
+def canonical_rules(counts, pairs, in_coords, out_coords):
+    """Rules as rows (offset, in xyz b, out xyz b), sorted: independent of site numbering."""
+    counts = np.asarray(counts)
+    k = np.repeat(np.arange(len(counts)), counts).astype(np.int64)
+    ic, oc = _c4(in_coords)[pairs[:, 0]].astype(np.int64), _c4(out_coords)[pairs[:, 1]].astype(np.int64)
+    rows = np.concatenate([k[:, None], ic, oc], 1)
+    o = np.lexsort(tuple(rows[:, j] for j in range(rows.shape[1] - 1, -1, -1)))
+    return rows[o]
