@@ -1,0 +1,211 @@
+/*
+ * insc.h - C ABI of the MI355X (gfx950) sparse-convolution inference library.
+ *
+ * This is the drop-in boundary for the reference's native extension `sparseconvnet.SCN`
+ * (reference: sparseconvnet/SCN/pybind.cpp:153-258, sparseconvnet/SCN/sparseconvnet.h).
+ * The reference passes at::Tensor objects; here every argument is a plain pointer or size.
+ * Unless a parameter name starts with h_ it is a DEVICE pointer valid on the device bound
+ * with insc_init.  Every function returns 0 on success or a negative INSC_ERR_* code and
+ * never aborts the process (the reference calls assert/abort/exit on failure,
+ * CUDA/CUDPPWrapper.hpp:17-27); insc_last_error() gives the message of the calling thread's
+ * last failure.  `stream` is a hipStream_t passed as void* (NULL = the default stream);
+ * work is enqueued asynchronously on it and functions that hand a value back to the host
+ * (h_ arguments) synchronise that stream first.
+ *
+ * Feature matrices are row-major float32 with an explicit row stride `ld` (in floats), so
+ * a layer can read or write a column slice of a wider matrix (channel concatenation without
+ * a copy).  Site ids are int32; -1 means "no site".  Coordinates are int32 quadruples
+ * (x, y, z, batch) with 0 <= x,y,z <= 65535 and 0 <= batch <= 32767.
+ *
+ * Row subsets: the feature functions take `rows` (int32 list of output rows to compute, or
+ * NULL for rows 0..n_rows-1), `d_n_rows` (device int32 holding the list length, or NULL to
+ * use n_rows) and `n_rows` (the length, or an upper bound on *d_n_rows used to size the
+ * launch).  Rows not listed are left untouched: this is what the incremental path uses to
+ * recompute only dirty rows.
+ */
+#ifndef INSC_H
+#define INSC_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define INSC_OK 0
+#define INSC_ERR_ARG -1      /* bad argument (null pointer, negative size, unsupported shape) */
+#define INSC_ERR_HIP -2      /* a HIP runtime call failed; message holds hipGetErrorString */
+#define INSC_ERR_CAPACITY -3 /* a fixed-capacity structure would overflow */
+#define INSC_ERR_STATE -4    /* call order violated (e.g. library not initialised) */
+#define INSC_ERR_COORD -5    /* a coordinate is outside the representable range */
+
+typedef struct insc_grid insc_grid;
+
+/* Binds the library to a HIP device (hipSetDevice) and checks that it is a gfx950 part.
+ * No counterpart in the reference, which uses whatever device torch selected. */
+int insc_init(int device);
+const char *insc_last_error(void);
+const char *insc_version(void);
+
+/* ---------------------------------------------------------------------------------------
+ * Hash grid: the set of active sites of one spatial scale.  Replaces the reference's
+ * Multival_Point_Hashtable<3> over the CUDPP cuckoo hash (CUDA/CUDPPWrapper.hpp:736-1010)
+ * and GPU_SparseGrid (Metadata/Metadata.h:114-122).  Open addressing on 64-bit packed keys.
+ * Sites are numbered by first appearance in the inserted coordinate list (the numbering of
+ * the reference's CPU path, Metadata/IOLayersRules.h:69-79) and numbering is append-only:
+ * a later insert never renumbers existing sites.
+ * ------------------------------------------------------------------------------------- */
+int insc_grid_create(int64_t capacity_sites, insc_grid **out);
+int insc_grid_destroy(insc_grid *g);
+/* Forget all sites, keep the allocation (reference: Metadata<D>::clear, Metadata.cpp:68-75). */
+int insc_grid_clear(insc_grid *g, void *stream);
+/* Grow so that capacity_sites fit; rehashes the existing sites, ids unchanged. */
+int insc_grid_reserve(insc_grid *g, int64_t capacity_sites, void *stream);
+/* Insert P coordinates (duplicates allowed).  d_site_of_point[p] receives the site of row p.
+ * h_n_sites (nullable, host) receives the site count after the insert (synchronises).
+ * Replaces HashInputPointClouds + InsertAndCompactPointCloud (CUDPPWrapper.hpp:668-686,
+ * 766-796; kernels CUDPPWrapper.cu:72-100,212-231). */
+int insc_grid_insert(insc_grid *g, const int32_t *d_coords4, int64_t P, int32_t *d_site_of_point, int64_t *h_n_sites,
+                     void *stream);
+/* d_site[q] = site id of coordinate q, or -1.  Replaces Multival retrieve +
+ * _dMultivalHashGetValue (CUDPPWrapper.cu:144-160), whose miss value is 0xFFFFFFFF. */
+int insc_grid_query(const insc_grid *g, const int32_t *d_coords4, int64_t Q, int32_t *d_site, void *stream);
+/* Site count (synchronises `stream` if an insert is still in flight). */
+int insc_grid_size(insc_grid *g, int64_t *h_n_sites, void *stream);
+/* Device pointer to the [capacity,4] coordinate table; rows 0..n-1 are valid
+ * (reference: getAllPoints, read by Metadata<D>::getSpatialLocations, Metadata.cpp:793-821). */
+const int32_t *insc_grid_coords(const insc_grid *g);
+/* Device pointer to the int32 site counter. */
+const int32_t *insc_grid_count_ptr(const insc_grid *g);
+int64_t insc_grid_capacity(const insc_grid *g);
+
+/* ---------------------------------------------------------------------------------------
+ * Rulebooks.
+ * ------------------------------------------------------------------------------------- */
+/* Submanifold 3x3x3 neighbour map for sites [first, first+n): d_nbr[o*27+k] = id of the
+ * site at coordinate(o) + (dx,dy,dz), k = (dx+1)*9 + (dy+1)*3 + (dz+1), or -1.  With
+ * patch_reverse != 0 it also writes d_nbr[j*27 + 26-k] = o for every neighbour j found, which
+ * brings the rows of older sites up to date after an append.  Replaces
+ * SubmanifoldBuildObject (CUDA/SubmanifoldRules_cuda.cpp:38-228; kernels
+ * SubmanifoldRules_cuda.cu:45-77,91-114) - same relation and offset numbering, kept as a
+ * dense map instead of 27 compacted lists. */
+int insc_rulebook_ssc3(const insc_grid *g, int64_t first, int64_t n, int32_t *d_nbr, int patch_reverse, void *stream);
+/* The reference's list form of the same rulebook (RuleBook = 27 lists of (in,out) pairs,
+ * Metadata/Metadata.h:86): d_counts[k] pairs for offset k, lists back to back in d_pairs,
+ * each in ascending `out` order.  h_total (nullable) receives the pair count. */
+int insc_rulebook_pairs(const int32_t *d_nbr, int64_t N, int K, int32_t *d_counts, int32_t *d_pairs,
+                        int64_t pairs_capacity, int64_t *h_total, void *stream);
+/* Size-2 stride-2 rulebook for fine sites [first, first+n): inserts coordinate>>1 into the
+ * coarse grid, d_parent[i] = coarse site, d_offset[i] = (x&1)*4 + (y&1)*2 + (z&1), and if
+ * d_child != NULL, d_child[parent*8 + offset] = i (rows of new coarse sites must have been
+ * filled with -1 by the caller; child_rows = rows allocated for d_child, which must cover the
+ * coarse grid's capacity).  Replaces
+ * Convolution_InputSgToRulesAndOutputSg_FastDownSampleMode (Metadata/ConvolutionRules.h:344-380,
+ * kernel SubmanifoldRules_cuda.cu:744-780). */
+int insc_rulebook_down2(const insc_grid *fine, insc_grid *coarse, int64_t first, int64_t n, int32_t *d_parent,
+                        int32_t *d_offset, int32_t *d_child, int64_t child_rows, void *stream);
+/* A processing order for the sites first..first+n-1, written to d_order[first..first+n): a
+ * permutation of those ids that puts sites of one 16^3 block with the same neighbour pattern
+ * next to each other, so that row tiles of the convolution kernel skip whole filter offsets.
+ * Results of the convolution do not depend on it.  No counterpart in the reference (its chunk
+ * builder, SubmanifoldRules_cuda.cpp:572-1112, serves the same purpose for its
+ * shared-memory kernel). */
+int insc_order_build(const insc_grid *g, const int32_t *d_nbr, int64_t first, int64_t n, int32_t *d_order,
+                     void *stream);
+
+/* d_out = the sites of d_order[0..n) (or 0..n-1 if d_order is NULL) regrouped by their
+ * offset inside the parent cell (d_offset[site], 0..7), keeping the given order within a
+ * group.  A row tile of the deconvolution then uses a single weight slice.  No counterpart in
+ * the reference (its rulebook is already split by offset, Metadata/Metadata.h:86). */
+int insc_order_by_offset(const int32_t *d_order, const int32_t *d_offset, int64_t n, int32_t *d_out, void *stream);
+
+/* ---------------------------------------------------------------------------------------
+ * Feature kernels.
+ * ------------------------------------------------------------------------------------- */
+/* Output-stationary sparse convolution over a neighbour map:
+ *   out[o,:] = bias + sum_k  in[nbr[o*K+k], :] . W[k]      (terms with nbr = -1 skipped)
+ * K = 27 with an insc_rulebook_ssc3 map is SubmanifoldConvolution_updateOutput
+ * (CUDA/Convolution.cpp:152-218); K = 8 with a child map is Convolution_updateOutput for
+ * size 2 / stride 2 (CUDA/Convolution.cpp:52-81); K = 1 with d_nbr = NULL (identity map) is
+ * NetworkInNetwork_updateOutput (CUDA/NetworkInNetwork.cpp:9-25).  W is [K,Cin,Cout].
+ * h_muladds (nullable) receives the multiply-add count the reference returns (synchronises). */
+int insc_conv_nbr(const float *d_in, int64_t ld_in, float *d_out, int64_t ld_out, const float *d_W,
+                  const float *d_bias, const int32_t *d_nbr, int K, const int32_t *d_rows, const int32_t *d_n_rows,
+                  int64_t n_rows, int Cin, int Cout, double *h_muladds, void *stream);
+/* Size-2 stride-2 deconvolution: out[i,:] = bias + in[parent[i],:] . W[offset[i]]
+ * (Deconvolution_updateOutput, CUDA/Deconvolution.cpp:28-58: the convolution's rules with
+ * the roles of input and output swapped). */
+int insc_deconv_down2(const float *d_in, int64_t ld_in, float *d_out, int64_t ld_out, const float *d_W,
+                      const float *d_bias, const int32_t *d_parent, const int32_t *d_offset, const int32_t *d_rows,
+                      const int32_t *d_n_rows, int64_t n_rows, int Cin, int Cout, void *stream);
+/* Inference batch norm + leaky ReLU: y = x*w + b, y *= (y>0 ? 1 : leakiness),
+ * w = gamma*(var+eps)^-1/2, b = beta - mean*w; gamma/beta nullable
+ * (BatchNormalization_updateOutput with train=false, CUDA/BatchNormalization.cpp:39-61,
+ * kernel BatchNormalization.cu:78-107). */
+int insc_bn_leaky(const float *d_in, int64_t ld_in, float *d_out, int64_t ld_out, const float *d_mean,
+                  const float *d_var, const float *d_gamma, const float *d_beta, float eps, float leakiness,
+                  const int32_t *d_rows, const int32_t *d_n_rows, int64_t n_rows, int C, void *stream);
+/* out = a + b on the listed rows (AddTable, sparseconvnet/tables.py:28-40). */
+int insc_add(const float *d_a, int64_t ld_a, const float *d_b, int64_t ld_b, float *d_out, int64_t ld_out,
+             const int32_t *d_rows, const int32_t *d_n_rows, int64_t n_rows, int C, void *stream);
+/* out[r, :] = in[r, :] on the listed rows (column-slice copy used for JoinTable,
+ * sparseconvnet/tables.py:13-25). */
+int insc_copy_rows(const float *d_in, int64_t ld_in, float *d_out, int64_t ld_out, const int32_t *d_rows,
+                   const int32_t *d_n_rows, int64_t n_rows, int C, void *stream);
+
+/* Input layer accumulation: adds the P feature rows to the per-site running sums
+ * d_sum[site,:] (float32 [*,C]) and counts d_cnt[site], rows of one site in ascending row
+ * order (the order InputLayer_fp_ visits them, CUDA/IOLayers.cu:17-32).  The caller zeroes
+ * the rows of d_sum / d_cnt that belong to sites it has not accumulated into before.
+ * mode 1 keeps the first row of a site, mode 2 the last (CPU rule builder,
+ * Metadata/IOLayersRules.h:104-115), modes 0/3/4 sum. */
+int insc_input_accumulate(const float *d_feats, int64_t P, int C, const int32_t *d_site_of_point, int mode,
+                          float *d_sum, int32_t *d_cnt, int64_t n_sites_upper, void *stream);
+/* out[s,:] = sum[s,:] / cnt[s] (mode 4) or sum[s,:] (other modes) on the listed rows. */
+int insc_input_finish(const float *d_sum, const int32_t *d_cnt, int mode, float *d_out, int64_t ld_out,
+                      const int32_t *d_rows, const int32_t *d_n_rows, int64_t n_rows, int C, void *stream);
+/* Output layer: out[p,:] = in[site_of_point[p],:] (OutputLayer_updateOutput,
+ * CUDA/IOLayers.cpp:123-145: InputLayer_bp_ with multiplier 1). */
+int insc_output_gather(const float *d_in, int64_t ld_in, const int32_t *d_site_of_point, int64_t P, int C,
+                       float *d_out, void *stream);
+
+/* ---------------------------------------------------------------------------------------
+ * Dirty-site propagation for the incremental forward.  Masks are uint8 per site.
+ * The reference's incremental path does not dilate (CUDA/Convolution.cpp:221-303 computes
+ * residuals only at the increment's own sites); these functions implement the exact rule:
+ * a row must be recomputed iff any input it reads changed.
+ * ------------------------------------------------------------------------------------- */
+int insc_fill_u8(uint8_t *d_p, int64_t n, int value, void *stream);
+int insc_fill_i32(int32_t *d_p, int64_t n, int32_t value, void *stream);
+/* mask[site_of_point[p]] = 1 */
+int insc_dirty_mark(const int32_t *d_site_of_point, int64_t P, uint8_t *d_mask, void *stream);
+/* mask_out[j] = 1 for every j = nbr[i*27+k] >= 0 with mask_in[i] != 0 (includes i itself). */
+int insc_dirty_dilate3(const int32_t *d_nbr, const uint8_t *d_mask_in, uint8_t *d_mask_out, const int32_t *d_n,
+                       int64_t n_upper, void *stream);
+/* mask_coarse[parent[i]] = 1 for dirty fine i. */
+int insc_dirty_parents(const int32_t *d_parent, const uint8_t *d_mask_fine, uint8_t *d_mask_coarse,
+                       const int32_t *d_n_fine, int64_t n_upper, void *stream);
+/* mask_fine[i] |= mask_coarse[parent[i]]. */
+int insc_dirty_children(const int32_t *d_parent, const uint8_t *d_mask_coarse, uint8_t *d_mask_fine,
+                        const int32_t *d_n_fine, int64_t n_upper, void *stream);
+/* mask_out = mask_a | mask_b */
+int insc_dirty_or(const uint8_t *d_a, const uint8_t *d_b, uint8_t *d_out, const int32_t *d_n, int64_t n_upper,
+                  void *stream);
+/* d_rows = the sites s (taken in the sequence d_order[0..n) if given, else 0..n) with
+ * mask[s] != 0; *d_count = how many.  h_count nullable (synchronises). */
+int insc_dirty_compact(const uint8_t *d_mask, const int32_t *d_order, const int32_t *d_n, int64_t n_upper,
+                       int32_t *d_rows, int32_t *d_count, int64_t *h_count, void *stream);
+
+/* ---------------------------------------------------------------------------------------
+ * Device utilities exported for tests and callers.
+ * ------------------------------------------------------------------------------------- */
+/* Exclusive prefix sum of n int32 values; d_total (nullable) receives the sum. */
+int insc_scan_exclusive_i32(const int32_t *d_in, int32_t *d_out, int64_t n, int32_t *d_total, void *stream);
+/* Stable ascending sort of n (key,value) pairs on the low key_bits bits of the 64-bit keys.
+ * Keys and values are sorted in place (d_keys / d_vals hold the result). */
+int insc_sort_pairs_u64(uint64_t *d_keys, int32_t *d_vals, int64_t n, int key_bits, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* INSC_H */

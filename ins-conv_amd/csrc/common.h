@@ -1,0 +1,64 @@
+// Internal helpers shared by the HIP translation units of libinsc.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "../../include/insc.h"
+
+namespace insc {
+
+// ---- error reporting -------------------------------------------------------------------
+void set_error(const char *fmt, ...);
+int hip_fail(hipError_t e, const char *what, const char *file, int line);
+
+#define INSC_HIP(call)                                                        \
+  do {                                                                        \
+    hipError_t e__ = (call);                                                  \
+    if (e__ != hipSuccess) return insc::hip_fail(e__, #call, __FILE__, __LINE__); \
+  } while (0)
+
+#define INSC_REQUIRE(cond, code, ...) \
+  do {                                \
+    if (!(cond)) {                    \
+      insc::set_error(__VA_ARGS__);   \
+      return (code);                  \
+    }                                 \
+  } while (0)
+
+#define INSC_LAUNCH_CHECK() INSC_HIP(hipGetLastError())
+
+// ---- per-stream scratch memory ---------------------------------------------------------
+// Temporary device memory for scans, sorts and compactions.  One arena per (device, stream);
+// it only ever grows, so steady-state calls allocate nothing.  Work using an arena is
+// ordered by its stream.
+// Arena 0 belongs to the scan primitive, arena 1 to the sort primitive, arena 2 to the
+// API-level function that is running (none of which calls another arena-2 user).
+enum { WS_SCAN = 0, WS_SORT = 1, WS_API = 2 };
+int workspace(int which, hipStream_t stream, size_t bytes, void **out);
+
+// ---- device primitives (scan_sort.hip) -------------------------------------------------
+int scan_exclusive_i32(const int32_t *in, int32_t *out, int64_t n, int32_t *total, hipStream_t s);
+int sort_pairs_u64(uint64_t *keys, int32_t *vals, int64_t n, int key_bits, hipStream_t s);
+
+static inline int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
+static inline unsigned grid_for(int64_t n, int block, int64_t cap = 1 << 20) {
+  int64_t g = cdiv(n, block);
+  if (g < 1) g = 1;
+  if (g > cap) g = cap;
+  return (unsigned)g;
+}
+
+// ---- key packing ------------------------------------------------------------------------
+// 64-bit voxel key: batch:16 | z:16 | y:16 | x:16.  Ascending key order is (batch, z, y, x).
+#define INSC_EMPTY_KEY 0xFFFFFFFFFFFFFFFFull
+
+__host__ __device__ static inline bool coord_ok(int x, int y, int z, int b) {
+  return ((unsigned)x | (unsigned)y | (unsigned)z) < 65536u && (unsigned)b < 32768u;
+}
+__host__ __device__ static inline uint64_t pack_key(int x, int y, int z, int b) {
+  return ((uint64_t)(unsigned)b << 48) | ((uint64_t)(unsigned)z << 32) | ((uint64_t)(unsigned)y << 16) |
+         (uint64_t)(unsigned)x;
+}
+
+}  // namespace insc

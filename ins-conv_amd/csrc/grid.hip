@@ -1,0 +1,454 @@
+// Hash grid: open addressing on 64-bit packed voxel keys, 16-byte slots.
+//
+// Home slot: the eight voxels (x, y, z0..z0+7) of one z-run share one aligned group of eight
+// slots (128 bytes, one L2 line), voxel z at position z&7.  The three z-neighbours of a
+// 3x3x3 query therefore read the same line, and the lanes of a wavefront that handle
+// consecutive filter offsets probe it together.  Collisions move on linearly.
+//
+// Numbering: a site's id is its rank among first occurrences in the inserted list, offset by
+// the count before the call - deterministic and append-only.
+#include "common.h"
+
+namespace insc {
+
+struct __attribute__((aligned(16))) Slot {
+  unsigned long long key;
+  int val;
+  int pad;
+};
+
+constexpr int VAL_UNSET = 0x7FFFFFFF;
+// At load <= 0.5 probe runs are a handful of slots; the cap only bounds a corrupted table.
+constexpr int64_t MAX_PROBES = 1 << 16;
+constexpr int VAL_PENDING = 0x40000000;  // VAL_PENDING + p : claimed during this insert by row p
+
+}  // namespace insc
+
+struct insc_grid {
+  insc::Slot *table = nullptr;
+  int64_t n_slots = 0;         // power of two
+  int64_t capacity_sites = 0;  // rows of coords
+  int32_t *coords = nullptr;   // [capacity_sites, 4]
+  int32_t *d_n = nullptr;      // device site counter
+  int32_t *d_err = nullptr;    // device flag: bit0 bad coordinate, bit1 table full
+  int64_t n_upper = 0;         // host upper bound of the site count
+  int64_t n_exact = -1;        // host copy of the count, -1 = stale
+  // insert scratch, grown on demand
+  int32_t *slot_of_point = nullptr;
+  int32_t *flags = nullptr;
+  int64_t scratch_rows = 0;
+  int device = 0;
+};
+
+namespace insc {
+
+__device__ __forceinline__ uint64_t mix64(uint64_t h) {
+  h ^= h >> 33;
+  h *= 0xff51afd7ed558ccdull;
+  h ^= h >> 33;
+  h *= 0xc4ceb9fe1a85ec53ull;
+  h ^= h >> 33;
+  return h;
+}
+
+__device__ __forceinline__ int64_t home_slot(uint64_t key, int64_t mask) {
+  // drop z's low three bits from the hashed part, put them back as the position in the group
+  uint64_t zlow = (key >> 32) & 7ull;
+  uint64_t h = mix64(key & ~(7ull << 32));
+  return (int64_t)(((h << 3) | zlow) & (uint64_t)mask);
+}
+
+__device__ __forceinline__ int grid_find(const Slot *__restrict__ table, int64_t mask, uint64_t key) {
+  int64_t s = home_slot(key, mask);
+  for (int64_t probe = 0; probe <= mask && probe < MAX_PROBES; probe++) {
+    unsigned long long k = table[s].key;
+    if (k == key) return table[s].val;
+    if (k == INSC_EMPTY_KEY) return -1;
+    s = (s + 1) & mask;
+  }
+  return -1;
+}
+
+__global__ void grid_clear_kernel(Slot *table, int64_t n_slots, int32_t *d_n, int32_t *d_err) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (; i < n_slots; i += stride) {
+    Slot e;
+    e.key = INSC_EMPTY_KEY;
+    e.val = VAL_UNSET;
+    e.pad = 0;
+    table[i] = e;
+  }
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    *d_n = 0;
+    *d_err = 0;
+  }
+}
+
+// pass 1: claim a slot per distinct key; the smallest row index claiming a new slot wins it
+__global__ void grid_claim_kernel(Slot *table, int64_t mask, const int32_t *__restrict__ coords4, int64_t P,
+                                  int32_t *__restrict__ slot_of_point, int32_t *d_err) {
+  int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (p >= P) return;
+  int4 c = reinterpret_cast<const int4 *>(coords4)[p];
+  if (!coord_ok(c.x, c.y, c.z, c.w)) {
+    slot_of_point[p] = -1;
+    atomicOr(d_err, 1);
+    return;
+  }
+  uint64_t key = pack_key(c.x, c.y, c.z, c.w);
+  int64_t s = home_slot(key, mask);
+  int64_t found = -1;
+  for (int64_t probe = 0; probe <= mask && probe < MAX_PROBES; probe++) {
+    unsigned long long k = table[s].key;
+    if (k == INSC_EMPTY_KEY) k = atomicCAS(&table[s].key, INSC_EMPTY_KEY, (unsigned long long)key);
+    if (k == INSC_EMPTY_KEY || k == key) {
+      found = s;
+      break;
+    }
+    s = (s + 1) & mask;
+  }
+  if (found < 0) {
+    slot_of_point[p] = -1;
+    atomicOr(d_err, 2);
+    return;
+  }
+  slot_of_point[p] = (int32_t)found;
+  // existing sites hold ids < VAL_PENDING and are left alone by the min
+  atomicMin(&table[found].val, VAL_PENDING + (int)p);
+}
+
+__global__ void grid_flag_kernel(const Slot *__restrict__ table, const int32_t *__restrict__ slot_of_point, int64_t P,
+                                 int32_t *__restrict__ flags) {
+  int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (p >= P) return;
+  int s = slot_of_point[p];
+  flags[p] = (s >= 0 && table[s].val == VAL_PENDING + (int)p) ? 1 : 0;
+}
+
+// pass 3: winners take id = n_before + rank, publish it in the slot and record the coordinates
+__global__ void grid_assign_kernel(Slot *table, const int32_t *__restrict__ coords4,
+                                   const int32_t *__restrict__ slot_of_point, const int32_t *__restrict__ excl,
+                                   int64_t P, const int32_t *__restrict__ d_n, int32_t *__restrict__ site_coords,
+                                   int64_t capacity_sites, int32_t *d_err) {
+  int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (p >= P) return;
+  int s = slot_of_point[p];
+  if (s < 0 || table[s].val != VAL_PENDING + (int)p) return;
+  int id = *d_n + excl[p];
+  if (id >= capacity_sites) {
+    atomicOr(d_err, 2);
+    return;
+  }
+  table[s].val = id;
+  reinterpret_cast<int4 *>(site_coords)[id] = reinterpret_cast<const int4 *>(coords4)[p];
+}
+
+__global__ void grid_resolve_kernel(const Slot *__restrict__ table, const int32_t *__restrict__ slot_of_point,
+                                    int64_t P, int32_t *__restrict__ site_of_point, int32_t *d_n,
+                                    const int32_t *__restrict__ total) {
+  int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (p < P) {
+    int s = slot_of_point[p];
+    int v = (s >= 0) ? table[s].val : -1;
+    site_of_point[p] = (v >= 0 && v < VAL_PENDING) ? v : -1;
+  }
+}
+__global__ void grid_bump_kernel(int32_t *d_n, const int32_t *total) { *d_n += *total; }
+
+__global__ void grid_query_kernel(const Slot *__restrict__ table, int64_t mask, const int32_t *__restrict__ coords4,
+                                  int64_t Q, int32_t *__restrict__ out) {
+  int64_t q = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (q >= Q) return;
+  int4 c = reinterpret_cast<const int4 *>(coords4)[q];
+  int r = -1;
+  if (coord_ok(c.x, c.y, c.z, c.w)) r = grid_find(table, mask, pack_key(c.x, c.y, c.z, c.w));
+  out[q] = r;
+}
+
+// re-insert site i with value i (used after a resize; keys are unique so no min is needed)
+__global__ void grid_rehash_kernel(Slot *table, int64_t mask, const int32_t *__restrict__ site_coords,
+                                   const int32_t *__restrict__ d_n, int32_t *d_err) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= *d_n) return;
+  int4 c = reinterpret_cast<const int4 *>(site_coords)[i];
+  uint64_t key = pack_key(c.x, c.y, c.z, c.w);
+  int64_t s = home_slot(key, mask);
+  for (int64_t probe = 0; probe <= mask && probe < MAX_PROBES; probe++) {
+    unsigned long long k = atomicCAS(&table[s].key, INSC_EMPTY_KEY, (unsigned long long)key);
+    if (k == INSC_EMPTY_KEY) {
+      table[s].val = (int)i;
+      return;
+    }
+    s = (s + 1) & mask;
+  }
+  atomicOr(d_err, 2);
+}
+
+// 27-neighbour map, one thread per (site, offset); see insc_rulebook_ssc3
+__global__ void ssc3_nbr_kernel(const Slot *__restrict__ table, int64_t mask, const int32_t *__restrict__ site_coords,
+                                int64_t first, int64_t n, int32_t *__restrict__ nbr, int patch_reverse) {
+  int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= n * 27) return;
+  int64_t o = first + t / 27;
+  int k = (int)(t % 27);
+  int4 c = reinterpret_cast<const int4 *>(site_coords)[o];
+  int x = c.x + k / 9 - 1, y = c.y + (k / 3) % 3 - 1, z = c.z + k % 3 - 1;
+  int r = -1;
+  if (k == 13)
+    r = (int)o;
+  else if (coord_ok(x, y, z, c.w))
+    r = grid_find(table, mask, pack_key(x, y, z, c.w));
+  nbr[o * 27 + k] = r;
+  if (patch_reverse && r >= 0 && r < first) nbr[(int64_t)r * 27 + (26 - k)] = (int)o;
+}
+
+__global__ void down2_coords_kernel(const int32_t *__restrict__ fine_coords, int64_t first, int64_t n,
+                                    int32_t *__restrict__ half, int32_t *__restrict__ offset) {
+  int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= n) return;
+  int4 c = reinterpret_cast<const int4 *>(fine_coords)[first + t];
+  offset[first + t] = (c.x & 1) * 4 + (c.y & 1) * 2 + (c.z & 1);
+  reinterpret_cast<int4 *>(half)[t] = make_int4(c.x >> 1, c.y >> 1, c.z >> 1, c.w);
+}
+
+__global__ void down2_child_kernel(const int32_t *__restrict__ parent, const int32_t *__restrict__ offset,
+                                   int64_t first, int64_t n, int32_t *__restrict__ child) {
+  int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= n) return;
+  int64_t i = first + t;
+  int p = parent[i];
+  if (p >= 0) child[(int64_t)p * 8 + offset[i]] = (int)i;
+}
+
+static int grid_alloc_table(insc_grid *g, int64_t capacity_sites) {
+  int64_t slots = 1024;
+  while (slots < 2 * capacity_sites) slots <<= 1;
+  INSC_HIP(hipMalloc((void **)&g->table, sizeof(Slot) * (size_t)slots));
+  g->n_slots = slots;
+  return INSC_OK;
+}
+
+static int grid_sync_errors(insc_grid *g, hipStream_t s, const char *who) {
+  int32_t h[2];
+  INSC_HIP(hipMemcpyAsync(&h[0], g->d_n, sizeof(int32_t), hipMemcpyDeviceToHost, s));
+  INSC_HIP(hipMemcpyAsync(&h[1], g->d_err, sizeof(int32_t), hipMemcpyDeviceToHost, s));
+  INSC_HIP(hipStreamSynchronize(s));
+  g->n_exact = h[0];
+  g->n_upper = h[0];
+  if (h[1] & 1) {
+    set_error("%s: a coordinate is outside 0..65535 (batch 0..32767)", who);
+    return INSC_ERR_COORD;
+  }
+  if (h[1] & 2) {
+    set_error("%s: grid capacity %lld exceeded", who, (long long)g->capacity_sites);
+    return INSC_ERR_CAPACITY;
+  }
+  return INSC_OK;
+}
+
+}  // namespace insc
+
+using namespace insc;
+
+extern "C" {
+
+int insc_grid_create(int64_t capacity_sites, insc_grid **out) {
+  INSC_REQUIRE(out, INSC_ERR_ARG, "insc_grid_create: out is null");
+  INSC_REQUIRE(capacity_sites >= 0 && capacity_sites < (1ll << 30), INSC_ERR_ARG,
+               "insc_grid_create: capacity %lld out of range", (long long)capacity_sites);
+  if (capacity_sites < 1024) capacity_sites = 1024;
+  insc_grid *g = new insc_grid();
+  INSC_HIP(hipGetDevice(&g->device));
+  g->capacity_sites = capacity_sites;
+  int rc = grid_alloc_table(g, capacity_sites);
+  if (rc) {
+    delete g;
+    return rc;
+  }
+  INSC_HIP(hipMalloc((void **)&g->coords, sizeof(int32_t) * 4 * (size_t)capacity_sites));
+  INSC_HIP(hipMalloc((void **)&g->d_n, 256));
+  g->d_err = g->d_n + 16;
+  *out = g;
+  return insc_grid_clear(g, nullptr);
+}
+
+int insc_grid_destroy(insc_grid *g) {
+  if (!g) return INSC_OK;
+  (void)hipDeviceSynchronize();
+  if (g->table) (void)hipFree(g->table);
+  if (g->coords) (void)hipFree(g->coords);
+  if (g->d_n) (void)hipFree(g->d_n);
+  if (g->slot_of_point) (void)hipFree(g->slot_of_point);
+  if (g->flags) (void)hipFree(g->flags);
+  delete g;
+  return INSC_OK;
+}
+
+int insc_grid_clear(insc_grid *g, void *stream) {
+  INSC_REQUIRE(g, INSC_ERR_ARG, "insc_grid_clear: grid is null");
+  hipLaunchKernelGGL(grid_clear_kernel, dim3(grid_for(g->n_slots, 256, 8192)), dim3(256), 0, (hipStream_t)stream,
+                     g->table, g->n_slots, g->d_n, g->d_err);
+  INSC_LAUNCH_CHECK();
+  g->n_upper = 0;
+  g->n_exact = 0;
+  return INSC_OK;
+}
+
+int insc_grid_reserve(insc_grid *g, int64_t capacity_sites, void *stream) {
+  INSC_REQUIRE(g, INSC_ERR_ARG, "insc_grid_reserve: grid is null");
+  INSC_REQUIRE(capacity_sites < (1ll << 30), INSC_ERR_ARG, "insc_grid_reserve: capacity out of range");
+  if (capacity_sites <= g->capacity_sites) return INSC_OK;
+  hipStream_t s = (hipStream_t)stream;
+  INSC_HIP(hipStreamSynchronize(s));
+  int32_t *coords = nullptr;
+  INSC_HIP(hipMalloc((void **)&coords, sizeof(int32_t) * 4 * (size_t)capacity_sites));
+  INSC_HIP(hipMemcpyAsync(coords, g->coords, sizeof(int32_t) * 4 * (size_t)g->capacity_sites,
+                          hipMemcpyDeviceToDevice, s));
+  INSC_HIP(hipStreamSynchronize(s));
+  INSC_HIP(hipFree(g->coords));
+  g->coords = coords;
+  g->capacity_sites = capacity_sites;
+  if (g->n_slots < 2 * capacity_sites) {
+    INSC_HIP(hipFree(g->table));
+    g->table = nullptr;
+    int rc = grid_alloc_table(g, capacity_sites);
+    if (rc) return rc;
+    // clear the new table but keep the counter
+    int32_t n_keep = 0;
+    INSC_HIP(hipMemcpy(&n_keep, g->d_n, sizeof(int32_t), hipMemcpyDeviceToHost));
+    hipLaunchKernelGGL(grid_clear_kernel, dim3(grid_for(g->n_slots, 256, 8192)), dim3(256), 0, s, g->table,
+                       g->n_slots, g->d_n, g->d_err);
+    INSC_HIP(hipMemcpyAsync(g->d_n, &n_keep, sizeof(int32_t), hipMemcpyHostToDevice, s));
+    INSC_HIP(hipStreamSynchronize(s));
+    if (n_keep > 0) {
+      hipLaunchKernelGGL(grid_rehash_kernel, dim3(grid_for(n_keep, 256)), dim3(256), 0, s, g->table,
+                         g->n_slots - 1, g->coords, g->d_n, g->d_err);
+      INSC_LAUNCH_CHECK();
+    }
+    return grid_sync_errors(g, s, "insc_grid_reserve");
+  }
+  return INSC_OK;
+}
+
+int insc_grid_insert(insc_grid *g, const int32_t *d_coords4, int64_t P, int32_t *d_site_of_point, int64_t *h_n_sites,
+                     void *stream) {
+  INSC_REQUIRE(g, INSC_ERR_ARG, "insc_grid_insert: grid is null");
+  INSC_REQUIRE(P >= 0 && P < VAL_PENDING - 1, INSC_ERR_ARG, "insc_grid_insert: P=%lld out of range", (long long)P);
+  INSC_REQUIRE(P == 0 || (d_coords4 && d_site_of_point), INSC_ERR_ARG, "insc_grid_insert: null pointer");
+  hipStream_t s = (hipStream_t)stream;
+  if (P > 0) {
+    if (g->n_upper + P > g->capacity_sites) {
+      // the bound may be loose (duplicates): refresh it before growing
+      int rc = grid_sync_errors(g, s, "insc_grid_insert");
+      if (rc) return rc;
+      if (g->n_upper + P > g->capacity_sites) {
+        int64_t want = g->capacity_sites * 2;
+        if (want < g->n_upper + P) want = g->n_upper + P;
+        rc = insc_grid_reserve(g, want, stream);
+        if (rc) return rc;
+      }
+    }
+    if (g->scratch_rows < P) {
+      INSC_HIP(hipStreamSynchronize(s));
+      if (g->slot_of_point) INSC_HIP(hipFree(g->slot_of_point));
+      if (g->flags) INSC_HIP(hipFree(g->flags));
+      g->slot_of_point = g->flags = nullptr;
+      int64_t rows = P + P / 2;
+      INSC_HIP(hipMalloc((void **)&g->slot_of_point, sizeof(int32_t) * (size_t)rows));
+      INSC_HIP(hipMalloc((void **)&g->flags, sizeof(int32_t) * (size_t)(rows + 64)));
+      g->scratch_rows = rows;
+    }
+    const int64_t mask = g->n_slots - 1;
+    const unsigned nb = grid_for(P, 256);
+    int32_t *total = g->flags + g->scratch_rows;  // spare int after the flags
+    hipLaunchKernelGGL(grid_claim_kernel, dim3(nb), dim3(256), 0, s, g->table, mask, d_coords4, P, g->slot_of_point,
+                       g->d_err);
+    hipLaunchKernelGGL(grid_flag_kernel, dim3(nb), dim3(256), 0, s, g->table, g->slot_of_point, P, g->flags);
+    INSC_LAUNCH_CHECK();
+    int rc = scan_exclusive_i32(g->flags, g->flags, P, total, s);
+    if (rc) return rc;
+    hipLaunchKernelGGL(grid_assign_kernel, dim3(nb), dim3(256), 0, s, g->table, d_coords4, g->slot_of_point, g->flags,
+                       P, g->d_n, g->coords, g->capacity_sites, g->d_err);
+    hipLaunchKernelGGL(grid_resolve_kernel, dim3(nb), dim3(256), 0, s, g->table, g->slot_of_point, P,
+                       d_site_of_point, g->d_n, total);
+    hipLaunchKernelGGL(grid_bump_kernel, dim3(1), dim3(1), 0, s, g->d_n, total);
+    INSC_LAUNCH_CHECK();
+    g->n_upper += P;
+    g->n_exact = -1;
+  }
+  if (h_n_sites) {
+    int rc = grid_sync_errors(g, s, "insc_grid_insert");
+    if (rc) return rc;
+    *h_n_sites = g->n_exact;
+  }
+  return INSC_OK;
+}
+
+int insc_grid_query(const insc_grid *g, const int32_t *d_coords4, int64_t Q, int32_t *d_site, void *stream) {
+  INSC_REQUIRE(g, INSC_ERR_ARG, "insc_grid_query: grid is null");
+  INSC_REQUIRE(Q >= 0 && (Q == 0 || (d_coords4 && d_site)), INSC_ERR_ARG, "insc_grid_query: bad arguments");
+  if (Q == 0) return INSC_OK;
+  hipLaunchKernelGGL(grid_query_kernel, dim3(grid_for(Q, 256)), dim3(256), 0, (hipStream_t)stream, g->table,
+                     g->n_slots - 1, d_coords4, Q, d_site);
+  INSC_LAUNCH_CHECK();
+  return INSC_OK;
+}
+
+int insc_grid_size(insc_grid *g, int64_t *h_n_sites, void *stream) {
+  INSC_REQUIRE(g && h_n_sites, INSC_ERR_ARG, "insc_grid_size: null argument");
+  if (g->n_exact < 0) {
+    int rc = grid_sync_errors(g, (hipStream_t)stream, "insc_grid_size");
+    if (rc) return rc;
+  }
+  *h_n_sites = g->n_exact;
+  return INSC_OK;
+}
+
+const int32_t *insc_grid_coords(const insc_grid *g) { return g ? g->coords : nullptr; }
+const int32_t *insc_grid_count_ptr(const insc_grid *g) { return g ? g->d_n : nullptr; }
+int64_t insc_grid_capacity(const insc_grid *g) { return g ? g->capacity_sites : 0; }
+
+int insc_rulebook_ssc3(const insc_grid *g, int64_t first, int64_t n, int32_t *d_nbr, int patch_reverse,
+                       void *stream) {
+  INSC_REQUIRE(g, INSC_ERR_ARG, "insc_rulebook_ssc3: grid is null");
+  INSC_REQUIRE(first >= 0 && n >= 0 && first + n <= g->capacity_sites, INSC_ERR_ARG,
+               "insc_rulebook_ssc3: rows [%lld,%lld) outside capacity %lld", (long long)first,
+               (long long)(first + n), (long long)g->capacity_sites);
+  INSC_REQUIRE(n == 0 || d_nbr, INSC_ERR_ARG, "insc_rulebook_ssc3: d_nbr is null");
+  if (n == 0) return INSC_OK;
+  hipLaunchKernelGGL(ssc3_nbr_kernel, dim3(grid_for(n * 27, 256, 1ll << 30)), dim3(256), 0, (hipStream_t)stream,
+                     g->table, g->n_slots - 1, g->coords, first, n, d_nbr, patch_reverse);
+  INSC_LAUNCH_CHECK();
+  return INSC_OK;
+}
+
+int insc_rulebook_down2(const insc_grid *fine, insc_grid *coarse, int64_t first, int64_t n, int32_t *d_parent,
+                        int32_t *d_offset, int32_t *d_child, int64_t child_rows, void *stream) {
+  INSC_REQUIRE(fine && coarse && fine != coarse, INSC_ERR_ARG, "insc_rulebook_down2: bad grids");
+  INSC_REQUIRE(first >= 0 && n >= 0 && first + n <= fine->capacity_sites, INSC_ERR_ARG,
+               "insc_rulebook_down2: rows outside capacity");
+  INSC_REQUIRE(n == 0 || (d_parent && d_offset), INSC_ERR_ARG, "insc_rulebook_down2: null pointer");
+  if (n == 0) return INSC_OK;
+  hipStream_t s = (hipStream_t)stream;
+  void *ws;
+  int rc = workspace(WS_API, s, sizeof(int32_t) * 4 * (size_t)n, &ws);
+  if (rc) return rc;
+  int32_t *half = (int32_t *)ws;
+  hipLaunchKernelGGL(down2_coords_kernel, dim3(grid_for(n, 256)), dim3(256), 0, s, fine->coords, first, n, half,
+                     d_offset);
+  INSC_LAUNCH_CHECK();
+  rc = insc_grid_insert(coarse, half, n, d_parent + first, nullptr, stream);
+  if (rc) return rc;
+  if (d_child) {
+    INSC_REQUIRE(child_rows >= coarse->capacity_sites, INSC_ERR_CAPACITY,
+                 "insc_rulebook_down2: child map has %lld rows, coarse grid capacity is %lld", (long long)child_rows,
+                 (long long)coarse->capacity_sites);
+    hipLaunchKernelGGL(down2_child_kernel, dim3(grid_for(n, 256)), dim3(256), 0, s, d_parent, d_offset, first, n,
+                       d_child);
+    INSC_LAUNCH_CHECK();
+  }
+  return INSC_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,303 @@
+// Row-wise streaming kernels: inference batch norm + leaky ReLU, add, column-slice copy,
+// input-layer accumulation / mean, output-layer gather.  All are HBM-bandwidth bound: one
+// thread owns a fixed group of four channels and walks rows, so loads and stores are
+// 16-byte wide and coalesced along a row.
+#include "common.h"
+
+namespace insc {
+
+__device__ __forceinline__ int64_t row_count(const int32_t *d_n_rows, int64_t n_rows) {
+  return d_n_rows ? min((int64_t)*d_n_rows, n_rows) : n_rows;
+}
+
+// V = 4: float4 path (C, strides multiples of 4, 16-byte aligned bases); V = 1: scalar path
+template <int V>
+struct Vec;
+template <>
+struct Vec<4> {
+  typedef float4 T;
+  static __device__ __forceinline__ T ld(const float *p) { return *reinterpret_cast<const float4 *>(p); }
+  static __device__ __forceinline__ void st(float *p, T v) { *reinterpret_cast<float4 *>(p) = v; }
+};
+template <>
+struct Vec<1> {
+  typedef float T;
+  static __device__ __forceinline__ T ld(const float *p) { return *p; }
+  static __device__ __forceinline__ void st(float *p, T v) { *p = v; }
+};
+
+__device__ __forceinline__ float leaky(float o, float leak) { return o * ((o > 0.0f) ? 1.0f : leak); }
+
+template <int V>
+__global__ __launch_bounds__(256) void bn_kernel(const float *__restrict__ in, int64_t ld_in, float *__restrict__ out,
+                                                 int64_t ld_out, const float *__restrict__ mean,
+                                                 const float *__restrict__ var, const float *__restrict__ gamma,
+                                                 const float *__restrict__ beta, float eps, float leak,
+                                                 const int32_t *__restrict__ rows,
+                                                 const int32_t *__restrict__ d_n_rows, int64_t n_rows, int C) {
+  const int64_t n = row_count(d_n_rows, n_rows);
+  const int groups = C / V;  // channel groups per row
+  const int rpb = 256 / groups > 0 ? 256 / groups : 1;
+  const int g = threadIdx.x % groups, lr = threadIdx.x / groups;
+  if (lr >= rpb || groups > 256) return;
+  float w[V], b[V];
+#pragma unroll
+  for (int i = 0; i < V; i++) {
+    const int c = g * V + i;
+    const float invstd = 1.0f / sqrtf(var[c] + eps);
+    w[i] = invstd * (gamma ? gamma[c] : 1.0f);
+    b[i] = -mean[c] * w[i] + (beta ? beta[c] : 0.0f);
+  }
+  for (int64_t t = (int64_t)blockIdx.x * rpb + lr; t < n; t += (int64_t)gridDim.x * rpb) {
+    const int row = rows ? rows[t] : (int)t;
+    if (row < 0) continue;
+    typename Vec<V>::T x = Vec<V>::ld(in + (int64_t)row * ld_in + g * V);
+    float *xf = reinterpret_cast<float *>(&x);
+#pragma unroll
+    for (int i = 0; i < V; i++) xf[i] = leaky(xf[i] * w[i] + b[i], leak);
+    Vec<V>::st(out + (int64_t)row * ld_out + g * V, x);
+  }
+}
+
+// wide rows (more than 256 channel groups): one thread per element, any C
+__global__ __launch_bounds__(256) void bn_wide_kernel(const float *__restrict__ in, int64_t ld_in,
+                                                      float *__restrict__ out, int64_t ld_out,
+                                                      const float *__restrict__ mean, const float *__restrict__ var,
+                                                      const float *__restrict__ gamma, const float *__restrict__ beta,
+                                                      float eps, float leak, const int32_t *__restrict__ rows,
+                                                      const int32_t *__restrict__ d_n_rows, int64_t n_rows, int C) {
+  const int64_t n = row_count(d_n_rows, n_rows);
+  for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < n * C; e += (int64_t)gridDim.x * 256) {
+    const int64_t t = e / C;
+    const int c = (int)(e - t * C);
+    const int row = rows ? rows[t] : (int)t;
+    if (row < 0) continue;
+    const float wv = (gamma ? gamma[c] : 1.0f) / sqrtf(var[c] + eps);
+    const float bv = -mean[c] * wv + (beta ? beta[c] : 0.0f);
+    out[(int64_t)row * ld_out + c] = leaky(in[(int64_t)row * ld_in + c] * wv + bv, leak);
+  }
+}
+
+// out = a + b (HAS_B) or out = a, on listed rows
+template <int V, bool HAS_B>
+__global__ __launch_bounds__(256) void add_kernel(const float *__restrict__ a, int64_t ld_a,
+                                                  const float *__restrict__ b, int64_t ld_b, float *__restrict__ out,
+                                                  int64_t ld_out, const int32_t *__restrict__ rows,
+                                                  const int32_t *__restrict__ d_n_rows, int64_t n_rows, int C) {
+  const int64_t n = row_count(d_n_rows, n_rows);
+  const int groups = C / V;
+  for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < n * groups; e += (int64_t)gridDim.x * 256) {
+    const int64_t t = e / groups;
+    const int g = (int)(e - t * groups);
+    const int row = rows ? rows[t] : (int)t;
+    if (row < 0) continue;
+    typename Vec<V>::T x = Vec<V>::ld(a + (int64_t)row * ld_a + g * V);
+    if (HAS_B) {
+      typename Vec<V>::T y = Vec<V>::ld(b + (int64_t)row * ld_b + g * V);
+      float *xf = reinterpret_cast<float *>(&x);
+      const float *yf = reinterpret_cast<const float *>(&y);
+#pragma unroll
+      for (int i = 0; i < V; i++) xf[i] += yf[i];
+    }
+    Vec<V>::st(out + (int64_t)row * ld_out + g * V, x);
+  }
+}
+
+__global__ __launch_bounds__(256) void gather_rows_kernel(const float *__restrict__ in, int64_t ld_in,
+                                                          const int32_t *__restrict__ src, int64_t P, int C,
+                                                          float *__restrict__ out) {
+  for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < P * C; e += (int64_t)gridDim.x * 256) {
+    const int64_t p = e / C;
+    const int c = (int)(e - p * C);
+    const int s = src[p];
+    out[e] = (s >= 0) ? in[(int64_t)s * ld_in + c] : 0.0f;
+  }
+}
+
+// ---- input layer -----------------------------------------------------------------------
+__global__ void input_key_kernel(const int32_t *__restrict__ site_of_point, int64_t P, uint64_t *__restrict__ keys,
+                                 int32_t *__restrict__ vals) {
+  int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (p >= P) return;
+  keys[p] = (uint64_t)(uint32_t)site_of_point[p];  // -1 sorts last
+  vals[p] = (int)p;
+}
+
+// keys/vals sorted by site (stable: rows of one site ascending).  One thread per (sorted
+// position, channel); the thread at the head of a site's run sums the run in order.
+__global__ __launch_bounds__(256) void input_sum_kernel(const float *__restrict__ feats, int C,
+                                                        const uint64_t *__restrict__ keys,
+                                                        const int32_t *__restrict__ vals, int64_t P, int mode,
+                                                        float *__restrict__ sum, const int32_t *__restrict__ cnt) {
+  for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < P * C; e += (int64_t)gridDim.x * 256) {
+    const int64_t j = e / C;
+    const int c = (int)(e - j * C);
+    const uint64_t key = keys[j];
+    if (key == 0xFFFFFFFFull) continue;
+    if (j > 0 && keys[j - 1] == key) continue;  // not a head
+    const int64_t site = (int64_t)key;
+    float acc = sum[site * C + c];
+    const bool had = cnt[site] > 0;
+    if (mode == 1) {
+      if (!had) acc = feats[(int64_t)vals[j] * C + c];
+    } else if (mode == 2) {
+      int64_t q = j;
+      while (q + 1 < P && keys[q + 1] == key) q++;
+      acc = feats[(int64_t)vals[q] * C + c];
+    } else {
+      for (int64_t q = j; q < P && keys[q] == key; q++) acc += feats[(int64_t)vals[q] * C + c];
+    }
+    sum[site * C + c] = acc;
+  }
+}
+
+__global__ __launch_bounds__(256) void input_count_kernel(const uint64_t *__restrict__ keys, int64_t P,
+                                                          int32_t *__restrict__ cnt) {
+  int64_t j = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (j >= P) return;
+  const uint64_t key = keys[j];
+  if (key == 0xFFFFFFFFull) return;
+  if (j > 0 && keys[j - 1] == key) return;
+  int64_t q = j;
+  while (q + 1 < P && keys[q + 1] == key) q++;
+  cnt[(int64_t)key] += (int)(q - j + 1);
+}
+
+__global__ __launch_bounds__(256) void input_finish_kernel(const float *__restrict__ sum,
+                                                           const int32_t *__restrict__ cnt, int mode,
+                                                           float *__restrict__ out, int64_t ld_out,
+                                                           const int32_t *__restrict__ rows,
+                                                           const int32_t *__restrict__ d_n_rows, int64_t n_rows,
+                                                           int C) {
+  const int64_t n = row_count(d_n_rows, n_rows);
+  for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < n * C; e += (int64_t)gridDim.x * 256) {
+    const int64_t t = e / C;
+    const int c = (int)(e - t * C);
+    const int row = rows ? rows[t] : (int)t;
+    if (row < 0) continue;
+    float v = sum[(int64_t)row * C + c];
+    if (mode == 4) {
+      const int k = cnt[row];
+      if (k > 1) v = v / (float)k;
+    }
+    out[(int64_t)row * ld_out + c] = v;
+  }
+}
+
+static inline bool vec4_ok(const void *p, int64_t ld) { return ((uintptr_t)p % 16 == 0) && (ld % 4 == 0); }
+
+}  // namespace insc
+
+using namespace insc;
+
+extern "C" {
+
+int insc_bn_leaky(const float *d_in, int64_t ld_in, float *d_out, int64_t ld_out, const float *d_mean,
+                  const float *d_var, const float *d_gamma, const float *d_beta, float eps, float leakiness,
+                  const int32_t *d_rows, const int32_t *d_n_rows, int64_t n_rows, int C, void *stream) {
+  INSC_REQUIRE(n_rows >= 0 && C > 0 && ld_in >= C && ld_out >= C, INSC_ERR_ARG, "insc_bn_leaky: bad sizes");
+  INSC_REQUIRE(n_rows == 0 || (d_in && d_out && d_mean && d_var), INSC_ERR_ARG, "insc_bn_leaky: null pointer");
+  if (n_rows == 0) return INSC_OK;
+  hipStream_t s = (hipStream_t)stream;
+  const bool v4 = C % 4 == 0 && vec4_ok(d_in, ld_in) && vec4_ok(d_out, ld_out);
+  const int groups = v4 ? C / 4 : C;
+  if (groups <= 256) {
+    const int rpb = 256 / groups;
+    const unsigned nb = grid_for(n_rows, rpb * 4, 1 << 16);
+    if (v4)
+      hipLaunchKernelGGL(bn_kernel<4>, dim3(nb), dim3(256), 0, s, d_in, ld_in, d_out, ld_out, d_mean, d_var, d_gamma,
+                         d_beta, eps, leakiness, d_rows, d_n_rows, n_rows, C);
+    else
+      hipLaunchKernelGGL(bn_kernel<1>, dim3(nb), dim3(256), 0, s, d_in, ld_in, d_out, ld_out, d_mean, d_var, d_gamma,
+                         d_beta, eps, leakiness, d_rows, d_n_rows, n_rows, C);
+  } else {
+    hipLaunchKernelGGL(bn_wide_kernel, dim3(grid_for(n_rows * C, 1024, 1 << 16)), dim3(256), 0, s, d_in, ld_in, d_out,
+                       ld_out, d_mean, d_var, d_gamma, d_beta, eps, leakiness, d_rows, d_n_rows, n_rows, C);
+  }
+  INSC_LAUNCH_CHECK();
+  return INSC_OK;
+}
+
+int insc_add(const float *d_a, int64_t ld_a, const float *d_b, int64_t ld_b, float *d_out, int64_t ld_out,
+             const int32_t *d_rows, const int32_t *d_n_rows, int64_t n_rows, int C, void *stream) {
+  INSC_REQUIRE(n_rows >= 0 && C > 0 && ld_a >= C && ld_b >= C && ld_out >= C, INSC_ERR_ARG, "insc_add: bad sizes");
+  INSC_REQUIRE(n_rows == 0 || (d_a && d_b && d_out), INSC_ERR_ARG, "insc_add: null pointer");
+  if (n_rows == 0) return INSC_OK;
+  hipStream_t s = (hipStream_t)stream;
+  const bool v4 = C % 4 == 0 && vec4_ok(d_a, ld_a) && vec4_ok(d_b, ld_b) && vec4_ok(d_out, ld_out);
+  const unsigned nb = grid_for(n_rows * (v4 ? C / 4 : C), 1024, 1 << 16);
+  if (v4)
+    hipLaunchKernelGGL((add_kernel<4, true>), dim3(nb), dim3(256), 0, s, d_a, ld_a, d_b, ld_b, d_out, ld_out, d_rows,
+                       d_n_rows, n_rows, C);
+  else
+    hipLaunchKernelGGL((add_kernel<1, true>), dim3(nb), dim3(256), 0, s, d_a, ld_a, d_b, ld_b, d_out, ld_out, d_rows,
+                       d_n_rows, n_rows, C);
+  INSC_LAUNCH_CHECK();
+  return INSC_OK;
+}
+
+int insc_copy_rows(const float *d_in, int64_t ld_in, float *d_out, int64_t ld_out, const int32_t *d_rows,
+                   const int32_t *d_n_rows, int64_t n_rows, int C, void *stream) {
+  INSC_REQUIRE(n_rows >= 0 && C > 0 && ld_in >= C && ld_out >= C, INSC_ERR_ARG, "insc_copy_rows: bad sizes");
+  INSC_REQUIRE(n_rows == 0 || (d_in && d_out), INSC_ERR_ARG, "insc_copy_rows: null pointer");
+  if (n_rows == 0) return INSC_OK;
+  hipStream_t s = (hipStream_t)stream;
+  const bool v4 = C % 4 == 0 && vec4_ok(d_in, ld_in) && vec4_ok(d_out, ld_out);
+  const unsigned nb = grid_for(n_rows * (v4 ? C / 4 : C), 1024, 1 << 16);
+  if (v4)
+    hipLaunchKernelGGL((add_kernel<4, false>), dim3(nb), dim3(256), 0, s, d_in, ld_in, nullptr, 0, d_out, ld_out,
+                       d_rows, d_n_rows, n_rows, C);
+  else
+    hipLaunchKernelGGL((add_kernel<1, false>), dim3(nb), dim3(256), 0, s, d_in, ld_in, nullptr, 0, d_out, ld_out,
+                       d_rows, d_n_rows, n_rows, C);
+  INSC_LAUNCH_CHECK();
+  return INSC_OK;
+}
+
+int insc_input_accumulate(const float *d_feats, int64_t P, int C, const int32_t *d_site_of_point, int mode,
+                          float *d_sum, int32_t *d_cnt, int64_t n_sites_upper, void *stream) {
+  INSC_REQUIRE(P >= 0 && C > 0 && mode >= 0 && mode <= 4 && n_sites_upper >= 0, INSC_ERR_ARG,
+               "insc_input_accumulate: bad arguments");
+  INSC_REQUIRE(P == 0 || (d_feats && d_site_of_point && d_sum && d_cnt), INSC_ERR_ARG,
+               "insc_input_accumulate: null pointer");
+  if (P == 0) return INSC_OK;
+  hipStream_t s = (hipStream_t)stream;
+  void *ws;
+  int rc = workspace(WS_API, s, (sizeof(uint64_t) + sizeof(int32_t)) * (size_t)P + 256, &ws);
+  if (rc) return rc;
+  uint64_t *keys = (uint64_t *)ws;
+  int32_t *vals = (int32_t *)(keys + P);
+  hipLaunchKernelGGL(input_key_kernel, dim3(grid_for(P, 256)), dim3(256), 0, s, d_site_of_point, P, keys, vals);
+  INSC_LAUNCH_CHECK();
+  rc = sort_pairs_u64(keys, vals, P, 32, s);  // invalid rows carry 0xFFFFFFFF and must sort last
+  if (rc) return rc;
+  hipLaunchKernelGGL(input_sum_kernel, dim3(grid_for(P * C, 256, 1 << 16)), dim3(256), 0, s, d_feats, C, keys, vals,
+                     P, mode, d_sum, d_cnt);
+  hipLaunchKernelGGL(input_count_kernel, dim3(grid_for(P, 256)), dim3(256), 0, s, keys, P, d_cnt);
+  INSC_LAUNCH_CHECK();
+  return INSC_OK;
+}
+
+int insc_input_finish(const float *d_sum, const int32_t *d_cnt, int mode, float *d_out, int64_t ld_out,
+                      const int32_t *d_rows, const int32_t *d_n_rows, int64_t n_rows, int C, void *stream) {
+  INSC_REQUIRE(n_rows >= 0 && C > 0 && ld_out >= C, INSC_ERR_ARG, "insc_input_finish: bad sizes");
+  INSC_REQUIRE(n_rows == 0 || (d_sum && d_cnt && d_out), INSC_ERR_ARG, "insc_input_finish: null pointer");
+  if (n_rows == 0) return INSC_OK;
+  hipLaunchKernelGGL(input_finish_kernel, dim3(grid_for(n_rows * C, 256, 1 << 16)), dim3(256), 0, (hipStream_t)stream,
+                     d_sum, d_cnt, mode, d_out, ld_out, d_rows, d_n_rows, n_rows, C);
+  INSC_LAUNCH_CHECK();
+  return INSC_OK;
+}
+
+int insc_output_gather(const float *d_in, int64_t ld_in, const int32_t *d_site_of_point, int64_t P, int C,
+                       float *d_out, void *stream) {
+  INSC_REQUIRE(P >= 0 && C > 0 && ld_in >= C, INSC_ERR_ARG, "insc_output_gather: bad sizes");
+  INSC_REQUIRE(P == 0 || (d_in && d_site_of_point && d_out), INSC_ERR_ARG, "insc_output_gather: null pointer");
+  if (P == 0) return INSC_OK;
+  hipLaunchKernelGGL(gather_rows_kernel, dim3(grid_for(P * C, 256, 1 << 16)), dim3(256), 0, (hipStream_t)stream, d_in,
+                     ld_in, d_site_of_point, P, C, d_out);
+  INSC_LAUNCH_CHECK();
+  return INSC_OK;
+}
+
+}  // extern "C"

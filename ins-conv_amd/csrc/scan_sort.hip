@@ -1,0 +1,230 @@
+// Device-wide exclusive scan and stable LSD radix sort.  These replace the CUDPP scan /
+// compact / radix-sort calls the reference leans on (CUDA/CUDPPWrapper.hpp:30-217).
+#include "common.h"
+
+namespace insc {
+
+constexpr int SCAN_THREADS = 256;
+constexpr int SCAN_ITEMS = 8;
+constexpr int SCAN_TILE = SCAN_THREADS * SCAN_ITEMS;
+
+__device__ __forceinline__ int wave_incl_scan(int v) {
+  const int lane = threadIdx.x & 63;
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    int t = __shfl_up(v, d, 64);
+    if (lane >= d) v += t;
+  }
+  return v;
+}
+
+// exclusive scan of one value per thread across a 256-thread block; returns block total
+__device__ __forceinline__ int block_excl_scan(int v, int *total, int *lds /*[4]*/) {
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  int inc = wave_incl_scan(v);
+  if (lane == 63) lds[w] = inc;
+  __syncthreads();
+  int off = 0, tot = 0;
+#pragma unroll
+  for (int i = 0; i < SCAN_THREADS / 64; i++) {
+    int s = lds[i];
+    if (i < w) off += s;
+    tot += s;
+  }
+  __syncthreads();
+  *total = tot;
+  return off + inc - v;
+}
+
+__global__ __launch_bounds__(SCAN_THREADS) void scan_block_sums(const int32_t *__restrict__ in, int64_t n,
+                                                                int32_t *__restrict__ bsums) {
+  __shared__ int lds[4];
+  int64_t base = (int64_t)blockIdx.x * SCAN_TILE + (int64_t)threadIdx.x * SCAN_ITEMS;
+  int s = 0;
+#pragma unroll
+  for (int i = 0; i < SCAN_ITEMS; i++)
+    if (base + i < n) s += in[base + i];
+  int tot;
+  block_excl_scan(s, &tot, lds);
+  if (threadIdx.x == 0) bsums[blockIdx.x] = tot;
+}
+
+// single block: exclusive scan of bsums[0..nb) in place, total to *total (if non-null)
+__global__ __launch_bounds__(SCAN_THREADS) void scan_bsums(int32_t *__restrict__ bsums, int64_t nb,
+                                                           int32_t *__restrict__ total) {
+  __shared__ int lds[4];
+  int carry = 0;
+  for (int64_t base = 0; base < nb; base += SCAN_THREADS) {
+    int64_t i = base + threadIdx.x;
+    int v = (i < nb) ? bsums[i] : 0;
+    int tot;
+    int ex = block_excl_scan(v, &tot, lds);
+    if (i < nb) bsums[i] = carry + ex;
+    carry += tot;
+  }
+  if (threadIdx.x == 0 && total) *total = carry;
+}
+
+__global__ __launch_bounds__(SCAN_THREADS) void scan_final(const int32_t *__restrict__ in, int32_t *__restrict__ out,
+                                                           int64_t n, const int32_t *__restrict__ bsums) {
+  __shared__ int lds[4];
+  int64_t base = (int64_t)blockIdx.x * SCAN_TILE + (int64_t)threadIdx.x * SCAN_ITEMS;
+  int v[SCAN_ITEMS];
+  int s = 0;
+#pragma unroll
+  for (int i = 0; i < SCAN_ITEMS; i++) {
+    v[i] = (base + i < n) ? in[base + i] : 0;
+    s += v[i];
+  }
+  int tot;
+  int ex = block_excl_scan(s, &tot, lds) + bsums[blockIdx.x];
+#pragma unroll
+  for (int i = 0; i < SCAN_ITEMS; i++) {
+    if (base + i < n) out[base + i] = ex;
+    ex += v[i];
+  }
+}
+
+__global__ void scan_zero_total(int32_t *total) { *total = 0; }
+
+int scan_exclusive_i32(const int32_t *in, int32_t *out, int64_t n, int32_t *total, hipStream_t s) {
+  if (n <= 0) {
+    if (total) {
+      hipLaunchKernelGGL(scan_zero_total, dim3(1), dim3(1), 0, s, total);
+      INSC_LAUNCH_CHECK();
+    }
+    return INSC_OK;
+  }
+  int64_t nb = cdiv(n, SCAN_TILE);
+  void *ws;
+  int rc = workspace(WS_SCAN, s, sizeof(int32_t) * (size_t)nb, &ws);
+  if (rc) return rc;
+  int32_t *bsums = (int32_t *)ws;
+  hipLaunchKernelGGL(scan_block_sums, dim3((unsigned)nb), dim3(SCAN_THREADS), 0, s, in, n, bsums);
+  hipLaunchKernelGGL(scan_bsums, dim3(1), dim3(SCAN_THREADS), 0, s, bsums, nb, total);
+  hipLaunchKernelGGL(scan_final, dim3((unsigned)nb), dim3(SCAN_THREADS), 0, s, in, out, n, bsums);
+  INSC_LAUNCH_CHECK();
+  return INSC_OK;
+}
+
+// ---------------------------------------------------------------------------------------
+// radix sort: 8 bits per pass, 256 threads x 8 rounds per block, stable
+// ---------------------------------------------------------------------------------------
+constexpr int SORT_THREADS = 256;
+constexpr int SORT_ROUNDS = 8;
+constexpr int SORT_TILE = SORT_THREADS * SORT_ROUNDS;
+
+__global__ __launch_bounds__(SORT_THREADS) void sort_hist(const uint64_t *__restrict__ keys, int64_t n, int shift,
+                                                          int32_t *__restrict__ counts, int nb) {
+  __shared__ int h[256];
+  h[threadIdx.x] = 0;
+  __syncthreads();
+  int64_t base = (int64_t)blockIdx.x * SORT_TILE;
+#pragma unroll
+  for (int r = 0; r < SORT_ROUNDS; r++) {
+    int64_t i = base + r * SORT_THREADS + threadIdx.x;
+    if (i < n) atomicAdd(&h[(int)((keys[i] >> shift) & 255)], 1);
+  }
+  __syncthreads();
+  counts[(int64_t)threadIdx.x * nb + blockIdx.x] = h[threadIdx.x];
+}
+
+__global__ __launch_bounds__(SORT_THREADS) void sort_scatter(const uint64_t *__restrict__ keys_in,
+                                                             const int32_t *__restrict__ vals_in,
+                                                             uint64_t *__restrict__ keys_out,
+                                                             int32_t *__restrict__ vals_out, int64_t n, int shift,
+                                                             const int32_t *__restrict__ offsets, int nb) {
+  __shared__ int base[256];
+  __shared__ int wcount[SORT_THREADS / 64][256];
+  const int t = threadIdx.x, lane = t & 63, w = t >> 6;
+  base[t] = offsets[(int64_t)t * nb + blockIdx.x];
+  const int64_t tile = (int64_t)blockIdx.x * SORT_TILE;
+  for (int r = 0; r < SORT_ROUNDS; r++) {
+#pragma unroll
+    for (int i = 0; i < SORT_THREADS / 64; i++) wcount[i][t] = 0;
+    __syncthreads();
+    int64_t i = tile + r * SORT_THREADS + t;
+    bool valid = i < n;
+    uint64_t key = valid ? keys_in[i] : 0;
+    int val = valid ? vals_in[i] : 0;
+    int digit = (int)((key >> shift) & 255);
+    // lanes of this wave holding the same digit
+    uint64_t peers = __ballot(valid);
+#pragma unroll
+    for (int b = 0; b < 8; b++) {
+      uint64_t m = __ballot((digit >> b) & 1);
+      peers &= ((digit >> b) & 1) ? m : ~m;
+    }
+    int rank_in_wave = __popcll(peers & ((1ull << lane) - 1ull));
+    if (valid && rank_in_wave == 0) wcount[w][digit] = __popcll(peers);
+    __syncthreads();
+    if (valid) {
+      int rank = base[digit] + rank_in_wave;
+      for (int i2 = 0; i2 < w; i2++) rank += wcount[i2][digit];
+      keys_out[rank] = key;
+      vals_out[rank] = val;
+    }
+    __syncthreads();
+    int add = 0;
+#pragma unroll
+    for (int i2 = 0; i2 < SORT_THREADS / 64; i2++) add += wcount[i2][t];
+    base[t] += add;
+    __syncthreads();
+  }
+}
+
+int sort_pairs_u64(uint64_t *keys, int32_t *vals, int64_t n, int key_bits, hipStream_t s) {
+  if (n <= 1 || key_bits <= 0) return INSC_OK;
+  if (key_bits > 64) key_bits = 64;
+  const int passes = (key_bits + 7) / 8;
+  const int64_t nb64 = cdiv(n, SORT_TILE);
+  if (nb64 > (1 << 22)) {
+    set_error("sort_pairs_u64: n=%lld too large", (long long)n);
+    return INSC_ERR_ARG;
+  }
+  const int nb = (int)nb64;
+  size_t off_keys = 0;
+  size_t off_vals = off_keys + sizeof(uint64_t) * (size_t)n;
+  size_t off_cnt = (off_vals + sizeof(int32_t) * (size_t)n + 255) & ~(size_t)255;
+  size_t bytes = off_cnt + sizeof(int32_t) * 256 * (size_t)nb;
+  void *ws;
+  int rc = workspace(WS_SORT, s, bytes, &ws);
+  if (rc) return rc;
+  uint64_t *k2 = (uint64_t *)((char *)ws + off_keys);
+  int32_t *v2 = (int32_t *)((char *)ws + off_vals);
+  int32_t *counts = (int32_t *)((char *)ws + off_cnt);
+  uint64_t *kin = keys, *kout = k2;
+  int32_t *vin = vals, *vout = v2;
+  for (int p = 0; p < passes; p++) {
+    int shift = 8 * p;
+    hipLaunchKernelGGL(sort_hist, dim3(nb), dim3(SORT_THREADS), 0, s, kin, n, shift, counts, nb);
+    rc = scan_exclusive_i32(counts, counts, 256 * (int64_t)nb, nullptr, s);
+    if (rc) return rc;
+    hipLaunchKernelGGL(sort_scatter, dim3(nb), dim3(SORT_THREADS), 0, s, kin, vin, kout, vout, n, shift, counts, nb);
+    INSC_LAUNCH_CHECK();
+    uint64_t *tk = kin; kin = kout; kout = tk;
+    int32_t *tv = vin; vin = vout; vout = tv;
+  }
+  if (kin != keys) {
+    INSC_HIP(hipMemcpyAsync(keys, kin, sizeof(uint64_t) * (size_t)n, hipMemcpyDeviceToDevice, s));
+    INSC_HIP(hipMemcpyAsync(vals, vin, sizeof(int32_t) * (size_t)n, hipMemcpyDeviceToDevice, s));
+  }
+  return INSC_OK;
+}
+
+}  // namespace insc
+
+extern "C" {
+
+int insc_scan_exclusive_i32(const int32_t *d_in, int32_t *d_out, int64_t n, int32_t *d_total, void *stream) {
+  INSC_REQUIRE(n >= 0 && ((d_in && d_out) || n == 0), INSC_ERR_ARG, "insc_scan_exclusive_i32: bad arguments");
+  return insc::scan_exclusive_i32(d_in, d_out, n, d_total, (hipStream_t)stream);
+}
+
+int insc_sort_pairs_u64(uint64_t *d_keys, int32_t *d_vals, int64_t n, int key_bits, void *stream) {
+  INSC_REQUIRE(n >= 0 && ((d_keys && d_vals) || n == 0), INSC_ERR_ARG, "insc_sort_pairs_u64: bad arguments");
+  INSC_REQUIRE(key_bits >= 0 && key_bits <= 64, INSC_ERR_ARG, "insc_sort_pairs_u64: key_bits %d", key_bits);
+  return insc::sort_pairs_u64(d_keys, d_vals, n, key_bits, (hipStream_t)stream);
+}
+
+}  // extern "C"

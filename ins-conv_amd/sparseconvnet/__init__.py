@@ -1,0 +1,22 @@
+"""MI355X-native drop-in for the inference path of the `sparseconvnet` package.
+
+Module classes keep the reference's names, constructor arguments and
+`forward(input, increment=False)` signature (sparseconvnet/__init__.py of the reference);
+everything below them runs in hand-written HIP kernels behind a C ABI.
+"""
+forward_pass_multiplyAdd_count = 0
+forward_pass_hidden_states = 0
+
+from .sparseConvNetTensor import SparseConvNetTensor  # noqa: E402
+from .metadata import Metadata  # noqa: E402
+from .sequential import Sequential  # noqa: E402
+from .tables import JoinTable, AddTable, ConcatTable  # noqa: E402
+from .identity import Identity  # noqa: E402
+from .ioLayers import InputLayer, OutputLayer  # noqa: E402
+from .submanifoldConvolution import SubmanifoldConvolution, ValidConvolution  # noqa: E402
+from .convolution import Convolution  # noqa: E402
+from .deconvolution import Deconvolution  # noqa: E402
+from .batchNormalization import BatchNormalization, BatchNormReLU, BatchNormLeakyReLU  # noqa: E402
+from .networkInNetwork import NetworkInNetwork  # noqa: E402
+from .networkArchitectures import UNet  # noqa: E402
+from .utils import toLongTensor, optionalTensor  # noqa: E402

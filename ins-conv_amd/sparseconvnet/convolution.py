@@ -1,0 +1,61 @@
+"""Strided Convolution (reference: sparseconvnet/convolution.py:13-80); size 2 / stride 2 only."""
+import torch
+from torch.nn import Module, Parameter
+
+import sparseconvnet
+
+from . import SCN, incremental
+from .sparseConvNetTensor import SparseConvNetTensor
+from .utils import StateBuf, optionalTensor, toLongTensor
+
+
+class Convolution(Module):
+    def __init__(self, dimension, nIn, nOut, filter_size, filter_stride, bias):
+        Module.__init__(self)
+        self.dimension = dimension
+        self.nIn = nIn
+        self.nOut = nOut
+        self.filter_size = toLongTensor(dimension, filter_size)
+        self.filter_volume = self.filter_size.prod().item()
+        self.filter_stride = toLongTensor(dimension, filter_stride)
+        std = (2.0 / nIn / self.filter_volume) ** 0.5
+        self.weight = Parameter(torch.Tensor(self.filter_volume, nIn, nOut).normal_(0, std))
+        if bias:
+            self.bias = Parameter(torch.Tensor(nOut).zero_())
+        self._state = StateBuf()
+
+    def forward(self, input, increment=False):
+        assert input.features.nelement() == 0 or input.features.size(1) == self.nIn
+        output = SparseConvNetTensor(None, input.metadata, None)
+        # the reference divides LongTensors with `/` (integer division on torch 1.1)
+        output.spatial_size = (input.spatial_size - self.filter_size) // self.filter_stride + 1
+        assert ((output.spatial_size - 1) * self.filter_stride + self.filter_size == input.spatial_size).all(), (
+            input.spatial_size, output.spatial_size, self.filter_size, self.filter_stride)
+        if not increment:
+            out = input.features.new_empty((0, self.nOut))
+            sparseconvnet.forward_pass_multiplyAdd_count += SCN.Convolution_updateOutput(
+                input.spatial_size, output.spatial_size, self.filter_size, self.filter_stride, input.metadata,
+                input.features, out, self.weight, optionalTensor(self, 'bias'))
+            sparseconvnet.forward_pass_hidden_states += out.nelement()
+            output.features = self._state.adopt(out)
+        else:
+            SCN._check_down(self.filter_size, self.filter_stride)
+            m = input.metadata
+            fine, coarse, down = m.down_rulebook(input.spatial_size, output.spatial_size)
+            m.ssc_rulebook(output.spatial_size)
+            d = incremental.parents(input.dirty, coarse, down)
+            out = self._state.grow(coarse.n, keep=min(coarse.n, self._state.buf.size(0)))
+            rows, count = d.rows(coarse.order.t)
+            SCN.conv_rows(input.features, out, self.weight.detach(), SCN._opt(optionalTensor(self, 'bias')),
+                          down.child.t, 8, rows, count, d.n_upper)
+            output.features = out
+            output.dirty = d
+        return output
+
+    def __repr__(self):
+        s = 'Convolution ' + str(self.nIn) + '->' + str(self.nOut) + ' C'
+        s += str(self.filter_size[0].item()) + '/' + str(self.filter_stride[0].item())
+        return s
+
+    def input_spatial_size(self, out_size):
+        return (out_size - 1) * self.filter_stride + self.filter_size

@@ -1,0 +1,180 @@
+"""GPU parity of the feature kernels against the CPU oracle, called through the reference's
+op names (sparseconvnet.SCN.*_updateOutput).  Tolerance: 1e-4 relative / 1e-5 absolute, the
+bound the north star states for float32 outputs."""
+import numpy as np
+import pytest
+import torch
+
+import scenes
+
+pytestmark = pytest.mark.gpu
+RTOL, ATOL = 1e-4, 1e-5
+SZ = torch.LongTensor([4096, 4096, 4096])
+
+
+@pytest.fixture(scope="module")
+def S():
+    from sparseconvnet import SCN
+    from sparseconvnet._lib import ensure_init
+
+    ensure_init(0)
+    return SCN
+
+
+def cu(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def setup_sites(S, pts, C, seed=0, mode=4):
+    rng = np.random.default_rng(seed)
+    f = rng.normal(size=(len(pts), C)).astype(np.float32)
+    m = S.Metadata_3()
+    out = torch.empty(0, device="cuda")
+    S.InputLayer_updateOutput(m, SZ, torch.from_numpy(pts.astype(np.int64)), cu(f), out, 0, mode)
+    return m, f, out
+
+
+@pytest.mark.parametrize("mode", [0, 1, 2, 3, 4])
+def test_input_output_layers(S, orc, mode):
+    rng = np.random.default_rng(1)
+    if mode == 0:
+        pts = scenes.boxes_scene(seed=4, n=5000)
+    else:
+        pts = np.concatenate([rng.integers(50, 62, (8000, 3)), np.zeros((8000, 1), np.int64)], 1).astype(np.int32)
+    m, f, out = setup_sites(S, pts, 3, seed=2, mode=mode)
+    sop, sc, cnt = orc.grid_build(pts)
+    if mode in (0, 3, 4):
+        ref = orc.input_forward(f, sop, cnt, mode=mode)
+    else:  # keep first (1) / last (2) row of each site, per Metadata/IOLayersRules.h:104-115
+        idx = np.zeros(len(sc), np.int64)
+        if mode == 1:
+            idx[sop[::-1]] = np.arange(len(pts))[::-1]
+        else:
+            idx[sop] = np.arange(len(pts))
+        ref = f[idx]
+    assert out.shape == ref.shape
+    np.testing.assert_allclose(out.cpu().numpy(), ref, rtol=RTOL, atol=ATOL)
+    o = torch.empty(0, device="cuda")
+    S.OutputLayer_updateOutput(m, out, o)
+    assert (o.cpu().numpy() == out.cpu().numpy()[sop]).all()
+    assert (o.cpu().numpy() == orc.output_forward(out.cpu().numpy(), sop)).all()
+
+
+@pytest.mark.parametrize("Cin,Cout,bias", [(16, 16, False), (32, 32, True), (64, 64, False), (3, 32, False),
+                                            (64, 32, True), (96, 96, False), (32, 20, True), (48, 224, False),
+                                            (384, 192, False), (5, 7, True), (32, 288, False)])
+def test_submanifold_convolution(S, orc, Cin, Cout, bias):
+    pts = scenes.boxes_scene(seed=1, n=20000 if Cin * Cout <= 4096 else 6000)
+    m, x, feats = setup_sites(S, pts, Cin, seed=Cin)
+    rng = np.random.default_rng(Cout)
+    W = (rng.normal(size=(27, Cin, Cout)) * (2.0 / Cin / 27) ** 0.5).astype(np.float32)
+    b = rng.normal(size=Cout).astype(np.float32) if bias else None
+    out = torch.empty(0, device="cuda")
+    flops = S.SubmanifoldConvolution_updateOutput(SZ, torch.LongTensor([3, 3, 3]), m, feats, out, cu(W),
+                                                  cu(b) if bias else torch.Tensor(), 1)
+    _, sc, _ = orc.grid_build(pts)
+    _, counts, pairs = orc.ssc_rules(sc)
+    ref, rflops = orc.conv_forward(feats.cpu().numpy(), W, b, pairs, counts, len(sc))
+    assert flops == rflops
+    np.testing.assert_allclose(out.cpu().numpy(), ref, rtol=RTOL, atol=ATOL)
+
+
+def test_submanifold_convolution_cfg1_vs_dense_conv3d(S):
+    """Workload 1 against the library routine directly (no oracle in the loop)."""
+    import torch.nn.functional as F
+
+    pts = scenes.boxes_scene(seed=1, n=20000)
+    m, x, feats = setup_sites(S, pts, 16, seed=1)
+    W = torch.randn(27, 16, 16, generator=torch.Generator().manual_seed(1)) * (2.0 / 16 / 27) ** 0.5
+    out = torch.empty(0, device="cuda")
+    S.SubmanifoldConvolution_updateOutput(SZ, torch.LongTensor([3, 3, 3]), m, feats, out, W.cuda(), torch.Tensor(), 1)
+    loc = m.getSpatialLocations(SZ)
+    G = 128
+    dense = torch.zeros(1, 16, G, G, G, dtype=torch.float64)
+    dense[0, :, loc[:, 0], loc[:, 1], loc[:, 2]] = feats.cpu().double().t()
+    w = W.double().reshape(3, 3, 3, 16, 16).permute(4, 3, 0, 1, 2)
+    ref = F.conv3d(dense, w, padding=1)[0, :, loc[:, 0], loc[:, 1], loc[:, 2]].t()
+    np.testing.assert_allclose(out.cpu().numpy(), ref.numpy(), rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("Cin,Cout", [(32, 64), (64, 96), (16, 8), (3, 5)])
+def test_strided_convolution_and_deconvolution(S, orc, Cin, Cout):
+    pts = scenes.boxes_scene(seed=5, n=15000)
+    m, x, feats = setup_sites(S, pts, Cin, seed=7)
+    rng = np.random.default_rng(8)
+    W = (rng.normal(size=(8, Cin, Cout)) * (2.0 / Cin / 8) ** 0.5).astype(np.float32)
+    two = torch.LongTensor([2, 2, 2])
+    out = torch.empty(0, device="cuda")
+    flops = S.Convolution_updateOutput(SZ, SZ // 2, two, two, m, feats, out, cu(W), torch.Tensor())
+    _, sc, _ = orc.grid_build(pts)
+    parent, off, cc = orc.down2_rules(sc)
+    counts, pairs = orc.down2_pairs(parent, off)
+    ref, rflops = orc.conv_forward(feats.cpu().numpy(), W, None, pairs, counts, len(cc))
+    assert flops == rflops and out.shape == ref.shape
+    np.testing.assert_allclose(out.cpu().numpy(), ref, rtol=RTOL, atol=ATOL)
+    # deconvolution back to the fine sites
+    W2 = (rng.normal(size=(8, Cout, Cin)) * (2.0 / Cout / 8) ** 0.5).astype(np.float32)
+    b2 = rng.normal(size=Cin).astype(np.float32)
+    back = torch.empty(0, device="cuda")
+    S.Deconvolution_updateOutput(SZ // 2, SZ, two, two, m, out, back, cu(W2), cu(b2))
+    ref2, _ = orc.conv_forward(ref, W2, b2, pairs, counts, len(sc), swap=True)
+    np.testing.assert_allclose(back.cpu().numpy(), ref2, rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("C,leak,affine", [(32, 0.0, True), (96, 0.333, True), (7, 1.0, False), (384, 0.0, True),
+                                           (2048, 0.0, True)])
+def test_batchnorm(S, orc, C, leak, affine):
+    rng = np.random.default_rng(C)
+    N = 5001
+    x = (rng.normal(size=(N, C)) * 2).astype(np.float32)
+    mean, var = rng.normal(size=C).astype(np.float32), rng.uniform(0.5, 2, C).astype(np.float32)
+    g = rng.uniform(0.5, 1.5, C).astype(np.float32) if affine else None
+    b = (rng.normal(size=C) * 0.1).astype(np.float32) if affine else None
+    out = torch.empty(0, device="cuda")
+    S.BatchNormalization_updateOutput(cu(x), out, None, None, cu(mean), cu(var), cu(g) if affine else torch.Tensor(),
+                                      cu(b) if affine else torch.Tensor(), 1e-4, 0.9, False, leak)
+    ref = orc.bn_forward(x, mean, var, g, b, 1e-4, leak)
+    np.testing.assert_allclose(out.cpu().numpy(), ref, rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("Cin,Cout,bias", [(64, 32, False), (384, 192, False), (32, 20, True), (6, 3, True)])
+def test_network_in_network(S, orc, Cin, Cout, bias):
+    rng = np.random.default_rng(Cin)
+    x = rng.normal(size=(7003, Cin)).astype(np.float32)
+    W = (rng.normal(size=(Cin, Cout)) * (2.0 / Cin) ** 0.5).astype(np.float32)
+    b = rng.normal(size=Cout).astype(np.float32) if bias else None
+    out = torch.empty(0, device="cuda")
+    flops = S.NetworkInNetwork_updateOutput(cu(x), out, cu(W), cu(b) if bias else torch.Tensor())
+    assert flops == 7003 * Cin * Cout
+    np.testing.assert_allclose(out.cpu().numpy(), orc.nin_forward(x, W, b), rtol=RTOL, atol=ATOL)
+
+
+def test_empty_input(S):
+    m = S.Metadata_3()
+    out = torch.empty(0, device="cuda")
+    S.InputLayer_updateOutput(m, SZ, torch.zeros((0, 3), dtype=torch.long), torch.zeros((0, 3), device="cuda"), out,
+                              0, 4)
+    assert out.shape == (0, 3)
+    o2 = torch.empty(0, device="cuda")
+    S.SubmanifoldConvolution_updateOutput(SZ, torch.LongTensor([3, 3, 3]), m, out, o2,
+                                          torch.zeros(27, 3, 8, device="cuda"), torch.Tensor(), 1)
+    assert o2.shape == (0, 8)
+
+
+def test_row_subset_leaves_other_rows_untouched(S, orc):
+    """The `rows` argument of the C ABI: listed rows are recomputed, the rest keep their bytes."""
+    pts = scenes.boxes_scene(seed=1, n=8000)
+    m, x, feats = setup_sites(S, pts, 32, seed=3)
+    sc = m.ssc_rulebook(SZ)
+    W = cu((np.random.default_rng(0).normal(size=(27, 32, 32)) * 0.05).astype(np.float32))
+    full = torch.empty(0, device="cuda")
+    S.SubmanifoldConvolution_updateOutput(SZ, torch.LongTensor([3, 3, 3]), m, feats, full, W, torch.Tensor(), 1)
+    out = torch.full_like(full, 123.0)
+    rows = torch.arange(0, sc.n, 3, dtype=torch.int32, device="cuda")
+    count = torch.tensor([len(rows) - 10], dtype=torch.int32, device="cuda")
+    S.conv_rows(feats, out, W, None, sc.nbr.t, 27, rows, count, len(rows))
+    done = rows[:len(rows) - 10].long()
+    assert torch.equal(out[done], full[done])  # bit-identical: a row's result does not depend on its tile
+    mask = torch.ones(sc.n, dtype=torch.bool, device="cuda")
+    mask[done] = False
+    assert bool((out[mask] == 123.0).all())

@@ -1,0 +1,191 @@
+"""GPU parity: scan / sort primitives, hash grid and rulebooks against the CPU oracle.
+Integer structures are compared bit-exactly: the HIP grid numbers sites by first appearance
+exactly like the oracle, so raw ids can be compared, and the canonical (sorted-by-coordinate)
+form is checked as well."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+import scenes
+
+pytestmark = pytest.mark.gpu
+I64 = ctypes.c_int64
+
+
+@pytest.fixture(scope="module")
+def S():
+    from sparseconvnet import SCN
+    from sparseconvnet._lib import ensure_init
+
+    ensure_init(0)
+    return SCN
+
+
+def dev(a, dtype=None):
+    t = torch.from_numpy(np.ascontiguousarray(a))
+    if dtype is not None:
+        t = t.to(dtype)
+    return t.cuda()
+
+
+@pytest.mark.parametrize("n", [0, 1, 63, 2048, 2049, 100003, 3000000])
+def test_scan(S, n):
+    from sparseconvnet._lib import lib, ptr, stream_ptr
+
+    rng = np.random.default_rng(n)
+    a = rng.integers(0, 5, n).astype(np.int32)
+    d_in = dev(a) if n else torch.empty(0, dtype=torch.int32, device="cuda")
+    d_out = torch.empty_like(d_in)
+    tot = torch.full((1,), -7, dtype=torch.int32, device="cuda")
+    lib.insc_scan_exclusive_i32(ptr(d_in), ptr(d_out), I64(n), ptr(tot), stream_ptr())
+    exp = np.concatenate([[0], np.cumsum(a)[:-1]]) if n else np.zeros(0)
+    assert (d_out.cpu().numpy() == exp).all()
+    assert int(tot.item()) == int(a.sum())
+
+
+@pytest.mark.parametrize("n,bits", [(1, 64), (1000, 16), (2048, 64), (50001, 40), (700000, 64), (300000, 3)])
+def test_sort_stable(S, n, bits):
+    from sparseconvnet._lib import lib, ptr, stream_ptr
+
+    rng = np.random.default_rng(n + bits)
+    hi = (1 << bits) - 1 if bits < 63 else (1 << 63) - 1
+    # few distinct values in part of the range so that stability matters
+    k = rng.integers(0, min(hi, 50) + 1, n).astype(np.uint64) if bits <= 16 else \
+        rng.integers(0, hi, n, dtype=np.int64).astype(np.uint64)
+    if bits == 64:
+        k |= (rng.integers(0, 2, n).astype(np.uint64) << np.uint64(63))
+    v = np.arange(n, dtype=np.int32)
+    dk = torch.from_numpy(k.view(np.int64)).cuda()
+    dv = dev(v)
+    lib.insc_sort_pairs_u64(ptr(dk), ptr(dv), I64(n), bits, stream_ptr())
+    order = np.argsort(k, kind="stable")
+    assert (dv.cpu().numpy() == v[order]).all()
+    assert (dk.cpu().numpy().view(np.uint64) == k[order]).all()
+
+
+def _insert(S, pts, capacity=None):
+    m = S.Metadata_3()
+    m._bind(torch.device("cuda", 0))
+    sc = m.scale((4096,) * 3, create_capacity=capacity or max(len(pts), 1))
+    sop = m.insert(sc, dev(pts, torch.int32)) if len(pts) else torch.empty(0, dtype=torch.int32)
+    return m, sc, sop
+
+
+@pytest.mark.parametrize("case", ["dups", "unique", "batched"])
+def test_grid_insert_matches_oracle(S, orc, case):
+    rng = np.random.default_rng(11)
+    if case == "dups":
+        pts = np.concatenate([rng.integers(0, 12, (20000, 3)), np.zeros((20000, 1), np.int64)], 1)
+    elif case == "unique":
+        pts = scenes.boxes_scene(seed=3, n=20000)
+    else:
+        pts = np.concatenate([rng.integers(100, 140, (30000, 3)), rng.integers(0, 5, (30000, 1))], 1)
+    pts = pts.astype(np.int32)
+    m, sc, sop = _insert(S, pts)
+    o_sop, o_sc, o_cnt = orc.grid_build(pts)
+    assert sc.n == len(o_sc)
+    assert (sop.cpu().numpy() == o_sop).all()
+    got = sc.coords_view().cpu().numpy()
+    assert (got == o_sc).all()
+    assert (orc.canonical_sites(got) == orc.canonical_sites(np.unique(pts, axis=0))).all()
+    assert (m.getSpatialLocations((4096,) * 3).numpy() == o_sc).all()
+
+
+def test_grid_query_append_and_grow(S, orc):
+    rng = np.random.default_rng(12)
+    a = rng.integers(0, 30, (5000, 3)).astype(np.int32)
+    a = np.concatenate([a, np.zeros((len(a), 1), np.int32)], 1)
+    m, sc, sop = _insert(S, a, capacity=1024)  # forces a rehash (capacity < sites)
+    b = rng.integers(0, 40, (9000, 3)).astype(np.int32)
+    b = np.concatenate([b, np.zeros((len(b), 1), np.int32)], 1)
+    sop_b = m.insert(sc, dev(b))
+    # append-only numbering == oracle numbering of the concatenated list
+    o_sop, o_sc, _ = orc.grid_build(np.concatenate([a, b], 0))
+    assert sc.n == len(o_sc)
+    assert (sop.cpu().numpy() == o_sop[:len(a)]).all()
+    assert (sop_b.cpu().numpy() == o_sop[len(a):]).all()
+    assert (sc.coords_view().cpu().numpy() == o_sc).all()
+    # queries: hits, misses, out-of-range coordinates
+    q = rng.integers(-2, 45, (20000, 3)).astype(np.int32)
+    q = np.concatenate([q, np.zeros((len(q), 1), np.int32)], 1)
+    q[:5, 0] = [70000, -1, 65536, 3, 3]
+    out = torch.empty(len(q), dtype=torch.int32, device="cuda")
+    from sparseconvnet._lib import lib, ptr, stream_ptr
+
+    lib.insc_grid_query(sc.grid, ptr(dev(q)), I64(len(q)), ptr(out), stream_ptr())
+    assert (out.cpu().numpy() == orc.grid_query(o_sc, q)).all()
+
+
+def test_grid_rejects_bad_coordinate(S):
+    from sparseconvnet._lib import InscError
+
+    pts = np.array([[1, 2, 3, 0], [70000, 1, 1, 0]], np.int32)
+    with pytest.raises(InscError):
+        _insert(S, pts)
+    pts = np.array([[1, 2, 3, 0], [1, -1, 1, 0]], np.int32)
+    with pytest.raises(InscError):
+        _insert(S, pts)
+
+
+@pytest.mark.parametrize("scene", ["cfg1", "random", "border"])
+def test_ssc_rulebook_matches_oracle(S, orc, scene):
+    if scene == "cfg1":
+        pts = scenes.boxes_scene(seed=1, n=20000)
+    elif scene == "random":
+        rng = np.random.default_rng(5)
+        pts = np.concatenate([rng.integers(0, 20, (6000, 3)), rng.integers(0, 2, (6000, 1))], 1).astype(np.int32)
+    else:  # sites on the coordinate borders: -1 and 65536 neighbours must not alias
+        rng = np.random.default_rng(6)
+        pts = np.concatenate([rng.choice([0, 1, 65534, 65535], (500, 3)), np.zeros((500, 1), np.int64)], 1).astype(np.int32)
+    m, sc, _ = _insert(S, pts)
+    m.ssc_rulebook((4096,) * 3)
+    o_sop, o_sc, _ = orc.grid_build(pts)
+    o_nbr, o_counts, o_pairs = orc.ssc_rules(o_sc)
+    assert (sc.nbr.t[:sc.n].cpu().numpy() == o_nbr).all()
+    counts, pairs = S.ssc_rulebook_lists(m, (4096,) * 3)
+    assert (counts.numpy() == o_counts).all()
+    assert (pairs.numpy() == o_pairs).all()
+    can = orc.canonical_rules(counts.numpy(), pairs.numpy(), o_sc, o_sc)
+    assert (can == orc.canonical_rules(o_counts, o_pairs, o_sc, o_sc)).all()
+    # the processing order is a permutation of the sites
+    assert (np.sort(sc.order.t[:sc.n].cpu().numpy()) == np.arange(sc.n)).all()
+
+
+def test_ssc_rulebook_incremental_patch(S, orc):
+    """Appending sites and patching the map equals building it from scratch."""
+    pts = scenes.boxes_scene(seed=9, n=12000)
+    m, sc, _ = _insert(S, pts[:7000])
+    m.ssc_rulebook((4096,) * 3)
+    m.insert(sc, dev(pts[7000:]))
+    m.ssc_rulebook((4096,) * 3)
+    _, o_sc, _ = orc.grid_build(pts)
+    o_nbr, _, _ = orc.ssc_rules(o_sc)
+    assert sc.n == len(o_sc)
+    assert (sc.nbr.t[:sc.n].cpu().numpy() == o_nbr).all()
+    assert (np.sort(sc.order.t[:sc.n].cpu().numpy()) == np.arange(sc.n)).all()
+
+
+def test_down2_rulebook_matches_oracle(S, orc):
+    pts = scenes.boxes_scene(seed=2, n=20000)
+    m, sc, _ = _insert(S, pts)
+    fine, coarse, d = m.down_rulebook((4096,) * 3, (2048,) * 3)
+    _, o_sc, _ = orc.grid_build(pts)
+    parent, off, cc = orc.down2_rules(o_sc)
+    assert coarse.n == len(cc)
+    assert (d.parent.t[:fine.n].cpu().numpy() == parent).all()
+    assert (d.offset.t[:fine.n].cpu().numpy() == off).all()
+    assert (coarse.coords_view().cpu().numpy() == cc).all()
+    child = d.child.t[:coarse.n].cpu().numpy()
+    exp = np.full((len(cc), 8), -1, np.int32)
+    exp[parent, off] = np.arange(len(parent))
+    assert (child == exp).all()
+    counts, pairs = S.down_rulebook_lists(m, (4096,) * 3, (2048,) * 3)
+    o_counts, o_pairs = orc.down2_pairs(parent, off)
+    can = orc.canonical_rules(counts.numpy(), pairs.numpy(), o_sc, cc)
+    assert (can == orc.canonical_rules(o_counts, o_pairs, o_sc, cc)).all()
+    # deconvolution order: a permutation, grouped by offset
+    bo = m.deconv_order(fine, d)[:fine.n].cpu().numpy()
+    assert (np.sort(bo) == np.arange(fine.n)).all()
+    assert (np.diff(off[bo]) >= 0).all()
