@@ -286,17 +286,42 @@ def _rows_args(rows, count, n_upper):
     return ptr(rows), ptr(count), I64(int(n_upper))
 
 
+def packed_weight(weight, K):
+    """Weights in the matrix-core operand layout.  The packed copy is kept on the tensor
+    object itself and reused until the tensor is modified in place or re-assigned."""
+    Cin, Cout = weight.size(-2), weight.size(-1)
+    if Cin % 16:
+        return None
+    tag = (weight._version, weight.data_ptr(), K, Cin, Cout)
+    hit = getattr(weight, "_insc_packed", None)
+    if hit is not None and hit[0] == tag:
+        return hit[1]
+    w = weight.detach()
+    if not w.is_contiguous():
+        w = w.contiguous()
+    n = int(lib.insc_conv_packed_floats(int(K), int(Cin), int(Cout)))
+    wp = torch.empty(n, dtype=torch.float32, device=weight.device)
+    lib.insc_conv_pack_weights(ptr(w), int(K), int(Cin), int(Cout), ptr(wp), stream_ptr())
+    try:
+        weight._insc_packed = (tag, wp)
+    except AttributeError:
+        pass
+    return wp
+
+
 def conv_rows(in_f, out_f, weight, bias, nbr, K, rows, count, n_rows):
     """insc_conv_nbr on a row subset; in_f/out_f may be column slices of wider buffers."""
     Cin, Cout = weight.size(-2), weight.size(-1)
-    lib.insc_conv_nbr(ptr(in_f), I64(_ld(in_f)), ptr(out_f), I64(_ld(out_f)), ptr(weight), ptr(bias), ptr(nbr), int(K),
-                      ptr(rows), ptr(count), I64(int(n_rows)), int(Cin), int(Cout), None, stream_ptr())
+    lib.insc_conv_nbr(ptr(in_f), I64(_ld(in_f)), ptr(out_f), I64(_ld(out_f)), ptr(weight),
+                      ptr(packed_weight(weight, K)), ptr(bias), ptr(nbr), int(K), ptr(rows), ptr(count),
+                      I64(int(n_rows)), int(Cin), int(Cout), None, stream_ptr())
 
 
 def deconv_rows(in_f, out_f, weight, bias, parent, offset, rows, count, n_rows):
     Cin, Cout = weight.size(-2), weight.size(-1)
-    lib.insc_deconv_down2(ptr(in_f), I64(_ld(in_f)), ptr(out_f), I64(_ld(out_f)), ptr(weight), ptr(bias), ptr(parent),
-                          ptr(offset), ptr(rows), ptr(count), I64(int(n_rows)), int(Cin), int(Cout), stream_ptr())
+    lib.insc_deconv_down2(ptr(in_f), I64(_ld(in_f)), ptr(out_f), I64(_ld(out_f)), ptr(weight),
+                          ptr(packed_weight(weight, 8)), ptr(bias), ptr(parent), ptr(offset), ptr(rows), ptr(count),
+                          I64(int(n_rows)), int(Cin), int(Cout), stream_ptr())
 
 
 def bn_rows(in_f, out_f, mean, var, gamma, beta, eps, leak, rows, count, n_rows):
@@ -386,7 +411,7 @@ def SubmanifoldConvolution_updateOutput(inputSize, filterSize, m, input_features
         raise NotImplementedError("only 3x3x3 submanifold convolutions with dilated_rate 1 are provided")
     input_features = _check_feats(input_features, "input_features")
     sc = m.ssc_rulebook(inputSize)
-    w, b = weight.detach().contiguous(), _opt(bias)
+    w, b = (weight if weight.is_contiguous() else weight.contiguous()), _opt(bias)
     if input_features.size(0) != sc.n or input_features.size(1) != w.size(1) or w.size(0) != 27:
         raise ValueError("feature / weight shapes do not match the active sites")
     _resize(output_features, sc.n, w.size(2), input_features)
@@ -407,7 +432,7 @@ def Convolution_updateOutput(inputSize, outputSize, filterSize, filterStride, m,
     _check_down(filterSize, filterStride)
     input_features = _check_feats(input_features, "input_features")
     fine, coarse, d = m.down_rulebook(inputSize, outputSize)
-    w, b = weight.detach().contiguous(), _opt(bias)
+    w, b = (weight if weight.is_contiguous() else weight.contiguous()), _opt(bias)
     if input_features.size(0) != fine.n or input_features.size(1) != w.size(1) or w.size(0) != 8:
         raise ValueError("feature / weight shapes do not match the active sites")
     _resize(output_features, coarse.n, w.size(2), input_features)
@@ -423,7 +448,7 @@ def Deconvolution_updateOutput(inputSize, outputSize, filterSize, filterStride, 
     _check_down(filterSize, filterStride)
     input_features = _check_feats(input_features, "input_features")
     fine, coarse, d = m.down_rulebook(outputSize, inputSize)
-    w, b = weight.detach().contiguous(), _opt(bias)
+    w, b = (weight if weight.is_contiguous() else weight.contiguous()), _opt(bias)
     if input_features.size(0) != coarse.n or input_features.size(1) != w.size(1) or w.size(0) != 8:
         raise ValueError("feature / weight shapes do not match the active sites")
     _resize(output_features, fine.n, w.size(2), input_features)
@@ -451,7 +476,7 @@ def BatchNormalization_updateOutput(input_features, output_features, saveMean, s
 def NetworkInNetwork_updateOutput(input_features, output_features, weight, bias):
     """cuda_NetworkInNetwork_updateOutput (CUDA/NetworkInNetwork.cpp:9-25)."""
     input_features = _check_feats(input_features, "input_features")
-    w, b = weight.detach().contiguous(), _opt(bias)
+    w, b = (weight if weight.is_contiguous() else weight.contiguous()), _opt(bias)
     n = input_features.size(0)
     _resize(output_features, n, w.size(1), input_features)
     if n:

@@ -46,7 +46,7 @@ class Convolution(Module):
             d = incremental.parents(input.dirty, coarse, down)
             out = self._state.grow(coarse.n, keep=min(coarse.n, self._state.buf.size(0)))
             rows, count = d.rows(coarse.order.t)
-            SCN.conv_rows(input.features, out, self.weight.detach(), SCN._opt(optionalTensor(self, 'bias')),
+            SCN.conv_rows(input.features, out, self.weight, SCN._opt(optionalTensor(self, 'bias')),
                           down.child.t, 8, rows, count, d.n_upper)
             output.features = out
             output.dirty = d

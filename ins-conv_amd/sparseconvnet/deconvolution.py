@@ -44,7 +44,7 @@ class Deconvolution(Module):
             d = incremental.children(input.dirty, fine, down)
             out = self._state.grow(fine.n, keep=min(fine.n, self._state.buf.size(0)))
             rows, count = d.rows(m.deconv_order(fine, down), tag="by_offset")
-            SCN.deconv_rows(input.features, out, self.weight.detach(), SCN._opt(optionalTensor(self, 'bias')),
+            SCN.deconv_rows(input.features, out, self.weight, SCN._opt(optionalTensor(self, 'bias')),
                             down.parent.t, down.offset.t, rows, count, d.n_upper)
             output.features = out
             output.dirty = d

@@ -34,7 +34,7 @@ class NetworkInNetwork(Module):
             n = input.features.size(0)
             out = self._state.grow(n, keep=min(n, self._state.buf.size(0)))
             rows, count = d.rows(d.scale.order.t)
-            SCN.conv_rows(input.features, out, self.weight.detach(), SCN._opt(optionalTensor(self, 'bias')), None, 1,
+            SCN.conv_rows(input.features, out, self.weight, SCN._opt(optionalTensor(self, 'bias')), None, 1,
                           rows, count, d.n_upper)
             output.features = out
             output.dirty = d

@@ -42,7 +42,7 @@ class SubmanifoldConvolution(Module):
             d = incremental.dilate(input.dirty)
             out = self._state.grow(sc.n, keep=min(sc.n, self._state.buf.size(0)))
             rows, count = d.rows(sc.order.t)
-            SCN.conv_rows(input.features, out, self.weight.detach(), SCN._opt(optionalTensor(self, 'bias')), sc.nbr.t,
+            SCN.conv_rows(input.features, out, self.weight, SCN._opt(optionalTensor(self, 'bias')), sc.nbr.t,
                           27, rows, count, d.n_upper)
             output.features = out
             output.dirty = d
