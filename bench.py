@@ -157,6 +157,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="ssc", choices=["ssc"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--roofline-only", action="store_true",
+                    help="run only the dominant-kernel measurement (short; used under rocprofv3)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU; --gpus %d is not supported (no collectives, no sharding)"
@@ -169,6 +171,9 @@ def main():
     torch.cuda.set_device(device)
 
     step, info, (x0, stack0) = ssc_workload(device)
+    if args.roofline_only:
+        print(json.dumps({"roofline": conv_roofline(x0, stack0, info["rules"], device, reps=10)}))
+        return
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()

@@ -59,11 +59,12 @@ __global__ __launch_bounds__(256) void conv_generic_kernel(const float *__restri
 }
 
 // ---------------------------------------------------------------------------------------
-// Weight packing.  The MFMA kernel wants, for filter offset k, input-channel chunk ch (32
-// channels) and output-channel block nb (32 channels), the 16 B-operand values of a lane
-// contiguous: lane = h*32 + j holds W[k][ch*32 + h*16 + s][nb*32 + j], s = 0..15.  One
-// wavefront then reads its 4 KB operand tile with four 16-byte loads per lane.  Channels
-// beyond Cin / Cout are zero.
+// Weight packing.  For filter offset k, input-channel chunk ch (32 channels) and
+// output-channel block nb (32 channels), lane = h*32 + j of the MFMA kernel needs the 16
+// B-operand values W[k][ch*32 + h*16 + s][nb*32 + j], s = 0..15.  The 4 KB tile is stored as
+// four 1 KB quarters; quarter q holds, for lane 0..63 in turn, the values s = 4q..4q+3.  One
+// 16-byte load per lane then reads a quarter fully coalesced.  Channels beyond Cin / Cout
+// are zero.
 // ---------------------------------------------------------------------------------------
 __host__ __device__ static inline int conv_nch(int Cin) { return (Cin + 31) / 32; }
 static inline int conv_nb_per_group(int Cout) {
@@ -79,7 +80,7 @@ __global__ void pack_weights_kernel(const float *__restrict__ W, int K, int Cin,
                                     float *__restrict__ Wp) {
   const int64_t total = (int64_t)K * nch * nbtp * 1024;
   for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < total; e += (int64_t)gridDim.x * blockDim.x) {
-    const int s = (int)(e & 15), lane = (int)((e >> 4) & 63);
+    const int s = (int)(((e >> 8) & 3) * 4 + (e & 3)), lane = (int)((e >> 2) & 63);
     int64_t q = e >> 10;
     const int nb = (int)(q % nbtp);
     q /= nbtp;
@@ -100,7 +101,7 @@ struct Frag {
 
 // Lanes whose row has no neighbour at the current offset read this row of zeros instead, so
 // the gather needs no branch and no select.
-__device__ __attribute__((aligned(64))) float g_zero_row[16];
+__device__ __attribute__((aligned(64))) float g_zero_row[16];  // all lanes read the first 16 bytes
 
 __device__ __forceinline__ Frag load_frag(const float *p) {
   Frag f;
@@ -109,18 +110,31 @@ __device__ __forceinline__ Frag load_frag(const float *p) {
   for (int i = 0; i < 4; i++) f.q[i] = p4[i];
   return f;
 }
+// weight tile: quarter q of the tile starts at q*256 floats, this lane's values at lane*4
+__device__ __forceinline__ Frag load_wfrag(const float *tile, int lane) {
+  Frag f;
+  const float4 *p4 = reinterpret_cast<const float4 *>(tile) + lane;
+#pragma unroll
+  for (int i = 0; i < 4; i++) f.q[i] = p4[i * 64];
+  return f;
+}
 __device__ __forceinline__ float frag_at(const Frag &f, int s) {
   const float4 v = f.q[s >> 2];
   return (s & 3) == 0 ? v.x : (s & 3) == 1 ? v.y : (s & 3) == 2 ? v.z : v.w;
 }
 
-template <int NB>
+// LDS row stride of the gather tile in floats: 32 channels + 4 of padding, so that both the
+// row-wise 16-byte writes and the column-block reads of the MFMA layout spread over all banks.
+constexpr int AT_LD = 36;
+
+template <int NB, int K, int MODE>
 __global__ __launch_bounds__(CONV_WAVES * 64) void conv_mfma_kernel(
     const float *__restrict__ in, int64_t ld_in, float *__restrict__ out, int64_t ld_out,
     const float *__restrict__ Wp, const float *__restrict__ bias, const int32_t *__restrict__ map0,
-    const int32_t *__restrict__ map1, int mode, int K, const int32_t *__restrict__ rows,
+    const int32_t *__restrict__ map1, const int32_t *__restrict__ rows,
     const int32_t *__restrict__ d_n_rows, int64_t n_rows, int Cin, int Cout, int nbtp) {
-  __shared__ int nbl[CONV_WAVES][TILE_M * MAXK];
+  __shared__ int nbl[CONV_WAVES][TILE_M * K];
+  __shared__ __attribute__((aligned(16))) float atile[CONV_WAVES][TILE_M * AT_LD];
   const int64_t n = d_n_rows ? min((int64_t)*d_n_rows, n_rows) : n_rows;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int r = lane & 31, h = lane >> 5;
@@ -131,23 +145,35 @@ __global__ __launch_bounds__(CONV_WAVES * 64) void conv_mfma_kernel(
   int my_row = -1;
   if (t0 + r < n) my_row = rows ? rows[t0 + r] : (int)(t0 + r);
 
-  // stage the tile's slice of the neighbour map in LDS and find the offsets it uses
+  // stage the tile's slice of the neighbour map in LDS and find the offsets it uses; all the
+  // loads are issued before the first one is consumed
   int *nl = nbl[wave];
   unsigned mymask = 0;
-  for (int e = lane; e < TILE_M * K; e += 64) {
+  constexpr int NSTAGE = (TILE_M * K + 63) / 64;
+  int staged[NSTAGE];
+#pragma unroll
+  for (int i = 0; i < NSTAGE; i++) {
+    const int e = i * 64 + lane;
     const int rr = e / K, kk = e - rr * K;
-    const int rid = __shfl(my_row, rr, 64);
+    const int rid = __shfl(my_row, rr & (TILE_M - 1), 64);
     int v = -1;
-    if (rid >= 0) {
-      if (mode == MAP_NBR)
+    if (e < TILE_M * K && rid >= 0) {
+      if (MODE == MAP_NBR)
         v = map0[(int64_t)rid * K + kk];
-      else if (mode == MAP_IDENTITY)
+      else if (MODE == MAP_IDENTITY)
         v = rid;
       else
         v = (map1[rid] == kk) ? map0[rid] : -1;
     }
-    nl[e] = v;
-    if (v >= 0) mymask |= 1u << kk;
+    staged[i] = v;
+  }
+#pragma unroll
+  for (int i = 0; i < NSTAGE; i++) {
+    const int e = i * 64 + lane;
+    if (e < TILE_M * K) {
+      nl[e] = staged[i];
+      if (staged[i] >= 0) mymask |= 1u << (e % K);
+    }
   }
 #pragma unroll
   for (int d = 32; d > 0; d >>= 1) mymask |= (unsigned)__shfl_xor((int)mymask, d, 64);
@@ -166,47 +192,97 @@ __global__ __launch_bounds__(CONV_WAVES * 64) void conv_mfma_kernel(
 
   if (rest) {
     const int64_t wtile = 1024;  // floats per (k, chunk, block) weight tile
-    int k = __builtin_ctz(rest);
+    // Work items of this tile: (active offset k, 32-channel chunk ch), in order.
+    struct Item {
+      int k, ch;
+    };
+    // next item, or the same item again with `last` set when there is none
+    auto advance = [&](Item it, bool &last) -> Item {
+      last = false;
+      if (it.ch + 1 < nch) {
+        it.ch++;
+      } else if (rest) {
+        it.k = __builtin_ctz(rest);
+        rest &= rest - 1;
+        it.ch = 0;
+      } else {
+        last = true;
+      }
+      return it;
+    };
+    // Gather of one item, coalesced: load i (0..3) of lane l reads 16 bytes of input row
+    // 8*i + l/8 at channel 4*(l%8), so eight lanes cover one 128-byte row segment and every
+    // quad of lanes reads 64 contiguous bytes.  Rows without a neighbour (and the upper half of
+    // a 16-channel tail chunk) read a row of zeros.
+    const int grow = lane >> 3, gcol = (lane & 7) * 4;
+    auto gather = [&](const Item &it) -> Frag {
+      Frag f;
+      const bool col_ok = it.ch * 32 + gcol < Cin;
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        const int src = nl[(8 * i + grow) * K + it.k];
+        const float *p = (src >= 0 && col_ok) ? in + (int64_t)src * ld_in + it.ch * 32 + gcol : g_zero_row;
+        f.q[i] = *reinterpret_cast<const float4 *>(p);
+      }
+      return f;
+    };
+    // through LDS into the MFMA A layout: lane (r, h) gets channels h*16 .. h*16+15 of row r
+    float *at = atile[wave];
+    auto transpose = [&](const Frag &g) -> Frag {
+#pragma unroll
+      for (int i = 0; i < 4; i++) *reinterpret_cast<float4 *>(at + (8 * i + grow) * AT_LD + gcol) = g.q[i];
+      Frag a;
+#pragma unroll
+      for (int q = 0; q < 4; q++) a.q[q] = *reinterpret_cast<const float4 *>(at + r * AT_LD + h * 16 + 4 * q);
+      return a;
+    };
+    auto wtile_of = [&](const Item &it, int b) -> const float * {
+      return Wp + (((int64_t)it.k * nch + it.ch) * nbtp + cb0 + b) * wtile;
+    };
+    Item it0;
+    it0.k = __builtin_ctz(rest);
     rest &= rest - 1;
-    int ch = 0;
-    int src = nl[r * K + k];
-    // the second half-wave of a 16-channel tail chunk has no input channels
-    bool a_on = src >= 0 && (h == 0 || Cin - ch * 32 >= 32);
-    Frag a_next = load_frag(a_on ? in + (int64_t)src * ld_in + ch * 32 + h * 16 : g_zero_row);
-    Frag b_pref = load_frag(Wp + (((int64_t)k * nch + ch) * nbtp + cb0) * wtile + lane * 16);
-    for (;;) {
-      const Frag a_cur = a_next;
-      bool has_next = true;
-      int k2 = k, ch2 = ch + 1, src2 = src;
-      if (ch2 == nch) {
-        if (rest == 0) {
-          has_next = false;
-        } else {
-          k2 = __builtin_ctz(rest);
-          rest &= rest - 1;
-          ch2 = 0;
-          src2 = nl[r * K + k2];
+    it0.ch = 0;
+    Frag g = gather(it0);
+    Frag bw[2];
+    bw[0] = load_wfrag(wtile_of(it0, 0), lane);
+    Frag a = transpose(g);
+    // Every load below is issued unconditionally (past the last item the current item is simply
+    // fetched again): a load under a branch would force the wait before the MFMAs to drain all
+    // outstanding loads, which serialises the pipeline.
+    bool done = false;
+    while (!done) {
+#pragma unroll
+      for (int u = 0; u < 2; u++) {
+        bool last;
+        const Item it1 = advance(it0, last);
+        g = gather(it1);  // in flight while this item runs on the matrix cores
+#pragma unroll
+        for (int b = 0; b < NB; b++) {
+          const int nn = u * NB + b;
+          if (b + 1 < NB)
+            bw[(nn + 1) % 2] = load_wfrag(wtile_of(it0, b + 1), lane);
+          else
+            bw[(nn + 1) % 2] = load_wfrag(wtile_of(it1, 0), lane);
+          // the loads above stay above the MFMAs (the scheduler otherwise sinks them to their
+          // consumers, i.e. behind the matrix work they are meant to overlap)
+          asm volatile("" ::: "memory");
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int s = 0; s < 16; s++)
+            acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(frag_at(a, s), frag_at(bw[nn % 2], s), acc[b], 0, 0, 0);
+        }
+        // keep the consumer of the gather behind the MFMAs: hoisting it would wait for the loads
+        // right after they were issued
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+        a = transpose(g);
+        it0 = it1;
+        if (last) {
+          done = true;
+          break;
         }
       }
-      if (has_next) {
-        a_on = src2 >= 0 && (h == 0 || Cin - ch2 * 32 >= 32);
-        a_next = load_frag(a_on ? in + (int64_t)src2 * ld_in + ch2 * 32 + h * 16 : g_zero_row);
-      }
-#pragma unroll
-      for (int b = 0; b < NB; b++) {
-        const Frag b_cur = b_pref;
-        if (b + 1 < NB)
-          b_pref = load_frag(Wp + (((int64_t)k * nch + ch) * nbtp + cb0 + b + 1) * wtile + lane * 16);
-        else if (has_next)
-          b_pref = load_frag(Wp + (((int64_t)k2 * nch + ch2) * nbtp + cb0) * wtile + lane * 16);
-#pragma unroll
-        for (int s = 0; s < 16; s++)
-          acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(frag_at(a_cur, s), frag_at(b_cur, s), acc[b], 0, 0, 0);
-      }
-      if (!has_next) break;
-      k = k2;
-      ch = ch2;
-      src = src2;
     }
   }
 
@@ -239,7 +315,7 @@ __global__ void count_rules_kernel(const int32_t *__restrict__ map0, int K, cons
 }
 
 static bool conv_uses_mfma(const float *in, int64_t ld_in, int Cin, int K) {
-  return Cin % 16 == 0 && ((uintptr_t)in % 16 == 0) && (ld_in % 4 == 0) && K <= MAXK;
+  return Cin % 16 == 0 && ((uintptr_t)in % 16 == 0) && (ld_in % 4 == 0) && (K == 27 || K == 8 || K == 1);
 }
 
 static int64_t packed_floats(int K, int Cin, int Cout) {
@@ -274,11 +350,23 @@ static int launch_conv(const float *in, int64_t ld_in, float *out, int64_t ld_ou
     const unsigned gx = (unsigned)cdiv(tiles, CONV_WAVES);
     const int NB = conv_nb_per_group(Cout), nbtp = conv_nbt_padded(Cout);
     dim3 grid(gx, (unsigned)(nbtp / NB)), block(CONV_WAVES * 64);
-#define INSC_CONV_CASE(NBV)                                                                                      \
-  case NBV:                                                                                                      \
-    hipLaunchKernelGGL(conv_mfma_kernel<NBV>, grid, block, 0, s, in, ld_in, out, ld_out, Wp, bias, map0, map1,   \
-                       mode, K, rows, d_n_rows, n_rows, Cin, Cout, nbtp);                                        \
+#define INSC_CONV_LAUNCH(NBV, KV, MV)                                                                          \
+  hipLaunchKernelGGL((conv_mfma_kernel<NBV, KV, MV>), grid, block, 0, s, in, ld_in, out, ld_out, Wp, bias, map0, \
+                     map1, rows, d_n_rows, n_rows, Cin, Cout, nbtp)
+#define INSC_CONV_CASE(NBV)                                      \
+  case NBV:                                                      \
+    if (mode == MAP_NBR && K == 27)                              \
+      INSC_CONV_LAUNCH(NBV, 27, MAP_NBR);                        \
+    else if (mode == MAP_NBR && K == 8)                          \
+      INSC_CONV_LAUNCH(NBV, 8, MAP_NBR);                         \
+    else if (mode == MAP_PARENT && K == 8)                       \
+      INSC_CONV_LAUNCH(NBV, 8, MAP_PARENT);                      \
+    else if (mode == MAP_IDENTITY && K == 1)                     \
+      INSC_CONV_LAUNCH(NBV, 1, MAP_IDENTITY);                    \
+    else                                                         \
+      shape_ok = false;                                          \
     break;
+    bool shape_ok = true;
     switch (NB) {
       INSC_CONV_CASE(1)
       INSC_CONV_CASE(2)
@@ -288,6 +376,11 @@ static int launch_conv(const float *in, int64_t ld_in, float *out, int64_t ld_ou
       INSC_CONV_CASE(6)
       INSC_CONV_CASE(7)
     }
+    if (!shape_ok) {
+      set_error("conv: no matrix-core kernel for K=%d with map mode %d", K, mode);
+      return INSC_ERR_ARG;
+    }
+#undef INSC_CONV_LAUNCH
 #undef INSC_CONV_CASE
   } else {
     if (!W) {
