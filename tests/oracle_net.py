@@ -1,0 +1,94 @@
+"""Runs a network built from the sparseconvnet mirror modules on the CPU oracle.
+
+The module tree (Sequential / ConcatTable / AddTable / JoinTable / layers) is walked exactly
+as Sequential.forward does, but every layer is evaluated with the oracle's restatement of the
+reference's CPU path, on numpy arrays.  Used to check whole-network results of the HIP path.
+"""
+import numpy as np
+
+from oracle import oracle as orc
+
+
+class OTensor(object):
+    def __init__(self, feats, size, ctx):
+        self.features, self.spatial_size, self.ctx = feats, tuple(int(v) for v in size), ctx
+
+
+class Ctx(object):
+    """Sites per spatial size and the rulebooks between them (the oracle's Metadata)."""
+
+    def __init__(self):
+        self.coords = {}
+        self.ssc = {}
+        self.down = {}
+
+    def ssc_rules(self, size):
+        if size not in self.ssc:
+            _, counts, pairs = orc.ssc_rules(self.coords[size])
+            self.ssc[size] = (counts, pairs)
+        return self.ssc[size]
+
+    def down_rules(self, fine, coarse):
+        if (fine, coarse) not in self.down:
+            parent, off, cc = orc.down2_rules(self.coords[fine])
+            self.coords[coarse] = cc
+            self.down[(fine, coarse)] = orc.down2_pairs(parent, off)
+        return self.down[(fine, coarse)]
+
+
+def _np(t):
+    return None if t is None else t.detach().cpu().numpy()
+
+
+def forward(module, x):
+    import sparseconvnet as scn
+
+    name = type(module).__name__
+    if isinstance(module, scn.InputLayer):
+        coords, feats = x[0], x[1]
+        ctx = Ctx()
+        size = tuple(int(v) for v in module.spatial_size.tolist())
+        sop, sc, cnt = orc.grid_build(np.asarray(coords))
+        ctx.coords[size] = sc
+        ctx.site_of_point = sop
+        f = orc.input_forward(np.asarray(feats, np.float32), sop, cnt, mode=module.mode)
+        return OTensor(f, size, ctx)
+    if isinstance(module, scn.OutputLayer):
+        return orc.output_forward(x.features, x.ctx.site_of_point)
+    if isinstance(module, scn.ConcatTable):
+        return [forward(m, x) for m in module._modules.values()]
+    if isinstance(module, scn.AddTable):
+        f = x[0].features
+        for t in x[1:]:
+            f = f + t.features
+        return OTensor(f.astype(np.float32), x[0].spatial_size, x[0].ctx)
+    if isinstance(module, scn.JoinTable):
+        return OTensor(np.concatenate([t.features for t in x], 1), x[0].spatial_size, x[0].ctx)
+    if isinstance(module, scn.Sequential):
+        for m in module:
+            x = forward(m, x)
+        return x
+    if isinstance(module, scn.Identity):
+        return x
+    bias = _np(getattr(module, "bias", None))
+    if isinstance(module, scn.SubmanifoldConvolution):
+        counts, pairs = x.ctx.ssc_rules(x.spatial_size)
+        f, _ = orc.conv_forward(x.features, _np(module.weight), bias, pairs, counts, len(x.features))
+        return OTensor(f, x.spatial_size, x.ctx)
+    if isinstance(module, scn.Convolution):
+        coarse = tuple(s // 2 for s in x.spatial_size)
+        counts, pairs = x.ctx.down_rules(x.spatial_size, coarse)
+        f, _ = orc.conv_forward(x.features, _np(module.weight), bias, pairs, counts, len(x.ctx.coords[coarse]))
+        return OTensor(f, coarse, x.ctx)
+    if isinstance(module, scn.Deconvolution):
+        fine = tuple(s * 2 for s in x.spatial_size)
+        counts, pairs = x.ctx.down_rules(fine, x.spatial_size)
+        f, _ = orc.conv_forward(x.features, _np(module.weight), bias, pairs, counts, len(x.ctx.coords[fine]), swap=True)
+        return OTensor(f, fine, x.ctx)
+    if isinstance(module, scn.BatchNormalization):
+        f = orc.bn_forward(x.features, _np(module.running_mean), _np(module.running_var),
+                           _np(getattr(module, "weight", None)), bias, module.eps, module.leakiness)
+        return OTensor(f, x.spatial_size, x.ctx)
+    if isinstance(module, scn.NetworkInNetwork):
+        return OTensor(orc.nin_forward(x.features, _np(module.weight), bias), x.spatial_size, x.ctx)
+    raise NotImplementedError(name)
