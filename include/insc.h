@@ -205,6 +205,49 @@ int insc_dirty_compact(const uint8_t *d_mask, const int32_t *d_order, const int3
                        int32_t *d_rows, int32_t *d_count, int64_t *h_count, void *stream);
 
 /* ---------------------------------------------------------------------------------------
+ * Network executor: a whole network (input layer, 3^3 submanifold convolutions, 2/2
+ * convolutions and deconvolutions, batch norm + ReLU, 1x1 layers, add, channel join, output
+ * layer) run from one host call, full or incremental.  It plays the part of the reference's
+ * Python module graph plus its per-module saved state (sparseconvnet/sequential.py:20-25,
+ * submanifoldConvolution.py:53-54, batchNormalization.py:60-61, ioLayers.py:69,106-107):
+ * a full frame corresponds to Model(x, increment=False), an incremental frame to
+ * Model(x, increment=True) (demo.py:26-38), except that the incremental result equals a full
+ * forward over all points seen so far.
+ *
+ * Scales are numbered 0 (input resolution) upward, one per 2/2 convolution.  Tensor 0 is the
+ * input layer's output; weight, bias and batch-norm pointers are device pointers that must
+ * outlive the net.
+ * ------------------------------------------------------------------------------------- */
+typedef struct insc_net insc_net;
+int insc_net_create(int n_levels, int in_channels, int input_mode, insc_net **out);
+int insc_net_destroy(insc_net *net);
+/* New feature matrix with `channels` columns at scale `level`. */
+int insc_net_tensor(insc_net *net, int level, int channels, int *out_id);
+/* Declare tensor `out` as the channel concatenation [a | b] (JoinTable): a and b become
+ * column slices of out's matrix, so their producers write in place and nothing is copied. */
+int insc_net_join(insc_net *net, int a, int b, int out);
+/* kind 0: submanifold 3^3, W [27,Cin,Cout]; 2: convolution 2/2 to the next coarser scale,
+ * W [8,Cin,Cout]; 3: deconvolution 2/2 to the next finer scale; 4: 1x1, W [Cin,Cout]. */
+int insc_net_op_conv(insc_net *net, int kind, int in, int out, const float *d_W, const float *d_bias);
+int insc_net_op_bn(insc_net *net, int in, int out, const float *d_mean, const float *d_var, const float *d_gamma,
+                   const float *d_beta, float eps, float leakiness);
+int insc_net_op_add(insc_net *net, int a, int b, int out);
+/* Freeze the program; out_tensor feeds the output layer; capacity_sites is reserved at scale 0
+ * (half of it at each coarser scale; everything grows on demand). */
+int insc_net_finalize(insc_net *net, int out_tensor, int64_t capacity_sites, void *stream);
+/* Re-pack the weights after the caller changed them in place. */
+int insc_net_refresh_weights(insc_net *net, void *stream);
+/* One frame: d_coords int32 [P,coord_cols] (x,y,z[,batch]), d_feats float32 [P,in_channels].
+ * increment == 0 forgets all state and runs a full forward; increment != 0 appends the points
+ * and recomputes only the rows they affect.  d_out (nullable) receives one row of the output
+ * tensor per point of this frame (out_all == 0) or per point since the last full frame.
+ * Returns when the frame has completed. */
+int insc_net_forward(insc_net *net, const int32_t *d_coords, int coord_cols, const float *d_feats, int64_t P,
+                     int increment, float *d_out, int out_all, int64_t *h_n_sites, void *stream);
+int insc_net_tensor_view(insc_net *net, int tensor, float **d_ptr, int64_t *ld, int64_t *rows, int *channels);
+int insc_net_counts(insc_net *net, int64_t *h_sites_per_level, int64_t *h_points);
+
+/* ---------------------------------------------------------------------------------------
  * Device utilities exported for tests and callers.
  * ------------------------------------------------------------------------------------- */
 /* Exclusive prefix sum of n int32 values; d_total (nullable) receives the sum. */

@@ -41,6 +41,27 @@ int workspace(int which, hipStream_t stream, size_t bytes, void **out);
 int scan_exclusive_i32(const int32_t *in, int32_t *out, int64_t n, int32_t *total, hipStream_t s);
 int sort_pairs_u64(uint64_t *keys, int32_t *vals, int64_t n, int key_bits, hipStream_t s);
 
+// ---- feature kernels shared with the network executor (conv.hip, pointwise.hip) ----------
+enum { MAP_NBR = 0, MAP_IDENTITY = 1, MAP_PARENT = 2 };
+// tile_flags: one byte per 32-row tile of `rows` (matrix-core kernel); row_mask: one byte per
+// site (generic kernel and the streaming kernels).  Null = everything.
+int launch_conv(const float *in, int64_t ld_in, float *out, int64_t ld_out, const float *W, const float *Wp,
+                const float *bias, const int32_t *map0, const int32_t *map1, int mode, int K, const int32_t *rows,
+                const int32_t *d_n_rows, int64_t n_rows, int Cin, int Cout, const uint8_t *tile_flags,
+                const uint8_t *row_mask, hipStream_t s);
+int64_t packed_floats(int K, int Cin, int Cout);
+int pack_weights(const float *W, int K, int Cin, int Cout, float *Wp, hipStream_t s);
+int launch_bn(const float *in, int64_t ld_in, float *out, int64_t ld_out, const float *mean, const float *var,
+              const float *gamma, const float *beta, float eps, float leak, const int32_t *rows,
+              const int32_t *d_n_rows, int64_t n_rows, int C, const uint8_t *row_mask, hipStream_t s);
+// out = a + b (b != null) or out = a
+int launch_add(const float *a, int64_t ld_a, const float *b, int64_t ld_b, float *out, int64_t ld_out,
+               const int32_t *rows, const int32_t *d_n_rows, int64_t n_rows, int C, const uint8_t *row_mask,
+               hipStream_t s);
+int launch_input_finish(const float *sum, const int32_t *cnt, int mode, float *out, int64_t ld_out,
+                        const int32_t *rows, const int32_t *d_n_rows, int64_t n_rows, int C,
+                        const uint8_t *row_mask, hipStream_t s);
+
 static inline int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
 static inline unsigned grid_for(int64_t n, int block, int64_t cap = 1 << 20) {
   int64_t g = cdiv(n, block);

@@ -14,7 +14,6 @@ namespace insc {
 
 typedef float f16v __attribute__((ext_vector_type(16)));
 
-enum { MAP_NBR = 0, MAP_IDENTITY = 1, MAP_PARENT = 2 };
 
 constexpr int CONV_WAVES = 4;
 constexpr int TILE_M = 32;
@@ -32,14 +31,15 @@ __global__ __launch_bounds__(256) void conv_generic_kernel(const float *__restri
                                                            const int32_t *__restrict__ map1, int mode, int K,
                                                            const int32_t *__restrict__ rows,
                                                            const int32_t *__restrict__ d_n_rows, int64_t n_rows,
-                                                           int Cin, int Cout) {
+                                                           int Cin, int Cout,
+                                                           const uint8_t *__restrict__ row_mask) {
   const int64_t n = d_n_rows ? min((int64_t)*d_n_rows, n_rows) : n_rows;
   const int cpb = 256 / Cout > 0 ? 256 / Cout : 1;  // rows per block (Cout <= 256)
   const int lr = threadIdx.x / Cout, co = threadIdx.x % Cout;
   if (lr >= cpb) return;
   for (int64_t t = (int64_t)blockIdx.x * cpb + lr; t < n; t += (int64_t)gridDim.x * cpb) {
     const int row = rows ? rows[t] : (int)t;
-    if (row < 0) continue;
+    if (row < 0 || (row_mask && !row_mask[row])) continue;
     float acc = bias ? bias[co] : 0.0f;
     for (int k = 0; k < K; k++) {
       int src;
@@ -132,7 +132,8 @@ __global__ __launch_bounds__(CONV_WAVES * 64) void conv_mfma_kernel(
     const float *__restrict__ in, int64_t ld_in, float *__restrict__ out, int64_t ld_out,
     const float *__restrict__ Wp, const float *__restrict__ bias, const int32_t *__restrict__ map0,
     const int32_t *__restrict__ map1, const int32_t *__restrict__ rows,
-    const int32_t *__restrict__ d_n_rows, int64_t n_rows, int Cin, int Cout, int nbtp) {
+    const int32_t *__restrict__ d_n_rows, int64_t n_rows, int Cin, int Cout, int nbtp,
+    const uint8_t *__restrict__ tile_flags) {
   __shared__ int nbl[CONV_WAVES][TILE_M * K];
   __shared__ __attribute__((aligned(16))) float atile[CONV_WAVES][TILE_M * AT_LD];
   const int64_t n = d_n_rows ? min((int64_t)*d_n_rows, n_rows) : n_rows;
@@ -142,8 +143,10 @@ __global__ __launch_bounds__(CONV_WAVES * 64) void conv_mfma_kernel(
   const int cb0 = blockIdx.y * NB;  // first output-channel block of this column group
   const int nch = conv_nch(Cin);
 
+  // a tile is skipped when it lies beyond the row count or, with tile flags, is not marked
+  const bool live = t0 < n && (!tile_flags || tile_flags[t0 >> 5]);
   int my_row = -1;
-  if (t0 + r < n) my_row = rows ? rows[t0 + r] : (int)(t0 + r);
+  if (live && t0 + r < n) my_row = rows ? rows[t0 + r] : (int)(t0 + r);
 
   // stage the tile's slice of the neighbour map in LDS and find the offsets it uses; all the
   // loads are issued before the first one is consumed
@@ -178,7 +181,7 @@ __global__ __launch_bounds__(CONV_WAVES * 64) void conv_mfma_kernel(
 #pragma unroll
   for (int d = 32; d > 0; d >>= 1) mymask |= (unsigned)__shfl_xor((int)mymask, d, 64);
   __syncthreads();
-  if (t0 >= n) return;  // whole wavefront idle; no barrier follows
+  if (!live) return;  // whole wavefront idle; no barrier follows
   unsigned rest = (unsigned)__builtin_amdgcn_readfirstlane((int)mymask);
 
   f16v acc[NB];
@@ -318,11 +321,11 @@ static bool conv_uses_mfma(const float *in, int64_t ld_in, int Cin, int K) {
   return Cin % 16 == 0 && ((uintptr_t)in % 16 == 0) && (ld_in % 4 == 0) && (K == 27 || K == 8 || K == 1);
 }
 
-static int64_t packed_floats(int K, int Cin, int Cout) {
+int64_t packed_floats(int K, int Cin, int Cout) {
   return (int64_t)K * conv_nch(Cin) * conv_nbt_padded(Cout) * 1024;
 }
 
-static int pack_weights(const float *W, int K, int Cin, int Cout, float *Wp, hipStream_t s) {
+int pack_weights(const float *W, int K, int Cin, int Cout, float *Wp, hipStream_t s) {
   const int64_t total = packed_floats(K, Cin, Cout);
   hipLaunchKernelGGL(pack_weights_kernel, dim3(grid_for(total, 256, 4096)), dim3(256), 0, s, W, K, Cin, Cout,
                      conv_nch(Cin), conv_nbt_padded(Cout), Wp);
@@ -332,10 +335,10 @@ static int pack_weights(const float *W, int K, int Cin, int Cout, float *Wp, hip
 
 // W: raw [K,Cin,Cout] weights (always needed by the generic kernel); Wp: packed weights or
 // null, in which case they are packed into scratch memory first.
-static int launch_conv(const float *in, int64_t ld_in, float *out, int64_t ld_out, const float *W, const float *Wp,
-                       const float *bias, const int32_t *map0, const int32_t *map1, int mode, int K,
-                       const int32_t *rows, const int32_t *d_n_rows, int64_t n_rows, int Cin, int Cout,
-                       hipStream_t s) {
+int launch_conv(const float *in, int64_t ld_in, float *out, int64_t ld_out, const float *W, const float *Wp,
+                const float *bias, const int32_t *map0, const int32_t *map1, int mode, int K, const int32_t *rows,
+                const int32_t *d_n_rows, int64_t n_rows, int Cin, int Cout, const uint8_t *tile_flags,
+                const uint8_t *row_mask, hipStream_t s) {
   if (n_rows == 0) return INSC_OK;
   if (conv_uses_mfma(in, ld_in, Cin, K)) {
     if (!Wp) {
@@ -352,7 +355,7 @@ static int launch_conv(const float *in, int64_t ld_in, float *out, int64_t ld_ou
     dim3 grid(gx, (unsigned)(nbtp / NB)), block(CONV_WAVES * 64);
 #define INSC_CONV_LAUNCH(NBV, KV, MV)                                                                          \
   hipLaunchKernelGGL((conv_mfma_kernel<NBV, KV, MV>), grid, block, 0, s, in, ld_in, out, ld_out, Wp, bias, map0, \
-                     map1, rows, d_n_rows, n_rows, Cin, Cout, nbtp)
+                     map1, rows, d_n_rows, n_rows, Cin, Cout, nbtp, tile_flags)
 #define INSC_CONV_CASE(NBV)                                      \
   case NBV:                                                      \
     if (mode == MAP_NBR && K == 27)                              \
@@ -393,7 +396,7 @@ static int launch_conv(const float *in, int64_t ld_in, float *out, int64_t ld_ou
     }
     const int cpb = 256 / Cout;
     hipLaunchKernelGGL(conv_generic_kernel, dim3(grid_for(n_rows, cpb, 65536)), dim3(256), 0, s, in, ld_in, out,
-                       ld_out, W, bias, map0, map1, mode, K, rows, d_n_rows, n_rows, Cin, Cout);
+                       ld_out, W, bias, map0, map1, mode, K, rows, d_n_rows, n_rows, Cin, Cout, row_mask);
   }
   INSC_LAUNCH_CHECK();
   return INSC_OK;
@@ -426,7 +429,7 @@ int insc_conv_nbr(const float *d_in, int64_t ld_in, float *d_out, int64_t ld_out
   INSC_REQUIRE(d_nbr || K == 1, INSC_ERR_ARG, "insc_conv_nbr: a null map needs K == 1");
   hipStream_t s = (hipStream_t)stream;
   int rc = launch_conv(d_in, ld_in, d_out, ld_out, d_W, d_Wp, d_bias, d_nbr, nullptr,
-                       d_nbr ? MAP_NBR : MAP_IDENTITY, K, d_rows, d_n_rows, n_rows, Cin, Cout, s);
+                       d_nbr ? MAP_NBR : MAP_IDENTITY, K, d_rows, d_n_rows, n_rows, Cin, Cout, nullptr, nullptr, s);
   if (rc) return rc;
   if (h_muladds) {
     unsigned long long h = 0;
@@ -463,7 +466,7 @@ int insc_deconv_down2(const float *d_in, int64_t ld_in, float *d_out, int64_t ld
   INSC_REQUIRE(n_rows == 0 || (d_in && d_out && (d_W || d_Wp) && d_parent && d_offset), INSC_ERR_ARG,
                "insc_deconv_down2: null pointer");
   return launch_conv(d_in, ld_in, d_out, ld_out, d_W, d_Wp, d_bias, d_parent, d_offset, MAP_PARENT, 8, d_rows,
-                     d_n_rows, n_rows, Cin, Cout, (hipStream_t)stream);
+                     d_n_rows, n_rows, Cin, Cout, nullptr, nullptr, (hipStream_t)stream);
 }
 
 }  // extern "C"

@@ -1,0 +1,53 @@
+// Internal view of the hash grid, shared by grid.hip and the network executor.
+#pragma once
+#include "common.h"
+
+namespace insc {
+
+struct __attribute__((aligned(16))) Slot {
+  unsigned long long key;
+  int val;
+  int pad;
+};
+
+constexpr int VAL_UNSET = 0x7FFFFFFF;
+// At load <= 0.5 probe runs are a handful of slots; the cap only bounds a corrupted table.
+constexpr int64_t MAX_PROBES = 1 << 16;
+constexpr int VAL_PENDING = 0x40000000;  // VAL_PENDING + p : claimed during this insert by row p
+
+}  // namespace insc
+
+struct insc_grid {
+  insc::Slot *table = nullptr;
+  int64_t n_slots = 0;         // power of two
+  int64_t capacity_sites = 0;  // rows of coords
+  int32_t *coords = nullptr;   // [capacity_sites, 4]
+  int32_t *d_n = nullptr;      // device site counter; d_n[1] = the count before the last insert
+  int32_t *d_err = nullptr;    // device flag: bit0 bad coordinate, bit1 table full
+  int64_t n_upper = 0;         // host upper bound of the site count
+  int64_t n_exact = -1;        // host copy of the count, -1 = stale
+  // insert scratch, grown on demand
+  int32_t *slot_of_point = nullptr;
+  int32_t *flags = nullptr;
+  int64_t scratch_rows = 0;
+  int device = 0;
+};
+
+namespace insc {
+
+// Point coordinate that the insert skips silently (site -1, no error): used to pad a fixed-size
+// launch whose real length is only known on the device.
+constexpr int32_t COORD_SKIP = INT32_MIN;
+
+// Device-side variants used inside a frame: nothing here synchronises with the host.
+// All of them act on the sites added by the grid's most recent insert, [*d_n_prev, *d_n).
+int grid_insert_nosync(insc_grid *g, const int32_t *d_coords4, int64_t P, int32_t *d_site_of_point, hipStream_t s);
+int ssc3_new_sites(const insc_grid *g, int32_t *d_nbr, int64_t n_new_upper, hipStream_t s);
+int down2_new_sites(const insc_grid *fine, insc_grid *coarse, int64_t n_new_upper, int32_t *d_parent,
+                    int32_t *d_offset, int32_t *d_child, hipStream_t s);
+// order[i] = pos[i] = i for the new sites (appended in id order)
+int order_append_new_sites(const insc_grid *g, int32_t *d_order, int32_t *d_pos, int64_t n_new_upper, hipStream_t s);
+// device pointer to the site count before the most recent insert
+static inline const int32_t *grid_n_prev_ptr(const insc_grid *g) { return g->d_n + 1; }
+
+}  // namespace insc

@@ -8,37 +8,7 @@
 // Numbering: a site's id is its rank among first occurrences in the inserted list, offset by
 // the count before the call - deterministic and append-only.
 #include "common.h"
-
-namespace insc {
-
-struct __attribute__((aligned(16))) Slot {
-  unsigned long long key;
-  int val;
-  int pad;
-};
-
-constexpr int VAL_UNSET = 0x7FFFFFFF;
-// At load <= 0.5 probe runs are a handful of slots; the cap only bounds a corrupted table.
-constexpr int64_t MAX_PROBES = 1 << 16;
-constexpr int VAL_PENDING = 0x40000000;  // VAL_PENDING + p : claimed during this insert by row p
-
-}  // namespace insc
-
-struct insc_grid {
-  insc::Slot *table = nullptr;
-  int64_t n_slots = 0;         // power of two
-  int64_t capacity_sites = 0;  // rows of coords
-  int32_t *coords = nullptr;   // [capacity_sites, 4]
-  int32_t *d_n = nullptr;      // device site counter
-  int32_t *d_err = nullptr;    // device flag: bit0 bad coordinate, bit1 table full
-  int64_t n_upper = 0;         // host upper bound of the site count
-  int64_t n_exact = -1;        // host copy of the count, -1 = stale
-  // insert scratch, grown on demand
-  int32_t *slot_of_point = nullptr;
-  int32_t *flags = nullptr;
-  int64_t scratch_rows = 0;
-  int device = 0;
-};
+#include "grid.h"
 
 namespace insc {
 
@@ -80,7 +50,8 @@ __global__ void grid_clear_kernel(Slot *table, int64_t n_slots, int32_t *d_n, in
     table[i] = e;
   }
   if (blockIdx.x == 0 && threadIdx.x == 0) {
-    *d_n = 0;
+    d_n[0] = 0;
+    d_n[1] = 0;
     *d_err = 0;
   }
 }
@@ -91,6 +62,10 @@ __global__ void grid_claim_kernel(Slot *table, int64_t mask, const int32_t *__re
   int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (p >= P) return;
   int4 c = reinterpret_cast<const int4 *>(coords4)[p];
+  if (c.x == COORD_SKIP) {
+    slot_of_point[p] = -1;
+    return;
+  }
   if (!coord_ok(c.x, c.y, c.z, c.w)) {
     slot_of_point[p] = -1;
     atomicOr(d_err, 1);
@@ -154,7 +129,10 @@ __global__ void grid_resolve_kernel(const Slot *__restrict__ table, const int32_
     site_of_point[p] = (v >= 0 && v < VAL_PENDING) ? v : -1;
   }
 }
-__global__ void grid_bump_kernel(int32_t *d_n, const int32_t *total) { *d_n += *total; }
+__global__ void grid_bump_kernel(int32_t *d_n, const int32_t *total) {
+  d_n[1] = d_n[0];
+  d_n[0] += *total;
+}
 
 __global__ void grid_query_kernel(const Slot *__restrict__ table, int64_t mask, const int32_t *__restrict__ coords4,
                                   int64_t Q, int32_t *__restrict__ out) {
@@ -221,6 +199,62 @@ __global__ void down2_child_kernel(const int32_t *__restrict__ parent, const int
   if (p >= 0) child[(int64_t)p * 8 + offset[i]] = (int)i;
 }
 
+// ---- variants over the sites added by the last insert, [d_n[1], d_n[0]) --------------------
+__global__ void ssc3_nbr_new_kernel(const Slot *__restrict__ table, int64_t mask,
+                                    const int32_t *__restrict__ site_coords, const int32_t *__restrict__ d_n,
+                                    int32_t *__restrict__ nbr) {
+  const int64_t first = d_n[1], n = (int64_t)d_n[0] - first;
+  int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= n * 27) return;
+  int64_t o = first + t / 27;
+  int k = (int)(t % 27);
+  int4 c = reinterpret_cast<const int4 *>(site_coords)[o];
+  int x = c.x + k / 9 - 1, y = c.y + (k / 3) % 3 - 1, z = c.z + k % 3 - 1;
+  int r = -1;
+  if (k == 13)
+    r = (int)o;
+  else if (coord_ok(x, y, z, c.w))
+    r = grid_find(table, mask, pack_key(x, y, z, c.w));
+  nbr[o * 27 + k] = r;
+  if (r >= 0 && r < first) nbr[(int64_t)r * 27 + (26 - k)] = (int)o;
+}
+
+__global__ void down2_coords_new_kernel(const int32_t *__restrict__ fine_coords, const int32_t *__restrict__ d_n,
+                                        int64_t n_upper, int32_t *__restrict__ half, int32_t *__restrict__ offset) {
+  const int64_t first = d_n[1], n = (int64_t)d_n[0] - first;
+  int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= n_upper) return;
+  if (t >= n) {
+    reinterpret_cast<int4 *>(half)[t] = make_int4(COORD_SKIP, 0, 0, 0);
+    return;
+  }
+  int4 c = reinterpret_cast<const int4 *>(fine_coords)[first + t];
+  offset[first + t] = (c.x & 1) * 4 + (c.y & 1) * 2 + (c.z & 1);
+  reinterpret_cast<int4 *>(half)[t] = make_int4(c.x >> 1, c.y >> 1, c.z >> 1, c.w);
+}
+
+// parent_tmp[t] = coarse site of new fine site first+t
+__global__ void down2_link_new_kernel(const int32_t *__restrict__ parent_tmp, const int32_t *__restrict__ d_n,
+                                      int32_t *__restrict__ parent, const int32_t *__restrict__ offset,
+                                      int32_t *__restrict__ child) {
+  const int64_t first = d_n[1], n = (int64_t)d_n[0] - first;
+  int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= n) return;
+  const int64_t i = first + t;
+  const int p = parent_tmp[t];
+  parent[i] = p;
+  if (p >= 0 && child) child[(int64_t)p * 8 + offset[i]] = (int)i;
+}
+
+__global__ void order_append_kernel(const int32_t *__restrict__ d_n, int32_t *__restrict__ order,
+                                    int32_t *__restrict__ pos) {
+  const int64_t first = d_n[1], n = (int64_t)d_n[0] - first;
+  int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= n) return;
+  order[first + t] = (int)(first + t);
+  if (pos) pos[first + t] = (int)(first + t);
+}
+
 static int grid_alloc_table(insc_grid *g, int64_t capacity_sites) {
   int64_t slots = 1024;
   while (slots < 2 * capacity_sites) slots <<= 1;
@@ -244,6 +278,90 @@ static int grid_sync_errors(insc_grid *g, hipStream_t s, const char *who) {
     set_error("%s: grid capacity %lld exceeded", who, (long long)g->capacity_sites);
     return INSC_ERR_CAPACITY;
   }
+  return INSC_OK;
+}
+
+static int grid_ensure_scratch(insc_grid *g, int64_t P, hipStream_t s) {
+  if (g->scratch_rows < P) {
+    INSC_HIP(hipStreamSynchronize(s));
+    if (g->slot_of_point) INSC_HIP(hipFree(g->slot_of_point));
+    if (g->flags) INSC_HIP(hipFree(g->flags));
+    g->slot_of_point = g->flags = nullptr;
+    int64_t rows = P + P / 2;
+    INSC_HIP(hipMalloc((void **)&g->slot_of_point, sizeof(int32_t) * (size_t)rows));
+    INSC_HIP(hipMalloc((void **)&g->flags, sizeof(int32_t) * (size_t)(rows + 64)));
+    g->scratch_rows = rows;
+  }
+  return INSC_OK;
+}
+
+// the insert proper: the caller has made sure that P more sites fit
+static int grid_insert_launch(insc_grid *g, const int32_t *d_coords4, int64_t P, int32_t *d_site_of_point,
+                              hipStream_t s) {
+  int rc = grid_ensure_scratch(g, P, s);
+  if (rc) return rc;
+  const int64_t mask = g->n_slots - 1;
+  const unsigned nb = grid_for(P, 256);
+  int32_t *total = g->flags + g->scratch_rows;  // spare int after the flags
+  hipLaunchKernelGGL(grid_claim_kernel, dim3(nb), dim3(256), 0, s, g->table, mask, d_coords4, P, g->slot_of_point,
+                     g->d_err);
+  hipLaunchKernelGGL(grid_flag_kernel, dim3(nb), dim3(256), 0, s, g->table, g->slot_of_point, P, g->flags);
+  INSC_LAUNCH_CHECK();
+  rc = scan_exclusive_i32(g->flags, g->flags, P, total, s);
+  if (rc) return rc;
+  hipLaunchKernelGGL(grid_assign_kernel, dim3(nb), dim3(256), 0, s, g->table, d_coords4, g->slot_of_point, g->flags,
+                     P, g->d_n, g->coords, g->capacity_sites, g->d_err);
+  hipLaunchKernelGGL(grid_resolve_kernel, dim3(nb), dim3(256), 0, s, g->table, g->slot_of_point, P, d_site_of_point,
+                     g->d_n, total);
+  hipLaunchKernelGGL(grid_bump_kernel, dim3(1), dim3(1), 0, s, g->d_n, total);
+  INSC_LAUNCH_CHECK();
+  g->n_upper += P;
+  g->n_exact = -1;
+  return INSC_OK;
+}
+
+int grid_insert_nosync(insc_grid *g, const int32_t *d_coords4, int64_t P, int32_t *d_site_of_point, hipStream_t s) {
+  if (P <= 0) return INSC_OK;
+  if (g->n_upper + P > g->capacity_sites) {
+    set_error("grid_insert_nosync: %lld sites + %lld points exceed capacity %lld", (long long)g->n_upper,
+              (long long)P, (long long)g->capacity_sites);
+    return INSC_ERR_CAPACITY;
+  }
+  return grid_insert_launch(g, d_coords4, P, d_site_of_point, s);
+}
+
+int ssc3_new_sites(const insc_grid *g, int32_t *d_nbr, int64_t n_new_upper, hipStream_t s) {
+  if (n_new_upper <= 0) return INSC_OK;
+  hipLaunchKernelGGL(ssc3_nbr_new_kernel, dim3(grid_for(n_new_upper * 27, 256, 1ll << 30)), dim3(256), 0, s, g->table,
+                     g->n_slots - 1, g->coords, g->d_n, d_nbr);
+  INSC_LAUNCH_CHECK();
+  return INSC_OK;
+}
+
+int down2_new_sites(const insc_grid *fine, insc_grid *coarse, int64_t n_new_upper, int32_t *d_parent,
+                    int32_t *d_offset, int32_t *d_child, hipStream_t s) {
+  if (n_new_upper <= 0) return INSC_OK;
+  void *ws;
+  int rc = workspace(WS_API, s, sizeof(int32_t) * 5 * (size_t)n_new_upper, &ws);
+  if (rc) return rc;
+  int32_t *half = (int32_t *)ws;
+  int32_t *parent_tmp = half + 4 * n_new_upper;
+  const unsigned nb = grid_for(n_new_upper, 256);
+  hipLaunchKernelGGL(down2_coords_new_kernel, dim3(nb), dim3(256), 0, s, fine->coords, fine->d_n, n_new_upper, half,
+                     d_offset);
+  INSC_LAUNCH_CHECK();
+  rc = grid_insert_nosync(coarse, half, n_new_upper, parent_tmp, s);
+  if (rc) return rc;
+  hipLaunchKernelGGL(down2_link_new_kernel, dim3(nb), dim3(256), 0, s, parent_tmp, fine->d_n, d_parent, d_offset,
+                     d_child);
+  INSC_LAUNCH_CHECK();
+  return INSC_OK;
+}
+
+int order_append_new_sites(const insc_grid *g, int32_t *d_order, int32_t *d_pos, int64_t n_new_upper, hipStream_t s) {
+  if (n_new_upper <= 0) return INSC_OK;
+  hipLaunchKernelGGL(order_append_kernel, dim3(grid_for(n_new_upper, 256)), dim3(256), 0, s, g->d_n, d_order, d_pos);
+  INSC_LAUNCH_CHECK();
   return INSC_OK;
 }
 
@@ -349,33 +467,8 @@ int insc_grid_insert(insc_grid *g, const int32_t *d_coords4, int64_t P, int32_t 
         if (rc) return rc;
       }
     }
-    if (g->scratch_rows < P) {
-      INSC_HIP(hipStreamSynchronize(s));
-      if (g->slot_of_point) INSC_HIP(hipFree(g->slot_of_point));
-      if (g->flags) INSC_HIP(hipFree(g->flags));
-      g->slot_of_point = g->flags = nullptr;
-      int64_t rows = P + P / 2;
-      INSC_HIP(hipMalloc((void **)&g->slot_of_point, sizeof(int32_t) * (size_t)rows));
-      INSC_HIP(hipMalloc((void **)&g->flags, sizeof(int32_t) * (size_t)(rows + 64)));
-      g->scratch_rows = rows;
-    }
-    const int64_t mask = g->n_slots - 1;
-    const unsigned nb = grid_for(P, 256);
-    int32_t *total = g->flags + g->scratch_rows;  // spare int after the flags
-    hipLaunchKernelGGL(grid_claim_kernel, dim3(nb), dim3(256), 0, s, g->table, mask, d_coords4, P, g->slot_of_point,
-                       g->d_err);
-    hipLaunchKernelGGL(grid_flag_kernel, dim3(nb), dim3(256), 0, s, g->table, g->slot_of_point, P, g->flags);
-    INSC_LAUNCH_CHECK();
-    int rc = scan_exclusive_i32(g->flags, g->flags, P, total, s);
+    int rc = grid_insert_launch(g, d_coords4, P, d_site_of_point, s);
     if (rc) return rc;
-    hipLaunchKernelGGL(grid_assign_kernel, dim3(nb), dim3(256), 0, s, g->table, d_coords4, g->slot_of_point, g->flags,
-                       P, g->d_n, g->coords, g->capacity_sites, g->d_err);
-    hipLaunchKernelGGL(grid_resolve_kernel, dim3(nb), dim3(256), 0, s, g->table, g->slot_of_point, P,
-                       d_site_of_point, g->d_n, total);
-    hipLaunchKernelGGL(grid_bump_kernel, dim3(1), dim3(1), 0, s, g->d_n, total);
-    INSC_LAUNCH_CHECK();
-    g->n_upper += P;
-    g->n_exact = -1;
   }
   if (h_n_sites) {
     int rc = grid_sync_errors(g, s, "insc_grid_insert");

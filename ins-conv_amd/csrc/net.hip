@@ -1,0 +1,841 @@
+// Network executor: runs a whole sparse U-Net style network, full or incremental, from one
+// host call.  It owns the per-scale hash grids, rulebooks, cached feature matrices and the
+// dirty-set bookkeeping, and enqueues every kernel of a frame back to back on one stream with
+// no host round trip inside an incremental frame.
+//
+// The reference keeps this state spread over Python module attributes (save_meta,
+// save_input_feats, save_output: sparseconvnet/submanifoldConvolution.py:53-54,
+// batchNormalization.py:60-61, ioLayers.py:69,106-107) and a Metadata object per frame
+// (Metadata/Metadata.h:218-386); here it is one object with an explicit program.
+#include <algorithm>
+#include <map>
+#include <set>
+#include <vector>
+
+#include "common.h"
+#include "grid.h"
+
+namespace insc {
+
+enum OpKind { OP_SSC, OP_BN, OP_CONV, OP_DECONV, OP_NIN, OP_ADD, OP_COPY, OP_JOIN };
+enum DirtyKind { D_INPUT, D_DILATE, D_PARENTS, D_CHILDREN, D_UNION };
+
+struct Level {
+  insc_grid *grid = nullptr;
+  int64_t cap = 0;
+  int32_t *nbr = nullptr;       // [cap,27]
+  int32_t *order = nullptr;     // [cap] processing order of the 3^3 convolutions
+  int32_t *pos = nullptr;       // [cap] inverse of order
+  int32_t *parent = nullptr;    // [cap] site at the next coarser level
+  int32_t *offset = nullptr;    // [cap] position inside the parent cell
+  int32_t *child = nullptr;     // [cap_coarse,8] (owned by the FINE level's link)
+  int64_t child_rows = 0;
+  int32_t *bo_order = nullptr;  // [cap] fine sites grouped by offset (deconvolution order)
+  int32_t *bo_pos = nullptr;    // [cap]
+  int64_t n = 0;                // exact count after the last completed frame
+  int64_t n_upper = 0;          // bound valid during the frame being enqueued
+  int64_t new_upper = 0;        // bound on sites added in this frame
+};
+
+struct Buffer {
+  int level = 0;
+  int ld = 0;
+  float *p = nullptr;
+  int64_t rows = 0;
+};
+
+struct Tensor {
+  int level = 0, C = 0, buf = -1, col0 = 0, dirty = -1;
+};
+
+struct Op {
+  int kind = 0, in0 = -1, in1 = -1, out = -1;
+  const float *W = nullptr, *bias = nullptr, *mean = nullptr, *var = nullptr, *gamma = nullptr, *beta = nullptr;
+  float *Wp = nullptr;  // packed weights, owned
+  float eps = 0, leak = 0;
+  int Cin = 0, Cout = 0;
+};
+
+struct DirtyNode {
+  int kind = 0, level = 0, src0 = -1, src1 = -1;
+  bool tiles_by_offset = false;  // tile flags follow the deconvolution order
+  uint8_t *mask = nullptr;       // [cap] one byte per site
+  uint8_t *tflag = nullptr;      // [cap/32+1] one byte per 32-row tile of the level's order
+  uint8_t *tflag_bo = nullptr;   // same for the by-offset order (only if some deconvolution needs it)
+  std::set<int> ancestors;
+};
+
+}  // namespace insc
+
+struct insc_net {
+  int n_levels = 0, in_channels = 0, mode = 4;
+  bool finalized = false, have_state = false;
+  std::vector<insc::Level> levels;
+  std::vector<insc::Buffer> buffers;
+  std::vector<insc::Tensor> tensors;
+  std::vector<insc::Op> ops;
+  std::vector<insc::DirtyNode> dirty;
+  std::map<std::vector<int>, int> dirty_index;
+  // input layer state
+  float *in_sum = nullptr;
+  int32_t *in_cnt = nullptr;
+  int32_t *chain_head = nullptr;  // [cap0] per-site list head, -1 when idle
+  int32_t *chain_next = nullptr;  // [points_cap]
+  int32_t *site_of_point = nullptr;  // all points since the last full frame
+  int64_t points_cap = 0, n_points = 0, n_points_frame = 0;
+  uint8_t *mask_arena = nullptr;
+  size_t mask_arena_bytes = 0;
+  int32_t *h_counts = nullptr;  // pinned: per level count, error flags
+  int out_tensor = -1;
+};
+
+namespace insc {
+
+// -----------------------------------------------------------------------------------------
+// kernels private to the executor
+// -----------------------------------------------------------------------------------------
+__global__ void invert_perm_kernel(const int32_t *__restrict__ order, int64_t n, int32_t *__restrict__ pos) {
+  int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t < n) pos[order[t]] = (int)t;
+}
+
+// Input layer, step 1: thread p pushes itself on the list of its site.
+__global__ void chain_push_kernel(const int32_t *__restrict__ sop, int64_t P, int32_t *__restrict__ head,
+                                  int32_t *__restrict__ next) {
+  int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (p >= P) return;
+  const int s = sop[p];
+  next[p] = (s >= 0) ? atomicExch(&head[s], (int)p) : -1;
+}
+
+// Input layer, step 2: the row left at the head of a site's list owns the site.  It adds the
+// rows of the list to the running sum in ascending row order (the order InputLayer_fp_ visits
+// them, CUDA/IOLayers.cu:17-32) and resets the head.  Lists are short (rows of one voxel in one
+// frame); each pass picks the smallest row index not yet added.
+__global__ void chain_sum_kernel(const float *__restrict__ feats, int C, const int32_t *__restrict__ sop, int64_t P,
+                                 int32_t *__restrict__ head, const int32_t *__restrict__ next,
+                                 float *__restrict__ sum, int32_t *__restrict__ cnt, uint8_t *__restrict__ mask,
+                                 uint8_t *__restrict__ tflag, const int32_t *__restrict__ pos) {
+  int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (p >= P) return;
+  const int s = sop[p];
+  if (s < 0 || head[s] != (int)p) return;
+  int done = -1, n = 0;
+  for (;;) {
+    int best = 0x7fffffff;
+    for (int q = (int)p; q >= 0; q = next[q])
+      if (q > done && q < best) best = q;
+    if (best == 0x7fffffff) break;
+    for (int c = 0; c < C; c++) sum[(int64_t)s * C + c] += feats[(int64_t)best * C + c];
+    done = best;
+    n++;
+  }
+  cnt[s] += n;
+  head[s] = -1;
+  if (mask) {
+    mask[s] = 1;
+    tflag[pos[s] >> 5] = 1;
+  }
+}
+
+__global__ void dirty_dilate_kernel(const int32_t *__restrict__ nbr, const uint8_t *__restrict__ mask_in,
+                                    uint8_t *__restrict__ mask_out, uint8_t *__restrict__ tflag,
+                                    const int32_t *__restrict__ pos, uint8_t *__restrict__ tflag_bo,
+                                    const int32_t *__restrict__ bo_pos, const int32_t *__restrict__ d_n,
+                                    int64_t n_upper) {
+  const int64_t n = min((int64_t)*d_n, n_upper);
+  int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= n * 27) return;
+  if (!mask_in[t / 27]) return;
+  const int j = nbr[t];
+  if (j < 0) return;
+  mask_out[j] = 1;
+  tflag[pos[j] >> 5] = 1;
+  if (tflag_bo) tflag_bo[bo_pos[j] >> 5] = 1;
+}
+
+__global__ void dirty_parents_kernel(const int32_t *__restrict__ parent, const uint8_t *__restrict__ mask_fine,
+                                     uint8_t *__restrict__ mask_out, uint8_t *__restrict__ tflag,
+                                     const int32_t *__restrict__ pos, const int32_t *__restrict__ d_n_fine,
+                                     int64_t n_upper) {
+  const int64_t n = min((int64_t)*d_n_fine, n_upper);
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n || !mask_fine[i]) return;
+  const int j = parent[i];
+  if (j < 0) return;
+  mask_out[j] = 1;
+  tflag[pos[j] >> 5] = 1;
+}
+
+__global__ void dirty_children_kernel(const int32_t *__restrict__ parent, const uint8_t *__restrict__ mask_coarse,
+                                      uint8_t *__restrict__ mask_out, uint8_t *__restrict__ tflag,
+                                      const int32_t *__restrict__ pos, uint8_t *__restrict__ tflag_bo,
+                                      const int32_t *__restrict__ bo_pos, const int32_t *__restrict__ d_n_fine,
+                                      int64_t n_upper) {
+  const int64_t n = min((int64_t)*d_n_fine, n_upper);
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const int j = parent[i];
+  if (j < 0 || !mask_coarse[j]) return;
+  mask_out[i] = 1;
+  tflag[pos[i] >> 5] = 1;
+  if (tflag_bo) tflag_bo[bo_pos[i] >> 5] = 1;
+}
+
+__global__ void dirty_union_kernel(const uint8_t *__restrict__ a, const uint8_t *__restrict__ b,
+                                   uint8_t *__restrict__ mask_out, uint8_t *__restrict__ tflag,
+                                   const int32_t *__restrict__ pos, uint8_t *__restrict__ tflag_bo,
+                                   const int32_t *__restrict__ bo_pos, const int32_t *__restrict__ d_n,
+                                   int64_t n_upper) {
+  const int64_t n = min((int64_t)*d_n, n_upper);
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n || !(a[i] | b[i])) return;
+  mask_out[i] = 1;
+  tflag[pos[i] >> 5] = 1;
+  if (tflag_bo) tflag_bo[bo_pos[i] >> 5] = 1;
+}
+
+__global__ void fill_bytes_kernel(uint4 *p, size_t n16) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (; i < n16; i += stride) p[i] = make_uint4(0, 0, 0, 0);
+}
+
+__global__ void gather_out_kernel(const float *__restrict__ in, int64_t ld_in, const int32_t *__restrict__ sop,
+                                  int64_t P, int C, float *__restrict__ out) {
+  for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < P * C; e += (int64_t)gridDim.x * 256) {
+    const int64_t p = e / C;
+    const int c = (int)(e - p * C);
+    const int s = sop[p];
+    out[e] = (s >= 0) ? in[(int64_t)s * ld_in + c] : 0.0f;
+  }
+}
+
+__global__ void coords_to_int4_kernel(const int32_t *__restrict__ in, int cols, int64_t P, int32_t *__restrict__ out) {
+  int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (p >= P) return;
+  const int32_t *c = in + p * cols;
+  reinterpret_cast<int4 *>(out)[p] = make_int4(c[0], c[1], c[2], cols > 3 ? c[3] : 0);
+}
+
+// -----------------------------------------------------------------------------------------
+// host side
+// -----------------------------------------------------------------------------------------
+template <typename T>
+static int dev_alloc(T **p, size_t count) {
+  *p = nullptr;
+  if (count == 0) count = 1;
+  INSC_HIP(hipMalloc((void **)p, sizeof(T) * count));
+  return INSC_OK;
+}
+
+template <typename T>
+static int dev_grow(T **p, size_t old_count, size_t new_count, hipStream_t s) {
+  T *q = nullptr;
+  INSC_HIP(hipMalloc((void **)&q, sizeof(T) * (new_count ? new_count : 1)));
+  if (*p && old_count) INSC_HIP(hipMemcpyAsync(q, *p, sizeof(T) * old_count, hipMemcpyDeviceToDevice, s));
+  INSC_HIP(hipStreamSynchronize(s));
+  if (*p) INSC_HIP(hipFree(*p));
+  *p = q;
+  return INSC_OK;
+}
+
+static int fill_i32(int32_t *p, int64_t n, int32_t v, hipStream_t s) { return insc_fill_i32(p, n, v, (void *)s); }
+
+static float *tensor_ptr(insc_net *net, int t) {
+  const Tensor &T = net->tensors[t];
+  return net->buffers[T.buf].p + T.col0;
+}
+static int64_t tensor_ld(insc_net *net, int t) { return net->buffers[net->tensors[t].buf].ld; }
+
+static int dirty_node(insc_net *net, int kind, int level, int a, int b) {
+  std::vector<int> key = {kind, level, a, b};
+  auto it = net->dirty_index.find(key);
+  if (it != net->dirty_index.end()) return it->second;
+  DirtyNode d;
+  d.kind = kind;
+  d.level = level;
+  d.src0 = a;
+  d.src1 = b;
+  if (a >= 0) d.ancestors = net->dirty[a].ancestors;
+  if (b >= 0) d.ancestors.insert(net->dirty[b].ancestors.begin(), net->dirty[b].ancestors.end());
+  const int id = (int)net->dirty.size();
+  d.ancestors.insert(id);
+  net->dirty.push_back(d);
+  net->dirty_index[key] = id;
+  return id;
+}
+
+// Every propagation rule only grows a set, so a set derived from another contains it and the
+// union of the two is the derived one.
+static int dirty_union(insc_net *net, int a, int b) {
+  if (a == b) return a;
+  if (net->dirty[b].ancestors.count(a)) return b;
+  if (net->dirty[a].ancestors.count(b)) return a;
+  return dirty_node(net, D_UNION, net->dirty[a].level, std::min(a, b), std::max(a, b));
+}
+
+// (re)allocate everything that is sized by the capacity of level l
+static int level_reserve(insc_net *net, int l, int64_t cap, hipStream_t s) {
+  Level &L = net->levels[l];
+  if (cap <= L.cap) return INSC_OK;
+  cap = std::max<int64_t>(cap, 1024);
+  cap = (cap + 31) / 32 * 32;
+  int rc;
+  if (!L.grid) {
+    rc = insc_grid_create(cap, &L.grid);
+  } else {
+    rc = insc_grid_reserve(L.grid, cap, (void *)s);
+  }
+  if (rc) return rc;
+  const int64_t old = L.cap;
+  if ((rc = dev_grow(&L.nbr, (size_t)old * 27, (size_t)cap * 27, s))) return rc;
+  if ((rc = dev_grow(&L.order, (size_t)old, (size_t)cap, s))) return rc;
+  if ((rc = dev_grow(&L.pos, (size_t)old, (size_t)cap, s))) return rc;
+  if (l + 1 < net->n_levels) {
+    if ((rc = dev_grow(&L.parent, (size_t)old, (size_t)cap, s))) return rc;
+    if ((rc = dev_grow(&L.offset, (size_t)old, (size_t)cap, s))) return rc;
+    if ((rc = dev_grow(&L.bo_order, (size_t)old, (size_t)cap, s))) return rc;
+    if ((rc = dev_grow(&L.bo_pos, (size_t)old, (size_t)cap, s))) return rc;
+  }
+  if (l > 0) {  // child map of the link from the finer level has one row per site of this level
+    Level &F = net->levels[l - 1];
+    if ((rc = dev_grow(&F.child, (size_t)F.child_rows * 8, (size_t)cap * 8, s))) return rc;
+    if ((rc = fill_i32(F.child + F.child_rows * 8, (cap - F.child_rows) * 8, -1, s))) return rc;
+    F.child_rows = cap;
+  }
+  if (l == 0) {
+    if ((rc = dev_grow(&net->in_sum, (size_t)old * net->in_channels, (size_t)cap * net->in_channels, s))) return rc;
+    if ((rc = dev_grow(&net->in_cnt, (size_t)old, (size_t)cap, s))) return rc;
+    if ((rc = dev_grow(&net->chain_head, (size_t)old, (size_t)cap, s))) return rc;
+    INSC_HIP(hipMemsetAsync(net->in_sum + old * net->in_channels, 0, sizeof(float) * (cap - old) * net->in_channels, s));
+    INSC_HIP(hipMemsetAsync(net->in_cnt + old, 0, sizeof(int32_t) * (cap - old), s));
+    if ((rc = fill_i32(net->chain_head + old, cap - old, -1, s))) return rc;
+  }
+  for (Buffer &B : net->buffers)
+    if (B.level == l) {
+      if ((rc = dev_grow(&B.p, (size_t)B.rows * B.ld, (size_t)cap * B.ld, s))) return rc;
+      B.rows = cap;
+    }
+  L.cap = cap;
+  // masks of this level live in the arena: rebuild it
+  size_t bytes = 0;
+  for (DirtyNode &d : net->dirty) {
+    const int64_t c = net->levels[d.level].cap;
+    bytes += ((size_t)c + 255) / 256 * 256 * 1 + 3 * (((size_t)c / 32 + 1 + 255) / 256 * 256);
+  }
+  if (bytes > net->mask_arena_bytes) {
+    INSC_HIP(hipStreamSynchronize(s));
+    if (net->mask_arena) INSC_HIP(hipFree(net->mask_arena));
+    INSC_HIP(hipMalloc((void **)&net->mask_arena, bytes));
+    net->mask_arena_bytes = bytes;
+  }
+  size_t off = 0;
+  for (DirtyNode &d : net->dirty) {
+    const size_t c = (size_t)net->levels[d.level].cap;
+    const size_t mb = (c + 255) / 256 * 256, tb = (c / 32 + 1 + 255) / 256 * 256;
+    d.mask = net->mask_arena + off;
+    d.tflag = d.mask + mb;
+    d.tflag_bo = d.tflag + tb;
+    off += mb + 3 * tb;
+  }
+  return INSC_OK;
+}
+
+static int points_reserve(insc_net *net, int64_t need, hipStream_t s) {
+  if (need <= net->points_cap) return INSC_OK;
+  const int64_t cap = std::max<int64_t>(need + need / 2, 4096);
+  int rc;
+  if ((rc = dev_grow(&net->site_of_point, (size_t)net->n_points, (size_t)cap, s))) return rc;
+  if ((rc = dev_grow(&net->chain_next, 0, (size_t)cap, s))) return rc;
+  net->points_cap = cap;
+  return INSC_OK;
+}
+
+static int sync_counts(insc_net *net, hipStream_t s, const char *who) {
+  const int L = net->n_levels;
+  for (int l = 0; l < L; l++) {
+    INSC_HIP(hipMemcpyAsync(net->h_counts + 2 * l, net->levels[l].grid->d_n, sizeof(int32_t),
+                            hipMemcpyDeviceToHost, s));
+    INSC_HIP(hipMemcpyAsync(net->h_counts + 2 * l + 1, net->levels[l].grid->d_err, sizeof(int32_t),
+                            hipMemcpyDeviceToHost, s));
+  }
+  INSC_HIP(hipStreamSynchronize(s));
+  for (int l = 0; l < L; l++) {
+    Level &Lv = net->levels[l];
+    Lv.n = Lv.n_upper = net->h_counts[2 * l];
+    Lv.grid->n_exact = Lv.grid->n_upper = Lv.n;
+    const int err = net->h_counts[2 * l + 1];
+    if (err & 1) {
+      set_error("%s: a coordinate is outside 0..65535 (batch 0..32767)", who);
+      return INSC_ERR_COORD;
+    }
+    if (err & 2) {
+      set_error("%s: capacity of scale %d exceeded", who, l);
+      return INSC_ERR_CAPACITY;
+    }
+  }
+  return INSC_OK;
+}
+
+// ---- one layer ------------------------------------------------------------------------
+static int run_op(insc_net *net, const Op &op, bool incremental, hipStream_t s) {
+  const Tensor &To = net->tensors[op.out];
+  const Level &Lo = net->levels[To.level];
+  const DirtyNode *d = incremental ? &net->dirty[To.dirty] : nullptr;
+  const int32_t *d_n = Lo.grid->d_n;
+  const int64_t n_up = Lo.n_upper;
+  float *out = tensor_ptr(net, op.out);
+  const int64_t ld_out = tensor_ld(net, op.out);
+  const float *in0 = tensor_ptr(net, op.in0);
+  const int64_t ld0 = tensor_ld(net, op.in0);
+  switch (op.kind) {
+    case OP_SSC:
+      return launch_conv(in0, ld0, out, ld_out, op.W, op.Wp, op.bias, Lo.nbr, nullptr, MAP_NBR, 27, Lo.order, d_n,
+                         n_up, op.Cin, op.Cout, d ? d->tflag : nullptr, d ? d->mask : nullptr, s);
+    case OP_NIN:
+      return launch_conv(in0, ld0, out, ld_out, op.W, op.Wp, op.bias, nullptr, nullptr, MAP_IDENTITY, 1, Lo.order,
+                         d_n, n_up, op.Cin, op.Cout, d ? d->tflag : nullptr, d ? d->mask : nullptr, s);
+    case OP_CONV: {
+      const Level &Lf = net->levels[To.level - 1];
+      return launch_conv(in0, ld0, out, ld_out, op.W, op.Wp, op.bias, Lf.child, nullptr, MAP_NBR, 8, Lo.order, d_n,
+                         n_up, op.Cin, op.Cout, d ? d->tflag : nullptr, d ? d->mask : nullptr, s);
+    }
+    case OP_DECONV:
+      return launch_conv(in0, ld0, out, ld_out, op.W, op.Wp, op.bias, Lo.parent, Lo.offset, MAP_PARENT, 8,
+                         Lo.bo_order, d_n, n_up, op.Cin, op.Cout, d ? d->tflag_bo : nullptr, d ? d->mask : nullptr,
+                         s);
+    case OP_BN:
+      return launch_bn(in0, ld0, out, ld_out, op.mean, op.var, op.gamma, op.beta, op.eps, op.leak, nullptr, d_n,
+                       n_up, op.Cout, d ? d->mask : nullptr, s);
+    case OP_ADD:
+      return launch_add(in0, ld0, tensor_ptr(net, op.in1), tensor_ld(net, op.in1), out, ld_out, nullptr, d_n, n_up,
+                        op.Cout, d ? d->mask : nullptr, s);
+    case OP_COPY:
+      return launch_add(in0, ld0, nullptr, 0, out, ld_out, nullptr, d_n, n_up, op.Cout, d ? d->mask : nullptr, s);
+    case OP_JOIN:
+      return INSC_OK;  // the inputs are column slices of the output
+  }
+  set_error("run_op: unknown op kind %d", op.kind);
+  return INSC_ERR_STATE;
+}
+
+static int run_dirty_node(insc_net *net, int id, hipStream_t s) {
+  DirtyNode &d = net->dirty[id];
+  const Level &L = net->levels[d.level];
+  uint8_t *tbo = d.tiles_by_offset ? d.tflag_bo : nullptr;
+  switch (d.kind) {
+    case D_INPUT:
+      return INSC_OK;  // marked by the input layer
+    case D_DILATE:
+      if (L.n_upper == 0) return INSC_OK;
+      hipLaunchKernelGGL(dirty_dilate_kernel, dim3(grid_for(L.n_upper * 27, 256, 1ll << 30)), dim3(256), 0, s, L.nbr,
+                         net->dirty[d.src0].mask, d.mask, d.tflag, L.pos, tbo, L.bo_pos, L.grid->d_n, L.n_upper);
+      break;
+    case D_PARENTS: {
+      const Level &F = net->levels[d.level - 1];
+      if (F.n_upper == 0) return INSC_OK;
+      hipLaunchKernelGGL(dirty_parents_kernel, dim3(grid_for(F.n_upper, 256)), dim3(256), 0, s, F.parent,
+                         net->dirty[d.src0].mask, d.mask, d.tflag, L.pos, F.grid->d_n, F.n_upper);
+      break;
+    }
+    case D_CHILDREN:
+      if (L.n_upper == 0) return INSC_OK;
+      hipLaunchKernelGGL(dirty_children_kernel, dim3(grid_for(L.n_upper, 256)), dim3(256), 0, s, L.parent,
+                         net->dirty[d.src0].mask, d.mask, d.tflag, L.pos, tbo, L.bo_pos, L.grid->d_n, L.n_upper);
+      break;
+    case D_UNION:
+      if (L.n_upper == 0) return INSC_OK;
+      hipLaunchKernelGGL(dirty_union_kernel, dim3(grid_for(L.n_upper, 256)), dim3(256), 0, s,
+                         net->dirty[d.src0].mask, net->dirty[d.src1].mask, d.mask, d.tflag, L.pos, tbo, L.bo_pos,
+                         L.grid->d_n, L.n_upper);
+      break;
+  }
+  INSC_LAUNCH_CHECK();
+  return INSC_OK;
+}
+
+}  // namespace insc
+
+using namespace insc;
+
+extern "C" {
+
+int insc_net_create(int n_levels, int in_channels, int mode, insc_net **out) {
+  INSC_REQUIRE(out && n_levels >= 1 && n_levels <= 16 && in_channels >= 1, INSC_ERR_ARG,
+               "insc_net_create: bad arguments");
+  INSC_REQUIRE(mode == 0 || mode == 3 || mode == 4, INSC_ERR_ARG,
+               "insc_net_create: input mode %d (0, 3 and 4 are provided)", mode);
+  insc_net *net = new insc_net();
+  net->n_levels = n_levels;
+  net->in_channels = in_channels;
+  net->mode = mode;
+  net->levels.resize(n_levels);
+  // tensor 0: the input layer's output
+  Tensor t;
+  t.level = 0;
+  t.C = in_channels;
+  Buffer b;
+  b.level = 0;
+  b.ld = in_channels;
+  net->buffers.push_back(b);
+  t.buf = 0;
+  net->tensors.push_back(t);
+  INSC_HIP(hipHostMalloc((void **)&net->h_counts, sizeof(int32_t) * 64, hipHostMallocDefault));
+  *out = net;
+  return INSC_OK;
+}
+
+int insc_net_destroy(insc_net *net) {
+  if (!net) return INSC_OK;
+  (void)hipDeviceSynchronize();
+  for (Level &L : net->levels) {
+    if (L.grid) insc_grid_destroy(L.grid);
+    void *ps[] = {L.nbr, L.order, L.pos, L.parent, L.offset, L.child, L.bo_order, L.bo_pos};
+    for (void *p : ps)
+      if (p) (void)hipFree(p);
+  }
+  for (Buffer &B : net->buffers)
+    if (B.p) (void)hipFree(B.p);
+  for (Op &op : net->ops)
+    if (op.Wp) (void)hipFree(op.Wp);
+  void *ps[] = {net->in_sum, net->in_cnt, net->chain_head, net->chain_next, net->site_of_point, net->mask_arena};
+  for (void *p : ps)
+    if (p) (void)hipFree(p);
+  if (net->h_counts) (void)hipHostFree(net->h_counts);
+  delete net;
+  return INSC_OK;
+}
+
+/* New feature matrix with C channels at scale `level`; *out_id receives its id. */
+int insc_net_tensor(insc_net *net, int level, int C, int *out_id) {
+  INSC_REQUIRE(net && out_id && !net->finalized, INSC_ERR_STATE, "insc_net_tensor: net is null or finalized");
+  INSC_REQUIRE(level >= 0 && level < net->n_levels && C >= 1, INSC_ERR_ARG, "insc_net_tensor: bad level/channels");
+  Buffer b;
+  b.level = level;
+  b.ld = C;
+  net->buffers.push_back(b);
+  Tensor t;
+  t.level = level;
+  t.C = C;
+  t.buf = (int)net->buffers.size() - 1;
+  net->tensors.push_back(t);
+  *out_id = (int)net->tensors.size() - 1;
+  return INSC_OK;
+}
+
+/* Channel concatenation without copies: tensor `out` (Ca+Cb channels) is declared first, then
+ * a and b are re-homed as column slices of its matrix, so their producers write in place. */
+int insc_net_join(insc_net *net, int a, int b, int out) {
+  INSC_REQUIRE(net && !net->finalized, INSC_ERR_STATE, "insc_net_join: net is null or finalized");
+  const int nt = (int)net->tensors.size();
+  INSC_REQUIRE(a > 0 && a < nt && b > 0 && b < nt && out > 0 && out < nt && a != b, INSC_ERR_ARG,
+               "insc_net_join: bad tensor ids");
+  Tensor &A = net->tensors[a], &B = net->tensors[b], &O = net->tensors[out];
+  INSC_REQUIRE(A.level == O.level && B.level == O.level && A.C + B.C == O.C, INSC_ERR_ARG,
+               "insc_net_join: shapes do not add up");
+  INSC_REQUIRE(net->buffers[A.buf].ld == A.C && net->buffers[B.buf].ld == B.C && A.col0 == 0 && B.col0 == 0,
+               INSC_ERR_ARG, "insc_net_join: an input is already part of another join");
+  net->buffers[A.buf].ld = 0;  // the stand-alone matrices are no longer needed
+  net->buffers[B.buf].ld = 0;
+  A.buf = O.buf;
+  A.col0 = O.col0;
+  B.buf = O.buf;
+  B.col0 = O.col0 + A.C;
+  // no kernel runs for a join; the entry only carries the dirty-set rule (union of the inputs)
+  Op op;
+  op.kind = OP_JOIN;
+  op.in0 = a;
+  op.in1 = b;
+  op.out = out;
+  net->ops.push_back(op);
+  return INSC_OK;
+}
+
+static int add_op(insc_net *net, Op op) {
+  INSC_REQUIRE(net && !net->finalized, INSC_ERR_STATE, "insc_net_op: net is null or finalized");
+  const int nt = (int)net->tensors.size();
+  INSC_REQUIRE(op.in0 >= 0 && op.in0 < nt && op.out > 0 && op.out < nt && op.in1 < nt, INSC_ERR_ARG,
+               "insc_net_op: bad tensor ids");
+  net->ops.push_back(op);
+  return INSC_OK;
+}
+
+/* kind: 0 submanifold 3^3 (W [27,Cin,Cout]), 2 convolution 2/2 to the next coarser scale
+ * (W [8,Cin,Cout]), 3 deconvolution 2/2 to the next finer scale, 4 network-in-network
+ * (W [Cin,Cout]).  The weight and bias pointers must stay valid for the life of the net. */
+int insc_net_op_conv(insc_net *net, int kind, int in, int out, const float *d_W, const float *d_bias) {
+  INSC_REQUIRE(kind == OP_SSC || kind == OP_CONV || kind == OP_DECONV || kind == OP_NIN, INSC_ERR_ARG,
+               "insc_net_op_conv: bad kind %d", kind);
+  INSC_REQUIRE(net && d_W, INSC_ERR_ARG, "insc_net_op_conv: null argument");
+  const int nt = (int)net->tensors.size();
+  INSC_REQUIRE(in >= 0 && in < nt && out > 0 && out < nt, INSC_ERR_ARG, "insc_net_op_conv: bad tensor ids");
+  const Tensor &Ti = net->tensors[in], &To = net->tensors[out];
+  const int dl = kind == OP_CONV ? 1 : kind == OP_DECONV ? -1 : 0;
+  INSC_REQUIRE(To.level == Ti.level + dl, INSC_ERR_ARG, "insc_net_op_conv: scales of input and output do not fit");
+  Op op;
+  op.kind = kind;
+  op.in0 = in;
+  op.out = out;
+  op.W = d_W;
+  op.bias = d_bias;
+  op.Cin = Ti.C;
+  op.Cout = To.C;
+  return add_op(net, op);
+}
+
+int insc_net_op_bn(insc_net *net, int in, int out, const float *d_mean, const float *d_var, const float *d_gamma,
+                   const float *d_beta, float eps, float leakiness) {
+  INSC_REQUIRE(net && d_mean && d_var, INSC_ERR_ARG, "insc_net_op_bn: null argument");
+  const int nt = (int)net->tensors.size();
+  INSC_REQUIRE(in >= 0 && in < nt && out > 0 && out < nt, INSC_ERR_ARG, "insc_net_op_bn: bad tensor ids");
+  INSC_REQUIRE(net->tensors[in].C == net->tensors[out].C && net->tensors[in].level == net->tensors[out].level,
+               INSC_ERR_ARG, "insc_net_op_bn: shapes differ");
+  Op op;
+  op.kind = OP_BN;
+  op.in0 = in;
+  op.out = out;
+  op.mean = d_mean;
+  op.var = d_var;
+  op.gamma = d_gamma;
+  op.beta = d_beta;
+  op.eps = eps;
+  op.leak = leakiness;
+  op.Cin = op.Cout = net->tensors[out].C;
+  return add_op(net, op);
+}
+
+int insc_net_op_add(insc_net *net, int a, int b, int out) {
+  INSC_REQUIRE(net, INSC_ERR_ARG, "insc_net_op_add: null argument");
+  const int nt = (int)net->tensors.size();
+  INSC_REQUIRE(a >= 0 && a < nt && b >= 0 && b < nt && out > 0 && out < nt, INSC_ERR_ARG,
+               "insc_net_op_add: bad tensor ids");
+  INSC_REQUIRE(net->tensors[a].C == net->tensors[out].C && net->tensors[b].C == net->tensors[out].C &&
+                   net->tensors[a].level == net->tensors[out].level &&
+                   net->tensors[b].level == net->tensors[out].level,
+               INSC_ERR_ARG, "insc_net_op_add: shapes differ");
+  Op op;
+  op.kind = OP_ADD;
+  op.in0 = a;
+  op.in1 = b;
+  op.out = out;
+  op.Cin = op.Cout = net->tensors[out].C;
+  return add_op(net, op);
+}
+
+/* Freeze the program: derive the dirty-set dataflow, pack the weights, reserve capacity. */
+int insc_net_finalize(insc_net *net, int out_tensor, int64_t capacity_sites, void *stream) {
+  INSC_REQUIRE(net && !net->finalized, INSC_ERR_STATE, "insc_net_finalize: net is null or already finalized");
+  INSC_REQUIRE(out_tensor >= 0 && out_tensor < (int)net->tensors.size() && net->tensors[out_tensor].level == 0,
+               INSC_ERR_ARG, "insc_net_finalize: the output tensor must be at the input scale");
+  hipStream_t s = (hipStream_t)stream;
+  net->out_tensor = out_tensor;
+  // a tensor re-homed by a join whose producer is not in the program (the input) needs a copy;
+  // this cannot happen for tensor 0 because insc_net_join rejects it.
+  net->tensors[0].dirty = dirty_node(net, D_INPUT, 0, -1, -1);
+  for (Op &op : net->ops) {
+    const Tensor &Ti = net->tensors[op.in0];
+    Tensor &To = net->tensors[op.out];
+    INSC_REQUIRE(Ti.dirty >= 0, INSC_ERR_STATE, "insc_net_finalize: op reads a tensor that nothing produced");
+    switch (op.kind) {
+      case OP_SSC:
+        To.dirty = dirty_node(net, D_DILATE, To.level, Ti.dirty, -1);
+        break;
+      case OP_CONV:
+        To.dirty = dirty_node(net, D_PARENTS, To.level, Ti.dirty, -1);
+        break;
+      case OP_DECONV:
+        To.dirty = dirty_node(net, D_CHILDREN, To.level, Ti.dirty, -1);
+        net->dirty[To.dirty].tiles_by_offset = true;
+        break;
+      case OP_ADD:
+      case OP_JOIN:
+        INSC_REQUIRE(net->tensors[op.in1].dirty >= 0, INSC_ERR_STATE,
+                     "insc_net_finalize: op reads a tensor that nothing produced");
+        To.dirty = dirty_union(net, Ti.dirty, net->tensors[op.in1].dirty);
+        break;
+      default:
+        To.dirty = Ti.dirty;
+    }
+    if (op.kind == OP_SSC || op.kind == OP_CONV || op.kind == OP_DECONV || op.kind == OP_NIN) {
+      const int K = op.kind == OP_SSC ? 27 : op.kind == OP_NIN ? 1 : 8;
+      if (op.Cin % 16 == 0) {
+        const int64_t nf = packed_floats(K, op.Cin, op.Cout);
+        int rc = dev_alloc(&op.Wp, (size_t)nf);
+        if (rc) return rc;
+        rc = pack_weights(op.W, K, op.Cin, op.Cout, op.Wp, s);
+        if (rc) return rc;
+      }
+    }
+  }
+  net->finalized = true;
+  int64_t cap = std::max<int64_t>(capacity_sites, 1024);
+  for (int l = 0; l < net->n_levels; l++) {
+    int rc = level_reserve(net, l, cap, s);
+    if (rc) return rc;
+    cap = std::max<int64_t>(cap / 2, 1024);
+  }
+  INSC_HIP(hipStreamSynchronize(s));
+  return INSC_OK;
+}
+
+/* Re-pack the weights after the caller changed them in place. */
+int insc_net_refresh_weights(insc_net *net, void *stream) {
+  INSC_REQUIRE(net && net->finalized, INSC_ERR_STATE, "insc_net_refresh_weights: net is not finalized");
+  for (Op &op : net->ops)
+    if (op.Wp) {
+      const int K = op.kind == OP_SSC ? 27 : op.kind == OP_NIN ? 1 : 8;
+      int rc = pack_weights(op.W, K, op.Cin, op.Cout, op.Wp, (hipStream_t)stream);
+      if (rc) return rc;
+    }
+  return INSC_OK;
+}
+
+/* One frame.  d_coords: int32 [P, coord_cols] (x,y,z[,batch]); d_feats: float32 [P,in_channels].
+ * increment == 0: forget all state and run a full forward over these points.
+ * increment != 0: append the points to the scene of the previous frames and recompute only
+ *                 the rows they affect; the result equals a full forward over all points.
+ * d_out (nullable): one row of the output tensor per point - of this frame's points
+ * (out_all == 0, [P,C]) or of every point since the last full frame (out_all != 0).
+ * h_n_sites (nullable): receives the number of active sites at the input scale.
+ * The call returns after the frame has completed (it reads the site counts back). */
+int insc_net_forward(insc_net *net, const int32_t *d_coords, int coord_cols, const float *d_feats, int64_t P,
+                     int increment, float *d_out, int out_all, int64_t *h_n_sites, void *stream) {
+  INSC_REQUIRE(net && net->finalized, INSC_ERR_STATE, "insc_net_forward: net is not finalized");
+  INSC_REQUIRE(P >= 0 && (P == 0 || (d_coords && d_feats)) && (coord_cols == 3 || coord_cols == 4), INSC_ERR_ARG,
+               "insc_net_forward: bad arguments");
+  INSC_REQUIRE(!increment || net->have_state, INSC_ERR_STATE,
+               "insc_net_forward: incremental frame before any full frame");
+  hipStream_t s = (hipStream_t)stream;
+  const int L = net->n_levels;
+  const int C0 = net->in_channels;
+  int rc;
+  const bool inc = increment != 0;
+
+  if (!inc) {
+    for (int l = 0; l < L; l++) {
+      Level &Lv = net->levels[l];
+      if ((rc = insc_grid_clear(Lv.grid, stream))) return rc;
+      Lv.n = Lv.n_upper = 0;
+      if (l + 1 < L && Lv.child_rows)
+        if ((rc = fill_i32(Lv.child, Lv.child_rows * 8, -1, s))) return rc;
+    }
+    INSC_HIP(hipMemsetAsync(net->in_sum, 0, sizeof(float) * (size_t)net->levels[0].cap * C0, s));
+    INSC_HIP(hipMemsetAsync(net->in_cnt, 0, sizeof(int32_t) * (size_t)net->levels[0].cap, s));
+    net->n_points = 0;
+    net->have_state = false;
+  }
+  // capacity: every new point may be a new site at every scale
+  for (int l = 0; l < L; l++) {
+    Level &Lv = net->levels[l];
+    if (Lv.n + P > Lv.cap)
+      if ((rc = level_reserve(net, l, std::max(Lv.n + P, Lv.cap + Lv.cap / 2), s))) return rc;
+    Lv.new_upper = P;
+    Lv.n_upper = Lv.n + P;
+  }
+  if ((rc = points_reserve(net, net->n_points + P, s))) return rc;
+
+  if (inc && net->mask_arena_bytes) {
+    hipLaunchKernelGGL(fill_bytes_kernel, dim3(1024), dim3(256), 0, s, (uint4 *)net->mask_arena,
+                       net->mask_arena_bytes / 16);
+    INSC_LAUNCH_CHECK();
+  }
+
+  int32_t *sop = net->site_of_point + net->n_points;
+  if (P > 0) {
+    // ---- input scale: insert, accumulate --------------------------------------------------
+    void *ws;
+    if ((rc = workspace(WS_API, s, sizeof(int32_t) * 4 * (size_t)P, &ws))) return rc;
+    int32_t *c4 = (int32_t *)ws;
+    hipLaunchKernelGGL(coords_to_int4_kernel, dim3(grid_for(P, 256)), dim3(256), 0, s, d_coords, coord_cols, P, c4);
+    INSC_LAUNCH_CHECK();
+    Level &L0 = net->levels[0];
+    if ((rc = grid_insert_nosync(L0.grid, c4, P, sop, s))) return rc;
+    if ((rc = ssc3_new_sites(L0.grid, L0.nbr, P, s))) return rc;
+    if ((rc = order_append_new_sites(L0.grid, L0.order, L0.pos, P, s))) return rc;
+    DirtyNode &din = net->dirty[net->tensors[0].dirty];
+    const unsigned nb = grid_for(P, 256);
+    hipLaunchKernelGGL(chain_push_kernel, dim3(nb), dim3(256), 0, s, sop, P, net->chain_head, net->chain_next);
+    hipLaunchKernelGGL(chain_sum_kernel, dim3(nb), dim3(256), 0, s, d_feats, C0, sop, P, net->chain_head,
+                       net->chain_next, net->in_sum, net->in_cnt, inc ? din.mask : nullptr,
+                       inc ? din.tflag : nullptr, L0.pos);
+    INSC_LAUNCH_CHECK();
+    // ---- coarser scales --------------------------------------------------------------------
+    for (int l = 0; l + 1 < L; l++) {
+      Level &F = net->levels[l], &Cs = net->levels[l + 1];
+      if ((rc = down2_new_sites(F.grid, Cs.grid, P, F.parent, F.offset, F.child, s))) return rc;
+      if ((rc = order_append_new_sites(F.grid, F.bo_order, F.bo_pos, P, s))) return rc;
+      if ((rc = ssc3_new_sites(Cs.grid, Cs.nbr, P, s))) return rc;
+      if ((rc = order_append_new_sites(Cs.grid, Cs.order, Cs.pos, P, s))) return rc;
+    }
+  }
+  if (!inc) {
+    // A full frame may synchronise: learn the exact counts, then build the processing orders
+    // (pattern-sorted for the 3^3 convolutions, offset-grouped for the deconvolutions).
+    if ((rc = sync_counts(net, s, "insc_net_forward"))) return rc;
+    for (int l = 0; l < L; l++) {
+      Level &Lv = net->levels[l];
+      if (Lv.n == 0) continue;
+      if ((rc = insc_order_build(Lv.grid, Lv.nbr, 0, Lv.n, Lv.order, stream))) return rc;
+      hipLaunchKernelGGL(invert_perm_kernel, dim3(grid_for(Lv.n, 256)), dim3(256), 0, s, Lv.order, Lv.n, Lv.pos);
+      if (l + 1 < L) {
+        if ((rc = insc_order_by_offset(Lv.order, Lv.offset, Lv.n, Lv.bo_order, stream))) return rc;
+        hipLaunchKernelGGL(invert_perm_kernel, dim3(grid_for(Lv.n, 256)), dim3(256), 0, s, Lv.bo_order, Lv.n,
+                           Lv.bo_pos);
+      }
+      INSC_LAUNCH_CHECK();
+    }
+  }
+
+  // ---- input layer output ------------------------------------------------------------------
+  {
+    Level &L0 = net->levels[0];
+    const DirtyNode &din = net->dirty[net->tensors[0].dirty];
+    if ((rc = launch_input_finish(net->in_sum, net->in_cnt, net->mode, tensor_ptr(net, 0), tensor_ld(net, 0), nullptr,
+                                  L0.grid->d_n, L0.n_upper, C0, inc ? din.mask : nullptr, s)))
+      return rc;
+  }
+  // ---- dirty sets, then the layers ---------------------------------------------------------
+  if (inc)
+    for (int i = 0; i < (int)net->dirty.size(); i++)
+      if ((rc = run_dirty_node(net, i, s))) return rc;
+  for (const Op &op : net->ops)
+    if ((rc = run_op(net, op, inc, s))) return rc;
+
+  // ---- output layer ------------------------------------------------------------------------
+  const int64_t n_out_pts = out_all ? net->n_points + P : P;
+  if (d_out && n_out_pts > 0) {
+    const Tensor &To = net->tensors[net->out_tensor];
+    hipLaunchKernelGGL(gather_out_kernel, dim3(grid_for(n_out_pts * To.C, 256, 1 << 16)), dim3(256), 0, s,
+                       tensor_ptr(net, net->out_tensor), tensor_ld(net, net->out_tensor),
+                       out_all ? net->site_of_point : sop, n_out_pts, To.C, d_out);
+    INSC_LAUNCH_CHECK();
+  }
+  net->n_points += P;
+  net->have_state = true;
+  if ((rc = sync_counts(net, s, "insc_net_forward"))) return rc;
+  if (h_n_sites) *h_n_sites = net->levels[0].n;
+  return INSC_OK;
+}
+
+/* Inspection: device pointer, row stride and row count of a tensor (valid until the next
+ * frame that grows the scene past the reserved capacity). */
+int insc_net_tensor_view(insc_net *net, int tensor, float **d_ptr, int64_t *ld, int64_t *rows, int *channels) {
+  INSC_REQUIRE(net && net->finalized && tensor >= 0 && tensor < (int)net->tensors.size(), INSC_ERR_ARG,
+               "insc_net_tensor_view: bad arguments");
+  if (d_ptr) *d_ptr = tensor_ptr(net, tensor);
+  if (ld) *ld = tensor_ld(net, tensor);
+  if (rows) *rows = net->levels[net->tensors[tensor].level].n;
+  if (channels) *channels = net->tensors[tensor].C;
+  return INSC_OK;
+}
+
+int insc_net_counts(insc_net *net, int64_t *h_sites_per_level, int64_t *h_points) {
+  INSC_REQUIRE(net && net->finalized, INSC_ERR_ARG, "insc_net_counts: bad arguments");
+  if (h_sites_per_level)
+    for (int l = 0; l < net->n_levels; l++) h_sites_per_level[l] = net->levels[l].n;
+  if (h_points) *h_points = net->n_points;
+  return INSC_OK;
+}
+
+}  // extern "C"

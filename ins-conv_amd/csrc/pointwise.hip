@@ -34,7 +34,8 @@ __global__ __launch_bounds__(256) void bn_kernel(const float *__restrict__ in, i
                                                  const float *__restrict__ var, const float *__restrict__ gamma,
                                                  const float *__restrict__ beta, float eps, float leak,
                                                  const int32_t *__restrict__ rows,
-                                                 const int32_t *__restrict__ d_n_rows, int64_t n_rows, int C) {
+                                                 const int32_t *__restrict__ d_n_rows, int64_t n_rows, int C,
+                                                 const uint8_t *__restrict__ row_mask) {
   const int64_t n = row_count(d_n_rows, n_rows);
   const int groups = C / V;  // channel groups per row
   const int rpb = 256 / groups > 0 ? 256 / groups : 1;
@@ -50,7 +51,7 @@ __global__ __launch_bounds__(256) void bn_kernel(const float *__restrict__ in, i
   }
   for (int64_t t = (int64_t)blockIdx.x * rpb + lr; t < n; t += (int64_t)gridDim.x * rpb) {
     const int row = rows ? rows[t] : (int)t;
-    if (row < 0) continue;
+    if (row < 0 || (row_mask && !row_mask[row])) continue;
     typename Vec<V>::T x = Vec<V>::ld(in + (int64_t)row * ld_in + g * V);
     float *xf = reinterpret_cast<float *>(&x);
 #pragma unroll
@@ -65,13 +66,14 @@ __global__ __launch_bounds__(256) void bn_wide_kernel(const float *__restrict__ 
                                                       const float *__restrict__ mean, const float *__restrict__ var,
                                                       const float *__restrict__ gamma, const float *__restrict__ beta,
                                                       float eps, float leak, const int32_t *__restrict__ rows,
-                                                      const int32_t *__restrict__ d_n_rows, int64_t n_rows, int C) {
+                                                      const int32_t *__restrict__ d_n_rows, int64_t n_rows, int C,
+                                                      const uint8_t *__restrict__ row_mask) {
   const int64_t n = row_count(d_n_rows, n_rows);
   for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < n * C; e += (int64_t)gridDim.x * 256) {
     const int64_t t = e / C;
     const int c = (int)(e - t * C);
     const int row = rows ? rows[t] : (int)t;
-    if (row < 0) continue;
+    if (row < 0 || (row_mask && !row_mask[row])) continue;
     const float wv = (gamma ? gamma[c] : 1.0f) / sqrtf(var[c] + eps);
     const float bv = -mean[c] * wv + (beta ? beta[c] : 0.0f);
     out[(int64_t)row * ld_out + c] = leaky(in[(int64_t)row * ld_in + c] * wv + bv, leak);
@@ -83,14 +85,15 @@ template <int V, bool HAS_B>
 __global__ __launch_bounds__(256) void add_kernel(const float *__restrict__ a, int64_t ld_a,
                                                   const float *__restrict__ b, int64_t ld_b, float *__restrict__ out,
                                                   int64_t ld_out, const int32_t *__restrict__ rows,
-                                                  const int32_t *__restrict__ d_n_rows, int64_t n_rows, int C) {
+                                                  const int32_t *__restrict__ d_n_rows, int64_t n_rows, int C,
+                                                  const uint8_t *__restrict__ row_mask) {
   const int64_t n = row_count(d_n_rows, n_rows);
   const int groups = C / V;
   for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < n * groups; e += (int64_t)gridDim.x * 256) {
     const int64_t t = e / groups;
     const int g = (int)(e - t * groups);
     const int row = rows ? rows[t] : (int)t;
-    if (row < 0) continue;
+    if (row < 0 || (row_mask && !row_mask[row])) continue;
     typename Vec<V>::T x = Vec<V>::ld(a + (int64_t)row * ld_a + g * V);
     if (HAS_B) {
       typename Vec<V>::T y = Vec<V>::ld(b + (int64_t)row * ld_b + g * V);
@@ -168,13 +171,13 @@ __global__ __launch_bounds__(256) void input_finish_kernel(const float *__restri
                                                            float *__restrict__ out, int64_t ld_out,
                                                            const int32_t *__restrict__ rows,
                                                            const int32_t *__restrict__ d_n_rows, int64_t n_rows,
-                                                           int C) {
+                                                           int C, const uint8_t *__restrict__ row_mask) {
   const int64_t n = row_count(d_n_rows, n_rows);
   for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < n * C; e += (int64_t)gridDim.x * 256) {
     const int64_t t = e / C;
     const int c = (int)(e - t * C);
     const int row = rows ? rows[t] : (int)t;
-    if (row < 0) continue;
+    if (row < 0 || (row_mask && !row_mask[row])) continue;
     float v = sum[(int64_t)row * C + c];
     if (mode == 4) {
       const int k = cnt[row];
@@ -185,6 +188,64 @@ __global__ __launch_bounds__(256) void input_finish_kernel(const float *__restri
 }
 
 static inline bool vec4_ok(const void *p, int64_t ld) { return ((uintptr_t)p % 16 == 0) && (ld % 4 == 0); }
+
+int launch_bn(const float *d_in, int64_t ld_in, float *d_out, int64_t ld_out, const float *d_mean, const float *d_var,
+              const float *d_gamma, const float *d_beta, float eps, float leakiness, const int32_t *d_rows,
+              const int32_t *d_n_rows, int64_t n_rows, int C, const uint8_t *row_mask, hipStream_t s) {
+  if (n_rows == 0) return INSC_OK;
+  const bool v4 = C % 4 == 0 && vec4_ok(d_in, ld_in) && vec4_ok(d_out, ld_out);
+  const int groups = v4 ? C / 4 : C;
+  if (groups <= 256) {
+    const int rpb = 256 / groups;
+    const unsigned nb = grid_for(n_rows, rpb * 4, 1 << 16);
+    if (v4)
+      hipLaunchKernelGGL(bn_kernel<4>, dim3(nb), dim3(256), 0, s, d_in, ld_in, d_out, ld_out, d_mean, d_var, d_gamma,
+                         d_beta, eps, leakiness, d_rows, d_n_rows, n_rows, C, row_mask);
+    else
+      hipLaunchKernelGGL(bn_kernel<1>, dim3(nb), dim3(256), 0, s, d_in, ld_in, d_out, ld_out, d_mean, d_var, d_gamma,
+                         d_beta, eps, leakiness, d_rows, d_n_rows, n_rows, C, row_mask);
+  } else {
+    hipLaunchKernelGGL(bn_wide_kernel, dim3(grid_for(n_rows * C, 1024, 1 << 16)), dim3(256), 0, s, d_in, ld_in, d_out,
+                       ld_out, d_mean, d_var, d_gamma, d_beta, eps, leakiness, d_rows, d_n_rows, n_rows, C, row_mask);
+  }
+  INSC_LAUNCH_CHECK();
+  return INSC_OK;
+}
+
+int launch_add(const float *d_a, int64_t ld_a, const float *d_b, int64_t ld_b, float *d_out, int64_t ld_out,
+               const int32_t *d_rows, const int32_t *d_n_rows, int64_t n_rows, int C, const uint8_t *row_mask,
+               hipStream_t s) {
+  if (n_rows == 0) return INSC_OK;
+  const bool v4 = C % 4 == 0 && vec4_ok(d_a, ld_a) && (!d_b || vec4_ok(d_b, ld_b)) && vec4_ok(d_out, ld_out);
+  const unsigned nb = grid_for(n_rows * (v4 ? C / 4 : C), 1024, 1 << 16);
+  if (d_b) {
+    if (v4)
+      hipLaunchKernelGGL((add_kernel<4, true>), dim3(nb), dim3(256), 0, s, d_a, ld_a, d_b, ld_b, d_out, ld_out,
+                         d_rows, d_n_rows, n_rows, C, row_mask);
+    else
+      hipLaunchKernelGGL((add_kernel<1, true>), dim3(nb), dim3(256), 0, s, d_a, ld_a, d_b, ld_b, d_out, ld_out,
+                         d_rows, d_n_rows, n_rows, C, row_mask);
+  } else {
+    if (v4)
+      hipLaunchKernelGGL((add_kernel<4, false>), dim3(nb), dim3(256), 0, s, d_a, ld_a, d_b, ld_b, d_out, ld_out,
+                         d_rows, d_n_rows, n_rows, C, row_mask);
+    else
+      hipLaunchKernelGGL((add_kernel<1, false>), dim3(nb), dim3(256), 0, s, d_a, ld_a, d_b, ld_b, d_out, ld_out,
+                         d_rows, d_n_rows, n_rows, C, row_mask);
+  }
+  INSC_LAUNCH_CHECK();
+  return INSC_OK;
+}
+
+int launch_input_finish(const float *d_sum, const int32_t *d_cnt, int mode, float *d_out, int64_t ld_out,
+                        const int32_t *d_rows, const int32_t *d_n_rows, int64_t n_rows, int C,
+                        const uint8_t *row_mask, hipStream_t s) {
+  if (n_rows == 0) return INSC_OK;
+  hipLaunchKernelGGL(input_finish_kernel, dim3(grid_for(n_rows * C, 256, 1 << 16)), dim3(256), 0, s, d_sum, d_cnt,
+                     mode, d_out, ld_out, d_rows, d_n_rows, n_rows, C, row_mask);
+  INSC_LAUNCH_CHECK();
+  return INSC_OK;
+}
 
 }  // namespace insc
 
@@ -197,61 +258,23 @@ int insc_bn_leaky(const float *d_in, int64_t ld_in, float *d_out, int64_t ld_out
                   const int32_t *d_rows, const int32_t *d_n_rows, int64_t n_rows, int C, void *stream) {
   INSC_REQUIRE(n_rows >= 0 && C > 0 && ld_in >= C && ld_out >= C, INSC_ERR_ARG, "insc_bn_leaky: bad sizes");
   INSC_REQUIRE(n_rows == 0 || (d_in && d_out && d_mean && d_var), INSC_ERR_ARG, "insc_bn_leaky: null pointer");
-  if (n_rows == 0) return INSC_OK;
-  hipStream_t s = (hipStream_t)stream;
-  const bool v4 = C % 4 == 0 && vec4_ok(d_in, ld_in) && vec4_ok(d_out, ld_out);
-  const int groups = v4 ? C / 4 : C;
-  if (groups <= 256) {
-    const int rpb = 256 / groups;
-    const unsigned nb = grid_for(n_rows, rpb * 4, 1 << 16);
-    if (v4)
-      hipLaunchKernelGGL(bn_kernel<4>, dim3(nb), dim3(256), 0, s, d_in, ld_in, d_out, ld_out, d_mean, d_var, d_gamma,
-                         d_beta, eps, leakiness, d_rows, d_n_rows, n_rows, C);
-    else
-      hipLaunchKernelGGL(bn_kernel<1>, dim3(nb), dim3(256), 0, s, d_in, ld_in, d_out, ld_out, d_mean, d_var, d_gamma,
-                         d_beta, eps, leakiness, d_rows, d_n_rows, n_rows, C);
-  } else {
-    hipLaunchKernelGGL(bn_wide_kernel, dim3(grid_for(n_rows * C, 1024, 1 << 16)), dim3(256), 0, s, d_in, ld_in, d_out,
-                       ld_out, d_mean, d_var, d_gamma, d_beta, eps, leakiness, d_rows, d_n_rows, n_rows, C);
-  }
-  INSC_LAUNCH_CHECK();
-  return INSC_OK;
+  return launch_bn(d_in, ld_in, d_out, ld_out, d_mean, d_var, d_gamma, d_beta, eps, leakiness, d_rows, d_n_rows,
+                   n_rows, C, nullptr, (hipStream_t)stream);
 }
 
 int insc_add(const float *d_a, int64_t ld_a, const float *d_b, int64_t ld_b, float *d_out, int64_t ld_out,
              const int32_t *d_rows, const int32_t *d_n_rows, int64_t n_rows, int C, void *stream) {
   INSC_REQUIRE(n_rows >= 0 && C > 0 && ld_a >= C && ld_b >= C && ld_out >= C, INSC_ERR_ARG, "insc_add: bad sizes");
   INSC_REQUIRE(n_rows == 0 || (d_a && d_b && d_out), INSC_ERR_ARG, "insc_add: null pointer");
-  if (n_rows == 0) return INSC_OK;
-  hipStream_t s = (hipStream_t)stream;
-  const bool v4 = C % 4 == 0 && vec4_ok(d_a, ld_a) && vec4_ok(d_b, ld_b) && vec4_ok(d_out, ld_out);
-  const unsigned nb = grid_for(n_rows * (v4 ? C / 4 : C), 1024, 1 << 16);
-  if (v4)
-    hipLaunchKernelGGL((add_kernel<4, true>), dim3(nb), dim3(256), 0, s, d_a, ld_a, d_b, ld_b, d_out, ld_out, d_rows,
-                       d_n_rows, n_rows, C);
-  else
-    hipLaunchKernelGGL((add_kernel<1, true>), dim3(nb), dim3(256), 0, s, d_a, ld_a, d_b, ld_b, d_out, ld_out, d_rows,
-                       d_n_rows, n_rows, C);
-  INSC_LAUNCH_CHECK();
-  return INSC_OK;
+  return launch_add(d_a, ld_a, d_b, ld_b, d_out, ld_out, d_rows, d_n_rows, n_rows, C, nullptr, (hipStream_t)stream);
 }
 
 int insc_copy_rows(const float *d_in, int64_t ld_in, float *d_out, int64_t ld_out, const int32_t *d_rows,
                    const int32_t *d_n_rows, int64_t n_rows, int C, void *stream) {
   INSC_REQUIRE(n_rows >= 0 && C > 0 && ld_in >= C && ld_out >= C, INSC_ERR_ARG, "insc_copy_rows: bad sizes");
   INSC_REQUIRE(n_rows == 0 || (d_in && d_out), INSC_ERR_ARG, "insc_copy_rows: null pointer");
-  if (n_rows == 0) return INSC_OK;
-  hipStream_t s = (hipStream_t)stream;
-  const bool v4 = C % 4 == 0 && vec4_ok(d_in, ld_in) && vec4_ok(d_out, ld_out);
-  const unsigned nb = grid_for(n_rows * (v4 ? C / 4 : C), 1024, 1 << 16);
-  if (v4)
-    hipLaunchKernelGGL((add_kernel<4, false>), dim3(nb), dim3(256), 0, s, d_in, ld_in, nullptr, 0, d_out, ld_out,
-                       d_rows, d_n_rows, n_rows, C);
-  else
-    hipLaunchKernelGGL((add_kernel<1, false>), dim3(nb), dim3(256), 0, s, d_in, ld_in, nullptr, 0, d_out, ld_out,
-                       d_rows, d_n_rows, n_rows, C);
-  INSC_LAUNCH_CHECK();
-  return INSC_OK;
+  return launch_add(d_in, ld_in, nullptr, 0, d_out, ld_out, d_rows, d_n_rows, n_rows, C, nullptr,
+                    (hipStream_t)stream);
 }
 
 int insc_input_accumulate(const float *d_feats, int64_t P, int C, const int32_t *d_site_of_point, int mode,
@@ -282,11 +305,8 @@ int insc_input_finish(const float *d_sum, const int32_t *d_cnt, int mode, float 
                       const int32_t *d_rows, const int32_t *d_n_rows, int64_t n_rows, int C, void *stream) {
   INSC_REQUIRE(n_rows >= 0 && C > 0 && ld_out >= C, INSC_ERR_ARG, "insc_input_finish: bad sizes");
   INSC_REQUIRE(n_rows == 0 || (d_sum && d_cnt && d_out), INSC_ERR_ARG, "insc_input_finish: null pointer");
-  if (n_rows == 0) return INSC_OK;
-  hipLaunchKernelGGL(input_finish_kernel, dim3(grid_for(n_rows * C, 256, 1 << 16)), dim3(256), 0, (hipStream_t)stream,
-                     d_sum, d_cnt, mode, d_out, ld_out, d_rows, d_n_rows, n_rows, C);
-  INSC_LAUNCH_CHECK();
-  return INSC_OK;
+  return launch_input_finish(d_sum, d_cnt, mode, d_out, ld_out, d_rows, d_n_rows, n_rows, C, nullptr,
+                             (hipStream_t)stream);
 }
 
 int insc_output_gather(const float *d_in, int64_t ld_in, const int32_t *d_site_of_point, int64_t P, int C,

@@ -20,3 +20,4 @@ from .batchNormalization import BatchNormalization, BatchNormReLU, BatchNormLeak
 from .networkInNetwork import NetworkInNetwork  # noqa: E402
 from .networkArchitectures import UNet  # noqa: E402
 from .utils import toLongTensor, optionalTensor  # noqa: E402
+from .compiled import compile, CompiledNet  # noqa: E402

@@ -46,6 +46,19 @@ _SIGS = {
     "insc_dirty_children": [vp, vp, vp, vp, c_i64, vp],
     "insc_dirty_or": [vp, vp, vp, vp, c_i64, vp],
     "insc_dirty_compact": [vp, vp, vp, c_i64, vp, vp, ctypes.POINTER(c_i64), vp],
+    "insc_net_create": [c_int, c_int, c_int, ctypes.POINTER(vp)],
+    "insc_net_destroy": [vp],
+    "insc_net_tensor": [vp, c_int, c_int, ctypes.POINTER(c_int)],
+    "insc_net_join": [vp, c_int, c_int, c_int],
+    "insc_net_op_conv": [vp, c_int, c_int, c_int, vp, vp],
+    "insc_net_op_bn": [vp, c_int, c_int, vp, vp, vp, vp, c_f32, c_f32],
+    "insc_net_op_add": [vp, c_int, c_int, c_int],
+    "insc_net_finalize": [vp, c_int, c_i64, vp],
+    "insc_net_refresh_weights": [vp, vp],
+    "insc_net_forward": [vp, vp, c_int, vp, c_i64, c_int, vp, c_int, ctypes.POINTER(c_i64), vp],
+    "insc_net_tensor_view": [vp, c_int, ctypes.POINTER(vp), ctypes.POINTER(c_i64), ctypes.POINTER(c_i64),
+                             ctypes.POINTER(c_int)],
+    "insc_net_counts": [vp, ctypes.POINTER(c_i64), ctypes.POINTER(c_i64)],
     "insc_scan_exclusive_i32": [vp, vp, c_i64, vp, vp],
     "insc_sort_pairs_u64": [vp, vp, c_i64, c_int, vp],
 }

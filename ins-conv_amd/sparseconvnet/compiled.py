@@ -1,0 +1,152 @@
+"""Run a sparseconvnet module tree through the native network executor (insc_net_*).
+
+    net = scn.compile(sparse_model)          # Sequential starting with InputLayer, ending with OutputLayer
+    feats = net([coords, features, batch], increment=False)     # same call shape as the module
+    feats = net([new_coords, new_features, batch], increment=True)
+
+The module path issues one C call per layer from Python; this path hands the whole frame to
+one C call, so an incremental frame costs a few hundred kernel launches and no Python work.
+Results are bit-identical to the module path.  Parameters are read in place (device
+pointers); after modifying weights call `refresh()`.
+"""
+import ctypes
+
+import torch
+
+from . import SCN
+from ._lib import ensure_init, lib, ptr, stream_ptr
+
+I64 = ctypes.c_int64
+_KIND = {"ssc": 0, "conv": 2, "deconv": 3, "nin": 4}
+
+
+class CompiledNet(object):
+    def __init__(self, model, capacity_sites=1 << 18):
+        import sparseconvnet as scn
+
+        mods = list(model)
+        if not (isinstance(mods[0], scn.InputLayer) and isinstance(mods[-1], scn.OutputLayer)):
+            raise ValueError("the model must start with an InputLayer and end with an OutputLayer")
+        self.model = model
+        self.input_layer, self.output_layer = mods[0], mods[-1]
+        self.device = next(model.parameters()).device
+        if self.device.type != "cuda":
+            raise ValueError("move the model to the GPU before compiling it")
+        ensure_init(self.device.index or 0)
+        levels = 1 + sum(1 for m in model.modules() if isinstance(m, scn.Convolution))
+        first = next(m for m in model.modules() if hasattr(m, "nIn") or hasattr(m, "nPlanes"))
+        self.in_channels = getattr(first, "nIn", None) or first.nPlanes
+        self.h = ctypes.c_void_p()
+        lib.insc_net_create(levels, int(self.in_channels), int(self.input_layer.mode), ctypes.byref(self.h))
+        self._keep = []  # tensors whose storage the executor points into
+        self._level = {0: 0}
+        self._chan = {0: self.in_channels}
+        x = 0
+        for m in mods[1:-1]:
+            x = self._trace(m, x)
+        self.out_tensor = x
+        self.out_channels = self._chan[x]
+        lib.insc_net_finalize(self.h, int(x), I64(int(capacity_sites)), stream_ptr())
+
+    def __del__(self):
+        try:
+            if self.h:
+                lib.insc_net_destroy(self.h)
+                self.h = ctypes.c_void_p()
+        except Exception:
+            pass
+
+    # ---- tracing --------------------------------------------------------------------------
+    def _new(self, level, C):
+        t = ctypes.c_int(0)
+        lib.insc_net_tensor(self.h, int(level), int(C), ctypes.byref(t))
+        self._level[t.value], self._chan[t.value] = level, C
+        return t.value
+
+    def _dev(self, t):
+        if t is None:
+            return None
+        t = t.detach()
+        if not t.is_contiguous():
+            raise ValueError("parameters must be contiguous")
+        self._keep.append(t)
+        return ptr(t)
+
+    def _trace(self, m, x):
+        import sparseconvnet as scn
+
+        if isinstance(m, scn.ConcatTable):
+            return [self._trace(c, x) for c in m._modules.values()]
+        if isinstance(m, scn.Sequential):
+            for c in m:
+                x = self._trace(c, x)
+            return x
+        if isinstance(m, scn.Identity):
+            return x
+        if isinstance(m, scn.AddTable):
+            out = x[0]
+            for t in x[1:]:
+                o = self._new(self._level[out], self._chan[out])
+                lib.insc_net_op_add(self.h, out, t, o)
+                out = o
+            return out
+        if isinstance(m, scn.JoinTable):
+            if len(x) != 2:
+                raise NotImplementedError("JoinTable of two inputs")
+            o = self._new(self._level[x[0]], self._chan[x[0]] + self._chan[x[1]])
+            lib.insc_net_join(self.h, x[0], x[1], o)
+            return o
+        bias = getattr(m, "bias", None)
+        if isinstance(m, scn.BatchNormalization):
+            o = self._new(self._level[x], m.nPlanes)
+            lib.insc_net_op_bn(self.h, x, o, self._dev(m.running_mean), self._dev(m.running_var),
+                               self._dev(getattr(m, "weight", None)), self._dev(bias), ctypes.c_float(m.eps),
+                               ctypes.c_float(m.leakiness))
+            return o
+        if isinstance(m, scn.SubmanifoldConvolution):
+            if SCN._key(m.filter_size) != (3, 3, 3) or m.dilated_rate != 1:
+                raise NotImplementedError("3x3x3 submanifold convolutions with dilated_rate 1")
+            kind, dl = "ssc", 0
+        elif isinstance(m, scn.Convolution):
+            SCN._check_down(m.filter_size, m.filter_stride)
+            kind, dl = "conv", 1
+        elif isinstance(m, scn.Deconvolution):
+            SCN._check_down(m.filter_size, m.filter_stride)
+            kind, dl = "deconv", -1
+        elif isinstance(m, scn.NetworkInNetwork):
+            kind, dl = "nin", 0
+        else:
+            raise NotImplementedError("no executor op for %s" % type(m).__name__)
+        o = self._new(self._level[x] + dl, m.nOut)
+        lib.insc_net_op_conv(self.h, _KIND[kind], x, o, self._dev(m.weight), self._dev(bias))
+        return o
+
+    # ---- running --------------------------------------------------------------------------
+    def refresh(self):
+        lib.insc_net_refresh_weights(self.h, stream_ptr())
+
+    def __call__(self, input, increment=False, all_points=None):
+        coords, feats = input[0], input[1]
+        if all_points is None:
+            all_points = (not increment) or self.output_layer.all_points
+        c = coords.to(device=self.device, dtype=torch.int32).contiguous()
+        f = feats.detach().to(device=self.device, dtype=torch.float32).contiguous()
+        P = c.size(0)
+        n_pts = I64(0)
+        lib.insc_net_counts(self.h, None, ctypes.byref(n_pts))
+        rows = (n_pts.value if increment else 0) + P if all_points else P
+        out = torch.empty((rows, self.out_channels), dtype=torch.float32, device=self.device)
+        n = I64(0)
+        lib.insc_net_forward(self.h, ptr(c), int(c.size(1)), ptr(f), I64(P), int(bool(increment)), ptr(out),
+                             int(bool(all_points)), ctypes.byref(n), stream_ptr())
+        self.n_sites = int(n.value)
+        return out
+
+    def sites_per_level(self):
+        a = (I64 * 16)()
+        lib.insc_net_counts(self.h, a, None)
+        return [int(v) for v in a]
+
+
+def compile(model, capacity_sites=1 << 18):
+    return CompiledNet(model, capacity_sites)

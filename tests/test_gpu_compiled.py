@@ -1,0 +1,60 @@
+"""The native network executor (one C call per frame) against the per-layer module path:
+bit-identical outputs for full frames, incremental frames, and full recomputes."""
+import copy
+
+import numpy as np
+import pytest
+import torch
+
+from test_gpu_incremental import _frames, _inp
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("levels,m", [(3, 16), (7, 32)])
+def test_compiled_full_and_incremental(levels, m):
+    import sparseconvnet as scn
+    from netdefs import NaiveUNet
+
+    frames = _frames(6, seed=31)
+    model = NaiveUNet(m=m, levels=levels, seed=9).cuda()
+    ref_model = copy.deepcopy(model)
+    net = scn.compile(model.sparseModel, capacity_sites=4096)  # small: forces growth on later frames
+    all_pts, all_rgb = frames[0]
+    with torch.no_grad():
+        out = net(_inp(*frames[0]), increment=False)
+        ref = ref_model.sparseModel(_inp(all_pts, all_rgb), False)
+        assert out.shape == ref.shape
+        assert torch.equal(out, ref)
+        for f in range(1, len(frames)):
+            pts, rgb = frames[f]
+            out = net(_inp(pts, rgb), increment=True, all_points=True)
+            inc = net  # keep name for the error message below
+            all_pts = np.concatenate([all_pts, pts], 0)
+            all_rgb = np.concatenate([all_rgb, rgb], 0)
+            ref = ref_model.sparseModel(_inp(all_pts, all_rgb), False)
+            assert out.shape == ref.shape
+            assert torch.equal(out, ref), "frame %d: max diff %.3e" % (f, (out - ref).abs().max().item())
+        # increment rows only
+        pts, rgb = frames[1]
+        out = net(_inp(pts, rgb), increment=True)
+        all_pts = np.concatenate([all_pts, pts], 0)
+        all_rgb = np.concatenate([all_rgb, rgb], 0)
+        ref = ref_model.sparseModel(_inp(all_pts, all_rgb), False)
+        assert torch.equal(out, ref[-len(pts):])
+        # a new full frame forgets the scene
+        out = net(_inp(*frames[2]), increment=False)
+        ref = ref_model.sparseModel(_inp(*frames[2]), False)
+        assert torch.equal(out, ref)
+
+
+def test_compiled_rejects_incremental_without_state():
+    import sparseconvnet as scn
+    from netdefs import NaiveUNet
+    from sparseconvnet._lib import InscError
+
+    model = NaiveUNet(m=16, levels=2, seed=1).cuda()
+    net = scn.compile(model.sparseModel)
+    pts, rgb = _frames(2, seed=32)[0]
+    with pytest.raises(InscError):
+        net(_inp(pts, rgb), increment=True)
