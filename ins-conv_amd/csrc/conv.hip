@@ -69,7 +69,7 @@ __global__ __launch_bounds__(256) void conv_generic_kernel(const float *__restri
 __host__ __device__ static inline int conv_nch(int Cin) { return (Cin + 31) / 32; }
 static inline int conv_nb_per_group(int Cout) {
   const int nbt = (Cout + 31) / 32;
-  return nbt > 7 ? 4 : nbt;
+  return nbt > 4 ? 4 : nbt;
 }
 static inline int conv_nbt_padded(int Cout) {
   const int nbt = (Cout + 31) / 32, nb = conv_nb_per_group(Cout);
@@ -127,19 +127,29 @@ __device__ __forceinline__ float frag_at(const Frag &f, int s) {
 // row-wise 16-byte writes and the column-block reads of the MFMA layout spread over all banks.
 constexpr int AT_LD = 36;
 
-template <int NB, int K, int MODE>
-__global__ __launch_bounds__(CONV_WAVES * 64) void conv_mfma_kernel(
+// S == 1: every wavefront of the block owns a tile and walks all of its filter offsets.
+// S  > 1: the S wavefronts of a block share ONE tile; wavefront w takes the offsets k with
+//         k % S == w and the partial sums are added in wavefront order at the end.  This is for
+//         the coarse scales of a U-Net, where a layer has a handful of tiles but hundreds of
+//         channels and a single wavefront would run tens of thousands of dependent MFMAs.  Which
+//         terms a wavefront sums depends on k only, so a row's result is a function of S alone
+//         (S is a fixed property of the layer shape), never of the tile it happens to sit in.
+template <int NB, int K, int MODE, int S>
+__global__ __launch_bounds__((S == 1 ? CONV_WAVES : S) * 64) void conv_mfma_kernel(
     const float *__restrict__ in, int64_t ld_in, float *__restrict__ out, int64_t ld_out,
     const float *__restrict__ Wp, const float *__restrict__ bias, const int32_t *__restrict__ map0,
     const int32_t *__restrict__ map1, const int32_t *__restrict__ rows,
     const int32_t *__restrict__ d_n_rows, int64_t n_rows, int Cin, int Cout, int nbtp,
     const uint8_t *__restrict__ tile_flags) {
-  __shared__ int nbl[CONV_WAVES][TILE_M * K];
-  __shared__ __attribute__((aligned(16))) float atile[CONV_WAVES][TILE_M * AT_LD];
+  static_assert(S == 1 || NB == 1, "split tiles use one output block per wavefront");
+  constexpr int WAVES = S == 1 ? CONV_WAVES : S;
+  __shared__ int nbl[S == 1 ? WAVES : 1][TILE_M * K];
+  __shared__ __attribute__((aligned(16))) float atile[WAVES][TILE_M * AT_LD];
+  __shared__ float red[S > 1 ? S - 1 : 1][S > 1 ? 16 * 64 : 1];
   const int64_t n = d_n_rows ? min((int64_t)*d_n_rows, n_rows) : n_rows;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int r = lane & 31, h = lane >> 5;
-  const int64_t t0 = ((int64_t)blockIdx.x * CONV_WAVES + wave) * TILE_M;
+  const int64_t t0 = (S == 1 ? (int64_t)blockIdx.x * WAVES + wave : (int64_t)blockIdx.x) * TILE_M;
   const int cb0 = blockIdx.y * NB;  // first output-channel block of this column group
   const int nch = conv_nch(Cin);
 
@@ -150,13 +160,13 @@ __global__ __launch_bounds__(CONV_WAVES * 64) void conv_mfma_kernel(
 
   // stage the tile's slice of the neighbour map in LDS and find the offsets it uses; all the
   // loads are issued before the first one is consumed
-  int *nl = nbl[wave];
+  int *nl = nbl[S == 1 ? wave : 0];
   unsigned mymask = 0;
-  constexpr int NSTAGE = (TILE_M * K + 63) / 64;
+  constexpr int NSTAGE = (TILE_M * K + 64 * S - 1) / (64 * S);
   int staged[NSTAGE];
 #pragma unroll
   for (int i = 0; i < NSTAGE; i++) {
-    const int e = i * 64 + lane;
+    const int e = (S == 1 ? i : i * S + wave) * 64 + lane;
     const int rr = e / K, kk = e - rr * K;
     const int rid = __shfl(my_row, rr & (TILE_M - 1), 64);
     int v = -1;
@@ -172,23 +182,33 @@ __global__ __launch_bounds__(CONV_WAVES * 64) void conv_mfma_kernel(
   }
 #pragma unroll
   for (int i = 0; i < NSTAGE; i++) {
-    const int e = i * 64 + lane;
+    const int e = (S == 1 ? i : i * S + wave) * 64 + lane;
     if (e < TILE_M * K) {
       nl[e] = staged[i];
       if (staged[i] >= 0) mymask |= 1u << (e % K);
     }
   }
+  if (S == 1) {
 #pragma unroll
-  for (int d = 32; d > 0; d >>= 1) mymask |= (unsigned)__shfl_xor((int)mymask, d, 64);
+    for (int d = 32; d > 0; d >>= 1) mymask |= (unsigned)__shfl_xor((int)mymask, d, 64);
+  }
   __syncthreads();
-  if (!live) return;  // whole wavefront idle; no barrier follows
-  unsigned rest = (unsigned)__builtin_amdgcn_readfirstlane((int)mymask);
+  if (!live) return;  // the whole block (S > 1) or wavefront (S == 1) is idle; no barrier follows
+  unsigned rest;
+  if (S == 1) {
+    rest = (unsigned)__builtin_amdgcn_readfirstlane((int)mymask);
+  } else {
+    // offsets of this wavefront that some row of the tile uses
+    rest = 0;
+    for (int k = wave; k < K; k += S)
+      if (__ballot(nl[r * K + k] >= 0) != 0ull) rest |= 1u << k;
+  }
 
   f16v acc[NB];
 #pragma unroll
   for (int b = 0; b < NB; b++) {
     const int c = (cb0 + b) * 32 + r;
-    const float bv = (bias && c < Cout) ? bias[c] : 0.0f;
+    const float bv = (bias && c < Cout && (S == 1 || wave == 0)) ? bias[c] : 0.0f;
 #pragma unroll
     for (int v = 0; v < 16; v++) acc[b][v] = bv;
   }
@@ -289,6 +309,21 @@ __global__ __launch_bounds__(CONV_WAVES * 64) void conv_mfma_kernel(
     }
   }
 
+  if (S > 1) {
+    // partial sums of wavefronts 1..S-1 go through LDS and are added in wavefront order
+    if (wave > 0) {
+#pragma unroll
+      for (int v = 0; v < 16; v++) red[wave - 1][v * 64 + lane] = acc[0][v];
+    }
+    __syncthreads();
+    if (wave > 0) return;
+#pragma unroll
+    for (int w = 0; w < S - 1; w++) {
+#pragma unroll
+      for (int v = 0; v < 16; v++) acc[0][v] += red[w][v * 64 + lane];
+    }
+  }
+
   // D layout of the 32x32 MFMA: lane holds column (lane & 31), rows 8*(v/4) + 4*(lane>>5) + (v&3)
 #pragma unroll
   for (int v = 0; v < 16; v++) {
@@ -350,34 +385,52 @@ int launch_conv(const float *in, int64_t ld_in, float *out, int64_t ld_out, cons
       Wp = (const float *)ws;
     }
     const int64_t tiles = cdiv(n_rows, TILE_M);
-    const unsigned gx = (unsigned)cdiv(tiles, CONV_WAVES);
-    const int NB = conv_nb_per_group(Cout), nbtp = conv_nbt_padded(Cout);
-    dim3 grid(gx, (unsigned)(nbtp / NB)), block(CONV_WAVES * 64);
-#define INSC_CONV_LAUNCH(NBV, KV, MV)                                                                          \
-  hipLaunchKernelGGL((conv_mfma_kernel<NBV, KV, MV>), grid, block, 0, s, in, ld_in, out, ld_out, Wp, bias, map0, \
-                     map1, rows, d_n_rows, n_rows, Cin, Cout, nbtp, tile_flags)
+    const int nbt = (Cout + 31) / 32;
+    // Launch shape, a function of the layer shape only (so results never depend on the scene):
+    //  narrow layers (Cin < 96): each wavefront computes all output blocks of its tile (the
+    //    gathered rows are reused across them);
+    //  wide layers: one output block per wavefront (more wavefronts for the few tiles of a
+    //    coarse scale), and for 3^3 / 2^3 maps the offsets of a tile are split over S wavefronts.
+    const bool wide = Cin >= 96;
+    const int NB = wide ? 1 : conv_nb_per_group(Cout);
+    const int nbtp = conv_nbt_padded(Cout);
+    int S = 1;
+    if (wide && mode == MAP_NBR && K == 27) S = Cin >= 160 ? 8 : 4;
+    if (wide && mode == MAP_NBR && K == 8) S = 4;
+    const unsigned gx = (unsigned)(S == 1 ? cdiv(tiles, CONV_WAVES) : tiles);
+    dim3 grid(gx, (unsigned)(NB == 1 ? nbt : nbtp / NB)), block((S == 1 ? CONV_WAVES : S) * 64);
+    bool shape_ok = true;
+#define INSC_CONV_LAUNCH(NBV, KV, MV, SV)                                                                       \
+  hipLaunchKernelGGL((conv_mfma_kernel<NBV, KV, MV, SV>), grid, block, 0, s, in, ld_in, out, ld_out, Wp, bias,  \
+                     map0, map1, rows, d_n_rows, n_rows, Cin, Cout, nbtp, tile_flags)
 #define INSC_CONV_CASE(NBV)                                      \
   case NBV:                                                      \
     if (mode == MAP_NBR && K == 27)                              \
-      INSC_CONV_LAUNCH(NBV, 27, MAP_NBR);                        \
+      INSC_CONV_LAUNCH(NBV, 27, MAP_NBR, 1);                     \
     else if (mode == MAP_NBR && K == 8)                          \
-      INSC_CONV_LAUNCH(NBV, 8, MAP_NBR);                         \
+      INSC_CONV_LAUNCH(NBV, 8, MAP_NBR, 1);                      \
     else if (mode == MAP_PARENT && K == 8)                       \
-      INSC_CONV_LAUNCH(NBV, 8, MAP_PARENT);                      \
+      INSC_CONV_LAUNCH(NBV, 8, MAP_PARENT, 1);                   \
     else if (mode == MAP_IDENTITY && K == 1)                     \
-      INSC_CONV_LAUNCH(NBV, 1, MAP_IDENTITY);                    \
+      INSC_CONV_LAUNCH(NBV, 1, MAP_IDENTITY, 1);                 \
     else                                                         \
       shape_ok = false;                                          \
     break;
-    bool shape_ok = true;
-    switch (NB) {
-      INSC_CONV_CASE(1)
-      INSC_CONV_CASE(2)
-      INSC_CONV_CASE(3)
-      INSC_CONV_CASE(4)
-      INSC_CONV_CASE(5)
-      INSC_CONV_CASE(6)
-      INSC_CONV_CASE(7)
+    if (S == 8) {
+      INSC_CONV_LAUNCH(1, 27, MAP_NBR, 8);
+    } else if (S == 4 && K == 27) {
+      INSC_CONV_LAUNCH(1, 27, MAP_NBR, 4);
+    } else if (S == 4) {
+      INSC_CONV_LAUNCH(1, 8, MAP_NBR, 4);
+    } else {
+      switch (NB) {
+        INSC_CONV_CASE(1)
+        INSC_CONV_CASE(2)
+        INSC_CONV_CASE(3)
+        INSC_CONV_CASE(4)
+        default:
+          shape_ok = false;
+      }
     }
     if (!shape_ok) {
       set_error("conv: no matrix-core kernel for K=%d with map mode %d", K, mode);
