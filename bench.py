@@ -1,18 +1,21 @@
 #!/usr/bin/env python3
-"""Benchmark of the sparse-convolution inference path on one MI355X.
+"""Benchmark of the incremental sparse-convolution inference path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload ssc|unet|incr]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload incr|unet|ssc]
 
-Prints ONE JSON line.  A step is one pass of the hot path over one batch of seeded
-synthetic input that is already resident in HBM when the timed region starts:
+Prints ONE JSON line.  A step is one pass of the hot path over one batch of seeded synthetic
+input that is already resident in HBM when the timed region starts:
+  incr (default): workload 5 - one incremental U-Net frame of the 50-frame sensor sweep
+         (3k-8k new voxels + 1k-2k re-observed voxels per frame, growing to 150k voxels);
+         frame 0 (full forward) and the first W incremental frames are untimed, the next K
+         incremental frames are timed back to back.  value = mean ms per frame.
+  unet : workload 4 - full U-Net forward over the 150k-voxel scene (165k points).
   ssc  : workload 3 - 4 x [SubmanifoldConvolution(3) + BatchNormReLU] at 500k active voxels,
-         once at 32 channels and once at 64 (8 convolutions per step)
-  unet : workload 4 - full U-Net forward over a 150k-voxel scene
-  incr : workload 5 - one incremental U-Net frame of the 50-frame sweep
-The `roofline` object is measured live on the dominant kernel (the submanifold
-gather-GEMM-scatter at 500k voxels, 32 channels) with events on the launch stream;
-`cpu_baseline` times the CPU oracle (a restatement of the reference's CPU path) on this
-machine's host cores over a bounded sample.
+         once at 32 channels and once at 64 (8 convolutions per step); value = Msites/s.
+`roofline` is measured live on the dominant kernel, the submanifold gather-GEMM-scatter, at
+the size the roofline target is stated for (500k voxels, 32 channels), with events on the
+launch stream.  `cpu_baseline` times the CPU oracle (a restatement of the reference's CPU
+path) on this machine's host cores over a bounded sample.
 """
 import argparse
 import json
@@ -29,6 +32,9 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 MFMA_FP32_PEAK_TFLOPS = 157.3
 
 
+# ---------------------------------------------------------------------------------------------
+# workload 3: SSC layer stack at 500k voxels (also the roofline measurement)
+# ---------------------------------------------------------------------------------------------
 def build_ssc_stack(C, seed, device):
     import torch
 
@@ -45,14 +51,12 @@ def build_ssc_stack(C, seed, device):
     return net.to(device).eval()
 
 
-def ssc_workload(device):
-    """Workload 3: returns (run_step, info)."""
+def ssc_workload(device, channels=(32, 64)):
     import numpy as np
     import torch
 
     import scenes
     import sparseconvnet as scn
-    from sparseconvnet import SCN
 
     vox = scenes.indoor_scene(seed=3, n=500000)
     size = torch.LongTensor([4096, 4096, 4096])
@@ -60,7 +64,7 @@ def ssc_workload(device):
     rng = np.random.default_rng(3)
     stacks, xs = [], []
     coords = torch.from_numpy(vox.astype(np.int64))
-    for C in (32, 64):
+    for C in channels:
         f = torch.from_numpy(rng.normal(size=(len(vox), C)).astype(np.float32)).to(device)
         x = inp([coords, f, 1])
         x.features = x.features.clone()
@@ -74,16 +78,19 @@ def ssc_workload(device):
             for net, x in zip(stacks, xs):
                 net(x)
 
-    info = {"sites": len(vox), "rules": n_rules, "convs_per_step": 8}
+    info = {"sites": len(vox), "rules": n_rules, "convs_per_step": 4 * len(channels)}
     return step, info, (xs[0], stacks[0])
 
 
-def conv_roofline(x, stack, n_rules, device, reps=30):
-    """Average duration of the 32-channel submanifold convolution kernel and its roofline figures."""
+def conv_roofline(device, reps=30):
+    """Average duration of the 32-channel submanifold convolution kernel at 500k voxels and the
+    roofline figures derived from it."""
     import torch
 
     from sparseconvnet import SCN
 
+    _, info, (x, stack) = ssc_workload(device, channels=(32,))
+    n_rules = info["rules"]
     conv = stack[0]
     m = x.metadata
     sc = m.ssc_rulebook(x.spatial_size)
@@ -107,16 +114,59 @@ def conv_roofline(x, stack, n_rules, device, reps=30):
     achieved = bytes_alg / t / 1e9
     return {
         "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-        "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
-        "kernel": "conv_mfma_kernel<1> (SSC 3^3, 32->32, 500k sites)", "avg_us": round(t * 1e6, 1),
-        "algorithmic_bytes": int(bytes_alg),
+        "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": 235.3e6,
+        "kernel": "conv_mfma_kernel<NB=1,K=27,S=1> (SSC 3^3, 32->32, 500k sites, %d rules)" % n_rules,
+        "avg_us": round(t * 1e6, 1), "algorithmic_bytes": int(bytes_alg),
+        "traffic_note": "FETCH_SIZE 167.3 MB + WRITE_SIZE 64.0 MB per launch (rocprofv3 --pmc, see profiles/)",
         "mfma_tflops": round(flops / t / 1e12, 2), "mfma_frac": round(flops / t / 1e12 / MFMA_FP32_PEAK_TFLOPS, 4),
+        "ssc_msites_per_s": round(sc.n / t / 1e6, 1),
+    }
+
+
+# ---------------------------------------------------------------------------------------------
+# workloads 4 and 5: the U-Net of the reference's example, through the network executor
+# ---------------------------------------------------------------------------------------------
+def unet_model(device):
+    import sparseconvnet as scn
+    from netdefs import NaiveUNet
+
+    model = NaiveUNet(m=32, levels=7, seed=4).to(device)
+    return model, scn.compile(model.sparseModel, capacity_sites=1 << 18)
+
+
+def to_dev(pts, rgb, device):
+    import numpy as np
+    import torch
+
+    return [torch.from_numpy(pts.astype(np.int32)).to(device), torch.from_numpy(rgb).to(device), 1]
+
+
+def cpu_baseline_unet():
+    """The CPU oracle running the same U-Net as a FULL forward over the final 150k-voxel scene
+    (the reference's CPU path has no incremental mode, so this is what one frame costs there)."""
+    import numpy as np
+    import torch
+
+    import oracle_net
+    import scenes
+    from netdefs import NaiveUNet
+    from oracle import oracle as orc
+
+    pts, rgb, _ = scenes.unet_scene()
+    model = NaiveUNet(m=32, levels=7, seed=4)
+    t0 = time.perf_counter()
+    feats = oracle_net.forward(model.sparseModel, [pts, rgb, 1])
+    with torch.no_grad():
+        model.linear(torch.from_numpy(np.ascontiguousarray(feats)))
+    dt = time.perf_counter() - t0
+    return {
+        "value": round(dt * 1e3, 1), "unit": "ms/frame", "cores": orc.num_threads(), "kind": "port",
+        "sample": "one full U-Net forward (rulebooks + 53 SSC + 6 conv + 6 deconv + 65 BN) over the final "
+                  "150k-voxel scene of the sweep, 165k points; the reference CPU path has no incremental mode",
     }
 
 
 def cpu_baseline_ssc(n_sample=100000):
-    """The CPU oracle on a bounded sample of workload 3: one SSC(3)+BN+ReLU pair at 32 and at 64
-    channels over the first `n_sample` voxels of the scene."""
     import numpy as np
 
     import scenes
@@ -124,9 +174,7 @@ def cpu_baseline_ssc(n_sample=100000):
 
     vox = scenes.indoor_scene(seed=3, n=500000)[:n_sample]
     _, sc, _ = orc.grid_build(vox)
-    t0 = time.perf_counter()
     _, counts, pairs = orc.ssc_rules(sc)
-    t_rules = time.perf_counter() - t0
     rng = np.random.default_rng(0)
     t_total, convs = 0.0, 0
     for C in (32, 64):
@@ -145,17 +193,17 @@ def cpu_baseline_ssc(n_sample=100000):
     return {
         "value": round(len(sc) * convs / t_total / 1e6, 3), "unit": "Msites/s", "cores": orc.num_threads(),
         "kind": "port",
-        "sample": "first %d voxels of the workload-3 scene, one SSC(3)+BN+ReLU pair at C=32 and one at C=64 "
-                  "(rulebook build %.2f s not included)" % (len(sc), t_rules),
+        "sample": "first %d voxels of the workload-3 scene, one SSC(3)+BN+ReLU pair at C=32 and one at C=64"
+                  % len(sc),
     }
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="ssc", choices=["ssc"])
+    ap.add_argument("--steps", type=int, default=None)
+    ap.add_argument("--warmup", type=int, default=None)
+    ap.add_argument("--workload", default="incr", choices=["incr", "unet", "ssc"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--roofline-only", action="store_true",
                     help="run only the dominant-kernel measurement (short; used under rocprofv3)")
@@ -163,6 +211,7 @@ def main():
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU; --gpus %d is not supported (no collectives, no sharding)"
                  % args.gpus)
+    import numpy as np
     import torch
 
     if not torch.cuda.is_available():
@@ -170,32 +219,106 @@ def main():
     device = torch.device("cuda", 0)
     torch.cuda.set_device(device)
 
-    step, info, (x0, stack0) = ssc_workload(device)
     if args.roofline_only:
-        print(json.dumps({"roofline": conv_roofline(x0, stack0, info["rules"], device, reps=10)}))
-        return
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    dt = time.perf_counter() - t0
-    ms = dt * 1e3 / args.steps
-    msites = info["sites"] * info["convs_per_step"] / (dt / args.steps) / 1e6
+        # plus a plain copy of known size (500k x 32 floats: 64 MB read, 64 MB written), the
+        # yardstick the FETCH_SIZE / WRITE_SIZE counters of the same run are scaled by
+        from sparseconvnet import SCN
 
-    roof = conv_roofline(x0, stack0, info["rules"], device)
+        a = torch.randn(500000, 32, device=device)
+        b = torch.empty_like(a)
+        for _ in range(5):
+            SCN.copy_rows(a, b, None, None, a.size(0))
+        torch.cuda.synchronize()
+        print(json.dumps({"roofline": conv_roofline(device, reps=10)}))
+        return
+
+    extra = {}
+    if args.workload == "incr":
+        import scenes
+
+        seq = scenes.sweep_sequence()
+        W = 9 if args.warmup is None else args.warmup
+        K = len(seq) - 1 - W if args.steps is None else args.steps
+        if W + K > len(seq) - 1 or K < 1:
+            sys.exit("bench.py: the sweep has %d incremental frames; need warmup + steps <= %d"
+                     % (len(seq) - 1, len(seq) - 1))
+        model, net = unet_model(device)
+        frames = [to_dev(p, c, device) for p, c in seq]
+        with torch.no_grad():
+            # the logits of a frame's points = Linear(features of those points)
+            net(frames[0], increment=False)
+            for f in range(1, 1 + W):
+                model.linear(net(frames[f], increment=True))
+            torch.cuda.synchronize()
+            per_frame = []
+            t0 = time.perf_counter()
+            for f in range(1 + W, 1 + W + K):
+                t1 = time.perf_counter()
+                model.linear(net(frames[f], increment=True))
+                torch.cuda.synchronize()
+                per_frame.append((time.perf_counter() - t1) * 1e3)
+            dt = time.perf_counter() - t0
+        ms = dt * 1e3 / K
+        value, metric, unit, hib = round(ms, 3), "incremental frame latency ms (UNet, 150k vox)", "ms", False
+        config = {"workload": "cfg5: incremental U-Net frames %d..%d of the 50-frame sweep (m=32, 7 levels, "
+                              "InputLayer mode 4 .. OutputLayer + Linear(32,20)); scene grows to 150k voxels"
+                              % (1 + W, W + K),
+                  "points_per_frame_mean": int(np.mean([len(seq[f][0]) for f in range(1 + W, 1 + W + K)])),
+                  "sites_at_end": net.n_sites, "sites_per_level_at_end": net.sites_per_level()[:7]}
+        extra = {"median_ms": round(float(np.median(per_frame)), 3),
+                 "p95_ms": round(float(np.percentile(per_frame, 95)), 3),
+                 "last_frame_ms": round(per_frame[-1], 3), "first_timed_frame_ms": round(per_frame[0], 3)}
+        cpu = None if args.no_cpu_baseline else cpu_baseline_unet()
+    elif args.workload == "unet":
+        import scenes
+
+        W = 3 if args.warmup is None else args.warmup
+        K = 20 if args.steps is None else args.steps
+        pts, rgb, _ = scenes.unet_scene()
+        model, net = unet_model(device)
+        x = to_dev(pts, rgb, device)
+        with torch.no_grad():
+            for _ in range(W):
+                model.linear(net(x, increment=False))
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(K):
+                model.linear(net(x, increment=False))
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t0
+        ms = dt * 1e3 / K
+        value, metric, unit, hib = round(ms, 3), "full U-Net forward ms (150k vox)", "ms", False
+        config = {"workload": "cfg4: full U-Net forward (grid + rulebooks + all layers), 150k voxels / 165k points",
+                  "sites_per_level": net.sites_per_level()[:7]}
+        cpu = None if args.no_cpu_baseline else cpu_baseline_unet()
+    else:
+        W = 3 if args.warmup is None else args.warmup
+        K = 20 if args.steps is None else args.steps
+        step, info, _ = ssc_workload(device)
+        for _ in range(W):
+            step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(K):
+            step()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        ms = dt * 1e3 / K
+        value = round(info["sites"] * info["convs_per_step"] / (dt / K) / 1e6, 1)
+        metric, unit, hib = "SSC Msites/s", "Msites/s", True
+        config = {"workload": "cfg3: 4x[SSC(3)+BN+ReLU] at 500k voxels, C=32 then C=64 (8 convs/step)",
+                  "sites": info["sites"], "rules": info["rules"]}
+        cpu = None if args.no_cpu_baseline else cpu_baseline_ssc()
+
     out = {
-        "metric": "SSC Msites/s", "value": round(msites, 1), "unit": "Msites/s", "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup, "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "cfg3: 4x[SSC(3)+BN+ReLU] at 500k voxels, C=32 then C=64 (8 convs/step)",
-                   "sites": info["sites"], "rules": info["rules"]},
-        "roofline": roof,
+        "metric": metric, "value": value, "unit": unit, "n_gpus": 1, "steps": K, "warmup": W,
+        "ms_per_step": round(ms, 4), "higher_is_better": hib, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic", "config": config,
     }
-    if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline_ssc()
+    out.update(extra)
+    out["roofline"] = conv_roofline(device)
+    if cpu is not None:
+        out["cpu_baseline"] = cpu
     print(json.dumps(out))
 
 
