@@ -130,10 +130,13 @@ int insc_order_by_offset(const int32_t *d_order, const int32_t *d_offset, int64_
  * NetworkInNetwork_updateOutput (CUDA/NetworkInNetwork.cpp:9-25).  d_W is [K,Cin,Cout]; d_Wp
  * (nullable) is the same weights packed by insc_conv_pack_weights - give it to skip the
  * per-call packing (then d_W may be NULL when Cin is a multiple of 16).
- * h_muladds (nullable) receives the multiply-add count the reference returns (synchronises). */
-int insc_conv_nbr(const float *d_in, int64_t ld_in, float *d_out, int64_t ld_out, const float *d_W,
-                  const float *d_Wp, const float *d_bias, const int32_t *d_nbr, int K, const int32_t *d_rows,
-                  const int32_t *d_n_rows, int64_t n_rows, int Cin, int Cout, double *h_muladds, void *stream);
+ * n_in_rows = rows of d_in (the gather is bounds-checked against it; n_in_rows*ld_in*4 must stay
+ * below 4 GB).  h_muladds (nullable) receives the multiply-add count the reference returns
+ * (synchronises). */
+int insc_conv_nbr(const float *d_in, int64_t ld_in, int64_t n_in_rows, float *d_out, int64_t ld_out,
+                  const float *d_W, const float *d_Wp, const float *d_bias, const int32_t *d_nbr, int K,
+                  const int32_t *d_rows, const int32_t *d_n_rows, int64_t n_rows, int Cin, int Cout,
+                  double *h_muladds, void *stream);
 /* Weights in the operand layout of the matrix-core kernel (no counterpart in the reference,
  * whose kernels stage W[k] through shared memory per launch, CUDA/Convolution.cu:81-223).
  * insc_conv_packed_floats gives the size of d_Wp in floats. */
@@ -142,10 +145,10 @@ int insc_conv_pack_weights(const float *d_W, int K, int Cin, int Cout, float *d_
 /* Size-2 stride-2 deconvolution: out[i,:] = bias + in[parent[i],:] . W[offset[i]]
  * (Deconvolution_updateOutput, CUDA/Deconvolution.cpp:28-58: the convolution's rules with
  * the roles of input and output swapped). */
-int insc_deconv_down2(const float *d_in, int64_t ld_in, float *d_out, int64_t ld_out, const float *d_W,
-                      const float *d_Wp, const float *d_bias, const int32_t *d_parent, const int32_t *d_offset,
-                      const int32_t *d_rows, const int32_t *d_n_rows, int64_t n_rows, int Cin, int Cout,
-                      void *stream);
+int insc_deconv_down2(const float *d_in, int64_t ld_in, int64_t n_in_rows, float *d_out, int64_t ld_out,
+                      const float *d_W, const float *d_Wp, const float *d_bias, const int32_t *d_parent,
+                      const int32_t *d_offset, const int32_t *d_rows, const int32_t *d_n_rows, int64_t n_rows,
+                      int Cin, int Cout, void *stream);
 /* Inference batch norm + leaky ReLU: y = x*w + b, y *= (y>0 ? 1 : leakiness),
  * w = gamma*(var+eps)^-1/2, b = beta - mean*w; gamma/beta nullable
  * (BatchNormalization_updateOutput with train=false, CUDA/BatchNormalization.cpp:39-61,

@@ -45,10 +45,11 @@ int sort_pairs_u64(uint64_t *keys, int32_t *vals, int64_t n, int key_bits, hipSt
 enum { MAP_NBR = 0, MAP_IDENTITY = 1, MAP_PARENT = 2 };
 // tile_flags: one byte per 32-row tile of `rows` (matrix-core kernel); row_mask: one byte per
 // site (generic kernel and the streaming kernels).  Null = everything.
-int launch_conv(const float *in, int64_t ld_in, float *out, int64_t ld_out, const float *W, const float *Wp,
-                const float *bias, const int32_t *map0, const int32_t *map1, int mode, int K, const int32_t *rows,
-                const int32_t *d_n_rows, int64_t n_rows, int Cin, int Cout, const uint8_t *tile_flags,
-                const uint8_t *row_mask, hipStream_t s);
+// in_rows: rows of the input matrix (bounds the gather).
+int launch_conv(const float *in, int64_t ld_in, int64_t in_rows, float *out, int64_t ld_out, const float *W,
+                const float *Wp, const float *bias, const int32_t *map0, const int32_t *map1, int mode, int K,
+                const int32_t *rows, const int32_t *d_n_rows, int64_t n_rows, int Cin, int Cout,
+                const uint8_t *tile_flags, const uint8_t *row_mask, hipStream_t s);
 int64_t packed_floats(int K, int Cin, int Cout);
 int pack_weights(const float *W, int K, int Cin, int Cout, float *Wp, hipStream_t s);
 int launch_bn(const float *in, int64_t ld_in, float *out, int64_t ld_out, const float *mean, const float *var,

@@ -127,6 +127,29 @@ __device__ __forceinline__ float frag_at(const Frag &f, int s) {
 // row-wise 16-byte writes and the column-block reads of the MFMA layout spread over all banks.
 constexpr int AT_LD = 36;
 
+// Gather flavour.  DIRECT_GATHER: every lane reads the 64 bytes of its own input row that the
+// MFMA A operand needs, with buffer loads: one 32-bit offset per item, rows without a
+// neighbour get an out-of-range offset and the hardware returns zeros, and the weight tile is
+// addressed by a scalar offset - a handful of non-MFMA instructions per 16 MFMAs (ordinary
+// VALU work does not overlap with MFMAs on this part, so it is paid in matrix-core time).
+// Otherwise: coalesced 128-byte row segments, transposed through LDS into the A layout
+// (fewer cache-line touches per instruction, but ~100 extra instructions per item).
+#ifndef INSC_CONV_DIRECT
+#define INSC_CONV_DIRECT 1
+#endif
+constexpr bool DIRECT_GATHER = INSC_CONV_DIRECT != 0;
+
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+// offsets at or beyond this bound make a buffer load return zeros
+constexpr uint32_t BUF_OOB = 0xFFFFFF00u;
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *p, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p), 0, (int)bytes, 0x00020000);
+}
+__device__ __forceinline__ float4 buf_load16(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff) {
+  return __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(r, (int)voff, (int)soff, 0));
+}
+
 // S == 1: every wavefront of the block owns a tile and walks all of its filter offsets.
 // S  > 1: the S wavefronts of a block share ONE tile; wavefront w takes the offsets k with
 //         k % S == w and the partial sums are added in wavefront order at the end.  This is for
@@ -140,11 +163,11 @@ __global__ __launch_bounds__((S == 1 ? CONV_WAVES : S) * 64) void conv_mfma_kern
     const float *__restrict__ Wp, const float *__restrict__ bias, const int32_t *__restrict__ map0,
     const int32_t *__restrict__ map1, const int32_t *__restrict__ rows,
     const int32_t *__restrict__ d_n_rows, int64_t n_rows, int Cin, int Cout, int nbtp,
-    const uint8_t *__restrict__ tile_flags) {
+    const uint8_t *__restrict__ tile_flags, uint32_t in_bytes, uint32_t wp_bytes) {
   static_assert(S == 1 || NB == 1, "split tiles use one output block per wavefront");
   constexpr int WAVES = S == 1 ? CONV_WAVES : S;
   __shared__ int nbl[S == 1 ? WAVES : 1][TILE_M * K];
-  __shared__ __attribute__((aligned(16))) float atile[WAVES][TILE_M * AT_LD];
+  __shared__ __attribute__((aligned(16))) float atile[DIRECT_GATHER ? 1 : WAVES][DIRECT_GATHER ? 4 : TILE_M * AT_LD];
   __shared__ float red[S > 1 ? S - 1 : 1][S > 1 ? 16 * 64 : 1];
   const int64_t n = d_n_rows ? min((int64_t)*d_n_rows, n_rows) : n_rows;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -214,7 +237,6 @@ __global__ __launch_bounds__((S == 1 ? CONV_WAVES : S) * 64) void conv_mfma_kern
   }
 
   if (rest) {
-    const int64_t wtile = 1024;  // floats per (k, chunk, block) weight tile
     // Work items of this tile: (active offset k, 32-channel chunk ch), in order.
     struct Item {
       int k, ch;
@@ -233,77 +255,171 @@ __global__ __launch_bounds__((S == 1 ? CONV_WAVES : S) * 64) void conv_mfma_kern
       }
       return it;
     };
-    // Gather of one item, coalesced: load i (0..3) of lane l reads 16 bytes of input row
-    // 8*i + l/8 at channel 4*(l%8), so eight lanes cover one 128-byte row segment and every
-    // quad of lanes reads 64 contiguous bytes.  Rows without a neighbour (and the upper half of
-    // a 16-channel tail chunk) read a row of zeros.
-    const int grow = lane >> 3, gcol = (lane & 7) * 4;
-    auto gather = [&](const Item &it) -> Frag {
-      Frag f;
-      const bool col_ok = it.ch * 32 + gcol < Cin;
-#pragma unroll
-      for (int i = 0; i < 4; i++) {
-        const int src = nl[(8 * i + grow) * K + it.k];
-        const float *p = (src >= 0 && col_ok) ? in + (int64_t)src * ld_in + it.ch * 32 + gcol : g_zero_row;
-        f.q[i] = *reinterpret_cast<const float4 *>(p);
-      }
-      return f;
-    };
-    // through LDS into the MFMA A layout: lane (r, h) gets channels h*16 .. h*16+15 of row r
-    float *at = atile[wave];
-    auto transpose = [&](const Frag &g) -> Frag {
-#pragma unroll
-      for (int i = 0; i < 4; i++) *reinterpret_cast<float4 *>(at + (8 * i + grow) * AT_LD + gcol) = g.q[i];
-      Frag a;
-#pragma unroll
-      for (int q = 0; q < 4; q++) a.q[q] = *reinterpret_cast<const float4 *>(at + r * AT_LD + h * 16 + 4 * q);
-      return a;
-    };
-    auto wtile_of = [&](const Item &it, int b) -> const float * {
-      return Wp + (((int64_t)it.k * nch + it.ch) * nbtp + cb0 + b) * wtile;
-    };
     Item it0;
     it0.k = __builtin_ctz(rest);
     rest &= rest - 1;
     it0.ch = 0;
-    Frag g = gather(it0);
-    Frag bw[2];
-    bw[0] = load_wfrag(wtile_of(it0, 0), lane);
-    Frag a = transpose(g);
-    // Every load below is issued unconditionally (past the last item the current item is simply
+    // Pipeline: while item t runs on the matrix cores, the gathers of items t+1 and t+2 and the
+    // weight tile(s) of the next item(s) are in flight.  Register slots are compile-time (the
+    // loop bodies are unrolled) because copying a fragment would wait for the load that fills
+    // it.  Every load is issued unconditionally (past the last item the last item is simply
     // fetched again): a load under a branch would force the wait before the MFMAs to drain all
-    // outstanding loads, which serialises the pipeline.
-    bool done = false;
-    while (!done) {
+    // outstanding loads, which serialises the pipeline.  The sched_barrier / memory-clobber
+    // pairs keep the loads above the MFMAs they overlap and their consumers below.
+    bool last0, last1;
+    if constexpr (DIRECT_GATHER) {
+      const __amdgpu_buffer_rsrc_t rin = make_rsrc(in, in_bytes), rw = make_rsrc(Wp, wp_bytes);
+      const uint32_t ld4 = (uint32_t)ld_in * 4u, lane16 = (uint32_t)lane * 16u;
+      // lane (r, h) reads channels ch*32 + h*16 .. +15 of its own row; the second half-wave of
+      // a 16-channel tail chunk has no channels
+      auto gather = [&](const Item &it) -> Frag {
+        const int src = nl[r * K + it.k];
+        const bool on = src >= 0 && (h == 0 || Cin - it.ch * 32 >= 32);
+        const uint32_t voff = on ? (uint32_t)src * ld4 + (uint32_t)(it.ch * 128 + h * 64) : BUF_OOB;
+        Frag f;
 #pragma unroll
-      for (int u = 0; u < 2; u++) {
-        bool last;
-        const Item it1 = advance(it0, last);
-        g = gather(it1);  // in flight while this item runs on the matrix cores
+        for (int q = 0; q < 4; q++) f.q[q] = buf_load16(rin, voff + 16u * q, 0);
+        return f;
+      };
+      auto wload = [&](const Item &it, int b) -> Frag {
+        const uint32_t soff = (uint32_t)((((it.k * nch + it.ch) * nbtp) + cb0 + b) * 4096);
+        Frag f;
 #pragma unroll
-        for (int b = 0; b < NB; b++) {
-          const int nn = u * NB + b;
-          if (b + 1 < NB)
-            bw[(nn + 1) % 2] = load_wfrag(wtile_of(it0, b + 1), lane);
-          else
-            bw[(nn + 1) % 2] = load_wfrag(wtile_of(it1, 0), lane);
-          // the loads above stay above the MFMAs (the scheduler otherwise sinks them to their
-          // consumers, i.e. behind the matrix work they are meant to overlap)
+        for (int q = 0; q < 4; q++) f.q[q] = buf_load16(rw, lane16 + 1024u * q, soff);
+        return f;
+      };
+      Frag g[3];
+      g[0] = gather(it0);
+      Item it1 = advance(it0, last0);  // last0: it0 is the final item
+      g[1] = gather(it1);
+      if constexpr (S == 1) {
+        Frag bw[2];
+        bw[0] = wload(it0, 0);
+        bool done = false;
+        while (!done) {
+#pragma unroll
+          for (int u = 0; u < 6; u++) {
+            // item t = g[u%3] (arrived or arriving), t+1 = g[(u+1)%3] in flight, slot (u+2)%3 free
+            const Item it2 = advance(it1, last1);
+            g[(u + 2) % 3] = gather(it2);
+#pragma unroll
+            for (int b = 0; b < NB; b++) {
+              const int nn = u * NB + b;
+              bw[(nn + 1) % 2] = (b + 1 < NB) ? wload(it0, b + 1) : wload(it1, 0);
+              asm volatile("" ::: "memory");
+              __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+              for (int s = 0; s < 16; s++)
+                acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(frag_at(g[u % 3], s), frag_at(bw[nn % 2], s), acc[b],
+                                                              0, 0, 0);
+            }
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_sched_barrier(0);
+            if (last0) {
+              done = true;
+              break;
+            }
+            it0 = it1;
+            it1 = it2;
+            last0 = last1;
+          }
+        }
+      } else {
+        // few wavefronts per SIMD: the weight tiles are fetched two items ahead as well
+        Frag bw[3];
+        bw[0] = wload(it0, 0);
+        bw[1] = wload(it1, 0);
+        bool done = false;
+        while (!done) {
+#pragma unroll
+          for (int u = 0; u < 3; u++) {
+            const Item it2 = advance(it1, last1);
+            g[(u + 2) % 3] = gather(it2);
+            bw[(u + 2) % 3] = wload(it2, 0);
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int s = 0; s < 16; s++)
+              acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(frag_at(g[u % 3], s), frag_at(bw[u % 3], s), acc[0], 0,
+                                                            0, 0);
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_sched_barrier(0);
+            if (last0) {
+              done = true;
+              break;
+            }
+            it0 = it1;
+            it1 = it2;
+            last0 = last1;
+          }
+        }
+      }
+    } else {
+      const int64_t wtile = 1024;  // floats per (k, chunk, block) weight tile
+      // Gather of one item, coalesced: load i (0..3) of lane l reads 16 bytes of input row
+      // 8*i + l/8 at channel 4*(l%8), so eight lanes cover one 128-byte row segment and every
+      // quad of lanes reads 64 contiguous bytes.  Rows without a neighbour (and the upper half
+      // of a 16-channel tail chunk) read a row of zeros.
+      const int grow = lane >> 3, gcol = (lane & 7) * 4;
+      auto gather = [&](const Item &it) -> Frag {
+        Frag f;
+        const bool col_ok = it.ch * 32 + gcol < Cin;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          const int src = nl[(8 * i + grow) * K + it.k];
+          const float *p = (src >= 0 && col_ok) ? in + (int64_t)src * ld_in + it.ch * 32 + gcol : g_zero_row;
+          f.q[i] = *reinterpret_cast<const float4 *>(p);
+        }
+        return f;
+      };
+      // through LDS into the MFMA A layout: lane (r, h) gets channels h*16 .. h*16+15 of row r
+      float *at = atile[wave];
+      auto transpose = [&](const Frag &gg) -> Frag {
+#pragma unroll
+        for (int i = 0; i < 4; i++) *reinterpret_cast<float4 *>(at + (8 * i + grow) * AT_LD + gcol) = gg.q[i];
+        Frag a;
+#pragma unroll
+        for (int q = 0; q < 4; q++) a.q[q] = *reinterpret_cast<const float4 *>(at + r * AT_LD + h * 16 + 4 * q);
+        return a;
+      };
+      auto wtile_of = [&](const Item &it, int b) -> const float * {
+        return Wp + (((int64_t)it.k * nch + it.ch) * nbtp + cb0 + b) * wtile;
+      };
+      Frag g[2], bw[2];
+      g[0] = gather(it0);
+      bw[0] = load_wfrag(wtile_of(it0, 0), lane);
+      Item it1 = advance(it0, last0);
+      g[1] = gather(it1);
+      Frag a = transpose(g[0]);
+      bool done = false;
+      while (!done) {
+#pragma unroll
+        for (int u = 0; u < 2; u++) {
+          const Item it2 = advance(it1, last1);
+          g[u % 2] = gather(it2);
+#pragma unroll
+          for (int b = 0; b < NB; b++) {
+            const int nn = u * NB + b;
+            if (b + 1 < NB)
+              bw[(nn + 1) % 2] = load_wfrag(wtile_of(it0, b + 1), lane);
+            else
+              bw[(nn + 1) % 2] = load_wfrag(wtile_of(it1, 0), lane);
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int s = 0; s < 16; s++)
+              acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(frag_at(a, s), frag_at(bw[nn % 2], s), acc[b], 0, 0, 0);
+          }
           asm volatile("" ::: "memory");
           __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-          for (int s = 0; s < 16; s++)
-            acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(frag_at(a, s), frag_at(bw[nn % 2], s), acc[b], 0, 0, 0);
-        }
-        // keep the consumer of the gather behind the MFMAs: hoisting it would wait for the loads
-        // right after they were issued
-        asm volatile("" ::: "memory");
-        __builtin_amdgcn_sched_barrier(0);
-        a = transpose(g);
-        it0 = it1;
-        if (last) {
-          done = true;
-          break;
+          if (last0) {
+            done = true;
+            break;
+          }
+          a = transpose(g[(u + 1) % 2]);
+          it0 = it1;
+          it1 = it2;
+          last0 = last1;
         }
       }
     }
@@ -370,12 +486,20 @@ int pack_weights(const float *W, int K, int Cin, int Cout, float *Wp, hipStream_
 
 // W: raw [K,Cin,Cout] weights (always needed by the generic kernel); Wp: packed weights or
 // null, in which case they are packed into scratch memory first.
-int launch_conv(const float *in, int64_t ld_in, float *out, int64_t ld_out, const float *W, const float *Wp,
-                const float *bias, const int32_t *map0, const int32_t *map1, int mode, int K, const int32_t *rows,
-                const int32_t *d_n_rows, int64_t n_rows, int Cin, int Cout, const uint8_t *tile_flags,
-                const uint8_t *row_mask, hipStream_t s) {
+int launch_conv(const float *in, int64_t ld_in, int64_t in_rows, float *out, int64_t ld_out, const float *W,
+                const float *Wp, const float *bias, const int32_t *map0, const int32_t *map1, int mode, int K,
+                const int32_t *rows, const int32_t *d_n_rows, int64_t n_rows, int Cin, int Cout,
+                const uint8_t *tile_flags, const uint8_t *row_mask, hipStream_t s) {
   if (n_rows == 0) return INSC_OK;
   if (conv_uses_mfma(in, ld_in, Cin, K)) {
+    // the gather addresses rows with 32-bit byte offsets (buffer loads)
+    const int64_t in_bytes64 = in_rows * ld_in * 4, wp_bytes64 = packed_floats(K, Cin, Cout) * 4;
+    if (in_rows < 0 || in_bytes64 >= (int64_t)BUF_OOB || wp_bytes64 >= (int64_t)BUF_OOB) {
+      set_error("conv: input matrix (%lld rows x %lld floats) or weights exceed the 4 GB the kernel addresses",
+                (long long)in_rows, (long long)ld_in);
+      return INSC_ERR_ARG;
+    }
+    const uint32_t in_bytes = (uint32_t)in_bytes64, wp_bytes = (uint32_t)wp_bytes64;
     if (!Wp) {
       void *ws;
       int rc = workspace(WS_API, s, sizeof(float) * (size_t)packed_floats(K, Cin, Cout), &ws);
@@ -402,7 +526,7 @@ int launch_conv(const float *in, int64_t ld_in, float *out, int64_t ld_out, cons
     bool shape_ok = true;
 #define INSC_CONV_LAUNCH(NBV, KV, MV, SV)                                                                       \
   hipLaunchKernelGGL((conv_mfma_kernel<NBV, KV, MV, SV>), grid, block, 0, s, in, ld_in, out, ld_out, Wp, bias,  \
-                     map0, map1, rows, d_n_rows, n_rows, Cin, Cout, nbtp, tile_flags)
+                     map0, map1, rows, d_n_rows, n_rows, Cin, Cout, nbtp, tile_flags, in_bytes, wp_bytes)
 #define INSC_CONV_CASE(NBV)                                      \
   case NBV:                                                      \
     if (mode == MAP_NBR && K == 27)                              \
@@ -472,16 +596,18 @@ int insc_conv_pack_weights(const float *d_W, int K, int Cin, int Cout, float *d_
   return pack_weights(d_W, K, Cin, Cout, d_Wp, (hipStream_t)stream);
 }
 
-int insc_conv_nbr(const float *d_in, int64_t ld_in, float *d_out, int64_t ld_out, const float *d_W,
-                  const float *d_Wp, const float *d_bias, const int32_t *d_nbr, int K, const int32_t *d_rows,
-                  const int32_t *d_n_rows, int64_t n_rows, int Cin, int Cout, double *h_muladds, void *stream) {
+int insc_conv_nbr(const float *d_in, int64_t ld_in, int64_t n_in_rows, float *d_out, int64_t ld_out,
+                  const float *d_W, const float *d_Wp, const float *d_bias, const int32_t *d_nbr, int K,
+                  const int32_t *d_rows, const int32_t *d_n_rows, int64_t n_rows, int Cin, int Cout,
+                  double *h_muladds, void *stream) {
   INSC_REQUIRE(n_rows >= 0 && Cin > 0 && Cout > 0 && K > 0 && K <= MAXK, INSC_ERR_ARG,
                "insc_conv_nbr: bad sizes (n_rows=%lld Cin=%d Cout=%d K=%d)", (long long)n_rows, Cin, Cout, K);
   INSC_REQUIRE(ld_in >= Cin && ld_out >= Cout, INSC_ERR_ARG, "insc_conv_nbr: row stride smaller than channel count");
   INSC_REQUIRE(n_rows == 0 || (d_in && d_out && (d_W || d_Wp)), INSC_ERR_ARG, "insc_conv_nbr: null pointer");
   INSC_REQUIRE(d_nbr || K == 1, INSC_ERR_ARG, "insc_conv_nbr: a null map needs K == 1");
   hipStream_t s = (hipStream_t)stream;
-  int rc = launch_conv(d_in, ld_in, d_out, ld_out, d_W, d_Wp, d_bias, d_nbr, nullptr,
+  INSC_REQUIRE(n_in_rows >= 0, INSC_ERR_ARG, "insc_conv_nbr: n_in_rows is negative");
+  int rc = launch_conv(d_in, ld_in, n_in_rows, d_out, ld_out, d_W, d_Wp, d_bias, d_nbr, nullptr,
                        d_nbr ? MAP_NBR : MAP_IDENTITY, K, d_rows, d_n_rows, n_rows, Cin, Cout, nullptr, nullptr, s);
   if (rc) return rc;
   if (h_muladds) {
@@ -510,15 +636,16 @@ int insc_conv_nbr(const float *d_in, int64_t ld_in, float *d_out, int64_t ld_out
   return INSC_OK;
 }
 
-int insc_deconv_down2(const float *d_in, int64_t ld_in, float *d_out, int64_t ld_out, const float *d_W,
-                      const float *d_Wp, const float *d_bias, const int32_t *d_parent, const int32_t *d_offset,
-                      const int32_t *d_rows, const int32_t *d_n_rows, int64_t n_rows, int Cin, int Cout,
-                      void *stream) {
+int insc_deconv_down2(const float *d_in, int64_t ld_in, int64_t n_in_rows, float *d_out, int64_t ld_out,
+                      const float *d_W, const float *d_Wp, const float *d_bias, const int32_t *d_parent,
+                      const int32_t *d_offset, const int32_t *d_rows, const int32_t *d_n_rows, int64_t n_rows,
+                      int Cin, int Cout, void *stream) {
   INSC_REQUIRE(n_rows >= 0 && Cin > 0 && Cout > 0, INSC_ERR_ARG, "insc_deconv_down2: bad sizes");
   INSC_REQUIRE(ld_in >= Cin && ld_out >= Cout, INSC_ERR_ARG, "insc_deconv_down2: row stride too small");
   INSC_REQUIRE(n_rows == 0 || (d_in && d_out && (d_W || d_Wp) && d_parent && d_offset), INSC_ERR_ARG,
                "insc_deconv_down2: null pointer");
-  return launch_conv(d_in, ld_in, d_out, ld_out, d_W, d_Wp, d_bias, d_parent, d_offset, MAP_PARENT, 8, d_rows,
+  INSC_REQUIRE(n_in_rows >= 0, INSC_ERR_ARG, "insc_deconv_down2: n_in_rows is negative");
+  return launch_conv(d_in, ld_in, n_in_rows, d_out, ld_out, d_W, d_Wp, d_bias, d_parent, d_offset, MAP_PARENT, 8, d_rows,
                      d_n_rows, n_rows, Cin, Cout, nullptr, nullptr, (hipStream_t)stream);
 }
 

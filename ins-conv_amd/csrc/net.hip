@@ -389,20 +389,21 @@ static int run_op(insc_net *net, const Op &op, bool incremental, hipStream_t s) 
   const int64_t ld_out = tensor_ld(net, op.out);
   const float *in0 = tensor_ptr(net, op.in0);
   const int64_t ld0 = tensor_ld(net, op.in0);
+  const int64_t rows0 = net->buffers[net->tensors[op.in0].buf].rows;
   switch (op.kind) {
     case OP_SSC:
-      return launch_conv(in0, ld0, out, ld_out, op.W, op.Wp, op.bias, Lo.nbr, nullptr, MAP_NBR, 27, Lo.order, d_n,
+      return launch_conv(in0, ld0, rows0, out, ld_out, op.W, op.Wp, op.bias, Lo.nbr, nullptr, MAP_NBR, 27, Lo.order, d_n,
                          n_up, op.Cin, op.Cout, d ? d->tflag : nullptr, d ? d->mask : nullptr, s);
     case OP_NIN:
-      return launch_conv(in0, ld0, out, ld_out, op.W, op.Wp, op.bias, nullptr, nullptr, MAP_IDENTITY, 1, Lo.order,
+      return launch_conv(in0, ld0, rows0, out, ld_out, op.W, op.Wp, op.bias, nullptr, nullptr, MAP_IDENTITY, 1, Lo.order,
                          d_n, n_up, op.Cin, op.Cout, d ? d->tflag : nullptr, d ? d->mask : nullptr, s);
     case OP_CONV: {
       const Level &Lf = net->levels[To.level - 1];
-      return launch_conv(in0, ld0, out, ld_out, op.W, op.Wp, op.bias, Lf.child, nullptr, MAP_NBR, 8, Lo.order, d_n,
+      return launch_conv(in0, ld0, rows0, out, ld_out, op.W, op.Wp, op.bias, Lf.child, nullptr, MAP_NBR, 8, Lo.order, d_n,
                          n_up, op.Cin, op.Cout, d ? d->tflag : nullptr, d ? d->mask : nullptr, s);
     }
     case OP_DECONV:
-      return launch_conv(in0, ld0, out, ld_out, op.W, op.Wp, op.bias, Lo.parent, Lo.offset, MAP_PARENT, 8,
+      return launch_conv(in0, ld0, rows0, out, ld_out, op.W, op.Wp, op.bias, Lo.parent, Lo.offset, MAP_PARENT, 8,
                          Lo.bo_order, d_n, n_up, op.Cin, op.Cout, d ? d->tflag_bo : nullptr, d ? d->mask : nullptr,
                          s);
     case OP_BN:

@@ -312,14 +312,14 @@ def packed_weight(weight, K):
 def conv_rows(in_f, out_f, weight, bias, nbr, K, rows, count, n_rows):
     """insc_conv_nbr on a row subset; in_f/out_f may be column slices of wider buffers."""
     Cin, Cout = weight.size(-2), weight.size(-1)
-    lib.insc_conv_nbr(ptr(in_f), I64(_ld(in_f)), ptr(out_f), I64(_ld(out_f)), ptr(weight),
+    lib.insc_conv_nbr(ptr(in_f), I64(_ld(in_f)), I64(in_f.size(0)), ptr(out_f), I64(_ld(out_f)), ptr(weight),
                       ptr(packed_weight(weight, K)), ptr(bias), ptr(nbr), int(K), ptr(rows), ptr(count),
                       I64(int(n_rows)), int(Cin), int(Cout), None, stream_ptr())
 
 
 def deconv_rows(in_f, out_f, weight, bias, parent, offset, rows, count, n_rows):
     Cin, Cout = weight.size(-2), weight.size(-1)
-    lib.insc_deconv_down2(ptr(in_f), I64(_ld(in_f)), ptr(out_f), I64(_ld(out_f)), ptr(weight),
+    lib.insc_deconv_down2(ptr(in_f), I64(_ld(in_f)), I64(in_f.size(0)), ptr(out_f), I64(_ld(out_f)), ptr(weight),
                           ptr(packed_weight(weight, 8)), ptr(bias), ptr(parent), ptr(offset), ptr(rows), ptr(count),
                           I64(int(n_rows)), int(Cin), int(Cout), stream_ptr())
 
