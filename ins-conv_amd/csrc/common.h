@@ -45,11 +45,25 @@ int sort_pairs_u64(uint64_t *keys, int32_t *vals, int64_t n, int key_bits, hipSt
 enum { MAP_NBR = 0, MAP_IDENTITY = 1, MAP_PARENT = 2 };
 // tile_flags: one byte per 32-row tile of `rows` (matrix-core kernel); row_mask: one byte per
 // site (generic kernel and the streaming kernels).  Null = everything.
-// in_rows: rows of the input matrix (bounds the gather).
+// Optional fused inference batch norm + leaky ReLU behind a producing kernel:
+//   y = fmaf(x, w[c], b[c]); y *= (y > 0 ? 1 : leak)  ->  out2 (row stride ld2)
+// w, b are the per-channel scale / shift (bn_scale_shift).  The producer still writes its raw
+// result x to its own output unless that pointer is null.
+struct BnEpilogue {
+  const float *w = nullptr, *b = nullptr;
+  float leak = 0.0f;
+  float *out2 = nullptr;
+  int64_t ld2 = 0;
+};
+// w = gamma / sqrt(var + eps), b = beta - mean * w   (gamma / beta nullable)
+int bn_scale_shift(const float *mean, const float *var, const float *gamma, const float *beta, float eps, int C,
+                   float *w, float *b, hipStream_t s);
+
+// in_rows: rows of the input matrix (bounds the gather).  out may be null when ep.out2 is set.
 int launch_conv(const float *in, int64_t ld_in, int64_t in_rows, float *out, int64_t ld_out, const float *W,
                 const float *Wp, const float *bias, const int32_t *map0, const int32_t *map1, int mode, int K,
                 const int32_t *rows, const int32_t *d_n_rows, int64_t n_rows, int Cin, int Cout,
-                const uint8_t *tile_flags, const uint8_t *row_mask, hipStream_t s);
+                const uint8_t *tile_flags, const uint8_t *row_mask, hipStream_t s, BnEpilogue ep = BnEpilogue());
 int64_t packed_floats(int K, int Cin, int Cout);
 int pack_weights(const float *W, int K, int Cin, int Cout, float *Wp, hipStream_t s);
 int launch_bn(const float *in, int64_t ld_in, float *out, int64_t ld_out, const float *mean, const float *var,
@@ -58,7 +72,7 @@ int launch_bn(const float *in, int64_t ld_in, float *out, int64_t ld_out, const 
 // out = a + b (b != null) or out = a
 int launch_add(const float *a, int64_t ld_a, const float *b, int64_t ld_b, float *out, int64_t ld_out,
                const int32_t *rows, const int32_t *d_n_rows, int64_t n_rows, int C, const uint8_t *row_mask,
-               hipStream_t s);
+               hipStream_t s, BnEpilogue ep = BnEpilogue());
 int launch_input_finish(const float *sum, const int32_t *cnt, int mode, float *out, int64_t ld_out,
                         const int32_t *rows, const int32_t *d_n_rows, int64_t n_rows, int C,
                         const uint8_t *row_mask, hipStream_t s);

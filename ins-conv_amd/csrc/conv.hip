@@ -32,7 +32,7 @@ __global__ __launch_bounds__(256) void conv_generic_kernel(const float *__restri
                                                            const int32_t *__restrict__ rows,
                                                            const int32_t *__restrict__ d_n_rows, int64_t n_rows,
                                                            int Cin, int Cout,
-                                                           const uint8_t *__restrict__ row_mask) {
+                                                           const uint8_t *__restrict__ row_mask, BnEpilogue ep) {
   const int64_t n = d_n_rows ? min((int64_t)*d_n_rows, n_rows) : n_rows;
   const int cpb = 256 / Cout > 0 ? 256 / Cout : 1;  // rows per block (Cout <= 256)
   const int lr = threadIdx.x / Cout, co = threadIdx.x % Cout;
@@ -54,7 +54,11 @@ __global__ __launch_bounds__(256) void conv_generic_kernel(const float *__restri
       const float *w = W + (int64_t)k * Cin * Cout + co;
       for (int ci = 0; ci < Cin; ci++) acc = fmaf(x[ci], w[(int64_t)ci * Cout], acc);
     }
-    out[(int64_t)row * ld_out + co] = acc;
+    if (out) out[(int64_t)row * ld_out + co] = acc;
+    if (ep.out2) {
+      const float y = fmaf(acc, ep.w[co], ep.b[co]);
+      ep.out2[(int64_t)row * ep.ld2 + co] = y * ((y > 0.0f) ? 1.0f : ep.leak);
+    }
   }
 }
 
@@ -163,7 +167,7 @@ __global__ __launch_bounds__((S == 1 ? CONV_WAVES : S) * 64) void conv_mfma_kern
     const float *__restrict__ Wp, const float *__restrict__ bias, const int32_t *__restrict__ map0,
     const int32_t *__restrict__ map1, const int32_t *__restrict__ rows,
     const int32_t *__restrict__ d_n_rows, int64_t n_rows, int Cin, int Cout, int nbtp,
-    const uint8_t *__restrict__ tile_flags, uint32_t in_bytes, uint32_t wp_bytes) {
+    const uint8_t *__restrict__ tile_flags, uint32_t in_bytes, uint32_t wp_bytes, BnEpilogue ep) {
   static_assert(S == 1 || NB == 1, "split tiles use one output block per wavefront");
   constexpr int WAVES = S == 1 ? CONV_WAVES : S;
   __shared__ int nbl[S == 1 ? WAVES : 1][TILE_M * K];
@@ -440,16 +444,35 @@ __global__ __launch_bounds__((S == 1 ? CONV_WAVES : S) * 64) void conv_mfma_kern
     }
   }
 
+  // fused batch norm + leaky ReLU: per-channel scale / shift of this lane's columns
+  float ew[NB], eb[NB];
+#pragma unroll
+  for (int b = 0; b < NB; b++) {
+    const int c = (cb0 + b) * 32 + r;
+    ew[b] = (ep.out2 && c < Cout) ? ep.w[c] : 0.0f;
+    eb[b] = (ep.out2 && c < Cout) ? ep.b[c] : 0.0f;
+  }
   // D layout of the 32x32 MFMA: lane holds column (lane & 31), rows 8*(v/4) + 4*(lane>>5) + (v&3)
 #pragma unroll
   for (int v = 0; v < 16; v++) {
     const int i = 8 * (v >> 2) + 4 * h + (v & 3);
     const int rid = __shfl(my_row, i, 64);
     if (rid < 0) continue;
-    float *op = out + (int64_t)rid * ld_out + cb0 * 32 + r;
+    if (out) {
+      float *op = out + (int64_t)rid * ld_out + cb0 * 32 + r;
 #pragma unroll
-    for (int b = 0; b < NB; b++)
-      if ((cb0 + b) * 32 + r < Cout) op[b * 32] = acc[b][v];
+      for (int b = 0; b < NB; b++)
+        if ((cb0 + b) * 32 + r < Cout) op[b * 32] = acc[b][v];
+    }
+    if (ep.out2) {
+      float *op2 = ep.out2 + (int64_t)rid * ep.ld2 + cb0 * 32 + r;
+#pragma unroll
+      for (int b = 0; b < NB; b++)
+        if ((cb0 + b) * 32 + r < Cout) {
+          const float y = fmaf(acc[b][v], ew[b], eb[b]);
+          op2[b * 32] = y * ((y > 0.0f) ? 1.0f : ep.leak);
+        }
+    }
   }
 }
 
@@ -489,7 +512,7 @@ int pack_weights(const float *W, int K, int Cin, int Cout, float *Wp, hipStream_
 int launch_conv(const float *in, int64_t ld_in, int64_t in_rows, float *out, int64_t ld_out, const float *W,
                 const float *Wp, const float *bias, const int32_t *map0, const int32_t *map1, int mode, int K,
                 const int32_t *rows, const int32_t *d_n_rows, int64_t n_rows, int Cin, int Cout,
-                const uint8_t *tile_flags, const uint8_t *row_mask, hipStream_t s) {
+                const uint8_t *tile_flags, const uint8_t *row_mask, hipStream_t s, BnEpilogue ep) {
   if (n_rows == 0) return INSC_OK;
   if (conv_uses_mfma(in, ld_in, Cin, K)) {
     // the gather addresses rows with 32-bit byte offsets (buffer loads)
@@ -526,7 +549,7 @@ int launch_conv(const float *in, int64_t ld_in, int64_t in_rows, float *out, int
     bool shape_ok = true;
 #define INSC_CONV_LAUNCH(NBV, KV, MV, SV)                                                                       \
   hipLaunchKernelGGL((conv_mfma_kernel<NBV, KV, MV, SV>), grid, block, 0, s, in, ld_in, out, ld_out, Wp, bias,  \
-                     map0, map1, rows, d_n_rows, n_rows, Cin, Cout, nbtp, tile_flags, in_bytes, wp_bytes)
+                     map0, map1, rows, d_n_rows, n_rows, Cin, Cout, nbtp, tile_flags, in_bytes, wp_bytes, ep)
 #define INSC_CONV_CASE(NBV)                                      \
   case NBV:                                                      \
     if (mode == MAP_NBR && K == 27)                              \
@@ -573,7 +596,7 @@ int launch_conv(const float *in, int64_t ld_in, int64_t in_rows, float *out, int
     }
     const int cpb = 256 / Cout;
     hipLaunchKernelGGL(conv_generic_kernel, dim3(grid_for(n_rows, cpb, 65536)), dim3(256), 0, s, in, ld_in, out,
-                       ld_out, W, bias, map0, map1, mode, K, rows, d_n_rows, n_rows, Cin, Cout, row_mask);
+                       ld_out, W, bias, map0, map1, mode, K, rows, d_n_rows, n_rows, Cin, Cout, row_mask, ep);
   }
   INSC_LAUNCH_CHECK();
   return INSC_OK;

@@ -46,6 +46,7 @@ struct Buffer {
 
 struct Tensor {
   int level = 0, C = 0, buf = -1, col0 = 0, dirty = -1;
+  bool kept = true;  // false: nothing reads it any more (its batch norm moved into its producer)
 };
 
 struct Op {
@@ -54,6 +55,11 @@ struct Op {
   float *Wp = nullptr;  // packed weights, owned
   float eps = 0, leak = 0;
   int Cin = 0, Cout = 0;
+  // batch norm folded into the kernel that produces its input
+  float *bn_w = nullptr, *bn_b = nullptr;  // per-channel scale / shift of an OP_BN, owned
+  int fused_bn = -1;                       // producer side: index of the OP_BN it also computes
+  bool write_raw = true;                   // producer side: its own output has other readers
+  bool fused = false;                      // OP_BN side: computed by its producer, no kernel of its own
 };
 
 struct DirtyNode {
@@ -380,38 +386,48 @@ static int sync_counts(insc_net *net, hipStream_t s, const char *who) {
 
 // ---- one layer ------------------------------------------------------------------------
 static int run_op(insc_net *net, const Op &op, bool incremental, hipStream_t s) {
+  if (op.fused) return INSC_OK;
   const Tensor &To = net->tensors[op.out];
   const Level &Lo = net->levels[To.level];
   const DirtyNode *d = incremental ? &net->dirty[To.dirty] : nullptr;
   const int32_t *d_n = Lo.grid->d_n;
   const int64_t n_up = Lo.n_upper;
-  float *out = tensor_ptr(net, op.out);
+  float *out = op.write_raw ? tensor_ptr(net, op.out) : nullptr;
   const int64_t ld_out = tensor_ld(net, op.out);
+  BnEpilogue ep;
+  if (op.fused_bn >= 0) {
+    const Op &bn = net->ops[op.fused_bn];
+    ep.w = bn.bn_w;
+    ep.b = bn.bn_b;
+    ep.leak = bn.leak;
+    ep.out2 = tensor_ptr(net, bn.out);
+    ep.ld2 = tensor_ld(net, bn.out);
+  }
   const float *in0 = tensor_ptr(net, op.in0);
   const int64_t ld0 = tensor_ld(net, op.in0);
   const int64_t rows0 = net->buffers[net->tensors[op.in0].buf].rows;
   switch (op.kind) {
     case OP_SSC:
       return launch_conv(in0, ld0, rows0, out, ld_out, op.W, op.Wp, op.bias, Lo.nbr, nullptr, MAP_NBR, 27, Lo.order, d_n,
-                         n_up, op.Cin, op.Cout, d ? d->tflag : nullptr, d ? d->mask : nullptr, s);
+                         n_up, op.Cin, op.Cout, d ? d->tflag : nullptr, d ? d->mask : nullptr, s, ep);
     case OP_NIN:
       return launch_conv(in0, ld0, rows0, out, ld_out, op.W, op.Wp, op.bias, nullptr, nullptr, MAP_IDENTITY, 1, Lo.order,
-                         d_n, n_up, op.Cin, op.Cout, d ? d->tflag : nullptr, d ? d->mask : nullptr, s);
+                         d_n, n_up, op.Cin, op.Cout, d ? d->tflag : nullptr, d ? d->mask : nullptr, s, ep);
     case OP_CONV: {
       const Level &Lf = net->levels[To.level - 1];
       return launch_conv(in0, ld0, rows0, out, ld_out, op.W, op.Wp, op.bias, Lf.child, nullptr, MAP_NBR, 8, Lo.order, d_n,
-                         n_up, op.Cin, op.Cout, d ? d->tflag : nullptr, d ? d->mask : nullptr, s);
+                         n_up, op.Cin, op.Cout, d ? d->tflag : nullptr, d ? d->mask : nullptr, s, ep);
     }
     case OP_DECONV:
       return launch_conv(in0, ld0, rows0, out, ld_out, op.W, op.Wp, op.bias, Lo.parent, Lo.offset, MAP_PARENT, 8,
                          Lo.bo_order, d_n, n_up, op.Cin, op.Cout, d ? d->tflag_bo : nullptr, d ? d->mask : nullptr,
-                         s);
+                         s, ep);
     case OP_BN:
       return launch_bn(in0, ld0, out, ld_out, op.mean, op.var, op.gamma, op.beta, op.eps, op.leak, nullptr, d_n,
                        n_up, op.Cout, d ? d->mask : nullptr, s);
     case OP_ADD:
       return launch_add(in0, ld0, tensor_ptr(net, op.in1), tensor_ld(net, op.in1), out, ld_out, nullptr, d_n, n_up,
-                        op.Cout, d ? d->mask : nullptr, s);
+                        op.Cout, d ? d->mask : nullptr, s, ep);
     case OP_COPY:
       return launch_add(in0, ld0, nullptr, 0, out, ld_out, nullptr, d_n, n_up, op.Cout, d ? d->mask : nullptr, s);
     case OP_JOIN:
@@ -498,8 +514,11 @@ int insc_net_destroy(insc_net *net) {
   }
   for (Buffer &B : net->buffers)
     if (B.p) (void)hipFree(B.p);
-  for (Op &op : net->ops)
+  for (Op &op : net->ops) {
     if (op.Wp) (void)hipFree(op.Wp);
+    if (op.bn_w) (void)hipFree(op.bn_w);
+    if (op.bn_b) (void)hipFree(op.bn_b);
+  }
   void *ps[] = {net->in_sum, net->in_cnt, net->chain_head, net->chain_next, net->site_of_point, net->mask_arena};
   for (void *p : ps)
     if (p) (void)hipFree(p);
@@ -669,6 +688,41 @@ int insc_net_finalize(insc_net *net, int out_tensor, int64_t capacity_sites, voi
       }
     }
   }
+  // Fold each batch norm into the kernel that produces its input (one fewer pass over the rows
+  // and one fewer launch); the producer keeps writing its raw result only if something else
+  // reads it.  A tensor nothing reads any more loses its matrix.
+  {
+    const int nt = (int)net->tensors.size();
+    std::vector<int> producer(nt, -1), readers(nt, 0);
+    for (int i = 0; i < (int)net->ops.size(); i++) {
+      const Op &op = net->ops[i];
+      if (op.kind != OP_JOIN) producer[op.out] = producer[op.out] == -1 ? i : -2;
+      readers[op.in0]++;
+      if (op.in1 >= 0) readers[op.in1]++;
+    }
+    readers[out_tensor]++;
+    for (int i = 0; i < (int)net->ops.size(); i++) {
+      Op &bn = net->ops[i];
+      if (bn.kind != OP_BN) continue;
+      int rc;
+      if ((rc = dev_alloc(&bn.bn_w, (size_t)bn.Cout))) return rc;
+      if ((rc = dev_alloc(&bn.bn_b, (size_t)bn.Cout))) return rc;
+      if ((rc = bn_scale_shift(bn.mean, bn.var, bn.gamma, bn.beta, bn.eps, bn.Cout, bn.bn_w, bn.bn_b, s))) return rc;
+      if (bn.in0 == bn.out || producer[bn.in0] < 0 || producer[bn.out] != i) continue;
+      Op &A = net->ops[producer[bn.in0]];
+      const bool can = A.kind == OP_SSC || A.kind == OP_CONV || A.kind == OP_DECONV || A.kind == OP_NIN || A.kind == OP_ADD;
+      if (!can || A.fused_bn >= 0 || producer[bn.in0] > i) continue;
+      A.fused_bn = i;
+      bn.fused = true;
+      A.write_raw = readers[bn.in0] > 1;
+      if (!A.write_raw) {
+        Tensor &T = net->tensors[bn.in0];
+        Buffer &B = net->buffers[T.buf];
+        if (T.col0 == 0 && B.ld == T.C) B.ld = 0;
+        T.kept = false;
+      }
+    }
+  }
   net->finalized = true;
   int64_t cap = std::max<int64_t>(capacity_sites, 1024);
   for (int l = 0; l < net->n_levels; l++) {
@@ -687,6 +741,12 @@ int insc_net_refresh_weights(insc_net *net, void *stream) {
     if (op.Wp) {
       const int K = op.kind == OP_SSC ? 27 : op.kind == OP_NIN ? 1 : 8;
       int rc = pack_weights(op.W, K, op.Cin, op.Cout, op.Wp, (hipStream_t)stream);
+      if (rc) return rc;
+    }
+  for (Op &op : net->ops)
+    if (op.bn_w) {
+      int rc = bn_scale_shift(op.mean, op.var, op.gamma, op.beta, op.eps, op.Cout, op.bn_w, op.bn_b,
+                              (hipStream_t)stream);
       if (rc) return rc;
     }
   return INSC_OK;
@@ -824,6 +884,9 @@ int insc_net_forward(insc_net *net, const int32_t *d_coords, int coord_cols, con
 int insc_net_tensor_view(insc_net *net, int tensor, float **d_ptr, int64_t *ld, int64_t *rows, int *channels) {
   INSC_REQUIRE(net && net->finalized && tensor >= 0 && tensor < (int)net->tensors.size(), INSC_ERR_ARG,
                "insc_net_tensor_view: bad arguments");
+  INSC_REQUIRE(net->tensors[tensor].kept, INSC_ERR_STATE,
+               "insc_net_tensor_view: tensor %d is not kept (its only reader, a batch norm, is computed by its producer)",
+               tensor);
   if (d_ptr) *d_ptr = tensor_ptr(net, tensor);
   if (ld) *ld = tensor_ld(net, tensor);
   if (rows) *rows = net->levels[net->tensors[tensor].level].n;

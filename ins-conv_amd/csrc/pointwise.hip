@@ -28,6 +28,16 @@ struct Vec<1> {
 
 __device__ __forceinline__ float leaky(float o, float leak) { return o * ((o > 0.0f) ? 1.0f : leak); }
 
+// per-channel scale / shift of inference batch norm; every kernel that normalises goes through
+// this one function so that fused and unfused paths give the same bits
+__device__ __forceinline__ void bn_coeffs(const float *__restrict__ mean, const float *__restrict__ var,
+                                          const float *__restrict__ gamma, const float *__restrict__ beta, float eps,
+                                          int c, float &w, float &b) {
+  const float invstd = 1.0f / sqrtf(var[c] + eps);
+  w = invstd * (gamma ? gamma[c] : 1.0f);
+  b = fmaf(-mean[c], w, beta ? beta[c] : 0.0f);
+}
+
 template <int V>
 __global__ __launch_bounds__(256) void bn_kernel(const float *__restrict__ in, int64_t ld_in, float *__restrict__ out,
                                                  int64_t ld_out, const float *__restrict__ mean,
@@ -44,10 +54,7 @@ __global__ __launch_bounds__(256) void bn_kernel(const float *__restrict__ in, i
   float w[V], b[V];
 #pragma unroll
   for (int i = 0; i < V; i++) {
-    const int c = g * V + i;
-    const float invstd = 1.0f / sqrtf(var[c] + eps);
-    w[i] = invstd * (gamma ? gamma[c] : 1.0f);
-    b[i] = -mean[c] * w[i] + (beta ? beta[c] : 0.0f);
+    bn_coeffs(mean, var, gamma, beta, eps, g * V + i, w[i], b[i]);
   }
   for (int64_t t = (int64_t)blockIdx.x * rpb + lr; t < n; t += (int64_t)gridDim.x * rpb) {
     const int row = rows ? rows[t] : (int)t;
@@ -55,7 +62,7 @@ __global__ __launch_bounds__(256) void bn_kernel(const float *__restrict__ in, i
     typename Vec<V>::T x = Vec<V>::ld(in + (int64_t)row * ld_in + g * V);
     float *xf = reinterpret_cast<float *>(&x);
 #pragma unroll
-    for (int i = 0; i < V; i++) xf[i] = leaky(xf[i] * w[i] + b[i], leak);
+    for (int i = 0; i < V; i++) xf[i] = leaky(fmaf(xf[i], w[i], b[i]), leak);
     Vec<V>::st(out + (int64_t)row * ld_out + g * V, x);
   }
 }
@@ -74,9 +81,9 @@ __global__ __launch_bounds__(256) void bn_wide_kernel(const float *__restrict__ 
     const int c = (int)(e - t * C);
     const int row = rows ? rows[t] : (int)t;
     if (row < 0 || (row_mask && !row_mask[row])) continue;
-    const float wv = (gamma ? gamma[c] : 1.0f) / sqrtf(var[c] + eps);
-    const float bv = -mean[c] * wv + (beta ? beta[c] : 0.0f);
-    out[(int64_t)row * ld_out + c] = leaky(in[(int64_t)row * ld_in + c] * wv + bv, leak);
+    float wv, bv;
+    bn_coeffs(mean, var, gamma, beta, eps, c, wv, bv);
+    out[(int64_t)row * ld_out + c] = leaky(fmaf(in[(int64_t)row * ld_in + c], wv, bv), leak);
   }
 }
 
@@ -86,7 +93,7 @@ __global__ __launch_bounds__(256) void add_kernel(const float *__restrict__ a, i
                                                   const float *__restrict__ b, int64_t ld_b, float *__restrict__ out,
                                                   int64_t ld_out, const int32_t *__restrict__ rows,
                                                   const int32_t *__restrict__ d_n_rows, int64_t n_rows, int C,
-                                                  const uint8_t *__restrict__ row_mask) {
+                                                  const uint8_t *__restrict__ row_mask, BnEpilogue ep) {
   const int64_t n = row_count(d_n_rows, n_rows);
   const int groups = C / V;
   for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < n * groups; e += (int64_t)gridDim.x * 256) {
@@ -102,8 +109,25 @@ __global__ __launch_bounds__(256) void add_kernel(const float *__restrict__ a, i
 #pragma unroll
       for (int i = 0; i < V; i++) xf[i] += yf[i];
     }
-    Vec<V>::st(out + (int64_t)row * ld_out + g * V, x);
+    if (out) Vec<V>::st(out + (int64_t)row * ld_out + g * V, x);
+    if (ep.out2) {
+      float *xf = reinterpret_cast<float *>(&x);
+#pragma unroll
+      for (int i = 0; i < V; i++) xf[i] = leaky(fmaf(xf[i], ep.w[g * V + i], ep.b[g * V + i]), ep.leak);
+      Vec<V>::st(ep.out2 + (int64_t)row * ep.ld2 + g * V, x);
+    }
   }
+}
+
+__global__ void bn_scale_shift_kernel(const float *__restrict__ mean, const float *__restrict__ var,
+                                      const float *__restrict__ gamma, const float *__restrict__ beta, float eps,
+                                      int C, float *__restrict__ w, float *__restrict__ b) {
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= C) return;
+  float wv, bv;
+  bn_coeffs(mean, var, gamma, beta, eps, c, wv, bv);
+  w[c] = wv;
+  b[c] = bv;
 }
 
 __global__ __launch_bounds__(256) void gather_rows_kernel(const float *__restrict__ in, int64_t ld_in,
@@ -212,26 +236,35 @@ int launch_bn(const float *d_in, int64_t ld_in, float *d_out, int64_t ld_out, co
   return INSC_OK;
 }
 
+int bn_scale_shift(const float *mean, const float *var, const float *gamma, const float *beta, float eps, int C,
+                   float *w, float *b, hipStream_t s) {
+  hipLaunchKernelGGL(bn_scale_shift_kernel, dim3(grid_for(C, 256)), dim3(256), 0, s, mean, var, gamma, beta, eps, C, w,
+                     b);
+  INSC_LAUNCH_CHECK();
+  return INSC_OK;
+}
+
 int launch_add(const float *d_a, int64_t ld_a, const float *d_b, int64_t ld_b, float *d_out, int64_t ld_out,
                const int32_t *d_rows, const int32_t *d_n_rows, int64_t n_rows, int C, const uint8_t *row_mask,
-               hipStream_t s) {
+               hipStream_t s, BnEpilogue ep) {
   if (n_rows == 0) return INSC_OK;
-  const bool v4 = C % 4 == 0 && vec4_ok(d_a, ld_a) && (!d_b || vec4_ok(d_b, ld_b)) && vec4_ok(d_out, ld_out);
+  const bool v4 = C % 4 == 0 && vec4_ok(d_a, ld_a) && (!d_b || vec4_ok(d_b, ld_b)) &&
+                  (!d_out || vec4_ok(d_out, ld_out)) && (!ep.out2 || vec4_ok(ep.out2, ep.ld2));
   const unsigned nb = grid_for(n_rows * (v4 ? C / 4 : C), 1024, 1 << 16);
   if (d_b) {
     if (v4)
       hipLaunchKernelGGL((add_kernel<4, true>), dim3(nb), dim3(256), 0, s, d_a, ld_a, d_b, ld_b, d_out, ld_out,
-                         d_rows, d_n_rows, n_rows, C, row_mask);
+                         d_rows, d_n_rows, n_rows, C, row_mask, ep);
     else
       hipLaunchKernelGGL((add_kernel<1, true>), dim3(nb), dim3(256), 0, s, d_a, ld_a, d_b, ld_b, d_out, ld_out,
-                         d_rows, d_n_rows, n_rows, C, row_mask);
+                         d_rows, d_n_rows, n_rows, C, row_mask, ep);
   } else {
     if (v4)
       hipLaunchKernelGGL((add_kernel<4, false>), dim3(nb), dim3(256), 0, s, d_a, ld_a, d_b, ld_b, d_out, ld_out,
-                         d_rows, d_n_rows, n_rows, C, row_mask);
+                         d_rows, d_n_rows, n_rows, C, row_mask, ep);
     else
       hipLaunchKernelGGL((add_kernel<1, false>), dim3(nb), dim3(256), 0, s, d_a, ld_a, d_b, ld_b, d_out, ld_out,
-                         d_rows, d_n_rows, n_rows, C, row_mask);
+                         d_rows, d_n_rows, n_rows, C, row_mask, ep);
   }
   INSC_LAUNCH_CHECK();
   return INSC_OK;
