@@ -103,49 +103,28 @@ struct Frag {
   float4 q[4];
 };
 
-// Lanes whose row has no neighbour at the current offset read this row of zeros instead, so
-// the gather needs no branch and no select.
-__device__ __attribute__((aligned(64))) float g_zero_row[16];  // all lanes read the first 16 bytes
-
-__device__ __forceinline__ Frag load_frag(const float *p) {
-  Frag f;
-  const float4 *p4 = reinterpret_cast<const float4 *>(p);
-#pragma unroll
-  for (int i = 0; i < 4; i++) f.q[i] = p4[i];
-  return f;
-}
-// weight tile: quarter q of the tile starts at q*256 floats, this lane's values at lane*4
-__device__ __forceinline__ Frag load_wfrag(const float *tile, int lane) {
-  Frag f;
-  const float4 *p4 = reinterpret_cast<const float4 *>(tile) + lane;
-#pragma unroll
-  for (int i = 0; i < 4; i++) f.q[i] = p4[i * 64];
-  return f;
-}
 __device__ __forceinline__ float frag_at(const Frag &f, int s) {
   const float4 v = f.q[s >> 2];
   return (s & 3) == 0 ? v.x : (s & 3) == 1 ? v.y : (s & 3) == 2 ? v.z : v.w;
 }
 
-// LDS row stride of the gather tile in floats: 32 channels + 4 of padding, so that both the
-// row-wise 16-byte writes and the column-block reads of the MFMA layout spread over all banks.
-constexpr int AT_LD = 36;
-
-// Gather flavour.  DIRECT_GATHER: every lane reads the 64 bytes of its own input row that the
-// MFMA A operand needs, with buffer loads: one 32-bit offset per item, rows without a
-// neighbour get an out-of-range offset and the hardware returns zeros, and the weight tile is
-// addressed by a scalar offset - a handful of non-MFMA instructions per 16 MFMAs (ordinary
-// VALU work does not overlap with MFMAs on this part, so it is paid in matrix-core time).
-// Otherwise: coalesced 128-byte row segments, transposed through LDS into the A layout
-// (fewer cache-line touches per instruction, but ~100 extra instructions per item).
-#ifndef INSC_CONV_DIRECT
-#define INSC_CONV_DIRECT 1
+// Gather: every lane reads the 64 bytes of its own input row that the MFMA A operand needs, with
+// buffer loads: one 32-bit offset per item, rows without a neighbour get an out-of-range offset
+// and the hardware returns zeros, and the weight tile is addressed by a scalar offset - a
+// handful of non-MFMA instructions per 16 MFMAs (ordinary VALU work does not overlap with MFMAs
+// on this part, so it is paid in matrix-core time).
+// Items in flight per wavefront (ring depth): whole-tile wavefronts, and wavefronts that share a
+// tile (few of them per SIMD, so each must cover more latency itself).
+#ifndef INSC_CONV_DEPTH
+#define INSC_CONV_DEPTH 3
 #endif
-constexpr bool DIRECT_GATHER = INSC_CONV_DIRECT != 0;
+#ifndef INSC_CONV_DEPTH_SPLIT
+#define INSC_CONV_DEPTH_SPLIT 4
+#endif
 
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 // offsets at or beyond this bound make a buffer load return zeros
-constexpr uint32_t BUF_OOB = 0xFFFFFF00u;
+constexpr uint32_t BUF_OOB = 0xFFFFF000u;  // room for the per-load immediate on top
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *p, uint32_t bytes) {
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p), 0, (int)bytes, 0x00020000);
@@ -171,7 +150,6 @@ __global__ __launch_bounds__((S == 1 ? CONV_WAVES : S) * 64) void conv_mfma_kern
   static_assert(S == 1 || NB == 1, "split tiles use one output block per wavefront");
   constexpr int WAVES = S == 1 ? CONV_WAVES : S;
   __shared__ int nbl[S == 1 ? WAVES : 1][TILE_M * K];
-  __shared__ __attribute__((aligned(16))) float atile[DIRECT_GATHER ? 1 : WAVES][DIRECT_GATHER ? 4 : TILE_M * AT_LD];
   __shared__ float red[S > 1 ? S - 1 : 1][S > 1 ? 16 * 64 : 1];
   const int64_t n = d_n_rows ? min((int64_t)*d_n_rows, n_rows) : n_rows;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -229,6 +207,7 @@ __global__ __launch_bounds__((S == 1 ? CONV_WAVES : S) * 64) void conv_mfma_kern
     rest = 0;
     for (int k = wave; k < K; k += S)
       if (__ballot(nl[r * K + k] >= 0) != 0ull) rest |= 1u << k;
+    rest = (unsigned)__builtin_amdgcn_readfirstlane((int)rest);
   }
 
   f16v acc[NB];
@@ -240,191 +219,111 @@ __global__ __launch_bounds__((S == 1 ? CONV_WAVES : S) * 64) void conv_mfma_kern
     for (int v = 0; v < 16; v++) acc[b][v] = bv;
   }
 
+  // per-channel scale / shift of the fused batch norm for this lane's columns (loaded here so
+  // that the latency is hidden behind the main loop)
+  float ew[NB], eb[NB];
+#pragma unroll
+  for (int b = 0; b < NB; b++) {
+    const int c = (cb0 + b) * 32 + r;
+    const bool on = ep.out2 && c < Cout && (S == 1 || wave == 0);
+    ew[b] = on ? ep.w[c] : 0.0f;
+    eb[b] = on ? ep.b[c] : 0.0f;
+  }
+
   if (rest) {
-    // Work items of this tile: (active offset k, 32-channel chunk ch), in order.
-    struct Item {
+    // Work items of this tile: (active offset k, 32-channel chunk ch), offsets ascending, chunks
+    // inside.  A cursor walks them with scalar selects only (no branches: a branchy iterator
+    // splits the loop body into many blocks and the load/MFMA overlap below is lost).  Past the
+    // last item it yields k = -1, and loads for such an item are sent out of range: they
+    // return zeros and move no data.
+    struct Cursor {
       int k, ch;
+      unsigned rest;
     };
-    // next item, or the same item again with `last` set when there is none
-    auto advance = [&](Item it, bool &last) -> Item {
-      last = false;
-      if (it.ch + 1 < nch) {
-        it.ch++;
-      } else if (rest) {
-        it.k = __builtin_ctz(rest);
-        rest &= rest - 1;
-        it.ch = 0;
-      } else {
-        last = true;
-      }
-      return it;
+    auto step = [&](const Cursor &c) -> Cursor {
+      const bool wrap = c.ch + 1 >= nch;
+      Cursor n;
+      n.ch = wrap ? 0 : c.ch + 1;
+      n.k = wrap ? (c.rest ? __builtin_ctz(c.rest) : -1) : c.k;
+      n.rest = wrap ? (c.rest & (c.rest - 1)) : c.rest;
+      return n;
     };
-    Item it0;
-    it0.k = __builtin_ctz(rest);
-    rest &= rest - 1;
-    it0.ch = 0;
-    // Pipeline: while item t runs on the matrix cores, the gathers of items t+1 and t+2 and the
-    // weight tile(s) of the next item(s) are in flight.  Register slots are compile-time (the
-    // loop bodies are unrolled) because copying a fragment would wait for the load that fills
-    // it.  Every load is issued unconditionally (past the last item the last item is simply
-    // fetched again): a load under a branch would force the wait before the MFMAs to drain all
-    // outstanding loads, which serialises the pipeline.  The sched_barrier / memory-clobber
-    // pairs keep the loads above the MFMAs they overlap and their consumers below.
-    bool last0, last1;
-    if constexpr (DIRECT_GATHER) {
-      const __amdgpu_buffer_rsrc_t rin = make_rsrc(in, in_bytes), rw = make_rsrc(Wp, wp_bytes);
-      const uint32_t ld4 = (uint32_t)ld_in * 4u, lane16 = (uint32_t)lane * 16u;
-      // lane (r, h) reads channels ch*32 + h*16 .. +15 of its own row; the second half-wave of
-      // a 16-channel tail chunk has no channels
-      auto gather = [&](const Item &it) -> Frag {
-        const int src = nl[r * K + it.k];
-        const bool on = src >= 0 && (h == 0 || Cin - it.ch * 32 >= 32);
-        const uint32_t voff = on ? (uint32_t)src * ld4 + (uint32_t)(it.ch * 128 + h * 64) : BUF_OOB;
-        Frag f;
+    const int nitems = __builtin_popcount(rest) * nch;
+    Cursor first;
+    first.k = __builtin_ctz(rest);
+    first.ch = 0;
+    first.rest = rest & (rest - 1);
+
+    const __amdgpu_buffer_rsrc_t rin = make_rsrc(in, in_bytes), rw = make_rsrc(Wp, wp_bytes);
+    const uint32_t ld4 = (uint32_t)ld_in * 4u, lane16 = (uint32_t)lane * 16u;
+    // lane (r, h) reads channels ch*32 + h*16 .. +15 of its own row; the second half-wave of a
+    // 16-channel tail chunk has no channels
+    auto gather = [&](const Cursor &c) -> Frag {
+      const int src = nl[r * K + (c.k < 0 ? 0 : c.k)];
+      const bool on = c.k >= 0 && src >= 0 && (h == 0 || Cin - c.ch * 32 >= 32);
+      const uint32_t voff = on ? (uint32_t)src * ld4 + (uint32_t)(c.ch * 128 + h * 64) : BUF_OOB;
+      Frag f;
 #pragma unroll
-        for (int q = 0; q < 4; q++) f.q[q] = buf_load16(rin, voff + 16u * q, 0);
-        return f;
-      };
-      auto wload = [&](const Item &it, int b) -> Frag {
-        const uint32_t soff = (uint32_t)((((it.k * nch + it.ch) * nbtp) + cb0 + b) * 4096);
-        Frag f;
+      for (int q = 0; q < 4; q++) f.q[q] = buf_load16(rin, voff + 16u * q, 0);
+      return f;
+    };
+    auto wload = [&](const Cursor &c, int b) -> Frag {
+      const int tile = ((c.k < 0 ? 0 : c.k) * nch + c.ch) * nbtp + cb0 + b;
+      const uint32_t soff = (uint32_t)__builtin_amdgcn_readfirstlane(tile * 4096);
+      const uint32_t voff = c.k >= 0 ? lane16 : BUF_OOB;
+      Frag f;
 #pragma unroll
-        for (int q = 0; q < 4; q++) f.q[q] = buf_load16(rw, lane16 + 1024u * q, soff);
-        return f;
-      };
-      Frag g[3];
-      g[0] = gather(it0);
-      Item it1 = advance(it0, last0);  // last0: it0 is the final item
-      g[1] = gather(it1);
-      if constexpr (S == 1) {
-        Frag bw[2];
-        bw[0] = wload(it0, 0);
-        bool done = false;
-        while (!done) {
+      for (int q = 0; q < 4; q++) f.q[q] = buf_load16(rw, voff + 1024u * q, soff);
+      return f;
+    };
+
+    // Pipeline: while item t runs on the matrix cores, the gathers of items t+1 .. t+D-1 are in
+    // flight; so are their weight tiles when a wavefront owns a single output block (otherwise
+    // the weight tiles of the (item, block) sequence are fetched one step ahead).  Register
+    // slots are compile-time (the body is unrolled over a full turn of the rings) because
+    // copying a fragment would wait for the load that fills it.  Every load is issued
+    // unconditionally: a load under a branch would force the wait before the MFMAs to drain
+    // all outstanding loads.  The sched_barrier / memory-clobber pairs keep the loads above the
+    // MFMAs they overlap and their consumers below.
+    constexpr int D = S == 1 ? INSC_CONV_DEPTH : INSC_CONV_DEPTH_SPLIT;
+    constexpr bool WRING = NB == 1;                         // weight tiles ride in the same ring
+    constexpr int TURN = (WRING || NB % 2 == 0) ? D : (D % 2 == 0 ? D : 2 * D);
+    Frag g[D], bw[WRING ? D : 2];
+    Cursor ci = first;  // next item to issue
 #pragma unroll
-          for (int u = 0; u < 6; u++) {
-            // item t = g[u%3] (arrived or arriving), t+1 = g[(u+1)%3] in flight, slot (u+2)%3 free
-            const Item it2 = advance(it1, last1);
-            g[(u + 2) % 3] = gather(it2);
+    for (int d = 0; d < D - 1; d++) {
+      g[d] = gather(ci);
+      if constexpr (WRING) bw[d] = wload(ci, 0);
+      ci = step(ci);
+    }
+    Cursor c0 = first, c1 = step(first);  // item on the matrix cores and its successor
+    if constexpr (!WRING) bw[0] = wload(c0, 0);
+    // One loop turn = TURN items; the last turn may run past the last item: those steps issue
+    // out-of-range loads and skip their MFMAs (a uniform branch around the MFMAs only).
+    for (int t0i = 0; t0i < nitems; t0i += TURN) {
 #pragma unroll
-            for (int b = 0; b < NB; b++) {
-              const int nn = u * NB + b;
-              bw[(nn + 1) % 2] = (b + 1 < NB) ? wload(it0, b + 1) : wload(it1, 0);
-              asm volatile("" ::: "memory");
-              __builtin_amdgcn_sched_barrier(0);
+      for (int u = 0; u < TURN; u++) {
+        g[(u + D - 1) % D] = gather(ci);
+        if constexpr (WRING) bw[(u + D - 1) % D] = wload(ci, 0);
+        ci = step(ci);
+        const bool real = t0i + u < nitems;
 #pragma unroll
-              for (int s = 0; s < 16; s++)
-                acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(frag_at(g[u % 3], s), frag_at(bw[nn % 2], s), acc[b],
-                                                              0, 0, 0);
-            }
-            asm volatile("" ::: "memory");
-            __builtin_amdgcn_sched_barrier(0);
-            if (last0) {
-              done = true;
-              break;
-            }
-            it0 = it1;
-            it1 = it2;
-            last0 = last1;
-          }
-        }
-      } else {
-        // few wavefronts per SIMD: the weight tiles are fetched two items ahead as well
-        Frag bw[3];
-        bw[0] = wload(it0, 0);
-        bw[1] = wload(it1, 0);
-        bool done = false;
-        while (!done) {
-#pragma unroll
-          for (int u = 0; u < 3; u++) {
-            const Item it2 = advance(it1, last1);
-            g[(u + 2) % 3] = gather(it2);
-            bw[(u + 2) % 3] = wload(it2, 0);
-            asm volatile("" ::: "memory");
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int s = 0; s < 16; s++)
-              acc[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(frag_at(g[u % 3], s), frag_at(bw[u % 3], s), acc[0], 0,
-                                                            0, 0);
-            asm volatile("" ::: "memory");
-            __builtin_amdgcn_sched_barrier(0);
-            if (last0) {
-              done = true;
-              break;
-            }
-            it0 = it1;
-            it1 = it2;
-            last0 = last1;
-          }
-        }
-      }
-    } else {
-      const int64_t wtile = 1024;  // floats per (k, chunk, block) weight tile
-      // Gather of one item, coalesced: load i (0..3) of lane l reads 16 bytes of input row
-      // 8*i + l/8 at channel 4*(l%8), so eight lanes cover one 128-byte row segment and every
-      // quad of lanes reads 64 contiguous bytes.  Rows without a neighbour (and the upper half
-      // of a 16-channel tail chunk) read a row of zeros.
-      const int grow = lane >> 3, gcol = (lane & 7) * 4;
-      auto gather = [&](const Item &it) -> Frag {
-        Frag f;
-        const bool col_ok = it.ch * 32 + gcol < Cin;
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-          const int src = nl[(8 * i + grow) * K + it.k];
-          const float *p = (src >= 0 && col_ok) ? in + (int64_t)src * ld_in + it.ch * 32 + gcol : g_zero_row;
-          f.q[i] = *reinterpret_cast<const float4 *>(p);
-        }
-        return f;
-      };
-      // through LDS into the MFMA A layout: lane (r, h) gets channels h*16 .. h*16+15 of row r
-      float *at = atile[wave];
-      auto transpose = [&](const Frag &gg) -> Frag {
-#pragma unroll
-        for (int i = 0; i < 4; i++) *reinterpret_cast<float4 *>(at + (8 * i + grow) * AT_LD + gcol) = gg.q[i];
-        Frag a;
-#pragma unroll
-        for (int q = 0; q < 4; q++) a.q[q] = *reinterpret_cast<const float4 *>(at + r * AT_LD + h * 16 + 4 * q);
-        return a;
-      };
-      auto wtile_of = [&](const Item &it, int b) -> const float * {
-        return Wp + (((int64_t)it.k * nch + it.ch) * nbtp + cb0 + b) * wtile;
-      };
-      Frag g[2], bw[2];
-      g[0] = gather(it0);
-      bw[0] = load_wfrag(wtile_of(it0, 0), lane);
-      Item it1 = advance(it0, last0);
-      g[1] = gather(it1);
-      Frag a = transpose(g[0]);
-      bool done = false;
-      while (!done) {
-#pragma unroll
-        for (int u = 0; u < 2; u++) {
-          const Item it2 = advance(it1, last1);
-          g[u % 2] = gather(it2);
-#pragma unroll
-          for (int b = 0; b < NB; b++) {
-            const int nn = u * NB + b;
-            if (b + 1 < NB)
-              bw[(nn + 1) % 2] = load_wfrag(wtile_of(it0, b + 1), lane);
-            else
-              bw[(nn + 1) % 2] = load_wfrag(wtile_of(it1, 0), lane);
-            asm volatile("" ::: "memory");
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int s = 0; s < 16; s++)
-              acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(frag_at(a, s), frag_at(bw[nn % 2], s), acc[b], 0, 0, 0);
-          }
+        for (int b = 0; b < NB; b++) {
+          const int nn = u * NB + b;
+          if constexpr (!WRING) bw[(nn + 1) % 2] = (b + 1 < NB) ? wload(c0, b + 1) : wload(c1, 0);
           asm volatile("" ::: "memory");
           __builtin_amdgcn_sched_barrier(0);
-          if (last0) {
-            done = true;
-            break;
+          const Frag &bf = bw[WRING ? u % D : nn % 2];
+          if (real) {
+#pragma unroll
+            for (int s = 0; s < 16; s++)
+              acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(frag_at(g[u % D], s), frag_at(bf, s), acc[b], 0, 0, 0);
           }
-          a = transpose(g[(u + 1) % 2]);
-          it0 = it1;
-          it1 = it2;
-          last0 = last1;
         }
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+        c0 = c1;
+        c1 = step(c1);
       }
     }
   }
@@ -444,28 +343,23 @@ __global__ __launch_bounds__((S == 1 ? CONV_WAVES : S) * 64) void conv_mfma_kern
     }
   }
 
-  // fused batch norm + leaky ReLU: per-channel scale / shift of this lane's columns
-  float ew[NB], eb[NB];
+  // D layout of the 32x32 MFMA: lane holds column (lane & 31), rows 8*(v/4) + 4*(lane>>5) + (v&3).
+  // All row ids are fetched from their lanes first, then the stores go out back to back.
+  int rid[16];
 #pragma unroll
-  for (int b = 0; b < NB; b++) {
-    const int c = (cb0 + b) * 32 + r;
-    ew[b] = (ep.out2 && c < Cout) ? ep.w[c] : 0.0f;
-    eb[b] = (ep.out2 && c < Cout) ? ep.b[c] : 0.0f;
-  }
-  // D layout of the 32x32 MFMA: lane holds column (lane & 31), rows 8*(v/4) + 4*(lane>>5) + (v&3)
+  for (int v = 0; v < 16; v++) rid[v] = __shfl(my_row, 8 * (v >> 2) + 4 * h + (v & 3), 64);
 #pragma unroll
   for (int v = 0; v < 16; v++) {
-    const int i = 8 * (v >> 2) + 4 * h + (v & 3);
-    const int rid = __shfl(my_row, i, 64);
-    if (rid < 0) continue;
+    if (rid[v] < 0) continue;
     if (out) {
-      float *op = out + (int64_t)rid * ld_out + cb0 * 32 + r;
+      float *op = out + (int64_t)rid[v] * ld_out + cb0 * 32 + r;
 #pragma unroll
       for (int b = 0; b < NB; b++)
         if ((cb0 + b) * 32 + r < Cout) op[b * 32] = acc[b][v];
     }
     if (ep.out2) {
-      float *op2 = ep.out2 + (int64_t)rid * ep.ld2 + cb0 * 32 + r;
+      // fused batch norm + leaky ReLU
+      float *op2 = ep.out2 + (int64_t)rid[v] * ep.ld2 + cb0 * 32 + r;
 #pragma unroll
       for (int b = 0; b < NB; b++)
         if ((cb0 + b) * 32 + r < Cout) {
