@@ -36,6 +36,7 @@ int hip_fail(hipError_t e, const char *what, const char *file, int line);
 // API-level function that is running (none of which calls another arena-2 user).
 enum { WS_SCAN = 0, WS_SORT = 1, WS_API = 2 };
 int workspace(int which, hipStream_t stream, size_t bytes, void **out);
+int device_cus();
 
 // ---- device primitives (scan_sort.hip) -------------------------------------------------
 int scan_exclusive_i32(const int32_t *in, int32_t *out, int64_t n, int32_t *total, hipStream_t s);

@@ -8,6 +8,8 @@
 // fp32 in, fp32 accumulate).  Accumulators stay in registers for all offsets, so every
 // output row is written exactly once and no atomics are needed: the result of a row does
 // not depend on which other rows share its tile, nor on the launch shape.
+#include <algorithm>
+
 #include "common.h"
 
 namespace insc {
@@ -134,8 +136,8 @@ __device__ __forceinline__ float4 buf_load16(__amdgpu_buffer_rsrc_t r, uint32_t 
 }
 
 // S == 1: every wavefront of the block owns a tile and walks all of its filter offsets.
-// S  > 1: the S wavefronts of a block share ONE tile; wavefront w takes the offsets k with
-//         k % S == w and the partial sums are added in wavefront order at the end.  This is for
+// S  > 1: the S wavefronts of a block share ONE tile; the (offset, channel chunk) items are dealt
+//         out round robin and the partial sums are added in wavefront order at the end.  This is for
 //         the coarse scales of a U-Net, where a layer has a handful of tiles but hundreds of
 //         channels and a single wavefront would run tens of thousands of dependent MFMAs.  Which
 //         terms a wavefront sums depends on k only, so a row's result is a function of S alone
@@ -151,6 +153,7 @@ __global__ __launch_bounds__((S == 1 ? CONV_WAVES : S) * 64) void conv_mfma_kern
   constexpr int WAVES = S == 1 ? CONV_WAVES : S;
   __shared__ int nbl[S == 1 ? WAVES : 1][TILE_M * K];
   __shared__ float red[S > 1 ? S - 1 : 1][S > 1 ? 16 * 64 : 1];
+  __shared__ unsigned wmask[S];
   const int64_t n = d_n_rows ? min((int64_t)*d_n_rows, n_rows) : n_rows;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int r = lane & 31, h = lane >> 5;
@@ -193,21 +196,34 @@ __global__ __launch_bounds__((S == 1 ? CONV_WAVES : S) * 64) void conv_mfma_kern
       if (staged[i] >= 0) mymask |= 1u << (e % K);
     }
   }
-  if (S == 1) {
 #pragma unroll
-    for (int d = 32; d > 0; d >>= 1) mymask |= (unsigned)__shfl_xor((int)mymask, d, 64);
-  }
+  for (int d = 32; d > 0; d >>= 1) mymask |= (unsigned)__shfl_xor((int)mymask, d, 64);
+  if (S > 1 && lane == 0) wmask[wave] = mymask;
   __syncthreads();
   if (!live) return;  // the whole block (S > 1) or wavefront (S == 1) is idle; no barrier follows
-  unsigned rest;
+  // Offsets some row of the tile uses.  With S wavefronts per tile, the (offset k, chunk ch)
+  // items are dealt out by (k * nch + ch) % S: wavefront w takes, of offset k, the chunks
+  // ch0(k), ch0(k) + S, ... with ch0(k) = (w - k * nch) mod S.  The deal depends on k, ch and
+  // the layer shape only, so a row's sum is formed the same way whatever tile it sits in.
+  unsigned rest;  // offsets that hold at least one item of this wavefront
+  int nitems = 0;
   if (S == 1) {
     rest = (unsigned)__builtin_amdgcn_readfirstlane((int)mymask);
+    nitems = __builtin_popcount(rest) * nch;
   } else {
-    // offsets of this wavefront that some row of the tile uses
+    unsigned act = 0;
+#pragma unroll
+    for (int w = 0; w < S; w++) act |= wmask[w];
+    act = (unsigned)__builtin_amdgcn_readfirstlane((int)act);
     rest = 0;
-    for (int k = wave; k < K; k += S)
-      if (__ballot(nl[r * K + k] >= 0) != 0ull) rest |= 1u << k;
-    rest = (unsigned)__builtin_amdgcn_readfirstlane((int)rest);
+    for (unsigned m = act; m; m &= m - 1) {
+      const int k = __builtin_ctz(m);
+      const int c0 = (wave - k * nch) & (S - 1);
+      if (c0 < nch) {
+        rest |= 1u << k;
+        nitems += (nch - c0 + S - 1) / S;
+      }
+    }
   }
 
   f16v acc[NB];
@@ -240,18 +256,19 @@ __global__ __launch_bounds__((S == 1 ? CONV_WAVES : S) * 64) void conv_mfma_kern
       int k, ch;
       unsigned rest;
     };
+    auto ch0 = [&](int k) -> int { return S == 1 ? 0 : ((wave - k * nch) & (S - 1)); };
     auto step = [&](const Cursor &c) -> Cursor {
-      const bool wrap = c.ch + 1 >= nch;
+      const bool wrap = c.ch + S >= nch;
+      const int nk = c.rest ? __builtin_ctz(c.rest) : -1;
       Cursor n;
-      n.ch = wrap ? 0 : c.ch + 1;
-      n.k = wrap ? (c.rest ? __builtin_ctz(c.rest) : -1) : c.k;
+      n.ch = wrap ? ch0(nk) : c.ch + S;
+      n.k = wrap ? nk : c.k;
       n.rest = wrap ? (c.rest & (c.rest - 1)) : c.rest;
       return n;
     };
-    const int nitems = __builtin_popcount(rest) * nch;
     Cursor first;
     first.k = __builtin_ctz(rest);
-    first.ch = 0;
+    first.ch = ch0(first.k);
     first.rest = rest & (rest - 1);
 
     const __amdgpu_buffer_rsrc_t rin = make_rsrc(in, in_bytes), rw = make_rsrc(Wp, wp_bytes);
@@ -285,7 +302,7 @@ __global__ __launch_bounds__((S == 1 ? CONV_WAVES : S) * 64) void conv_mfma_kern
     // unconditionally: a load under a branch would force the wait before the MFMAs to drain
     // all outstanding loads.  The sched_barrier / memory-clobber pairs keep the loads above the
     // MFMAs they overlap and their consumers below.
-    constexpr int D = S == 1 ? INSC_CONV_DEPTH : INSC_CONV_DEPTH_SPLIT;
+    constexpr int D = (S == 1 || S >= 16) ? INSC_CONV_DEPTH : INSC_CONV_DEPTH_SPLIT;
     constexpr bool WRING = NB == 1;                         // weight tiles ride in the same ring
     constexpr int TURN = (WRING || NB % 2 == 0) ? D : (D % 2 == 0 ? D : 2 * D);
     Frag g[D], bw[WRING ? D : 2];
@@ -370,6 +387,209 @@ __global__ __launch_bounds__((S == 1 ? CONV_WAVES : S) * 64) void conv_mfma_kern
   }
 }
 
+// ---------------------------------------------------------------------------------------
+// Narrow 3^3 layers (Cin <= 32, Cout <= 32): the whole packed filter (27 tiles of 4 KB) stays in
+// LDS for the life of the block, so the only traffic between L2 and the CU is the gather itself
+// - with the weight tiles re-read per item that path carries twice the bytes and bounds the
+// kernel.  Blocks are persistent: block b owns every gridDim.x-th tile and its wavefronts draw
+// them one by one.
+// The sums are formed exactly as in conv_mfma_kernel<1, 27, MAP_NBR, 1> (offsets ascending,
+// same MFMA sequence), so both kernels give the same bits.
+// ---------------------------------------------------------------------------------------
+constexpr int WL_WAVES = 12;
+constexpr int WL_DEPTH = 4;
+
+__global__ __launch_bounds__(WL_WAVES * 64) void conv_wlds_kernel(
+    const float *__restrict__ in, int64_t ld_in, float *__restrict__ out, int64_t ld_out,
+    const float *__restrict__ Wp, const float *__restrict__ bias, const int32_t *__restrict__ map0,
+    const int32_t *__restrict__ rows, const int32_t *__restrict__ d_n_rows, int64_t n_rows, int Cin, int Cout,
+    const uint8_t *__restrict__ tile_flags, uint32_t in_bytes, uint32_t map_bytes, BnEpilogue ep) {
+  constexpr int K = 27;
+  constexpr int NSTAGE = (TILE_M * K + 63) / 64;
+  __shared__ __attribute__((aligned(16))) float wl[K * 1024];
+  __shared__ int nbl[WL_WAVES][TILE_M * K];
+  __shared__ int next_turn;
+  const int64_t n = d_n_rows ? min((int64_t)*d_n_rows, n_rows) : n_rows;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int r = lane & 31, h = lane >> 5;
+
+  // the filter: 27 KB-quarters x 4, copied as is (already in per-lane order)
+  {
+    const float4 *src = reinterpret_cast<const float4 *>(Wp);
+    float4 *dst = reinterpret_cast<float4 *>(wl);
+    for (int i = threadIdx.x; i < K * 256; i += WL_WAVES * 64) dst[i] = src[i];
+  }
+  if (threadIdx.x == 0) next_turn = 0;
+  __syncthreads();
+
+  const int64_t ntiles = (n + TILE_M - 1) / TILE_M;
+  int *nl = nbl[wave];
+  const __amdgpu_buffer_rsrc_t rin = make_rsrc(in, in_bytes), rmap = make_rsrc(map0, map_bytes);
+  // the outputs are addressed with 32-bit byte offsets as well; rows that do not exist get an
+  // out-of-range offset and the hardware drops the store
+  const __amdgpu_buffer_rsrc_t rout = make_rsrc(out, out ? BUF_OOB : 0u), rout2 = make_rsrc(ep.out2, ep.out2 ? BUF_OOB : 0u);
+  const uint32_t ld4 = (uint32_t)ld_in * 4u, ldo4 = (uint32_t)ld_out * 4u, ldo24 = (uint32_t)ep.ld2 * 4u;
+  const bool half_on = h == 0 || Cin >= 32;  // a 16-channel layer has nothing for the upper half-wave
+  const int col = r;
+  const float bv = (bias && col < Cout) ? bias[col] : 0.0f;
+  const float ew = (ep.out2 && col < Cout) ? ep.w[col] : 0.0f;
+  const float eb = (ep.out2 && col < Cout) ? ep.b[col] : 0.0f;
+
+  // Block b owns the tiles b, b + gridDim.x, ...; its wavefronts draw them from a counter in LDS
+  // (tile costs differ by 3x: a fixed deal per wavefront leaves the slowest one far behind).
+  // draw(): the next tile of this block that has work, or ntiles.
+  auto draw = [&]() -> int64_t {
+    for (;;) {
+      int v = 0;
+      if (lane == 0) v = atomicAdd(&next_turn, 1);
+      const int64_t t = (int64_t)__builtin_amdgcn_readfirstlane(v) * gridDim.x + blockIdx.x;
+      if (t >= ntiles) return ntiles;
+      if (!tile_flags || tile_flags[t]) return t;
+    }
+  };
+  auto load_row = [&](int64_t t) -> int {
+    const int64_t p = t * TILE_M + r;
+    return (t < ntiles && p < n) ? (rows ? rows[p] : (int)p) : -1;
+  };
+  // issue the loads of a tile's slice of the neighbour map; bit i of the result: element i of
+  // this lane exists (a load sent out of range returns 0, which would pass for a site)
+  auto stage_issue = [&](int my_row, int (&st)[NSTAGE]) -> unsigned {
+    int srow[NSTAGE];
+    unsigned valid = 0;
+#pragma unroll
+    for (int i = 0; i < NSTAGE; i++) srow[i] = __shfl(my_row, ((i * 64 + lane) / K) & (TILE_M - 1), 64);
+#pragma unroll
+    for (int i = 0; i < NSTAGE; i++) {
+      const int e = i * 64 + lane;
+      const int kk = e - (e / K) * K;
+      const bool ok = e < TILE_M * K && srow[i] >= 0;
+      if (ok) valid |= 1u << i;
+      st[i] = __builtin_amdgcn_raw_buffer_load_b32(rmap, (int)(ok ? (uint32_t)(srow[i] * K + kk) * 4u : BUF_OOB), 0, 0);
+    }
+    return valid;
+  };
+
+  // Software pipeline over tiles: while tile t is computed, the neighbour-map slice of the next
+  // tile and the row ids of the one after it are in flight.
+  int64_t t = draw();
+  int my_row = load_row(t);
+  int st[NSTAGE];
+  unsigned valid = stage_issue(my_row, st);
+  int64_t tn = t < ntiles ? draw() : ntiles;
+  int my_row_n = load_row(tn);
+
+  while (t < ntiles) {
+    // neighbour-map slice -> LDS (private to the wavefront), and the offsets the tile uses
+    unsigned mymask = 0;
+#pragma unroll
+    for (int i = 0; i < NSTAGE; i++) {
+      const int e = i * 64 + lane;
+      if (e < TILE_M * K) {
+        const bool have = ((valid >> i) & 1u) && st[i] >= 0;
+        nl[e] = have ? st[i] : -1;
+        if (have) mymask |= 1u << (e % K);
+      }
+    }
+#pragma unroll
+    for (int d = 32; d > 0; d >>= 1) mymask |= (unsigned)__shfl_xor((int)mymask, d, 64);
+    unsigned rest = (unsigned)__builtin_amdgcn_readfirstlane((int)mymask);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+    // next tile's loads
+    int stn[NSTAGE];
+    const unsigned valid_n = stage_issue(my_row_n, stn);
+    const int64_t tnn = tn < ntiles ? draw() : ntiles;
+    const int my_row_nn = load_row(tnn);
+
+    f16v acc;
+#pragma unroll
+    for (int v = 0; v < 16; v++) acc[v] = bv;
+
+    if (rest) {
+      const int nitems = __builtin_popcount(rest);
+      // cursor over the active offsets, branch-free; -1 past the end (loads go out of range)
+      auto next_k = [&]() -> int {
+        const int k = rest ? __builtin_ctz(rest) : -1;
+        rest &= rest - 1;
+        return k;
+      };
+      auto gather = [&](int k) -> Frag {
+        const int src = nl[r * K + (k < 0 ? 0 : k)];
+        const bool on = k >= 0 && src >= 0 && half_on;
+        const uint32_t voff = on ? (uint32_t)src * ld4 + (uint32_t)(h * 64) : BUF_OOB;
+        Frag f;
+#pragma unroll
+        for (int q = 0; q < 4; q++) f.q[q] = buf_load16(rin, voff + 16u * q, 0);
+        return f;
+      };
+      auto wread = [&](int k) -> Frag {
+        const float4 *p = reinterpret_cast<const float4 *>(wl + (k < 0 ? 0 : k) * 1024) + lane;
+        Frag f;
+#pragma unroll
+        for (int q = 0; q < 4; q++) f.q[q] = p[q * 64];
+        return f;
+      };
+      constexpr int D = WL_DEPTH;
+      Frag g[D];
+      int kq[D];  // offsets of the items in the ring
+#pragma unroll
+      for (int d = 0; d < D - 1; d++) {
+        kq[d] = next_k();
+        g[d] = gather(kq[d]);
+      }
+      for (int i0 = 0; i0 < nitems; i0 += D) {
+#pragma unroll
+        for (int u = 0; u < D; u++) {
+          kq[(u + D - 1) % D] = next_k();
+          g[(u + D - 1) % D] = gather(kq[(u + D - 1) % D]);
+          const Frag bf = wread(kq[u]);
+          asm volatile("" ::: "memory");
+          __builtin_amdgcn_sched_barrier(0);
+          if (i0 + u < nitems) {
+#pragma unroll
+            for (int s = 0; s < 16; s++)
+              acc = __builtin_amdgcn_mfma_f32_32x32x2f32(frag_at(g[u], s), frag_at(bf, s), acc, 0, 0, 0);
+          }
+          asm volatile("" ::: "memory");
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+    }
+
+    // D layout of the 32x32 MFMA: lane holds column (lane & 31), rows 8*(v/4) + 4*(lane>>5) + (v&3)
+    int rid[16];
+#pragma unroll
+    for (int v = 0; v < 16; v++) rid[v] = __shfl(my_row, 8 * (v >> 2) + 4 * h + (v & 3), 64);
+    const uint32_t col4 = (uint32_t)col * 4u;
+#pragma unroll
+    for (int v = 0; v < 16; v++) {
+      const bool ok = rid[v] >= 0 && col < Cout;
+      const float av = acc[v];  // (a bit cast applied to the vector element itself reads element 0)
+      if (out)
+        __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(av), rout,
+                                              (int)(ok ? __umul24((unsigned)rid[v], ldo4) + col4 : BUF_OOB), 0, 0);
+      if (ep.out2) {
+        // fused batch norm + leaky ReLU
+        const float y = fmaf(av, ew, eb);
+        __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(y * ((y > 0.0f) ? 1.0f : ep.leak)), rout2,
+                                              (int)(ok ? __umul24((unsigned)rid[v], ldo24) + col4 : BUF_OOB), 0, 0);
+      }
+    }
+    // the next tile overwrites this wavefront's LDS slice: all lanes must be done reading it
+    __builtin_amdgcn_wave_barrier();
+
+    t = tn;
+    my_row = my_row_n;
+    valid = valid_n;
+#pragma unroll
+    for (int i = 0; i < NSTAGE; i++) st[i] = stn[i];
+    tn = tnn;
+    my_row_n = my_row_nn;
+  }
+}
+
 __global__ void count_rules_kernel(const int32_t *__restrict__ map0, int K, const int32_t *__restrict__ rows,
                                    const int32_t *__restrict__ d_n_rows, int64_t n_rows,
                                    unsigned long long *__restrict__ total) {
@@ -426,18 +646,33 @@ int launch_conv(const float *in, int64_t ld_in, int64_t in_rows, float *out, int
       Wp = (const float *)ws;
     }
     const int64_t tiles = cdiv(n_rows, TILE_M);
+    const int64_t map_bytes64 = in_rows * 27 * 4;  // the neighbour map has a row per input site
+    // (row ids and row strides go through 24-bit multiplies; outputs have a row per input site)
+    const bool small_ids = in_rows < (1 << 24) && ld_out * 4 < (1 << 24) && ep.ld2 * 4 < (1 << 24) &&
+                           in_rows * ld_out * 4 < (int64_t)BUF_OOB && in_rows * ep.ld2 * 4 < (int64_t)BUF_OOB;
+    if (mode == MAP_NBR && K == 27 && Cin <= 32 && Cout <= 32 && map_bytes64 < (int64_t)BUF_OOB && small_ids) {
+      const uint32_t map_bytes = (uint32_t)map_bytes64;
+      // persistent blocks, a multiple of the XCD count, at most one per compute unit
+      const int64_t want = cdiv(tiles, WL_WAVES);
+      const unsigned nblk = (unsigned)std::min<int64_t>(device_cus(), want);
+      hipLaunchKernelGGL(conv_wlds_kernel, dim3(nblk), dim3(WL_WAVES * 64), 0, s, in, ld_in, out, ld_out, Wp, bias,
+                         map0, rows, d_n_rows, n_rows, Cin, Cout, tile_flags, in_bytes, map_bytes, ep);
+      INSC_LAUNCH_CHECK();
+      return INSC_OK;
+    }
     const int nbt = (Cout + 31) / 32;
     // Launch shape, a function of the layer shape only (so results never depend on the scene):
-    //  narrow layers (Cin < 96): each wavefront computes all output blocks of its tile (the
-    //    gathered rows are reused across them);
-    //  wide layers: one output block per wavefront (more wavefronts for the few tiles of a
-    //    coarse scale), and for 3^3 / 2^3 maps the offsets of a tile are split over S wavefronts.
-    const bool wide = Cin >= 96;
-    const int NB = wide ? 1 : conv_nb_per_group(Cout);
+    //  Cin < 64: each wavefront computes all output blocks of its tile (the gathered rows are
+    //    reused across them);
+    //  wider layers sit at the coarse scales of a U-Net, which have few tiles: one output block
+    //    per wavefront, and for 3^3 / 2^3 maps the items of a tile are dealt to S wavefronts
+    //    (S grows with Cin: 2, 4, 8 for 3^3).
+    const bool split = Cin >= 64 && mode == MAP_NBR && K > 1;
+    const int NB0 = split ? 1 : conv_nb_per_group(Cout);
     const int nbtp = conv_nbt_padded(Cout);
     int S = 1;
-    if (wide && mode == MAP_NBR && K == 27) S = Cin >= 160 ? 8 : 4;
-    if (wide && mode == MAP_NBR && K == 8) S = 4;
+    if (split) S = K == 27 ? (Cin >= 160 ? 8 : Cin >= 128 ? 4 : 2) : (Cin >= 96 ? 4 : 1);
+    const int NB = (S == 1 && Cin >= 96) ? 1 : NB0;
     const unsigned gx = (unsigned)(S == 1 ? cdiv(tiles, CONV_WAVES) : tiles);
     dim3 grid(gx, (unsigned)(NB == 1 ? nbt : nbtp / NB)), block((S == 1 ? CONV_WAVES : S) * 64);
     bool shape_ok = true;
@@ -457,12 +692,22 @@ int launch_conv(const float *in, int64_t ld_in, int64_t in_rows, float *out, int
     else                                                         \
       shape_ok = false;                                          \
     break;
-    if (S == 8) {
-      INSC_CONV_LAUNCH(1, 27, MAP_NBR, 8);
-    } else if (S == 4 && K == 27) {
-      INSC_CONV_LAUNCH(1, 27, MAP_NBR, 4);
-    } else if (S == 4) {
-      INSC_CONV_LAUNCH(1, 8, MAP_NBR, 4);
+    if (S > 1 && mode == MAP_NBR && K == 27) {
+      switch (S) {
+        case 2: INSC_CONV_LAUNCH(1, 27, MAP_NBR, 2); break;
+        case 4: INSC_CONV_LAUNCH(1, 27, MAP_NBR, 4); break;
+        case 8: INSC_CONV_LAUNCH(1, 27, MAP_NBR, 8); break;
+        default: shape_ok = false;
+      }
+    } else if (S > 1 && mode == MAP_NBR && K == 8) {
+      switch (S) {
+        case 2: INSC_CONV_LAUNCH(1, 8, MAP_NBR, 2); break;
+        case 4: INSC_CONV_LAUNCH(1, 8, MAP_NBR, 4); break;
+        case 8: INSC_CONV_LAUNCH(1, 8, MAP_NBR, 8); break;
+        default: shape_ok = false;
+      }
+    } else if (S > 1) {
+      shape_ok = false;
     } else {
       switch (NB) {
         INSC_CONV_CASE(1)

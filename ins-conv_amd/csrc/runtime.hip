@@ -56,6 +56,7 @@ static int arena_get(int which, hipStream_t stream, size_t bytes, void **out) {
 }
 int workspace(int which, hipStream_t stream, size_t bytes, void **out) { return arena_get(which, stream, bytes, out); }
 
+
 __global__ void fill_u8_kernel(uint8_t *p, int64_t n, uint8_t v) {
   int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   int64_t stride = (int64_t)gridDim.x * blockDim.x;
@@ -67,6 +68,21 @@ __global__ void fill_i32_kernel(int32_t *p, int64_t n, int32_t v) {
   for (; i < n; i += stride) p[i] = v;
 }
 
+}  // namespace insc
+
+namespace insc {
+// compute units of the current device (queried once per device)
+int device_cus() {
+  static int cus[64] = {0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (!cus[dev]) {
+    int v = 0;
+    if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0) v = 256;
+    cus[dev] = v;
+  }
+  return cus[dev];
+}
 }  // namespace insc
 
 using namespace insc;
