@@ -249,6 +249,12 @@ int insc_net_forward(insc_net *net, const int32_t *d_coords, int coord_cols, con
                      int increment, float *d_out, int out_all, int64_t *h_n_sites, void *stream);
 int insc_net_tensor_view(insc_net *net, int tensor, float **d_ptr, int64_t *ld, int64_t *rows, int *channels);
 int insc_net_counts(insc_net *net, int64_t *h_sites_per_level, int64_t *h_points);
+/* Phase timing (the reference brackets the same phases with easy_profiler blocks,
+ * Metadata/Metadata.cpp:442-509, CUDA/Convolution.cpp:152-218).  enable != 0: every frame
+ * records four stream events; h_ms4 then receives the GPU time in ms of the last frame's phases:
+ * [0] grids, rulebooks and input accumulation, [1] dirty-set propagation, [2] the layers,
+ * [3] output gather and count read-back. */
+int insc_net_profile(insc_net *net, int enable, float *h_ms4);
 
 /* ---------------------------------------------------------------------------------------
  * Device utilities exported for tests and callers.

@@ -93,6 +93,9 @@ struct insc_net {
   size_t mask_arena_bytes = 0;
   int32_t *h_counts = nullptr;  // pinned: per level count, error flags
   int out_tensor = -1;
+  bool profiling = false;
+  hipEvent_t ev[5] = {nullptr, nullptr, nullptr, nullptr, nullptr};
+  bool ev_valid = false;
 };
 
 namespace insc {
@@ -523,6 +526,8 @@ int insc_net_destroy(insc_net *net) {
   for (void *p : ps)
     if (p) (void)hipFree(p);
   if (net->h_counts) (void)hipHostFree(net->h_counts);
+  for (hipEvent_t e : net->ev)
+    if (e) (void)hipEventDestroy(e);
   delete net;
   return INSC_OK;
 }
@@ -802,6 +807,7 @@ int insc_net_forward(insc_net *net, const int32_t *d_coords, int coord_cols, con
     INSC_LAUNCH_CHECK();
   }
 
+  if (net->profiling) INSC_HIP(hipEventRecord(net->ev[0], s));
   int32_t *sop = net->site_of_point + net->n_points;
   if (P > 0) {
     // ---- input scale: insert, accumulate --------------------------------------------------
@@ -857,11 +863,14 @@ int insc_net_forward(insc_net *net, const int32_t *d_coords, int coord_cols, con
       return rc;
   }
   // ---- dirty sets, then the layers ---------------------------------------------------------
+  if (net->profiling) INSC_HIP(hipEventRecord(net->ev[1], s));
   if (inc)
     for (int i = 0; i < (int)net->dirty.size(); i++)
       if ((rc = run_dirty_node(net, i, s))) return rc;
+  if (net->profiling) INSC_HIP(hipEventRecord(net->ev[2], s));
   for (const Op &op : net->ops)
     if ((rc = run_op(net, op, inc, s))) return rc;
+  if (net->profiling) INSC_HIP(hipEventRecord(net->ev[3], s));
 
   // ---- output layer ------------------------------------------------------------------------
   const int64_t n_out_pts = out_all ? net->n_points + P : P;
@@ -874,7 +883,9 @@ int insc_net_forward(insc_net *net, const int32_t *d_coords, int coord_cols, con
   }
   net->n_points += P;
   net->have_state = true;
+  if (net->profiling) INSC_HIP(hipEventRecord(net->ev[4], s));
   if ((rc = sync_counts(net, s, "insc_net_forward"))) return rc;
+  net->ev_valid = net->profiling;
   if (h_n_sites) *h_n_sites = net->levels[0].n;
   return INSC_OK;
 }
@@ -891,6 +902,20 @@ int insc_net_tensor_view(insc_net *net, int tensor, float **d_ptr, int64_t *ld, 
   if (ld) *ld = tensor_ld(net, tensor);
   if (rows) *rows = net->levels[net->tensors[tensor].level].n;
   if (channels) *channels = net->tensors[tensor].C;
+  return INSC_OK;
+}
+
+int insc_net_profile(insc_net *net, int enable, float *h_ms4) {
+  INSC_REQUIRE(net, INSC_ERR_ARG, "insc_net_profile: null net");
+  if (h_ms4) {
+    INSC_REQUIRE(net->ev_valid, INSC_ERR_STATE, "insc_net_profile: no frame has been timed yet");
+    INSC_HIP(hipEventSynchronize(net->ev[4]));
+    for (int i = 0; i < 4; i++) INSC_HIP(hipEventElapsedTime(h_ms4 + i, net->ev[i], net->ev[i + 1]));
+  }
+  if (enable && !net->ev[0])
+    for (int i = 0; i < 5; i++) INSC_HIP(hipEventCreate(&net->ev[i]));
+  net->profiling = enable != 0;
+  if (!enable) net->ev_valid = false;
   return INSC_OK;
 }
 

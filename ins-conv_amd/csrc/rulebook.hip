@@ -37,7 +37,11 @@ __device__ __forceinline__ uint64_t spread3(uint64_t v) {  // 12 bits -> every t
   return v;
 }
 
-// sort key: batch (12 bits) | Morton code of the 16^3 block (36 bits) | hash of the neighbour pattern (16 bits)
+// sort key: batch (7 bits) | Morton code of the 64^3 block (30 bits) | neighbour pattern (27 bits).
+// Sites with the same pattern inside a block end up in the same tiles, so a tile skips the
+// offsets none of its rows has; larger blocks give purer tiles (the gather locality they cost
+// matters less than the matrix-core work they save).  The order is a heuristic only: batches
+// beyond 127 share groups, which is harmless.
 __global__ void order_key_kernel(const int32_t *__restrict__ coords, const int32_t *__restrict__ nbr, int64_t first,
                                  int64_t n, uint64_t *__restrict__ keys, int32_t *__restrict__ vals) {
   int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -46,11 +50,9 @@ __global__ void order_key_kernel(const int32_t *__restrict__ coords, const int32
   int4 c = reinterpret_cast<const int4 *>(coords)[i];
   uint32_t m = 0;
   for (int k = 0; k < 27; k++) m |= (nbr[i * 27 + k] >= 0 ? 1u : 0u) << k;
-  uint32_t h = m * 2654435761u;
-  h ^= h >> 15;
-  uint64_t mort = spread3((uint64_t)(c.x >> 4)) | (spread3((uint64_t)(c.y >> 4)) << 1) |
-                  (spread3((uint64_t)(c.z >> 4)) << 2);
-  keys[t] = ((uint64_t)(c.w & 4095) << 52) | (mort << 16) | (uint64_t)(h & 0xffff);
+  const uint64_t mort = spread3((uint64_t)(c.x >> 6)) | (spread3((uint64_t)(c.y >> 6)) << 1) |
+                        (spread3((uint64_t)(c.z >> 6)) << 2);
+  keys[t] = ((uint64_t)(c.w & 127) << 57) | ((mort & 0x3fffffffull) << 27) | (uint64_t)m;
   vals[t] = (int)i;
 }
 

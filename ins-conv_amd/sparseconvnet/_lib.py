@@ -59,6 +59,7 @@ _SIGS = {
     "insc_net_tensor_view": [vp, c_int, ctypes.POINTER(vp), ctypes.POINTER(c_i64), ctypes.POINTER(c_i64),
                              ctypes.POINTER(c_int)],
     "insc_net_counts": [vp, ctypes.POINTER(c_i64), ctypes.POINTER(c_i64)],
+    "insc_net_profile": [vp, c_int, ctypes.POINTER(ctypes.c_float)],
     "insc_scan_exclusive_i32": [vp, vp, c_i64, vp, vp],
     "insc_sort_pairs_u64": [vp, vp, c_i64, c_int, vp],
 }

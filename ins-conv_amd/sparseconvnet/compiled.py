@@ -140,6 +140,17 @@ class CompiledNet(object):
         lib.insc_net_forward(self.h, ptr(c), int(c.size(1)), ptr(f), I64(P), int(bool(increment)), ptr(out),
                              int(bool(all_points)), ctypes.byref(n), stream_ptr())
         self.n_sites = int(n.value)
+        self._timed = getattr(self, "_profiling", False)
+        return out
+
+    def profile(self, enable=True):
+        """Switch phase timing on/off; returns the last timed frame's phases in ms as a dict
+        (structure, dirty, layers, output), or None if no frame was timed yet."""
+        ms = (ctypes.c_float * 4)()
+        have = getattr(self, "_profiling", False)
+        lib.insc_net_profile(self.h, int(bool(enable)), ms if have and getattr(self, "_timed", False) else None)
+        out = dict(zip(("structure", "dirty", "layers", "output"), [float(v) for v in ms])) if have and getattr(self, "_timed", False) else None
+        self._profiling, self._timed = bool(enable), False
         return out
 
     def sites_per_level(self):
