@@ -34,9 +34,11 @@ int hip_fail(hipError_t e, const char *what, const char *file, int line);
 // ordered by its stream.
 // Arena 0 belongs to the scan primitive, arena 1 to the sort primitive, arena 2 to the
 // API-level function that is running (none of which calls another arena-2 user).
-enum { WS_SCAN = 0, WS_SORT = 1, WS_API = 2 };
+enum { WS_SCAN = 0, WS_SORT = 1, WS_API = 2, WS_CONV = 3 };
 int workspace(int which, hipStream_t stream, size_t bytes, void **out);
 int device_cus();
+// `count` int32 counters per (device, stream), zero at kernel start; users leave them at zero
+int zero_counters(hipStream_t stream, size_t count, int32_t **out);
 
 // ---- device primitives (scan_sort.hip) -------------------------------------------------
 int scan_exclusive_i32(const int32_t *in, int32_t *out, int64_t n, int32_t *total, hipStream_t s);

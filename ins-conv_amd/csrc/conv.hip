@@ -142,13 +142,17 @@ __device__ __forceinline__ float4 buf_load16(__amdgpu_buffer_rsrc_t r, uint32_t 
 //         channels and a single wavefront would run tens of thousands of dependent MFMAs.  Which
 //         terms a wavefront sums depends on k only, so a row's result is a function of S alone
 //         (S is a fixed property of the layer shape), never of the tile it happens to sit in.
+//         With gridDim.z = G > 1 the deal goes over S * G wavefronts in G blocks (different
+//         compute units): a coarse scale has so few tiles that the matrix cores of the few
+//         units holding them would bound the layer.
 template <int NB, int K, int MODE, int S>
 __global__ __launch_bounds__((S == 1 ? CONV_WAVES : S) * 64) void conv_mfma_kernel(
     const float *__restrict__ in, int64_t ld_in, float *__restrict__ out, int64_t ld_out,
     const float *__restrict__ Wp, const float *__restrict__ bias, const int32_t *__restrict__ map0,
     const int32_t *__restrict__ map1, const int32_t *__restrict__ rows,
     const int32_t *__restrict__ d_n_rows, int64_t n_rows, int Cin, int Cout, int nbtp,
-    const uint8_t *__restrict__ tile_flags, uint32_t in_bytes, uint32_t wp_bytes, BnEpilogue ep) {
+    const uint8_t *__restrict__ tile_flags, uint32_t in_bytes, uint32_t wp_bytes, BnEpilogue ep,
+    float *__restrict__ part, int32_t *__restrict__ pcount) {
   static_assert(S == 1 || NB == 1, "split tiles use one output block per wavefront");
   constexpr int WAVES = S == 1 ? CONV_WAVES : S;
   __shared__ int nbl[S == 1 ? WAVES : 1][TILE_M * K];
@@ -160,7 +164,11 @@ __global__ __launch_bounds__((S == 1 ? CONV_WAVES : S) * 64) void conv_mfma_kern
   const int64_t t0 = (S == 1 ? (int64_t)blockIdx.x * WAVES + wave : (int64_t)blockIdx.x) * TILE_M;
   const int cb0 = blockIdx.y * NB;  // first output-channel block of this column group
   const int nch = conv_nch(Cin);
+  // the items of a tile are dealt to S wavefronts in each of G = gridDim.z blocks
+  const int G = S == 1 ? 1 : (int)gridDim.z, ST = S * G, ws = wave * G + (S == 1 ? 0 : (int)blockIdx.z);
 
+  // blocks beyond the row count leave at once (launches are sized by an upper bound of it)
+  if ((S == 1 ? (int64_t)blockIdx.x * WAVES : (int64_t)blockIdx.x) * TILE_M >= n) return;
   // a tile is skipped when it lies beyond the row count or, with tile flags, is not marked
   const bool live = t0 < n && (!tile_flags || tile_flags[t0 >> 5]);
   int my_row = -1;
@@ -218,10 +226,10 @@ __global__ __launch_bounds__((S == 1 ? CONV_WAVES : S) * 64) void conv_mfma_kern
     rest = 0;
     for (unsigned m = act; m; m &= m - 1) {
       const int k = __builtin_ctz(m);
-      const int c0 = (wave - k * nch) & (S - 1);
+      const int c0 = (ws - k * nch) & (ST - 1);
       if (c0 < nch) {
         rest |= 1u << k;
-        nitems += (nch - c0 + S - 1) / S;
+        nitems += (nch - c0 + ST - 1) / ST;
       }
     }
   }
@@ -230,7 +238,7 @@ __global__ __launch_bounds__((S == 1 ? CONV_WAVES : S) * 64) void conv_mfma_kern
 #pragma unroll
   for (int b = 0; b < NB; b++) {
     const int c = (cb0 + b) * 32 + r;
-    const float bv = (bias && c < Cout && (S == 1 || wave == 0)) ? bias[c] : 0.0f;
+    const float bv = (bias && c < Cout && (S == 1 || ws == 0)) ? bias[c] : 0.0f;
 #pragma unroll
     for (int v = 0; v < 16; v++) acc[b][v] = bv;
   }
@@ -256,12 +264,12 @@ __global__ __launch_bounds__((S == 1 ? CONV_WAVES : S) * 64) void conv_mfma_kern
       int k, ch;
       unsigned rest;
     };
-    auto ch0 = [&](int k) -> int { return S == 1 ? 0 : ((wave - k * nch) & (S - 1)); };
+    auto ch0 = [&](int k) -> int { return S == 1 ? 0 : ((ws - k * nch) & (ST - 1)); };
     auto step = [&](const Cursor &c) -> Cursor {
-      const bool wrap = c.ch + S >= nch;
+      const bool wrap = c.ch + ST >= nch;
       const int nk = c.rest ? __builtin_ctz(c.rest) : -1;
       Cursor n;
-      n.ch = wrap ? ch0(nk) : c.ch + S;
+      n.ch = wrap ? ch0(nk) : c.ch + ST;
       n.k = wrap ? nk : c.k;
       n.rest = wrap ? (c.rest & (c.rest - 1)) : c.rest;
       return n;
@@ -357,6 +365,33 @@ __global__ __launch_bounds__((S == 1 ? CONV_WAVES : S) * 64) void conv_mfma_kern
     for (int w = 0; w < S - 1; w++) {
 #pragma unroll
       for (int v = 0; v < 16; v++) acc[0][v] += red[w][v * 64 + lane];
+    }
+    if (G > 1) {
+      // The G blocks of a (tile, output block) leave their sums in memory; the one that arrives
+      // last adds them in block order (so the result does not depend on the arrival order),
+      // writes the rows and puts the arrival counter back to zero.  Nobody waits for anybody.
+      const int unit = (int)(blockIdx.x * gridDim.y + blockIdx.y);
+      float *mine = part + ((int64_t)unit * G + blockIdx.z) * 1024;
+#pragma unroll
+      // (stores and loads of the sums go past the XCD-local L2 - device-scope atomics - so that no
+      // cache write-back or invalidation is needed: a full fence flushes the whole L2 and costs
+      // more than the layer)
+      for (int v = 0; v < 16; v++)
+        __hip_atomic_store(mine + v * 64 + lane, acc[0][v], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the stores have been acknowledged
+      int old = 0;
+      if (lane == 0) old = atomicAdd(pcount + unit, 1);
+      if (__builtin_amdgcn_readfirstlane(old) != G - 1) return;
+      const float *all = part + (int64_t)unit * G * 1024;
+#pragma unroll
+      for (int v = 0; v < 16; v++)
+        acc[0][v] = __hip_atomic_load(all + v * 64 + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      for (int gg = 1; gg < G; gg++) {
+#pragma unroll
+        for (int v = 0; v < 16; v++)
+          acc[0][v] += __hip_atomic_load(all + gg * 1024 + v * 64 + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+      if (lane == 0) pcount[unit] = 0;
     }
   }
 
@@ -673,12 +708,25 @@ int launch_conv(const float *in, int64_t ld_in, int64_t in_rows, float *out, int
     int S = 1;
     if (split) S = K == 27 ? (Cin >= 160 ? 8 : Cin >= 128 ? 4 : 2) : (Cin >= 96 ? 4 : 1);
     const int NB = (S == 1 && Cin >= 96) ? 1 : NB0;
+    const int G = (split && K == 27) ? (Cin >= 160 ? 4 : Cin >= 128 ? 2 : 1) : 1;
+    if (G > 1) S = 4;
     const unsigned gx = (unsigned)(S == 1 ? cdiv(tiles, CONV_WAVES) : tiles);
-    dim3 grid(gx, (unsigned)(NB == 1 ? nbt : nbtp / NB)), block((S == 1 ? CONV_WAVES : S) * 64);
+    dim3 grid(gx, (unsigned)(NB == 1 ? nbt : nbtp / NB), (unsigned)G), block((S == 1 ? CONV_WAVES : S) * 64);
+    float *part = nullptr;
+    int32_t *pcount = nullptr;
+    if (G > 1) {
+      const size_t units = (size_t)gx * grid.y;
+      void *ws;
+      int rc = workspace(WS_CONV, s, units * G * 1024 * sizeof(float), &ws);
+      if (rc) return rc;
+      part = (float *)ws;
+      if ((rc = zero_counters(s, units, &pcount))) return rc;
+    }
     bool shape_ok = true;
 #define INSC_CONV_LAUNCH(NBV, KV, MV, SV)                                                                       \
   hipLaunchKernelGGL((conv_mfma_kernel<NBV, KV, MV, SV>), grid, block, 0, s, in, ld_in, out, ld_out, Wp, bias,  \
-                     map0, map1, rows, d_n_rows, n_rows, Cin, Cout, nbtp, tile_flags, in_bytes, wp_bytes, ep)
+                     map0, map1, rows, d_n_rows, n_rows, Cin, Cout, nbtp, tile_flags, in_bytes, wp_bytes, ep, part,  \
+                     pcount)
 #define INSC_CONV_CASE(NBV)                                      \
   case NBV:                                                      \
     if (mode == MAP_NBR && K == 27)                              \

@@ -56,6 +56,34 @@ static int arena_get(int which, hipStream_t stream, size_t bytes, void **out) {
 }
 int workspace(int which, hipStream_t stream, size_t bytes, void **out) { return arena_get(which, stream, bytes, out); }
 
+// int32 counters per (device, stream) that are zero whenever a kernel starts: zeroed when the
+// block is created or grown, and every kernel that uses them puts them back to zero.
+struct Counters {
+  int32_t *p = nullptr;
+  size_t count = 0;
+};
+static std::map<std::pair<int, hipStream_t>, Counters> g_counters;
+int zero_counters(hipStream_t stream, size_t count, int32_t **out) {
+  int dev = 0;
+  INSC_HIP(hipGetDevice(&dev));
+  std::lock_guard<std::mutex> lk(g_ws_mu);
+  Counters &c = g_counters[std::make_pair(dev, stream)];
+  if (c.count < count) {
+    if (c.p) {
+      INSC_HIP(hipStreamSynchronize(stream));
+      INSC_HIP(hipFree(c.p));
+      c.p = nullptr;
+      c.count = 0;
+    }
+    size_t want = count < 16384 ? 16384 : count + count / 2;
+    INSC_HIP(hipMalloc((void **)&c.p, want * sizeof(int32_t)));
+    INSC_HIP(hipMemsetAsync(c.p, 0, want * sizeof(int32_t), stream));
+    c.count = want;
+  }
+  *out = c.p;
+  return INSC_OK;
+}
+
 
 __global__ void fill_u8_kernel(uint8_t *p, int64_t n, uint8_t v) {
   int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
