@@ -1,7 +1,7 @@
 // Network executor: runs a whole sparse U-Net style network, full or incremental, from one
 // host call.  It owns the per-scale hash grids, rulebooks, cached feature matrices and the
 // dirty-set bookkeeping, and enqueues every kernel of a frame back to back on one stream with
-// no host round trip inside an incremental frame.
+// one host round trip per incremental frame (the site counts, read back once the grids are updated).
 //
 // The reference keeps this state spread over Python module attributes (save_meta,
 // save_input_feats, save_output: sparseconvnet/submanifoldConvolution.py:53-54,
@@ -852,6 +852,12 @@ int insc_net_forward(insc_net *net, const int32_t *d_coords, int coord_cols, con
       }
       INSC_LAUNCH_CHECK();
     }
+  } else {
+    // An incremental frame learns the exact counts here as well: one short host round trip
+    // (tens of microseconds) buys launches sized to the real number of tiles.  With the bound
+    // "every new point is a new site at every scale" a coarse scale of 70 sites would be
+    // launched for thousands, and idle blocks cost more than the convolution itself.
+    if ((rc = sync_counts(net, s, "insc_net_forward"))) return rc;
   }
 
   // ---- input layer output ------------------------------------------------------------------
@@ -884,7 +890,7 @@ int insc_net_forward(insc_net *net, const int32_t *d_coords, int coord_cols, con
   net->n_points += P;
   net->have_state = true;
   if (net->profiling) INSC_HIP(hipEventRecord(net->ev[4], s));
-  if ((rc = sync_counts(net, s, "insc_net_forward"))) return rc;
+  INSC_HIP(hipStreamSynchronize(s));  // the counts are known already; the call returns when the frame is done
   net->ev_valid = net->profiling;
   if (h_n_sites) *h_n_sites = net->levels[0].n;
   return INSC_OK;
