@@ -49,7 +49,7 @@ enum { MAP_NBR = 0, MAP_IDENTITY = 1, MAP_PARENT = 2 };
 // tile_flags: one byte per 32-row tile of `rows` (matrix-core kernel); row_mask: one byte per
 // site (generic kernel and the streaming kernels).  Null = everything.
 // Optional fused inference batch norm + leaky ReLU behind a producing kernel:
-//   y = fmaf(x, w[c], b[c]); y *= (y > 0 ? 1 : leak)  ->  out2 (row stride ld2)
+//   y = fmaf(x, w[c], b[c]); y *= (y > 0 ? 1 : leak)  ->  out2 (row stride ld2), out2 nullable
 // w, b are the per-channel scale / shift (bn_scale_shift).  The producer still writes its raw
 // result x to its own output unless that pointer is null.
 struct BnEpilogue {
@@ -57,6 +57,10 @@ struct BnEpilogue {
   float leak = 0.0f;
   float *out2 = nullptr;
   int64_t ld2 = 0;
+  // optional residual: x = producer result + res[row][c] before anything is written (the
+  // element-wise sum of a residual block, folded into the convolution that ends the block)
+  const float *res = nullptr;
+  int64_t ldr = 0;
 };
 // w = gamma / sqrt(var + eps), b = beta - mean * w   (gamma / beta nullable)
 int bn_scale_shift(const float *mean, const float *var, const float *gamma, const float *beta, float eps, int C,

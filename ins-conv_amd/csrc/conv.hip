@@ -56,6 +56,7 @@ __global__ __launch_bounds__(256) void conv_generic_kernel(const float *__restri
       const float *w = W + (int64_t)k * Cin * Cout + co;
       for (int ci = 0; ci < Cin; ci++) acc = fmaf(x[ci], w[(int64_t)ci * Cout], acc);
     }
+    if (ep.res) acc += ep.res[(int64_t)row * ep.ldr + co];
     if (out) out[(int64_t)row * ld_out + co] = acc;
     if (ep.out2) {
       const float y = fmaf(acc, ep.w[co], ep.b[co]);
@@ -403,6 +404,12 @@ __global__ __launch_bounds__((S == 1 ? CONV_WAVES : S) * 64) void conv_mfma_kern
 #pragma unroll
   for (int v = 0; v < 16; v++) {
     if (rid[v] < 0) continue;
+    if (ep.res) {
+      const float *rp = ep.res + (int64_t)rid[v] * ep.ldr + cb0 * 32 + r;
+#pragma unroll
+      for (int b = 0; b < NB; b++)
+        if ((cb0 + b) * 32 + r < Cout) acc[b][v] += rp[b * 32];
+    }
     if (out) {
       float *op = out + (int64_t)rid[v] * ld_out + cb0 * 32 + r;
 #pragma unroll
@@ -601,7 +608,8 @@ __global__ __launch_bounds__(WL_WAVES * 64) void conv_wlds_kernel(
 #pragma unroll
     for (int v = 0; v < 16; v++) {
       const bool ok = rid[v] >= 0 && col < Cout;
-      const float av = acc[v];  // (a bit cast applied to the vector element itself reads element 0)
+      float av = acc[v];  // (a bit cast applied to the vector element itself reads element 0)
+      if (ep.res && ok) av += ep.res[(int64_t)rid[v] * ep.ldr + col];
       if (out)
         __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(av), rout,
                                               (int)(ok ? __umul24((unsigned)rid[v], ldo4) + col4 : BUF_OOB), 0, 0);

@@ -57,9 +57,10 @@ struct Op {
   int Cin = 0, Cout = 0;
   // batch norm folded into the kernel that produces its input
   float *bn_w = nullptr, *bn_b = nullptr;  // per-channel scale / shift of an OP_BN, owned
+  int fused_add = -1;                      // convolution side: index of the OP_ADD it also computes
   int fused_bn = -1;                       // producer side: index of the OP_BN it also computes
   bool write_raw = true;                   // producer side: its own output has other readers
-  bool fused = false;                      // OP_BN side: computed by its producer, no kernel of its own
+  bool fused = false;                      // OP_BN / OP_ADD side: computed by its producer, no kernel of its own
 };
 
 struct DirtyNode {
@@ -395,11 +396,19 @@ static int run_op(insc_net *net, const Op &op, bool incremental, hipStream_t s) 
   const DirtyNode *d = incremental ? &net->dirty[To.dirty] : nullptr;
   const int32_t *d_n = Lo.grid->d_n;
   const int64_t n_up = Lo.n_upper;
-  float *out = op.write_raw ? tensor_ptr(net, op.out) : nullptr;
-  const int64_t ld_out = tensor_ld(net, op.out);
+  // a convolution that also forms the sum of its residual block writes what the OP_ADD would
+  const Op *add = op.fused_add >= 0 ? &net->ops[op.fused_add] : nullptr;
+  const Op &tail = add ? *add : op;  // the op whose outputs this kernel writes
+  float *out = tail.write_raw ? tensor_ptr(net, tail.out) : nullptr;
+  const int64_t ld_out = tensor_ld(net, tail.out);
   BnEpilogue ep;
-  if (op.fused_bn >= 0) {
-    const Op &bn = net->ops[op.fused_bn];
+  if (add) {
+    const int other = add->in0 == op.out ? add->in1 : add->in0;
+    ep.res = tensor_ptr(net, other);
+    ep.ldr = tensor_ld(net, other);
+  }
+  if (tail.fused_bn >= 0) {
+    const Op &bn = net->ops[tail.fused_bn];
     ep.w = bn.bn_w;
     ep.b = bn.bn_b;
     ep.leak = bn.leak;
@@ -725,6 +734,42 @@ int insc_net_finalize(insc_net *net, int out_tensor, int64_t capacity_sites, voi
         Buffer &B = net->buffers[T.buf];
         if (T.col0 == 0 && B.ld == T.C) B.ld = 0;
         T.kept = false;
+      }
+    }
+  }
+  // Fold the element-wise sum that ends a residual block into the convolution that feeds it
+  // (the other operand must exist by then and both must be due on the same rows).
+  {
+    const int nt = (int)net->tensors.size();
+    std::vector<int> producer(nt, -1), readers(nt, 0);
+    for (int i = 0; i < (int)net->ops.size(); i++) {
+      const Op &op = net->ops[i];
+      if (op.kind != OP_JOIN) producer[op.out] = producer[op.out] == -1 ? i : -2;
+      readers[op.in0]++;
+      if (op.in1 >= 0) readers[op.in1]++;
+    }
+    readers[out_tensor]++;
+    for (int i = 0; i < (int)net->ops.size(); i++) {
+      Op &add = net->ops[i];
+      if (add.kind != OP_ADD || add.fused || add.in0 == add.in1) continue;
+      for (int side = 0; side < 2; side++) {
+        const int x = side ? add.in0 : add.in1, other = side ? add.in1 : add.in0;  // prefer in1 (the block body)
+        const int a = producer[x];
+        if (a < 0 || a > i || readers[x] != 1) continue;
+        Op &A = net->ops[a];
+        const bool conv = A.kind == OP_SSC || A.kind == OP_CONV || A.kind == OP_DECONV || A.kind == OP_NIN;
+        if (!conv || A.fused_bn >= 0 || A.fused_add >= 0) continue;
+        if (other != 0 && (producer[other] < 0 || producer[other] > a)) continue;  // not computed yet when A runs
+        if (!net->tensors[other].kept) continue;
+        if (net->tensors[x].dirty != net->tensors[add.out].dirty) continue;
+        if (add.out == x || add.out == other) continue;
+        A.fused_add = i;
+        add.fused = true;
+        Tensor &T = net->tensors[x];
+        Buffer &B = net->buffers[T.buf];
+        if (T.col0 == 0 && B.ld == T.C) B.ld = 0;
+        T.kept = false;
+        break;
       }
     }
   }
