@@ -47,6 +47,12 @@ int down2_new_sites(const insc_grid *fine, insc_grid *coarse, int64_t n_new_uppe
                     int32_t *d_offset, int32_t *d_child, hipStream_t s);
 // order[i] = pos[i] = i for the new sites (appended in id order)
 int order_append_new_sites(const insc_grid *g, int32_t *d_order, int32_t *d_pos, int64_t n_new_upper, hipStream_t s);
+// the same, with the new sites sorted among themselves by the key of insc_order_build (needs their
+// rows of the neighbour map) / grouped by their position inside the parent cell
+int order_append_new_sites_sorted(const insc_grid *g, const int32_t *d_nbr, int32_t *d_order, int32_t *d_pos,
+                                  int64_t n_new_upper, hipStream_t s);
+int order_append_new_sites_by_offset(const insc_grid *g, const int32_t *d_offset, const int32_t *d_pos_in_order,
+                                     int32_t *d_order, int32_t *d_pos, int64_t n_new_upper, hipStream_t s);
 // device pointer to the site count before the most recent insert
 static inline const int32_t *grid_n_prev_ptr(const insc_grid *g) { return g->d_n + 1; }
 

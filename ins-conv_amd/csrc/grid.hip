@@ -358,9 +358,105 @@ int down2_new_sites(const insc_grid *fine, insc_grid *coarse, int64_t n_new_uppe
   return INSC_OK;
 }
 
+// The sites of the last insert, appended to a processing order sorted among themselves (one
+// workgroup, bitonic sort in LDS): tiles made of sites in arrival order use every filter offset
+// and gather from all over the scene, which costs a convolution a quarter of its speed.
+//   MODE 0: key = Morton code of the 64^3 block | neighbour pattern (the key of insc_order_build)
+//   MODE 1: key = position inside the parent cell | position in the MODE 0 order (`aux`)
+// More new sites than SORT_NEW_MAX keep their arrival order (any order gives the same results).
+constexpr int SORT_NEW_MAX = 8192;
+__device__ __forceinline__ uint64_t spread3_10(uint64_t v) {  // 10 bits -> every third bit
+  v &= 0x3ff;
+  v = (v | (v << 16)) & 0x30000ffull;
+  v = (v | (v << 8)) & 0x300f00full;
+  v = (v | (v << 4)) & 0x30c30c3ull;
+  v = (v | (v << 2)) & 0x9249249ull;
+  return v;
+}
+template <int MODE>
+__global__ __launch_bounds__(1024) void order_append_sorted_kernel(const int32_t *__restrict__ d_n,
+                                                                   const int32_t *__restrict__ coords,
+                                                                   const int32_t *__restrict__ nbr,
+                                                                   const int32_t *__restrict__ offset,
+                                                                   const int32_t *__restrict__ aux,
+                                                                   int32_t *__restrict__ order,
+                                                                   int32_t *__restrict__ pos) {
+  // one 64-bit word per new site: sort key in the upper 51 bits, index of the site among the
+  // new ones in the lower 13
+  __shared__ uint64_t key[SORT_NEW_MAX];
+  const int first = d_n[1], n = d_n[0] - first;
+  const int tid = threadIdx.x;
+  if (n <= 0) return;
+  if (n > SORT_NEW_MAX) {
+    for (int i = tid; i < n; i += 1024) {
+      order[first + i] = first + i;
+      if (pos) pos[first + i] = first + i;
+    }
+    return;
+  }
+  int N = 2;
+  while (N < n) N <<= 1;
+  for (int i = tid; i < N; i += 1024) {
+    uint64_t k = ~0ull;
+    if (i < n) {
+      const int v = first + i;
+      if (MODE == 0) {
+        const int4 c = reinterpret_cast<const int4 *>(coords)[v];
+        uint32_t m = 0;
+        for (int j = 0; j < 27; j++) m |= (nbr[(int64_t)v * 27 + j] >= 0 ? 1u : 0u) << j;
+        // (8 bits of block coordinate per axis: blocks 16384 voxels apart share a group, harmless)
+        const uint64_t mort = spread3_10((uint64_t)((c.x >> 6) & 255)) | (spread3_10((uint64_t)((c.y >> 6) & 255)) << 1) |
+                              (spread3_10((uint64_t)((c.z >> 6) & 255)) << 2);
+        k = (mort << 27) | (uint64_t)m;
+      } else {
+        k = ((uint64_t)(offset[v] & 7) << 32) | (uint32_t)aux[v];
+      }
+      k = (k << 13) | (uint64_t)i;
+    }
+    key[i] = k;
+  }
+  __syncthreads();
+  for (int k = 2; k <= N; k <<= 1) {
+    for (int j = k >> 1; j > 0; j >>= 1) {
+      for (int p = tid; p < (N >> 1); p += 1024) {
+        const int i = ((p & ~(j - 1)) << 1) | (p & (j - 1)), x = i | j;
+        const uint64_t a = key[i], b = key[x];
+        if ((a > b) == ((i & k) == 0)) {
+          key[i] = b;
+          key[x] = a;
+        }
+      }
+      __syncthreads();
+    }
+  }
+  for (int i = tid; i < n; i += 1024) {
+    const int v = first + (int)(key[i] & 8191);
+    order[first + i] = v;
+    if (pos) pos[v] = first + i;
+  }
+}
+
 int order_append_new_sites(const insc_grid *g, int32_t *d_order, int32_t *d_pos, int64_t n_new_upper, hipStream_t s) {
   if (n_new_upper <= 0) return INSC_OK;
   hipLaunchKernelGGL(order_append_kernel, dim3(grid_for(n_new_upper, 256)), dim3(256), 0, s, g->d_n, d_order, d_pos);
+  INSC_LAUNCH_CHECK();
+  return INSC_OK;
+}
+
+int order_append_new_sites_sorted(const insc_grid *g, const int32_t *d_nbr, int32_t *d_order, int32_t *d_pos,
+                                  int64_t n_new_upper, hipStream_t s) {
+  if (n_new_upper <= 0) return INSC_OK;
+  hipLaunchKernelGGL(order_append_sorted_kernel<0>, dim3(1), dim3(1024), 0, s, g->d_n, g->coords, d_nbr, nullptr,
+                     nullptr, d_order, d_pos);
+  INSC_LAUNCH_CHECK();
+  return INSC_OK;
+}
+
+int order_append_new_sites_by_offset(const insc_grid *g, const int32_t *d_offset, const int32_t *d_pos_in_order,
+                                     int32_t *d_order, int32_t *d_pos, int64_t n_new_upper, hipStream_t s) {
+  if (n_new_upper <= 0) return INSC_OK;
+  hipLaunchKernelGGL(order_append_sorted_kernel<1>, dim3(1), dim3(1024), 0, s, g->d_n, nullptr, nullptr, d_offset,
+                     d_pos_in_order, d_order, d_pos);
   INSC_LAUNCH_CHECK();
   return INSC_OK;
 }

@@ -864,7 +864,9 @@ int insc_net_forward(insc_net *net, const int32_t *d_coords, int coord_cols, con
     Level &L0 = net->levels[0];
     if ((rc = grid_insert_nosync(L0.grid, c4, P, sop, s))) return rc;
     if ((rc = ssc3_new_sites(L0.grid, L0.nbr, P, s))) return rc;
-    if ((rc = order_append_new_sites(L0.grid, L0.order, L0.pos, P, s))) return rc;
+    if ((rc = inc ? order_append_new_sites_sorted(L0.grid, L0.nbr, L0.order, L0.pos, P, s)
+                  : order_append_new_sites(L0.grid, L0.order, L0.pos, P, s)))
+      return rc;
     DirtyNode &din = net->dirty[net->tensors[0].dirty];
     const unsigned nb = grid_for(P, 256);
     hipLaunchKernelGGL(chain_push_kernel, dim3(nb), dim3(256), 0, s, sop, P, net->chain_head, net->chain_next);
@@ -876,9 +878,13 @@ int insc_net_forward(insc_net *net, const int32_t *d_coords, int coord_cols, con
     for (int l = 0; l + 1 < L; l++) {
       Level &F = net->levels[l], &Cs = net->levels[l + 1];
       if ((rc = down2_new_sites(F.grid, Cs.grid, P, F.parent, F.offset, F.child, s))) return rc;
-      if ((rc = order_append_new_sites(F.grid, F.bo_order, F.bo_pos, P, s))) return rc;
+      if ((rc = inc ? order_append_new_sites_by_offset(F.grid, F.offset, F.pos, F.bo_order, F.bo_pos, P, s)
+                    : order_append_new_sites(F.grid, F.bo_order, F.bo_pos, P, s)))
+        return rc;
       if ((rc = ssc3_new_sites(Cs.grid, Cs.nbr, P, s))) return rc;
-      if ((rc = order_append_new_sites(Cs.grid, Cs.order, Cs.pos, P, s))) return rc;
+      if ((rc = inc ? order_append_new_sites_sorted(Cs.grid, Cs.nbr, Cs.order, Cs.pos, P, s)
+                    : order_append_new_sites(Cs.grid, Cs.order, Cs.pos, P, s)))
+        return rc;
     }
   }
   if (!inc) {
