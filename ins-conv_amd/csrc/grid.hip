@@ -134,6 +134,69 @@ __global__ void grid_bump_kernel(int32_t *d_n, const int32_t *total) {
   d_n[0] += *total;
 }
 
+// Passes 2-4 and the counter update in one workgroup, for inserts of up to FINISH_SMALL_MAX rows
+// (an incremental frame): thread t owns a contiguous run of rows, so the ids come out in row
+// order exactly as from the scan-based passes.
+constexpr int FINISH_SMALL_MAX = 16384;
+__global__ __launch_bounds__(1024) void grid_finish_small_kernel(Slot *table, const int32_t *__restrict__ coords4,
+                                                                 const int32_t *__restrict__ slot_of_point, int P,
+                                                                 int32_t *d_n, int32_t *__restrict__ site_coords,
+                                                                 int64_t capacity_sites, int32_t *d_err,
+                                                                 int32_t *__restrict__ site_of_point) {
+  __shared__ int wave_total[16];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int per = (P + 1023) / 1024, p0 = tid * per;
+  const int n_before = d_n[0];
+  unsigned win = 0;
+  int cnt = 0;
+  for (int j = 0; j < per; j++) {
+    const int p = p0 + j;
+    if (p < P) {
+      const int s = slot_of_point[p];
+      if (s >= 0 && table[s].val == VAL_PENDING + p) {
+        win |= 1u << j;
+        cnt++;
+      }
+    }
+  }
+  // exclusive scan of cnt over the workgroup
+  int incl = cnt;
+  for (int d = 1; d < 64; d <<= 1) {
+    const int v = __shfl_up(incl, d, 64);
+    if (lane >= d) incl += v;
+  }
+  if (lane == 63) wave_total[wave] = incl;
+  __syncthreads();
+  int base = n_before + incl - cnt, total = 0;
+  for (int w = 0; w < 16; w++) {
+    if (w < wave) base += wave_total[w];
+    total += wave_total[w];
+  }
+  for (int j = 0; j < per; j++) {
+    if (!((win >> j) & 1u)) continue;
+    const int p = p0 + j, id = base++;
+    if (id >= capacity_sites) {
+      atomicOr(d_err, 2);
+      continue;
+    }
+    table[slot_of_point[p]].val = id;
+    reinterpret_cast<int4 *>(site_coords)[id] = reinterpret_cast<const int4 *>(coords4)[p];
+  }
+  __threadfence_block();
+  __syncthreads();
+  for (int j = 0; j < per; j++) {
+    const int p = p0 + j;
+    if (p >= P) break;
+    const int s = slot_of_point[p];
+    const int v = (s >= 0) ? table[s].val : -1;
+    site_of_point[p] = (v >= 0 && v < VAL_PENDING) ? v : -1;
+  }
+  if (tid == 0) {
+    d_n[1] = n_before;
+    d_n[0] = n_before + total;
+  }
+}
+
 __global__ void grid_query_kernel(const Slot *__restrict__ table, int64_t mask, const int32_t *__restrict__ coords4,
                                   int64_t Q, int32_t *__restrict__ out) {
   int64_t q = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -305,6 +368,14 @@ static int grid_insert_launch(insc_grid *g, const int32_t *d_coords4, int64_t P,
   int32_t *total = g->flags + g->scratch_rows;  // spare int after the flags
   hipLaunchKernelGGL(grid_claim_kernel, dim3(nb), dim3(256), 0, s, g->table, mask, d_coords4, P, g->slot_of_point,
                      g->d_err);
+  if (P <= FINISH_SMALL_MAX) {
+    hipLaunchKernelGGL(grid_finish_small_kernel, dim3(1), dim3(1024), 0, s, g->table, d_coords4, g->slot_of_point,
+                       (int)P, g->d_n, g->coords, g->capacity_sites, g->d_err, d_site_of_point);
+    INSC_LAUNCH_CHECK();
+    g->n_upper += P;
+    g->n_exact = -1;
+    return INSC_OK;
+  }
   hipLaunchKernelGGL(grid_flag_kernel, dim3(nb), dim3(256), 0, s, g->table, g->slot_of_point, P, g->flags);
   INSC_LAUNCH_CHECK();
   rc = scan_exclusive_i32(g->flags, g->flags, P, total, s);
