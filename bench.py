@@ -125,6 +125,112 @@ def conv_roofline(device, reps=30):
 
 
 # ---------------------------------------------------------------------------------------------
+# the bandwidth-bound kernels of the path, one C call each, against the HBM roofline
+# ---------------------------------------------------------------------------------------------
+def kernel_table(device, reps=20):
+    """us per call, achieved GB/s on ALGORITHMIC bytes and fraction of the HBM peak for the hash
+    grid, the rulebooks, batch norm and the input/output layers, on the workload-2 scene (200k
+    voxels, 1024^3, plus 10 % repeated points) and, for the feature kernels, 500k x 32 floats."""
+    import ctypes
+
+    import numpy as np
+    import torch
+
+    import scenes
+    from sparseconvnet._lib import lib, ptr, stream_ptr
+
+    I64 = ctypes.c_int64
+    st = stream_ptr()
+    rng = np.random.default_rng(2)
+    vox = scenes.planes_boxes_scene(seed=2, n=200000).astype(np.int32)
+    pts = np.concatenate([vox, vox[rng.integers(0, len(vox), len(vox) // 10)]])
+    pts = pts[rng.permutation(len(pts))]
+    if pts.shape[1] == 3:
+        pts = np.concatenate([pts, np.zeros((len(pts), 1), np.int32)], 1)
+    P, N = len(pts), len(vox)
+    c4 = torch.from_numpy(np.ascontiguousarray(pts[:, :4])).to(device)
+    sop = torch.empty(P, dtype=torch.int32, device=device)
+    grid, coarse = ctypes.c_void_p(), ctypes.c_void_p()
+    lib.insc_grid_create(I64(2 * N), ctypes.byref(grid))
+    lib.insc_grid_create(I64(N), ctypes.byref(coarse))
+    n_sites = I64(0)
+    nbr = torch.empty((N, 27), dtype=torch.int32, device=device)
+    parent = torch.empty(N, dtype=torch.int32, device=device)
+    offset = torch.empty(N, dtype=torch.int32, device=device)
+    child = torch.empty((N, 8), dtype=torch.int32, device=device)
+    C, NF = 32, 500000
+    x = torch.randn(NF, C, device=device)
+    y = torch.empty_like(x)
+    mean, var = torch.zeros(C, device=device), torch.ones(C, device=device)
+    fp = torch.randn(P, C, device=device)
+    acc = torch.zeros(N, C, device=device)
+    cnt = torch.zeros(N, dtype=torch.int32, device=device)
+    outp = torch.empty(P, C, device=device)
+
+    def timed(fn, pre=None):
+        for _ in range(2):
+            if pre:
+                pre()
+            fn()
+        torch.cuda.synchronize()
+        total = 0.0
+        for _ in range(reps):
+            if pre:
+                pre()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            fn()
+            e1.record()
+            torch.cuda.synchronize()
+            total += e0.elapsed_time(e1)
+        return total * 1e-3 / reps
+
+    rows = []
+
+    def add(name, sec, nbytes, note):
+        gbs = nbytes / sec / 1e9
+        rows.append({"kernel": name, "us": round(sec * 1e6, 1), "algorithmic_bytes": int(nbytes),
+                     "GB/s": round(gbs, 1), "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4), "units": note})
+
+    t = timed(lambda: lib.insc_grid_insert(grid, ptr(c4), I64(P), ptr(sop), ctypes.byref(n_sites), st),
+              pre=lambda: lib.insc_grid_clear(grid, st))
+    add("hash grid insert (claim, scan, assign, resolve; incl. count read-back)", t, P * 32, "%d points -> %d sites" % (P, n_sites.value))
+    t = timed(lambda: lib.insc_grid_query(grid, ptr(c4), I64(P), ptr(sop), st))
+    add("hash grid query", t, P * 28, "%d queries" % P)
+    t = timed(lambda: lib.insc_rulebook_ssc3(grid, I64(0), I64(N), ptr(nbr), 0, st))
+    add("SSC 3^3 rulebook (dense neighbour map, 27 probes per site)", t, N * (16 + 27 * 8 + 27 * 4), "%d sites" % N)
+
+    def down():
+        lib.insc_rulebook_down2(grid, coarse, I64(0), I64(N), ptr(parent), ptr(offset), ptr(child), I64(N), st)
+
+    def down_pre():
+        lib.insc_grid_clear(coarse, st)
+        child.fill_(-1)
+
+    t = timed(down, pre=down_pre)
+    add("stride-2 rulebook (coarse grid insert + parent/offset/child maps)", t, N * 36, "%d fine sites" % N)
+    t = timed(lambda: lib.insc_bn_leaky(ptr(x), I64(C), ptr(y), I64(C), ptr(mean), ptr(var), None, None,
+                                         ctypes.c_float(1e-4), ctypes.c_float(0.0), None, None, I64(NF), C, st))
+    add("batch norm + ReLU (eval)", t, NF * C * 8, "%d x %d" % (NF, C))
+
+    def inp():
+        lib.insc_input_accumulate(ptr(fp), I64(P), C, ptr(sop), 4, ptr(acc), ptr(cnt), I64(N), st)
+        lib.insc_input_finish(ptr(acc), ptr(cnt), 4, ptr(y), I64(C), None, None, I64(N), C, st)
+
+    def inp_pre():
+        acc.zero_()
+        cnt.zero_()
+
+    t = timed(inp, pre=inp_pre)
+    add("input layer (mode 4: per-voxel mean)", t, P * (4 * C + 4) + N * 4 * C, "%d points x %d -> %d sites" % (P, C, N))
+    t = timed(lambda: lib.insc_output_gather(ptr(y), I64(C), ptr(sop), I64(P), C, ptr(outp), st))
+    add("output layer (row gather)", t, P * (4 * C + 4) + P * 4 * C, "%d points x %d" % (P, C))
+    lib.insc_grid_destroy(grid)
+    lib.insc_grid_destroy(coarse)
+    return rows
+
+
+# ---------------------------------------------------------------------------------------------
 # workloads 4 and 5: the U-Net of the reference's example, through the network executor
 # ---------------------------------------------------------------------------------------------
 def unet_model(device):
@@ -206,6 +312,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=None)
     ap.add_argument("--workload", default="incr", choices=["incr", "unet", "ssc"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--kernels-only", action="store_true",
+                    help="print only the table of bandwidth-bound kernels")
     ap.add_argument("--roofline-only", action="store_true",
                     help="run only the dominant-kernel measurement (short; used under rocprofv3)")
     args = ap.parse_args()
@@ -220,6 +328,9 @@ def main():
     device = torch.device("cuda", 0)
     torch.cuda.set_device(device)
 
+    if args.kernels_only:
+        print(json.dumps({"kernels": kernel_table(device)}))
+        return
     if args.roofline_only:
         # plus a plain copy of known size (500k x 32 floats: 64 MB read, 64 MB written), the
         # yardstick the FETCH_SIZE / WRITE_SIZE counters of the same run are scaled by
@@ -318,6 +429,7 @@ def main():
     }
     out.update(extra)
     out["roofline"] = conv_roofline(device)
+    out["kernels"] = kernel_table(device)
     if cpu is not None:
         out["cpu_baseline"] = cpu
     print(json.dumps(out))

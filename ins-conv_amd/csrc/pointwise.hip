@@ -142,52 +142,61 @@ __global__ __launch_bounds__(256) void gather_rows_kernel(const float *__restric
 }
 
 // ---- input layer -----------------------------------------------------------------------
-__global__ void input_key_kernel(const int32_t *__restrict__ site_of_point, int64_t P, uint64_t *__restrict__ keys,
-                                 int32_t *__restrict__ vals) {
+// Input layer.  The rows of one site are chained: every row pushes itself on its site's list
+// (an atomic exchange on the list head), and the row left at the head owns the site.  The owner
+// visits the rows of the list in ascending row order - the order InputLayer_fp_ adds them in
+// (CUDA/IOLayers.cu:17-32), so the float sum has the reference's rounding - and the lists are
+// short (rows of one voxel in one call).
+__global__ void input_push_kernel(const int32_t *__restrict__ sop, int64_t P, int32_t *__restrict__ head,
+                                  int32_t *__restrict__ next) {
   int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (p >= P) return;
-  keys[p] = (uint64_t)(uint32_t)site_of_point[p];  // -1 sorts last
-  vals[p] = (int)p;
+  const int s = sop[p];
+  next[p] = (s >= 0) ? atomicExch(&head[s], (int)p) : -1;
 }
 
-// keys/vals sorted by site (stable: rows of one site ascending).  One thread per (sorted
-// position, channel); the thread at the head of a site's run sums the run in order.
-__global__ __launch_bounds__(256) void input_sum_kernel(const float *__restrict__ feats, int C,
-                                                        const uint64_t *__restrict__ keys,
-                                                        const int32_t *__restrict__ vals, int64_t P, int mode,
-                                                        float *__restrict__ sum, const int32_t *__restrict__ cnt) {
+// one thread per (row, channel); only the threads of a list's head row work
+__global__ __launch_bounds__(256) void input_reduce_kernel(const float *__restrict__ feats, int C,
+                                                           const int32_t *__restrict__ sop, int64_t P,
+                                                           const int32_t *__restrict__ head,
+                                                           const int32_t *__restrict__ next, int mode,
+                                                           float *__restrict__ sum, const int32_t *__restrict__ cnt) {
   for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < P * C; e += (int64_t)gridDim.x * 256) {
-    const int64_t j = e / C;
-    const int c = (int)(e - j * C);
-    const uint64_t key = keys[j];
-    if (key == 0xFFFFFFFFull) continue;
-    if (j > 0 && keys[j - 1] == key) continue;  // not a head
-    const int64_t site = (int64_t)key;
-    float acc = sum[site * C + c];
-    const bool had = cnt[site] > 0;
-    if (mode == 1) {
-      if (!had) acc = feats[(int64_t)vals[j] * C + c];
-    } else if (mode == 2) {
-      int64_t q = j;
-      while (q + 1 < P && keys[q + 1] == key) q++;
-      acc = feats[(int64_t)vals[q] * C + c];
+    const int64_t p = e / C;
+    const int c = (int)(e - p * C);
+    const int s = sop[p];
+    if (s < 0 || head[s] != (int)p) continue;
+    float acc = sum[(int64_t)s * C + c];
+    if (mode == 1 || mode == 2) {  // keep the first / the last row of the site
+      int pick = (int)p;
+      for (int q = (int)p; q >= 0; q = next[q]) pick = mode == 1 ? min(pick, q) : max(pick, q);
+      if (mode == 2 || cnt[s] == 0) acc = feats[(int64_t)pick * C + c];
     } else {
-      for (int64_t q = j; q < P && keys[q] == key; q++) acc += feats[(int64_t)vals[q] * C + c];
+      int done = -1;
+      for (;;) {
+        int best = 0x7fffffff;
+        for (int q = (int)p; q >= 0; q = next[q])
+          if (q > done && q < best) best = q;
+        if (best == 0x7fffffff) break;
+        acc += feats[(int64_t)best * C + c];
+        done = best;
+      }
     }
-    sum[site * C + c] = acc;
+    sum[(int64_t)s * C + c] = acc;
   }
 }
 
-__global__ __launch_bounds__(256) void input_count_kernel(const uint64_t *__restrict__ keys, int64_t P,
-                                                          int32_t *__restrict__ cnt) {
-  int64_t j = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (j >= P) return;
-  const uint64_t key = keys[j];
-  if (key == 0xFFFFFFFFull) return;
-  if (j > 0 && keys[j - 1] == key) return;
-  int64_t q = j;
-  while (q + 1 < P && keys[q + 1] == key) q++;
-  cnt[(int64_t)key] += (int)(q - j + 1);
+// counts the rows of every list and empties it
+__global__ void input_count_kernel(const int32_t *__restrict__ sop, int64_t P, int32_t *__restrict__ head,
+                                   const int32_t *__restrict__ next, int32_t *__restrict__ cnt) {
+  int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (p >= P) return;
+  const int s = sop[p];
+  if (s < 0 || head[s] != (int)p) return;
+  int n = 0;
+  for (int q = (int)p; q >= 0; q = next[q]) n++;
+  cnt[s] += n;
+  head[s] = -1;
 }
 
 __global__ __launch_bounds__(256) void input_finish_kernel(const float *__restrict__ sum,
@@ -319,17 +328,15 @@ int insc_input_accumulate(const float *d_feats, int64_t P, int C, const int32_t 
   if (P == 0) return INSC_OK;
   hipStream_t s = (hipStream_t)stream;
   void *ws;
-  int rc = workspace(WS_API, s, (sizeof(uint64_t) + sizeof(int32_t)) * (size_t)P + 256, &ws);
+  int rc = workspace(WS_API, s, sizeof(int32_t) * (size_t)(P + n_sites_upper) + 256, &ws);
   if (rc) return rc;
-  uint64_t *keys = (uint64_t *)ws;
-  int32_t *vals = (int32_t *)(keys + P);
-  hipLaunchKernelGGL(input_key_kernel, dim3(grid_for(P, 256)), dim3(256), 0, s, d_site_of_point, P, keys, vals);
-  INSC_LAUNCH_CHECK();
-  rc = sort_pairs_u64(keys, vals, P, 32, s);  // invalid rows carry 0xFFFFFFFF and must sort last
-  if (rc) return rc;
-  hipLaunchKernelGGL(input_sum_kernel, dim3(grid_for(P * C, 256, 1 << 16)), dim3(256), 0, s, d_feats, C, keys, vals,
-                     P, mode, d_sum, d_cnt);
-  hipLaunchKernelGGL(input_count_kernel, dim3(grid_for(P, 256)), dim3(256), 0, s, keys, P, d_cnt);
+  int32_t *next = (int32_t *)ws, *head = next + P;
+  if (n_sites_upper > 0 && (rc = insc_fill_i32(head, n_sites_upper, -1, stream))) return rc;
+  const unsigned nb = grid_for(P, 256);
+  hipLaunchKernelGGL(input_push_kernel, dim3(nb), dim3(256), 0, s, d_site_of_point, P, head, next);
+  hipLaunchKernelGGL(input_reduce_kernel, dim3(grid_for(P * C, 256, 1 << 16)), dim3(256), 0, s, d_feats, C,
+                     d_site_of_point, P, head, next, mode, d_sum, d_cnt);
+  hipLaunchKernelGGL(input_count_kernel, dim3(nb), dim3(256), 0, s, d_site_of_point, P, head, next, d_cnt);
   INSC_LAUNCH_CHECK();
   return INSC_OK;
 }
