@@ -105,7 +105,7 @@ int insc_rulebook_pairs(const int32_t *d_nbr, int64_t N, int K, int32_t *d_count
 int insc_rulebook_down2(const insc_grid *fine, insc_grid *coarse, int64_t first, int64_t n, int32_t *d_parent,
                         int32_t *d_offset, int32_t *d_child, int64_t child_rows, void *stream);
 /* A processing order for the sites first..first+n-1, written to d_order[first..first+n): a
- * permutation of those ids that puts sites of one 16^3 block with the same neighbour pattern
+ * permutation of those ids that puts sites of one 64^3 block with the same neighbour pattern
  * next to each other, so that row tiles of the convolution kernel skip whole filter offsets.
  * Results of the convolution do not depend on it.  No counterpart in the reference (its chunk
  * builder, SubmanifoldRules_cuda.cpp:572-1112, serves the same purpose for its
