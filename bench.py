@@ -96,13 +96,14 @@ def conv_roofline(device, reps=30):
     sc = m.ssc_rulebook(x.spatial_size)
     out = torch.empty((sc.n, conv.nOut), device=device)
     w = conv.weight
+    plan = m.ssc_plan(sc)  # built once per rulebook, like the neighbour map and the order
     for _ in range(3):
-        SCN.conv_rows(x.features, out, w, None, sc.nbr.t, 27, sc.order.t, None, sc.n)
+        SCN.ssc_rows_planned(x.features, out, w, None, sc, plan)
     torch.cuda.synchronize()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     e0.record()
     for _ in range(reps):
-        SCN.conv_rows(x.features, out, w, None, sc.nbr.t, 27, sc.order.t, None, sc.n)
+        SCN.ssc_rows_planned(x.features, out, w, None, sc, plan)
     e1.record()
     torch.cuda.synchronize()
     t = e0.elapsed_time(e1) * 1e-3 / reps

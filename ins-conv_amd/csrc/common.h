@@ -66,11 +66,24 @@ struct BnEpilogue {
 int bn_scale_shift(const float *mean, const float *var, const float *gamma, const float *beta, float eps, int C,
                    float *w, float *b, hipStream_t s);
 
+// Tile plan of a 3^3 map for one processing order: map[k * ld + p] = neighbour k of the site at
+// position p of the order (-1: none; positions up to the end of the last 32-row tile are
+// filled), tmask[t] = offsets some row of tile t has.  Optional: kernels fall back to the
+// site-indexed map.
+struct TilePlan {
+  const int32_t *map = nullptr;
+  int64_t ld = 0;
+  const uint32_t *tmask = nullptr;
+};
+int build_tile_plan(const int32_t *nbr, const int32_t *order, const int32_t *d_n, int64_t n_rows, int64_t ld,
+                    int32_t *map, uint32_t *tmask, hipStream_t s);
+
 // in_rows: rows of the input matrix (bounds the gather).  out may be null when ep.out2 is set.
 int launch_conv(const float *in, int64_t ld_in, int64_t in_rows, float *out, int64_t ld_out, const float *W,
                 const float *Wp, const float *bias, const int32_t *map0, const int32_t *map1, int mode, int K,
                 const int32_t *rows, const int32_t *d_n_rows, int64_t n_rows, int Cin, int Cout,
-                const uint8_t *tile_flags, const uint8_t *row_mask, hipStream_t s, BnEpilogue ep = BnEpilogue());
+                const uint8_t *tile_flags, const uint8_t *row_mask, hipStream_t s, BnEpilogue ep = BnEpilogue(),
+                TilePlan plan = TilePlan());
 int64_t packed_floats(int K, int Cin, int Cout);
 int pack_weights(const float *W, int K, int Cin, int Cout, float *Wp, hipStream_t s);
 int launch_bn(const float *in, int64_t ld_in, float *out, int64_t ld_out, const float *mean, const float *var,

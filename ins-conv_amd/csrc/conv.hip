@@ -153,7 +153,7 @@ __global__ __launch_bounds__((S == 1 ? CONV_WAVES : S) * 64) void conv_mfma_kern
     const int32_t *__restrict__ map1, const int32_t *__restrict__ rows,
     const int32_t *__restrict__ d_n_rows, int64_t n_rows, int Cin, int Cout, int nbtp,
     const uint8_t *__restrict__ tile_flags, uint32_t in_bytes, uint32_t wp_bytes, BnEpilogue ep,
-    float *__restrict__ part, int32_t *__restrict__ pcount) {
+    float *__restrict__ part, int32_t *__restrict__ pcount, TilePlan plan) {
   static_assert(S == 1 || NB == 1, "split tiles use one output block per wavefront");
   constexpr int WAVES = S == 1 ? CONV_WAVES : S;
   __shared__ int nbl[S == 1 ? WAVES : 1][TILE_M * K];
@@ -176,37 +176,54 @@ __global__ __launch_bounds__((S == 1 ? CONV_WAVES : S) * 64) void conv_mfma_kern
   if (live && t0 + r < n) my_row = rows ? rows[t0 + r] : (int)(t0 + r);
 
   // stage the tile's slice of the neighbour map in LDS and find the offsets it uses; all the
-  // loads are issued before the first one is consumed
+  // loads are issued before the first one is consumed.  With a tile plan (the map transposed into
+  // processing order, one 128-byte run per (offset, tile), and the offsets of every tile) the
+  // loads are coalesced, need no row id and the LDS copy is offset-major.
+  const bool planned = MODE == MAP_NBR && K == 27 && plan.map != nullptr;
   int *nl = nbl[S == 1 ? wave : 0];
   unsigned mymask = 0;
   constexpr int NSTAGE = (TILE_M * K + 64 * S - 1) / (64 * S);
   int staged[NSTAGE];
+  if (planned) {
 #pragma unroll
-  for (int i = 0; i < NSTAGE; i++) {
-    const int e = (S == 1 ? i : i * S + wave) * 64 + lane;
-    const int rr = e / K, kk = e - rr * K;
-    const int rid = __shfl(my_row, rr & (TILE_M - 1), 64);
-    int v = -1;
-    if (e < TILE_M * K && rid >= 0) {
-      if (MODE == MAP_NBR)
-        v = map0[(int64_t)rid * K + kk];
-      else if (MODE == MAP_IDENTITY)
-        v = rid;
-      else
-        v = (map1[rid] == kk) ? map0[rid] : -1;
+    for (int i = 0; i < NSTAGE; i++) {
+      const int e = (S == 1 ? i : i * S + wave) * 64 + lane;  // e = k * 32 + row
+      staged[i] = (live && e < TILE_M * K) ? plan.map[(int64_t)(e >> 5) * plan.ld + t0 + (e & 31)] : -1;
     }
-    staged[i] = v;
-  }
+    if (live) mymask = plan.tmask[t0 >> 5];
 #pragma unroll
-  for (int i = 0; i < NSTAGE; i++) {
-    const int e = (S == 1 ? i : i * S + wave) * 64 + lane;
-    if (e < TILE_M * K) {
-      nl[e] = staged[i];
-      if (staged[i] >= 0) mymask |= 1u << (e % K);
+    for (int i = 0; i < NSTAGE; i++) {
+      const int e = (S == 1 ? i : i * S + wave) * 64 + lane;
+      if (e < TILE_M * K) nl[e] = staged[i];
     }
-  }
+  } else {
 #pragma unroll
-  for (int d = 32; d > 0; d >>= 1) mymask |= (unsigned)__shfl_xor((int)mymask, d, 64);
+    for (int i = 0; i < NSTAGE; i++) {
+      const int e = (S == 1 ? i : i * S + wave) * 64 + lane;
+      const int rr = e / K, kk = e - rr * K;
+      const int rid = __shfl(my_row, rr & (TILE_M - 1), 64);
+      int v = -1;
+      if (e < TILE_M * K && rid >= 0) {
+        if (MODE == MAP_NBR)
+          v = map0[(int64_t)rid * K + kk];
+        else if (MODE == MAP_IDENTITY)
+          v = rid;
+        else
+          v = (map1[rid] == kk) ? map0[rid] : -1;
+      }
+      staged[i] = v;
+    }
+#pragma unroll
+    for (int i = 0; i < NSTAGE; i++) {
+      const int e = (S == 1 ? i : i * S + wave) * 64 + lane;
+      if (e < TILE_M * K) {
+        nl[e] = staged[i];
+        if (staged[i] >= 0) mymask |= 1u << (e % K);
+      }
+    }
+#pragma unroll
+    for (int d = 32; d > 0; d >>= 1) mymask |= (unsigned)__shfl_xor((int)mymask, d, 64);
+  }
   if (S > 1 && lane == 0) wmask[wave] = mymask;
   __syncthreads();
   if (!live) return;  // the whole block (S > 1) or wavefront (S == 1) is idle; no barrier follows
@@ -285,7 +302,8 @@ __global__ __launch_bounds__((S == 1 ? CONV_WAVES : S) * 64) void conv_mfma_kern
     // lane (r, h) reads channels ch*32 + h*16 .. +15 of its own row; the second half-wave of a
     // 16-channel tail chunk has no channels
     auto gather = [&](const Cursor &c) -> Frag {
-      const int src = nl[r * K + (c.k < 0 ? 0 : c.k)];
+      const int kk = c.k < 0 ? 0 : c.k;
+      const int src = nl[planned ? kk * TILE_M + r : r * K + kk];
       const bool on = c.k >= 0 && src >= 0 && (h == 0 || Cin - c.ch * 32 >= 32);
       const uint32_t voff = on ? (uint32_t)src * ld4 + (uint32_t)(c.ch * 128 + h * 64) : BUF_OOB;
       Frag f;
@@ -445,7 +463,7 @@ __global__ __launch_bounds__(WL_WAVES * 64) void conv_wlds_kernel(
     const float *__restrict__ in, int64_t ld_in, float *__restrict__ out, int64_t ld_out,
     const float *__restrict__ Wp, const float *__restrict__ bias, const int32_t *__restrict__ map0,
     const int32_t *__restrict__ rows, const int32_t *__restrict__ d_n_rows, int64_t n_rows, int Cin, int Cout,
-    const uint8_t *__restrict__ tile_flags, uint32_t in_bytes, uint32_t map_bytes, BnEpilogue ep) {
+    const uint8_t *__restrict__ tile_flags, uint32_t in_bytes, uint32_t map_bytes, BnEpilogue ep, TilePlan plan) {
   constexpr int K = 27;
   constexpr int NSTAGE = (TILE_M * K + 63) / 64;
   __shared__ __attribute__((aligned(16))) float wl[K * 1024];
@@ -494,10 +512,24 @@ __global__ __launch_bounds__(WL_WAVES * 64) void conv_wlds_kernel(
     return (t < ntiles && p < n) ? (rows ? rows[p] : (int)p) : -1;
   };
   // issue the loads of a tile's slice of the neighbour map; bit i of the result: element i of
-  // this lane exists (a load sent out of range returns 0, which would pass for a site)
-  auto stage_issue = [&](int my_row, int (&st)[NSTAGE]) -> unsigned {
-    int srow[NSTAGE];
+  // this lane exists (a load sent out of range returns 0, which would pass for a site).  With a
+  // tile plan the slice is 27 coalesced runs that need no row id; the LDS copy is offset-major.
+  const bool planned = plan.map != nullptr;
+  const __amdgpu_buffer_rsrc_t rplan = make_rsrc(plan.map, planned ? (uint32_t)(plan.ld * K * 4) : 0u);
+  auto stage_issue = [&](int64_t tt, int my_row, int (&st)[NSTAGE]) -> unsigned {
     unsigned valid = 0;
+    if (planned) {
+#pragma unroll
+      for (int i = 0; i < NSTAGE; i++) {
+        const int e = i * 64 + lane;  // e = k * 32 + row
+        const bool ok = e < TILE_M * K && tt < ntiles;
+        if (ok) valid |= 1u << i;
+        const uint32_t voff = ok ? (uint32_t)((e >> 5) * (int)plan.ld + (int)(tt * TILE_M) + (e & 31)) * 4u : BUF_OOB;
+        st[i] = __builtin_amdgcn_raw_buffer_load_b32(rplan, (int)voff, 0, 0);
+      }
+      return valid;
+    }
+    int srow[NSTAGE];
 #pragma unroll
     for (int i = 0; i < NSTAGE; i++) srow[i] = __shfl(my_row, ((i * 64 + lane) / K) & (TILE_M - 1), 64);
 #pragma unroll
@@ -516,24 +548,33 @@ __global__ __launch_bounds__(WL_WAVES * 64) void conv_wlds_kernel(
   int64_t t = draw();
   int my_row = load_row(t);
   int st[NSTAGE];
-  unsigned valid = stage_issue(my_row, st);
+  unsigned valid = stage_issue(t, my_row, st);
   int64_t tn = t < ntiles ? draw() : ntiles;
   int my_row_n = load_row(tn);
 
   while (t < ntiles) {
     // neighbour-map slice -> LDS (private to the wavefront), and the offsets the tile uses
     unsigned mymask = 0;
+    if (planned) {
+      mymask = plan.tmask[t];
 #pragma unroll
-    for (int i = 0; i < NSTAGE; i++) {
-      const int e = i * 64 + lane;
-      if (e < TILE_M * K) {
-        const bool have = ((valid >> i) & 1u) && st[i] >= 0;
-        nl[e] = have ? st[i] : -1;
-        if (have) mymask |= 1u << (e % K);
+      for (int i = 0; i < NSTAGE; i++) {
+        const int e = i * 64 + lane;
+        if (e < TILE_M * K) nl[e] = st[i];
       }
-    }
+    } else {
 #pragma unroll
-    for (int d = 32; d > 0; d >>= 1) mymask |= (unsigned)__shfl_xor((int)mymask, d, 64);
+      for (int i = 0; i < NSTAGE; i++) {
+        const int e = i * 64 + lane;
+        if (e < TILE_M * K) {
+          const bool have = ((valid >> i) & 1u) && st[i] >= 0;
+          nl[e] = have ? st[i] : -1;
+          if (have) mymask |= 1u << (e % K);
+        }
+      }
+#pragma unroll
+      for (int d = 32; d > 0; d >>= 1) mymask |= (unsigned)__shfl_xor((int)mymask, d, 64);
+    }
     unsigned rest = (unsigned)__builtin_amdgcn_readfirstlane((int)mymask);
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
@@ -541,7 +582,7 @@ __global__ __launch_bounds__(WL_WAVES * 64) void conv_wlds_kernel(
 
     // next tile's loads
     int stn[NSTAGE];
-    const unsigned valid_n = stage_issue(my_row_n, stn);
+    const unsigned valid_n = stage_issue(tn, my_row_n, stn);
     const int64_t tnn = tn < ntiles ? draw() : ntiles;
     const int my_row_nn = load_row(tnn);
 
@@ -558,7 +599,8 @@ __global__ __launch_bounds__(WL_WAVES * 64) void conv_wlds_kernel(
         return k;
       };
       auto gather = [&](int k) -> Frag {
-        const int src = nl[r * K + (k < 0 ? 0 : k)];
+        const int kk = k < 0 ? 0 : k;
+        const int src = nl[planned ? kk * TILE_M + r : r * K + kk];
         const bool on = k >= 0 && src >= 0 && half_on;
         const uint32_t voff = on ? (uint32_t)src * ld4 + (uint32_t)(h * 64) : BUF_OOB;
         Frag f;
@@ -648,6 +690,40 @@ __global__ void count_rules_kernel(const int32_t *__restrict__ map0, int K, cons
   if ((threadIdx.x & 63) == 0 && c) atomicAdd(total, (unsigned long long)c);
 }
 
+// map[k * ld + p] = nbr[order[p]][k] for p < n, -1 up to the end of the last tile; tmask[t] = OR of
+// the offsets the rows of tile t have.  One thread per position; the writes of one offset are
+// coalesced across the wavefront.
+__global__ __launch_bounds__(256) void tile_plan_kernel(const int32_t *__restrict__ nbr,
+                                                        const int32_t *__restrict__ order,
+                                                        const int32_t *__restrict__ d_n, int64_t n_rows, int64_t ld,
+                                                        int32_t *__restrict__ map, uint32_t *__restrict__ tmask) {
+  const int64_t n = d_n ? min((int64_t)*d_n, n_rows) : n_rows;
+  const int64_t padded = (n + TILE_M - 1) / TILE_M * TILE_M;
+  const int64_t p = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (p >= padded) return;  // whole 32-lane groups leave together (padded is a multiple of 32)
+  const int site = p < n ? (order ? order[p] : (int)p) : -1;
+  unsigned m = 0;
+#pragma unroll
+  for (int k = 0; k < 27; k++) {
+    const int v = site >= 0 ? nbr[(int64_t)site * 27 + k] : -1;
+    map[(int64_t)k * ld + p] = v;
+    if (v >= 0) m |= 1u << k;
+  }
+#pragma unroll
+  for (int d = 16; d > 0; d >>= 1) m |= (unsigned)__shfl_xor((int)m, d, 64);
+  if ((threadIdx.x & 31) == 0) tmask[p >> 5] = m;
+}
+
+int build_tile_plan(const int32_t *nbr, const int32_t *order, const int32_t *d_n, int64_t n_rows, int64_t ld,
+                    int32_t *map, uint32_t *tmask, hipStream_t s) {
+  if (n_rows <= 0) return INSC_OK;
+  const int64_t padded = cdiv(n_rows, TILE_M) * TILE_M;
+  hipLaunchKernelGGL(tile_plan_kernel, dim3(grid_for(padded, 256)), dim3(256), 0, s, nbr, order, d_n, n_rows, ld, map,
+                     tmask);
+  INSC_LAUNCH_CHECK();
+  return INSC_OK;
+}
+
 static bool conv_uses_mfma(const float *in, int64_t ld_in, int Cin, int K) {
   return Cin % 16 == 0 && ((uintptr_t)in % 16 == 0) && (ld_in % 4 == 0) && (K == 27 || K == 8 || K == 1);
 }
@@ -669,8 +745,10 @@ int pack_weights(const float *W, int K, int Cin, int Cout, float *Wp, hipStream_
 int launch_conv(const float *in, int64_t ld_in, int64_t in_rows, float *out, int64_t ld_out, const float *W,
                 const float *Wp, const float *bias, const int32_t *map0, const int32_t *map1, int mode, int K,
                 const int32_t *rows, const int32_t *d_n_rows, int64_t n_rows, int Cin, int Cout,
-                const uint8_t *tile_flags, const uint8_t *row_mask, hipStream_t s, BnEpilogue ep) {
+                const uint8_t *tile_flags, const uint8_t *row_mask, hipStream_t s, BnEpilogue ep, TilePlan plan) {
   if (n_rows == 0) return INSC_OK;
+  if (plan.map && (mode != MAP_NBR || K != 27 || plan.ld * 27 * 4 >= (int64_t)BUF_OOB || plan.ld < cdiv(n_rows, TILE_M) * TILE_M))
+    plan = TilePlan();  // only the 3^3 map has a plan; an unusable one is ignored
   if (conv_uses_mfma(in, ld_in, Cin, K)) {
     // the gather addresses rows with 32-bit byte offsets (buffer loads)
     const int64_t in_bytes64 = in_rows * ld_in * 4, wp_bytes64 = packed_floats(K, Cin, Cout) * 4;
@@ -699,7 +777,7 @@ int launch_conv(const float *in, int64_t ld_in, int64_t in_rows, float *out, int
       const int64_t want = cdiv(tiles, WL_WAVES);
       const unsigned nblk = (unsigned)std::min<int64_t>(device_cus(), want);
       hipLaunchKernelGGL(conv_wlds_kernel, dim3(nblk), dim3(WL_WAVES * 64), 0, s, in, ld_in, out, ld_out, Wp, bias,
-                         map0, rows, d_n_rows, n_rows, Cin, Cout, tile_flags, in_bytes, map_bytes, ep);
+                         map0, rows, d_n_rows, n_rows, Cin, Cout, tile_flags, in_bytes, map_bytes, ep, plan);
       INSC_LAUNCH_CHECK();
       return INSC_OK;
     }
@@ -734,7 +812,7 @@ int launch_conv(const float *in, int64_t ld_in, int64_t in_rows, float *out, int
 #define INSC_CONV_LAUNCH(NBV, KV, MV, SV)                                                                       \
   hipLaunchKernelGGL((conv_mfma_kernel<NBV, KV, MV, SV>), grid, block, 0, s, in, ld_in, out, ld_out, Wp, bias,  \
                      map0, map1, rows, d_n_rows, n_rows, Cin, Cout, nbtp, tile_flags, in_bytes, wp_bytes, ep, part,  \
-                     pcount)
+                     pcount, plan)
 #define INSC_CONV_CASE(NBV)                                      \
   case NBV:                                                      \
     if (mode == MAP_NBR && K == 27)                              \
@@ -852,6 +930,31 @@ int insc_conv_nbr(const float *d_in, int64_t ld_in, int64_t n_in_rows, float *d_
     *h_muladds = (double)h * Cin * Cout;
   }
   return INSC_OK;
+}
+
+int insc_plan_build(const int32_t *d_nbr, const int32_t *d_order, const int32_t *d_n_rows, int64_t n_rows,
+                    int64_t plan_ld, int32_t *d_plan, uint32_t *d_tmask, void *stream) {
+  INSC_REQUIRE(n_rows >= 0 && plan_ld >= cdiv(n_rows, TILE_M) * TILE_M, INSC_ERR_ARG,
+               "insc_plan_build: plan_ld must cover the rows rounded up to a multiple of 32");
+  INSC_REQUIRE(n_rows == 0 || (d_nbr && d_plan && d_tmask), INSC_ERR_ARG, "insc_plan_build: null pointer");
+  return build_tile_plan(d_nbr, d_order, d_n_rows, n_rows, plan_ld, d_plan, d_tmask, (hipStream_t)stream);
+}
+
+int insc_conv_ssc_plan(const float *d_in, int64_t ld_in, int64_t n_in_rows, float *d_out, int64_t ld_out,
+                       const float *d_W, const float *d_Wp, const float *d_bias, const int32_t *d_nbr,
+                       const int32_t *d_plan, int64_t plan_ld, const uint32_t *d_tmask, const int32_t *d_order,
+                       const int32_t *d_n_rows, int64_t n_rows, int Cin, int Cout, void *stream) {
+  INSC_REQUIRE(n_rows >= 0 && Cin > 0 && Cout > 0 && n_in_rows >= 0, INSC_ERR_ARG, "insc_conv_ssc_plan: bad sizes");
+  INSC_REQUIRE(ld_in >= Cin && ld_out >= Cout, INSC_ERR_ARG, "insc_conv_ssc_plan: row stride smaller than channel count");
+  INSC_REQUIRE(n_rows == 0 || (d_in && d_out && (d_W || d_Wp) && d_nbr && d_plan && d_tmask), INSC_ERR_ARG,
+               "insc_conv_ssc_plan: null pointer");
+  INSC_REQUIRE(plan_ld >= cdiv(n_rows, TILE_M) * TILE_M, INSC_ERR_ARG, "insc_conv_ssc_plan: plan_ld too small");
+  TilePlan plan;
+  plan.map = d_plan;
+  plan.ld = plan_ld;
+  plan.tmask = d_tmask;
+  return launch_conv(d_in, ld_in, n_in_rows, d_out, ld_out, d_W, d_Wp, d_bias, d_nbr, nullptr, MAP_NBR, 27, d_order,
+                     d_n_rows, n_rows, Cin, Cout, nullptr, nullptr, (hipStream_t)stream, BnEpilogue(), plan);
 }
 
 int insc_deconv_down2(const float *d_in, int64_t ld_in, int64_t n_in_rows, float *d_out, int64_t ld_out,

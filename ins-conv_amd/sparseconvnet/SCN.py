@@ -92,6 +92,8 @@ class _Scale(object):
         self.nbr_n = 0
         self.order = _Buf(None, torch.int32, device)
         self.order_n = 0
+        self.plan = None  # tile plan of the 3^3 map in processing order: (map [27*ld] int32, tmask, ld)
+        self.plan_n = -1
         self.n_rules = None  # cached number of (in,out) pairs of the 3^3 rulebook
         self.n_rules_at = -1
         self.downs = {}
@@ -219,6 +221,19 @@ class Metadata_3(object):
             sc.nbr_n = sc.order_n = sc.n
         return sc
 
+    def ssc_plan(self, sc):
+        """Tile plan of the scale's 3^3 map (insc_plan_build), rebuilt when sites were added."""
+        if sc.plan_n != sc.n:
+            ld = (sc.n + 31) // 32 * 32
+            if sc.plan is None or sc.plan[2] < ld:
+                cap = max(ld, 1024)
+                sc.plan = (torch.empty(27 * cap, dtype=torch.int32, device=sc.device),
+                           torch.empty(cap // 32 + 1, dtype=torch.int32, device=sc.device), cap)
+            lib.insc_plan_build(ptr(sc.nbr.t), ptr(sc.order.t), None, I64(sc.n), I64(sc.plan[2]), ptr(sc.plan[0]),
+                                ptr(sc.plan[1]), stream_ptr())
+            sc.plan_n = sc.n
+        return sc.plan
+
     def n_ssc_rules(self, sc):
         if sc.n_rules_at != sc.n:
             # bookkeeping for the multiply-add counter only (not part of the computation)
@@ -315,6 +330,14 @@ def conv_rows(in_f, out_f, weight, bias, nbr, K, rows, count, n_rows):
     lib.insc_conv_nbr(ptr(in_f), I64(_ld(in_f)), I64(in_f.size(0)), ptr(out_f), I64(_ld(out_f)), ptr(weight),
                       ptr(packed_weight(weight, K)), ptr(bias), ptr(nbr), int(K), ptr(rows), ptr(count),
                       I64(int(n_rows)), int(Cin), int(Cout), None, stream_ptr())
+
+
+def ssc_rows_planned(in_f, out_f, weight, bias, sc, plan):
+    """insc_conv_ssc_plan over all sites of a scale in its processing order."""
+    Cin, Cout = weight.size(-2), weight.size(-1)
+    lib.insc_conv_ssc_plan(ptr(in_f), I64(_ld(in_f)), I64(in_f.size(0)), ptr(out_f), I64(_ld(out_f)), ptr(weight),
+                           ptr(packed_weight(weight, 27)), ptr(bias), ptr(sc.nbr.t), ptr(plan[0]), I64(plan[2]),
+                           ptr(plan[1]), ptr(sc.order.t), None, I64(int(sc.n)), int(Cin), int(Cout), stream_ptr())
 
 
 def deconv_rows(in_f, out_f, weight, bias, parent, offset, rows, count, n_rows):
@@ -417,7 +440,7 @@ def SubmanifoldConvolution_updateOutput(inputSize, filterSize, m, input_features
     _resize(output_features, sc.n, w.size(2), input_features)
     if sc.n == 0:
         return 0.0
-    conv_rows(input_features, output_features, w, b, sc.nbr.t, 27, sc.order.t, None, sc.n)
+    ssc_rows_planned(input_features, output_features, w, b, sc, m.ssc_plan(sc))
     return float(m.n_ssc_rules(sc)) * w.size(1) * w.size(2)
 
 
