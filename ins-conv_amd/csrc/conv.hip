@@ -66,6 +66,66 @@ __global__ __launch_bounds__(256) void conv_generic_kernel(const float *__restri
 }
 
 // ---------------------------------------------------------------------------------------
+// 3^3 layers with 1..4 input channels (the RGB stem of a U-Net): same thread layout and the same
+// order of operations as the generic kernel (so the same bits), but the 27 x CIN weights of a
+// thread's output channel stay in registers over all its rows, and the 27 neighbour ids and the
+// input values of a row are fetched in batches instead of one dependent load after the other.
+// ---------------------------------------------------------------------------------------
+template <int CIN>
+__global__ __launch_bounds__(256) void conv_stem_kernel(const float *__restrict__ in, int64_t ld_in,
+                                                        float *__restrict__ out, int64_t ld_out,
+                                                        const float *__restrict__ W, const float *__restrict__ bias,
+                                                        const int32_t *__restrict__ map0,
+                                                        const int32_t *__restrict__ rows,
+                                                        const int32_t *__restrict__ d_n_rows, int64_t n_rows,
+                                                        int Cout, const uint8_t *__restrict__ row_mask,
+                                                        BnEpilogue ep) {
+  constexpr int K = 27, GK = 9;  // offsets per batch
+  const int64_t n = d_n_rows ? min((int64_t)*d_n_rows, n_rows) : n_rows;
+  const int cpb = 256 / Cout;  // rows per block (Cout <= 256)
+  const int lr = threadIdx.x / Cout, co = threadIdx.x % Cout;
+  if (lr >= cpb) return;
+  float w[K][CIN];
+#pragma unroll
+  for (int k = 0; k < K; k++)
+#pragma unroll
+    for (int ci = 0; ci < CIN; ci++) w[k][ci] = W[((int64_t)k * CIN + ci) * Cout + co];
+  const float bv = bias ? bias[co] : 0.0f;
+  const float ew = ep.out2 ? ep.w[co] : 0.0f, eb = ep.out2 ? ep.b[co] : 0.0f;
+  for (int64_t t = (int64_t)blockIdx.x * cpb + lr; t < n; t += (int64_t)gridDim.x * cpb) {
+    const int row = rows ? rows[t] : (int)t;
+    if (row < 0 || (row_mask && !row_mask[row])) continue;
+    int src[K];
+#pragma unroll
+    for (int k = 0; k < K; k++) src[k] = map0[(int64_t)row * K + k];
+    float acc = bv;
+#pragma unroll
+    for (int g = 0; g < K / GK; g++) {
+      float x[GK][CIN];
+#pragma unroll
+      for (int j = 0; j < GK; j++) {
+        const float *p = in + (int64_t)max(src[g * GK + j], 0) * ld_in;
+#pragma unroll
+        for (int ci = 0; ci < CIN; ci++) x[j][ci] = p[ci];
+      }
+#pragma unroll
+      for (int j = 0; j < GK; j++) {
+        float a = acc;
+#pragma unroll
+        for (int ci = 0; ci < CIN; ci++) a = fmaf(x[j][ci], w[g * GK + j][ci], a);
+        acc = src[g * GK + j] >= 0 ? a : acc;
+      }
+    }
+    if (ep.res) acc += ep.res[(int64_t)row * ep.ldr + co];
+    if (out) out[(int64_t)row * ld_out + co] = acc;
+    if (ep.out2) {
+      const float y = fmaf(acc, ew, eb);
+      ep.out2[(int64_t)row * ep.ld2 + co] = y * ((y > 0.0f) ? 1.0f : ep.leak);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------
 // Weight packing.  For filter offset k, input-channel chunk ch (32 channels) and
 // output-channel block nb (32 channels), lane = h*32 + j of the MFMA kernel needs the 16
 // B-operand values W[k][ch*32 + h*16 + s][nb*32 + j], s = 0..15.  The 4 KB tile is stored as
@@ -788,11 +848,11 @@ int launch_conv(const float *in, int64_t ld_in, int64_t in_rows, float *out, int
     //  wider layers sit at the coarse scales of a U-Net, which have few tiles: one output block
     //    per wavefront, and for 3^3 / 2^3 maps the items of a tile are dealt to S wavefronts
     //    (S grows with Cin: 2, 4, 8 for 3^3).
-    const bool split = Cin >= 64 && mode == MAP_NBR && K > 1;
+    const bool split = Cin >= 64 && K > 1 && (mode == MAP_NBR || (mode == MAP_PARENT && Cin >= 96));
     const int NB0 = split ? 1 : conv_nb_per_group(Cout);
     const int nbtp = conv_nbt_padded(Cout);
     int S = 1;
-    if (split) S = K == 27 ? (Cin >= 160 ? 8 : Cin >= 128 ? 4 : 2) : (Cin >= 96 ? 4 : 1);
+    if (split) S = K == 27 ? (Cin >= 160 ? 8 : Cin >= 128 ? 4 : 2) : (Cin >= 96 ? 4 : 1);  // K == 8: conv and deconv
     const int NB = (S == 1 && Cin >= 96) ? 1 : NB0;
     const int G = (split && K == 27) ? (Cin >= 160 ? 4 : Cin >= 128 ? 2 : 1) : 1;
     if (G > 1) S = 4;
@@ -835,11 +895,11 @@ int launch_conv(const float *in, int64_t ld_in, int64_t in_rows, float *out, int
       }
     } else if (S > 1 && mode == MAP_NBR && K == 8) {
       switch (S) {
-        case 2: INSC_CONV_LAUNCH(1, 8, MAP_NBR, 2); break;
         case 4: INSC_CONV_LAUNCH(1, 8, MAP_NBR, 4); break;
-        case 8: INSC_CONV_LAUNCH(1, 8, MAP_NBR, 8); break;
         default: shape_ok = false;
       }
+    } else if (S == 4 && mode == MAP_PARENT && K == 8) {
+      INSC_CONV_LAUNCH(1, 8, MAP_PARENT, 4);
     } else if (S > 1) {
       shape_ok = false;
     } else {
@@ -868,6 +928,24 @@ int launch_conv(const float *in, int64_t ld_in, int64_t in_rows, float *out, int
       return INSC_ERR_ARG;
     }
     const int cpb = 256 / Cout;
+    if (mode == MAP_NBR && K == 27 && Cin <= 4) {
+      // enough blocks to fill the machine, few enough that the weights are fetched rarely
+      const dim3 sg(grid_for(n_rows, cpb, (unsigned)device_cus() * 8));
+#define INSC_STEM(CI)                                                                                          \
+  hipLaunchKernelGGL(conv_stem_kernel<CI>, sg, dim3(256), 0, s, in, ld_in, out, ld_out, W, bias, map0, rows, \
+                     d_n_rows, n_rows, Cout, row_mask, ep)
+      if (Cin == 1)
+        INSC_STEM(1);
+      else if (Cin == 2)
+        INSC_STEM(2);
+      else if (Cin == 3)
+        INSC_STEM(3);
+      else
+        INSC_STEM(4);
+#undef INSC_STEM
+      INSC_LAUNCH_CHECK();
+      return INSC_OK;
+    }
     hipLaunchKernelGGL(conv_generic_kernel, dim3(grid_for(n_rows, cpb, 65536)), dim3(256), 0, s, in, ld_in, out,
                        ld_out, W, bias, map0, map1, mode, K, rows, d_n_rows, n_rows, Cin, Cout, row_mask, ep);
   }
