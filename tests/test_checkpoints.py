@@ -1,0 +1,53 @@
+"""Checkpoint helpers and the offset-numbering conversion for weights trained against the
+reference's CPU rule generator (no GPU needed: modules are only constructed, the numerical
+check runs on the CPU oracle)."""
+import os
+
+import numpy as np
+import torch
+
+import scenes
+
+
+def test_checkpoint_round_trip(tmp_path):
+    import sparseconvnet as scn
+    from netdefs import NaiveUNet
+
+    a, b = NaiveUNet(m=8, levels=3, seed=1), NaiveUNet(m=8, levels=3, seed=2)
+    exp = str(tmp_path / "exp")
+    for epoch in (1, 2, 3, 4, 5):
+        scn.checkpoint_save(a, exp, "unet", epoch, use_cuda=False)
+    left = sorted(os.listdir(tmp_path))
+    # epochs whose number is a power of two survive, plus the latest (utils.py:228-233)
+    assert left == ["exp-0001-unet.pth", "exp-0002-unet.pth", "exp-0004-unet.pth", "exp-0005-unet.pth"]
+    nxt = scn.checkpoint_restore(b, exp, "unet", use_cuda=False)
+    assert nxt == 6
+    for (ka, va), (kb, vb) in zip(a.state_dict().items(), b.state_dict().items()):
+        assert ka == kb and torch.equal(va, vb)
+    assert scn.checkpoint_restore(b, exp, "unet", use_cuda=False, epoch=2) == 3
+    # parameter names and shapes are the reference's: [27|8, nIn, nOut] filters, BN running stats
+    sd = a.state_dict()
+    assert any(v.dim() == 3 and v.size(0) == 27 for v in sd.values())
+    assert any(v.dim() == 3 and v.size(0) == 8 for v in sd.values())
+    assert any(k.endswith("running_mean") for k in sd) and any(k.endswith("running_var") for k in sd)
+
+
+def test_zmajor_weights_convert_to_this_numbering(orc):
+    import sparseconvnet as scn
+
+    perm = scn.ssc_offset_permutation()
+    assert torch.equal(perm[perm], torch.arange(27))
+    for k in range(27):
+        dx, dy, dz = k // 9 - 1, (k // 3) % 3 - 1, k % 3 - 1
+        assert perm[k].item() == (dz + 1) * 9 + (dy + 1) * 3 + (dx + 1)
+    pts = scenes.boxes_scene(seed=1, n=3000)
+    _, sc, _ = orc.grid_build(pts)
+    rng = np.random.default_rng(0)
+    x = rng.normal(size=(len(sc), 8)).astype(np.float32)
+    Wz = rng.normal(size=(27, 8, 12)).astype(np.float32)  # trained against the z-major numbering
+    _, cz, pz = orc.ssc_rules(sc, zmajor=True)
+    ref, _ = orc.conv_forward(x, Wz, None, pz, cz, len(sc))
+    Wx = scn.convert_zmajor_state_dict({"w": torch.from_numpy(Wz), "b": torch.zeros(3)})["w"].numpy()
+    _, cx, px = orc.ssc_rules(sc, zmajor=False)
+    got, _ = orc.conv_forward(x, Wx, None, px, cx, len(sc))
+    np.testing.assert_allclose(got, ref, rtol=1e-4, atol=1e-5)  # (the two runs add the 27 terms in different orders)
