@@ -226,6 +226,16 @@ def kernel_table(device, reps=20):
     add("input layer (mode 4: per-voxel mean)", t, P * (4 * C + 4) + N * 4 * C, "%d points x %d -> %d sites" % (P, C, N))
     t = timed(lambda: lib.insc_output_gather(ptr(y), I64(C), ptr(sop), I64(P), C, ptr(outp), st))
     add("output layer (row gather)", t, P * (4 * C + 4) + P * 4 * C, "%d points x %d" % (P, C))
+    # label fusion: one frame of 20-class scores folded into the per-voxel (label, confidence) table
+    NCLS = 20
+    table = ctypes.c_void_p()
+    lib.insc_labels_create(I64(2 * N), 0, ctypes.c_float(5.0), ctypes.byref(table))
+    scores = torch.rand(P, NCLS, device=device)
+    lib.insc_labels_update(table, ptr(c4), ptr(scores), I64(NCLS), I64(P), NCLS, st)  # the voxels exist from here on
+    t = timed(lambda: lib.insc_labels_update(table, ptr(c4), ptr(scores), I64(NCLS), I64(P), NCLS, st))
+    add("label fusion update (argmax + per-voxel confidence rule)", t, P * (16 + 4 * NCLS + 12) + N * 16,
+        "%d points x %d classes -> %d voxels" % (P, NCLS, N))
+    lib.insc_labels_destroy(table)
     lib.insc_grid_destroy(grid)
     lib.insc_grid_destroy(coarse)
     return rows

@@ -271,6 +271,37 @@ int insc_net_counts(insc_net *net, int64_t *h_sites_per_level, int64_t *h_points
 int insc_net_profile(insc_net *net, int enable, float *h_ms4);
 
 /* ---------------------------------------------------------------------------------------
+ * Per-voxel label fusion over frames (Result<3> and ResultOfWeight, Metadata/resultHash.h:23-218;
+ * bound as SCN.Result_3 / SCN.ResultOfWeight, pybind.cpp:36-45,275-282).  The reference keeps a
+ * CPU hash map and handles points one by one; here the map is a hash grid plus device arrays.
+ * kind 0: (label, confidence) per voxel; kind 1: running scores per voxel (new = 0.5*old + row).
+ * Rows of one voxel inside a call are applied in ascending row order.
+ * `maximum` is truncated towards zero, as the reference does by storing it in an int member
+ * (resultHash.h:25,30): its default 0.7 acts as a ceiling of 0.
+ * ------------------------------------------------------------------------------------- */
+typedef struct insc_labels insc_labels;
+int insc_labels_create(int64_t capacity_voxels, int kind, float maximum, insc_labels **out);
+int insc_labels_destroy(insc_labels *l);
+int insc_labels_clear(insc_labels *l, void *stream);
+/* Result::set (resultHash.h:36-47): label = argmax of the row, confidence 0; the last row of a voxel wins. */
+int insc_labels_set(insc_labels *l, const int32_t *d_coords4, const float *d_scores, int64_t ld, int64_t P, int C,
+                    void *stream);
+/* Result::update (resultHash.h:49-101) for kind 0: a new voxel takes (argmax, max); a known one
+ * gains the row's maximum if the label agrees (up to the ceiling), loses it otherwise, and flips
+ * to the row's label when the confidence falls below zero.  ResultOfWeight::update
+ * (resultHash.h:158-170) for kind 1. */
+int insc_labels_update(insc_labels *l, const int32_t *d_coords4, const float *d_scores, int64_t ld, int64_t P, int C,
+                       void *stream);
+/* multiQuery (resultHash.h:110-118,179-187): label per coordinate, -1 for an unknown voxel. */
+int insc_labels_query(insc_labels *l, const int32_t *d_coords4, int64_t Q, int32_t *d_label, void *stream);
+int insc_labels_count(insc_labels *l, int64_t *h_n, void *stream);
+/* get_all_points_labels (resultHash.h:120-132,189-201): rows (x, y, z, label) of the first `rows`
+ * voxels; d_conf (nullable) receives the confidence (kind 0) or the best score (kind 1). */
+int insc_labels_export(insc_labels *l, int32_t *d_out4, float *d_conf, int64_t rows, void *stream);
+/* finalize (resultHash.h:134-145,203-214): forget every voxel that is not in the list. */
+int insc_labels_finalize(insc_labels *l, const int32_t *d_keep4, int64_t M, void *stream);
+
+/* ---------------------------------------------------------------------------------------
  * Device utilities exported for tests and callers.
  * ------------------------------------------------------------------------------------- */
 /* Exclusive prefix sum of n int32 values; d_total (nullable) receives the sum. */

@@ -34,7 +34,7 @@ int hip_fail(hipError_t e, const char *what, const char *file, int line);
 // ordered by its stream.
 // Arena 0 belongs to the scan primitive, arena 1 to the sort primitive, arena 2 to the
 // API-level function that is running (none of which calls another arena-2 user).
-enum { WS_SCAN = 0, WS_SORT = 1, WS_API = 2, WS_CONV = 3 };
+enum { WS_SCAN = 0, WS_SORT = 1, WS_API = 2, WS_CONV = 3, WS_LABELS = 4 };
 int workspace(int which, hipStream_t stream, size_t bytes, void **out);
 int device_cus();
 // `count` int32 counters per (device, stream), zero at kernel start; users leave them at zero

@@ -513,6 +513,91 @@ def n_rulebook_bits():
 
 
 # =========================================================================================
+# label fusion over frames (Result_3 / ResultOfWeight, pybind.cpp:36-45,275-282)
+# =========================================================================================
+class _Labels(object):
+    """Shared front end of the two label tables: the reference's method names and argument
+    shapes (Long [P,3] points, float [P,C] scores), tensors on either device."""
+    KIND = 0
+
+    def __init__(self, maximum=0.7, device=None):
+        self.device = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+        ensure_init(self.device.index or 0)
+        self.h = ctypes.c_void_p()
+        lib.insc_labels_create(I64(1 << 16), self.KIND, ctypes.c_float(float(maximum)), ctypes.byref(self.h))
+
+    def __del__(self):
+        try:
+            if self.h:
+                lib.insc_labels_destroy(self.h)
+                self.h = ctypes.c_void_p()
+        except Exception:
+            pass
+
+    def _args(self, ps, label):
+        if ps.dim() == 1:
+            ps, label = ps.unsqueeze(0), label.reshape(1, -1)
+        c4 = _coords4(ps[:, :3], self.device)
+        x = label.detach().to(device=self.device, dtype=torch.float32).contiguous()
+        if x.dim() != 2 or x.size(0) != c4.size(0):
+            raise ValueError("one row of scores per point is needed")
+        return c4, x
+
+    def update(self, ps, label):
+        if ps.dim() != 2:
+            raise ValueError("update takes a [P,3] list of points")  # the reference asserts the same
+        c4, x = self._args(ps, label)
+        lib.insc_labels_update(self.h, ptr(c4), ptr(x), I64(x.size(1)), I64(x.size(0)), int(x.size(1)), stream_ptr())
+
+    def multiQuery(self, ps):
+        c4 = _coords4(ps[:, :3], self.device)
+        out = torch.empty(c4.size(0), dtype=torch.int32, device=self.device)
+        lib.insc_labels_query(self.h, ptr(c4), I64(c4.size(0)), ptr(out), stream_ptr())
+        return out.cpu().long()
+
+    def query(self, p):
+        return int(self.multiQuery(p.reshape(1, -1))[0])
+
+    def __len__(self):
+        n = I64(0)
+        lib.insc_labels_count(self.h, ctypes.byref(n), stream_ptr())
+        return int(n.value)
+
+    def get_all_points_labels(self, with_confidence=False):
+        """Long [N,4] rows (x, y, z, label), in order of first appearance (the reference iterates
+        its hash map, i.e. in no particular order)."""
+        n = len(self)
+        out = torch.empty((n, 4), dtype=torch.int32, device=self.device)
+        conf = torch.empty(n, dtype=torch.float32, device=self.device) if with_confidence else None
+        lib.insc_labels_export(self.h, ptr(out), ptr(conf), I64(n), stream_ptr())
+        return (out.cpu().long(), conf.cpu()) if with_confidence else out.cpu().long()
+
+    def finalize(self, points):
+        c4 = _coords4(points[:, :3], self.device)
+        lib.insc_labels_finalize(self.h, ptr(c4), I64(c4.size(0)), stream_ptr())
+
+    def clear(self):
+        lib.insc_labels_clear(self.h, stream_ptr())
+
+
+class Result_3(_Labels):
+    """Result<3> (Metadata/resultHash.h:23-150): one (label, confidence) pair per voxel."""
+    KIND = 0
+
+    def set(self, ps, label):
+        c4, x = self._args(ps, label)
+        lib.insc_labels_set(self.h, ptr(c4), ptr(x), I64(x.size(1)), I64(x.size(0)), int(x.size(1)), stream_ptr())
+
+
+class ResultOfWeight(_Labels):
+    """ResultOfWeight (Metadata/resultHash.h:153-218): running scores per voxel, new = old/2 + row."""
+    KIND = 1
+
+    def __init__(self, device=None):
+        _Labels.__init__(self, 0.0, device)
+
+
+# =========================================================================================
 # canonical exports used by parity tests: the reference's list-form rulebooks
 # =========================================================================================
 def ssc_rulebook_lists(m, spatial_size):

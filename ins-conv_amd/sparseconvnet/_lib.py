@@ -62,6 +62,15 @@ _SIGS = {
                              ctypes.POINTER(c_int)],
     "insc_net_counts": [vp, ctypes.POINTER(c_i64), ctypes.POINTER(c_i64)],
     "insc_net_profile": [vp, c_int, ctypes.POINTER(ctypes.c_float)],
+    "insc_labels_create": [c_i64, c_int, c_f32, ctypes.POINTER(vp)],
+    "insc_labels_destroy": [vp],
+    "insc_labels_clear": [vp, vp],
+    "insc_labels_set": [vp, vp, vp, c_i64, c_i64, c_int, vp],
+    "insc_labels_update": [vp, vp, vp, c_i64, c_i64, c_int, vp],
+    "insc_labels_query": [vp, vp, c_i64, vp, vp],
+    "insc_labels_count": [vp, ctypes.POINTER(c_i64), vp],
+    "insc_labels_export": [vp, vp, vp, c_i64, vp],
+    "insc_labels_finalize": [vp, vp, c_i64, vp],
     "insc_scan_exclusive_i32": [vp, vp, c_i64, vp, vp],
     "insc_sort_pairs_u64": [vp, vp, c_i64, c_int, vp],
 }

@@ -178,3 +178,77 @@ def canonical_rules(counts, pairs, in_coords, out_coords):
     rows = np.concatenate([k[:, None], ic, oc], 1)
     o = np.lexsort(tuple(rows[:, j] for j in range(rows.shape[1] - 1, -1, -1)))
     return rows[o]
+
+
+# ---------------------------------------------------------------------------------------------
+# label fusion over frames (Metadata/resultHash.h).  Plain Python over a dict: small cases only.
+# ---------------------------------------------------------------------------------------------
+class ResultOracle(object):
+    """Result<3>::set / update / multiQuery / finalize (resultHash.h:36-145), rows applied one
+    after the other.  `maximum` lands in an int member there (resultHash.h:25,30), hence int()."""
+
+    def __init__(self, maximum=0.7):
+        self.maximum = int(maximum)
+        self.result = {}  # (x,y,z) -> [label, confidence]; insertion order = first appearance
+
+    def set(self, ps, scores):
+        for p, row in zip(np.asarray(ps), np.asarray(scores, np.float32)):
+            self.result[tuple(int(v) for v in p[:3])] = [int(np.argmax(row)), np.float32(0)]
+
+    def update(self, ps, scores):
+        ps, scores = np.asarray(ps), np.asarray(scores, np.float32)
+        idx, prob = scores.argmax(1), scores.max(1)  # label.max(1): value and first index
+        pre = []
+        for p in ps:  # first loop (:62-75): which rows find their voxel already there
+            k = tuple(int(v) for v in p[:3])
+            pre.append(k in self.result)
+            if k not in self.result:
+                self.result[k] = [0, np.float32(0)]
+        for i, p in enumerate(ps):  # second loop (:78-99)
+            e = self.result[tuple(int(v) for v in p[:3])]
+            val, mp = int(idx[i]), np.float32(prob[i])
+            if not pre[i]:
+                e[0], e[1] = val, mp
+            else:
+                if e[0] == val:
+                    e[1] = np.float32(min(np.float32(self.maximum), np.float32(e[1] + mp)))
+                else:
+                    e[1] = np.float32(e[1] - mp)
+                if e[1] < 0:
+                    e[0], e[1] = val, np.float32(-e[1])
+
+    def multi_query(self, ps):
+        return np.array([self.result.get(tuple(int(v) for v in p[:3]), [-1])[0] for p in np.asarray(ps)], np.int64)
+
+    def finalize(self, points):
+        keep = set(tuple(int(v) for v in p[:3]) for p in np.asarray(points))
+        self.result = {k: v for k, v in self.result.items() if k in keep}
+
+    def all_points_labels(self):
+        return np.array([list(k) + [v[0]] for k, v in self.result.items()], np.int64).reshape(-1, 4)
+
+    def confidences(self):
+        return np.array([v[1] for v in self.result.values()], np.float32)
+
+
+class ResultOfWeightOracle(object):
+    """ResultOfWeight::update / multiQuery / finalize (resultHash.h:158-214)."""
+
+    def __init__(self):
+        self.result = {}
+
+    def update(self, ps, scores):
+        for p, row in zip(np.asarray(ps), np.asarray(scores, np.float32)):
+            k = tuple(int(v) for v in p[:3])
+            self.result[k] = row.copy() if k not in self.result else (self.result[k] * np.float32(0.5) + row)
+
+    def multi_query(self, ps):
+        return np.array([int(np.argmax(self.result[k])) if k in self.result else -1
+                         for k in (tuple(int(v) for v in p[:3]) for p in np.asarray(ps))], np.int64)
+
+    def finalize(self, points):
+        keep = set(tuple(int(v) for v in p[:3]) for p in np.asarray(points))
+        self.result = {k: v for k, v in self.result.items() if k in keep}
+
+    def all_points_labels(self):
+        return np.array([list(k) + [int(np.argmax(v))] for k, v in self.result.items()], np.int64).reshape(-1, 4)
