@@ -302,6 +302,62 @@ int insc_labels_export(insc_labels *l, int32_t *d_out4, float *d_conf, int64_t r
 int insc_labels_finalize(insc_labels *l, const int32_t *d_keep4, int64_t M, void *stream);
 
 /* ---------------------------------------------------------------------------------------
+ * Residual frames: the reference's own incremental operators (Incre_*, pybind.cpp:218-258).
+ * The frame's points form a site set of their own (fresh grids g at every scale); `pre` names
+ * the grids and feature matrices saved by the last full forward.  d_pre_exist[i] = id of the
+ * frame's site i in the saved grid of the same scale or -1 (getPreExistMaps,
+ * Metadata/Metadata.cpp:609-626) - obtain it with insc_grid_query(pre, insc_grid_coords(g), n, ..).
+ * Features of sites that existed are differences to the saved state, features of new sites are
+ * plain values.  Nothing here changes the saved state.
+ * ------------------------------------------------------------------------------------- */
+/* d_nbr_pre[i*27+k] = id, in the saved grid, of the neighbour k of the frame's site i if that
+ * site is new (d_pre_exist[i] < 0), -1 otherwise; the centre offset is always -1.  The rules of
+ * IncreSubmanifoldBuildObject (CUDA/SubmanifoldRules_cuda.cpp:233-472, kernel
+ * SubmanifoldRules_cuda.cu:132-156) as a dense map. */
+int insc_incre_rulebook_ssc3(const insc_grid *g, const insc_grid *pre, const int32_t *d_pre_exist, int64_t n,
+                             int32_t *d_nbr_pre, void *stream);
+/* Input layer of a residual frame (cuda_Incre_InputLayer_updateOutput, CUDA/IOLayers.cpp:290-337;
+ * kernel IOLayers.cu:81-105).  d_sum / d_cnt: this frame's per-site sums and counts
+ * (insc_input_accumulate on the fresh grid); d_pre_out / d_pre_cnt: the saved input-layer output
+ * and point counts.  With na, pn the rule lengths (point counts for modes 3 and 4, 1 for modes 1
+ * and 2) and m = 1/(na+pn) in mode 4, 1 otherwise:
+ *   out = m*sum + pre_out*(pn*m - 1) for a voxel that existed, out = m*sum for a new one. */
+int insc_incre_input(const float *d_sum, const int32_t *d_cnt, int mode, const int32_t *d_pre_exist,
+                     const float *d_pre_out, int64_t ld_pre, const int32_t *d_pre_cnt, float *d_out, int64_t ld_out,
+                     int64_t n, int C, void *stream);
+/* 3^3 submanifold convolution of a residual frame (cuda_Incre_SubmanifoldConvolution_updateOutput,
+ * CUDA/Convolution.cpp:221-303):
+ *   out[i] = bias + sum_k in[nbr[i,k]].W[k] + sum_k pre_in[nbr_pre[i,k]].W[k]
+ * d_nbr is the frame's own map (insc_rulebook_ssc3 on g), d_nbr_pre the map of
+ * insc_incre_rulebook_ssc3; d_in has n rows, d_pre_in n_pre_rows. */
+int insc_incre_conv_ssc(const float *d_in, int64_t ld_in, const float *d_pre_in, int64_t ld_pre, int64_t n_pre_rows,
+                        float *d_out, int64_t ld_out, const float *d_W, const float *d_Wp, const float *d_bias,
+                        const int32_t *d_nbr, const int32_t *d_nbr_pre, int64_t n, int Cin, int Cout, void *stream);
+/* Batch norm + leaky ReLU of a residual frame (cuda_Incre_BatchNormalization_updateOutput,
+ * CUDA/BatchNormalization.cpp:63-91; kernel BatchNormalization.cu:112-150): with o = w*x + b,
+ *   out = leaky(o + w*pre_in[pe]) - pre_out[pe] for a site that existed, leaky(o) for a new one. */
+int insc_incre_bn_leaky(const float *d_in, int64_t ld_in, float *d_out, int64_t ld_out, const float *d_mean,
+                        const float *d_var, const float *d_gamma, const float *d_beta, float eps, float leakiness,
+                        const int32_t *d_pre_exist, const float *d_pre_in, int64_t ld_pre_in, const float *d_pre_out,
+                        int64_t ld_pre_out, int64_t n, int C, void *stream);
+/* Size-2 stride-2 deconvolution of a residual frame (cuda_Incre_Deconvolution_updateOutput,
+ * CUDA/Deconvolution.cpp:61-96; kernel Deconvolution.cu:84-150):
+ *   out[f] = bias + (in[c] + pre_in[pre_exist_in[c]] * [c existed and f is new]) . W[offset[f]],
+ * c = parent[f].  (The size-2 stride-2 convolution of a residual frame is insc_conv_nbr on the
+ * frame's own child map, Incre_Convolution_updateOutput, CUDA/Convolution.cpp:83-113.) */
+int insc_incre_deconv_down2(const float *d_in, int64_t ld_in, int64_t n_in_rows, const float *d_pre_in, int64_t ld_pre,
+                            int64_t n_pre_rows, float *d_out, int64_t ld_out, const float *d_W, const float *d_Wp,
+                            const float *d_bias, const int32_t *d_parent, const int32_t *d_offset,
+                            const int32_t *d_pre_exist_in, const int32_t *d_pre_exist_out, int64_t n_rows, int Cin,
+                            int Cout, void *stream);
+/* Output layer of a residual frame (cuda_Incre_OutputLayer_updateOutput, CUDA/IOLayers.cpp:339-368;
+ * kernel IOLayers.cu:122-141): out[p] = in[s] + pre_in[pre_exist[s]] (second term for sites that
+ * existed), s = site_of_point[p]. */
+int insc_incre_output(const float *d_in, int64_t ld_in, const float *d_pre_in, int64_t ld_pre,
+                      const int32_t *d_pre_exist, const int32_t *d_site_of_point, int64_t P, int C, float *d_out,
+                      void *stream);
+
+/* ---------------------------------------------------------------------------------------
  * Device utilities exported for tests and callers.
  * ------------------------------------------------------------------------------------- */
 /* Exclusive prefix sum of n int32 values; d_total (nullable) receives the sum. */

@@ -105,6 +105,19 @@ static inline unsigned grid_for(int64_t n, int block, int64_t cap = 1 << 20) {
   return (unsigned)g;
 }
 
+// ---- device helpers shared by the streaming kernels ------------------------------------
+__device__ __forceinline__ float leaky(float o, float leak) { return o * ((o > 0.0f) ? 1.0f : leak); }
+
+// per-channel scale / shift of inference batch norm; every kernel that normalises goes through
+// this one function so that fused and unfused paths give the same bits
+__device__ __forceinline__ void bn_coeffs(const float *__restrict__ mean, const float *__restrict__ var,
+                                          const float *__restrict__ gamma, const float *__restrict__ beta, float eps,
+                                          int c, float &w, float &b) {
+  const float invstd = 1.0f / sqrtf(var[c] + eps);
+  w = invstd * (gamma ? gamma[c] : 1.0f);
+  b = fmaf(-mean[c], w, beta ? beta[c] : 0.0f);
+}
+
 // ---- key packing ------------------------------------------------------------------------
 // 64-bit voxel key: batch:16 | z:16 | y:16 | x:16.  Ascending key order is (batch, z, y, x).
 #define INSC_EMPTY_KEY 0xFFFFFFFFFFFFFFFFull

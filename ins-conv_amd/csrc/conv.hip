@@ -827,10 +827,15 @@ int launch_conv(const float *in, int64_t ld_in, int64_t in_rows, float *out, int
       Wp = (const float *)ws;
     }
     const int64_t tiles = cdiv(n_rows, TILE_M);
-    const int64_t map_bytes64 = in_rows * 27 * 4;  // the neighbour map has a row per input site
-    // (row ids and row strides go through 24-bit multiplies; outputs have a row per input site)
-    const bool small_ids = in_rows < (1 << 24) && ld_out * 4 < (1 << 24) && ep.ld2 * 4 < (1 << 24) &&
-                           in_rows * ld_out * 4 < (int64_t)BUF_OOB && in_rows * ep.ld2 * 4 < (int64_t)BUF_OOB;
+    // Rows of the neighbour map and of the outputs: one per listed row, or - with a row list,
+    // which only 3^3 layers over one site set use - one per input site.  (The two differ when a
+    // layer gathers from another site set than the one it writes.)
+    const int64_t out_rows = rows ? in_rows : std::max(in_rows, n_rows);
+    const int64_t map_bytes64 = out_rows * 27 * 4;
+    // (row ids and row strides go through 24-bit multiplies)
+    const bool small_ids = in_rows < (1 << 24) && out_rows < (1 << 24) && ld_out * 4 < (1 << 24) &&
+                           ep.ld2 * 4 < (1 << 24) && out_rows * ld_out * 4 < (int64_t)BUF_OOB &&
+                           out_rows * ep.ld2 * 4 < (int64_t)BUF_OOB;
     if (mode == MAP_NBR && K == 27 && Cin <= 32 && Cout <= 32 && map_bytes64 < (int64_t)BUF_OOB && small_ids) {
       const uint32_t map_bytes = (uint32_t)map_bytes64;
       // persistent blocks, a multiple of the XCD count, at most one per compute unit

@@ -244,6 +244,24 @@ __global__ void ssc3_nbr_kernel(const Slot *__restrict__ table, int64_t mask, co
   if (patch_reverse && r >= 0 && r < first) nbr[(int64_t)r * 27 + (26 - k)] = (int)o;
 }
 
+// Neighbours, in another (saved) grid, of the sites that the saved grid does not hold; see
+// insc_incre_rulebook_ssc3
+__global__ void incre_ssc3_nbr_kernel(const Slot *__restrict__ pre_table, int64_t pre_mask,
+                                      const int32_t *__restrict__ site_coords,
+                                      const int32_t *__restrict__ pre_exist, int64_t n, int32_t *__restrict__ nbr) {
+  int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= n * 27) return;
+  int64_t o = t / 27;
+  int k = (int)(t % 27);
+  int r = -1;
+  if (pre_exist[o] < 0 && k != 13) {
+    int4 c = reinterpret_cast<const int4 *>(site_coords)[o];
+    int x = c.x + k / 9 - 1, y = c.y + (k / 3) % 3 - 1, z = c.z + k % 3 - 1;
+    if (coord_ok(x, y, z, c.w)) r = grid_find(pre_table, pre_mask, pack_key(x, y, z, c.w));
+  }
+  nbr[t] = r;
+}
+
 __global__ void down2_coords_kernel(const int32_t *__restrict__ fine_coords, int64_t first, int64_t n,
                                     int32_t *__restrict__ half, int32_t *__restrict__ offset) {
   int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -679,6 +697,18 @@ int insc_rulebook_ssc3(const insc_grid *g, int64_t first, int64_t n, int32_t *d_
   if (n == 0) return INSC_OK;
   hipLaunchKernelGGL(ssc3_nbr_kernel, dim3(grid_for(n * 27, 256, 1ll << 30)), dim3(256), 0, (hipStream_t)stream,
                      g->table, g->n_slots - 1, g->coords, first, n, d_nbr, patch_reverse);
+  INSC_LAUNCH_CHECK();
+  return INSC_OK;
+}
+
+int insc_incre_rulebook_ssc3(const insc_grid *g, const insc_grid *pre, const int32_t *d_pre_exist, int64_t n,
+                             int32_t *d_nbr_pre, void *stream) {
+  INSC_REQUIRE(g && pre && g != pre, INSC_ERR_ARG, "insc_incre_rulebook_ssc3: needs two different grids");
+  INSC_REQUIRE(n >= 0 && n <= g->capacity_sites, INSC_ERR_ARG, "insc_incre_rulebook_ssc3: n outside capacity");
+  INSC_REQUIRE(n == 0 || (d_pre_exist && d_nbr_pre), INSC_ERR_ARG, "insc_incre_rulebook_ssc3: null pointer");
+  if (n == 0) return INSC_OK;
+  hipLaunchKernelGGL(incre_ssc3_nbr_kernel, dim3(grid_for(n * 27, 256, 1ll << 30)), dim3(256), 0, (hipStream_t)stream,
+                     pre->table, pre->n_slots - 1, g->coords, d_pre_exist, n, d_nbr_pre);
   INSC_LAUNCH_CHECK();
   return INSC_OK;
 }

@@ -1,0 +1,200 @@
+// Residual frames: the reference's own incremental mode (its Incre_* operators).
+//
+// A frame's points get a site set of their own (a fresh grid at every scale); the features that
+// travel through the network are differences to the state saved by the last full forward for
+// sites that existed then, and plain values for sites that did not.  pre_exist[i] is the id the
+// frame's site i has in the saved site set of the same scale, or -1.  Every operator here is
+// exact for the rows it produces; the mode as a whole is an approximation because a 3^3
+// convolution leaves the rows around the frame's sites untouched.
+//
+// All kernels are streaming (one thread per channel group of a row); the two convolutions are
+// the ordinary kernels run twice, the second pass gathering the saved features.
+#include "common.h"
+#include "grid.h"
+
+namespace insc {
+
+// Input layer (InputLayer_inc_fp_, CUDA/IOLayers.cu:81-105): with n rows of this frame and pn
+// saved rows at a voxel, m = 1/(n+pn) for the mean (1 otherwise),
+//   out = m * sum_new + pre * (pn*m - 1)      for a voxel that existed,    out = m * sum_new  else.
+// n and pn are the lengths of the rule rows: 1 for modes 1 and 2, the number of points for 3, 4.
+__global__ __launch_bounds__(256) void incre_input_kernel(const float *__restrict__ sum,
+                                                          const int32_t *__restrict__ cnt, int mode,
+                                                          const int32_t *__restrict__ pre_exist,
+                                                          const float *__restrict__ pre_out, int64_t ld_pre,
+                                                          const int32_t *__restrict__ pre_cnt,
+                                                          float *__restrict__ out, int64_t ld_out, int64_t n, int C) {
+  for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < n * C; e += (int64_t)gridDim.x * 256) {
+    const int64_t row = e / C;
+    const int c = (int)(e - row * C);
+    const int pe = pre_exist[row];
+    const int na = mode >= 3 ? cnt[row] : 1;
+    const int pn = pe >= 0 ? (mode >= 3 ? pre_cnt[pe] : 1) : 0;
+    const float m = (mode == 4 && na > 0) ? 1.0f / (float)(na + pn) : 1.0f;
+    float v = m * sum[row * C + c];
+    if (pe >= 0) v = v + pre_out[(int64_t)pe * ld_pre + c] * ((float)pn * m - 1.0f);
+    out[row * ld_out + c] = v;
+  }
+}
+
+// Batch norm + leaky ReLU (Incre_BatchNormalization_f_test, CUDA/BatchNormalization.cu:112-150):
+//   o = w*x + b;  existing site: leaky(o + w*pre_in) - pre_out;  new site: leaky(o)
+__global__ __launch_bounds__(256) void incre_bn_kernel(const float *__restrict__ in, int64_t ld_in,
+                                                       float *__restrict__ out, int64_t ld_out,
+                                                       const float *__restrict__ mean, const float *__restrict__ var,
+                                                       const float *__restrict__ gamma, const float *__restrict__ beta,
+                                                       float eps, float leak, const int32_t *__restrict__ pre_exist,
+                                                       const float *__restrict__ pre_in, int64_t ld_pin,
+                                                       const float *__restrict__ pre_out, int64_t ld_pout, int64_t n,
+                                                       int C) {
+  for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < n * C; e += (int64_t)gridDim.x * 256) {
+    const int64_t row = e / C;
+    const int c = (int)(e - row * C);
+    float w, b;
+    bn_coeffs(mean, var, gamma, beta, eps, c, w, b);
+    const float o = fmaf(in[row * ld_in + c], w, b);
+    const int pe = pre_exist[row];
+    float y;
+    if (pe >= 0)
+      y = leaky(fmaf(pre_in[(int64_t)pe * ld_pin + c], w, o), leak) - pre_out[(int64_t)pe * ld_pout + c];
+    else
+      y = leaky(o, leak);
+    out[row * ld_out + c] = y;
+  }
+}
+
+// Deconvolution: which saved coarse row a fine site also reads (dDeconvolution_incre_KMxKN_forwardA,
+// CUDA/Deconvolution.cu:84-150: the saved input joins in when the coarse site existed and the
+// fine site did not).
+__global__ void incre_parent_kernel(const int32_t *__restrict__ parent, const int32_t *__restrict__ pre_exist_in,
+                                    const int32_t *__restrict__ pre_exist_out, int64_t n_fine, int64_t n_coarse,
+                                    int32_t *__restrict__ parent2) {
+  const int64_t f = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (f >= n_fine) return;
+  const int p = parent[f];
+  int r = -1;
+  if (p >= 0 && p < n_coarse && pre_exist_out[f] < 0) r = pre_exist_in[p];
+  parent2[f] = r;
+}
+
+// Output layer (InputLayer_inc_bp_, CUDA/IOLayers.cu:122-141): residual + saved value.
+__global__ __launch_bounds__(256) void incre_output_kernel(const float *__restrict__ in, int64_t ld_in,
+                                                           const float *__restrict__ pre_in, int64_t ld_pre,
+                                                           const int32_t *__restrict__ pre_exist,
+                                                           const int32_t *__restrict__ sop, int64_t P, int C,
+                                                           float *__restrict__ out) {
+  for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < P * C; e += (int64_t)gridDim.x * 256) {
+    const int64_t p = e / C;
+    const int c = (int)(e - p * C);
+    const int s = sop[p];
+    float v = 0.0f;
+    if (s >= 0) {
+      v = in[(int64_t)s * ld_in + c];
+      const int pe = pre_exist[s];
+      if (pe >= 0) v += pre_in[(int64_t)pe * ld_pre + c];
+    }
+    out[e] = v;
+  }
+}
+
+}  // namespace insc
+
+using namespace insc;
+
+extern "C" {
+
+int insc_incre_input(const float *d_sum, const int32_t *d_cnt, int mode, const int32_t *d_pre_exist,
+                     const float *d_pre_out, int64_t ld_pre, const int32_t *d_pre_cnt, float *d_out, int64_t ld_out,
+                     int64_t n, int C, void *stream) {
+  INSC_REQUIRE(n >= 0 && C > 0 && mode >= 0 && mode <= 4 && ld_out >= C && ld_pre >= C, INSC_ERR_ARG,
+               "insc_incre_input: bad arguments");
+  if (n == 0) return INSC_OK;
+  INSC_REQUIRE(d_sum && d_cnt && d_pre_exist && d_pre_out && d_pre_cnt && d_out, INSC_ERR_ARG,
+               "insc_incre_input: null pointer");
+  hipLaunchKernelGGL(incre_input_kernel, dim3(grid_for(n * C, 256, 1 << 16)), dim3(256), 0, (hipStream_t)stream, d_sum,
+                     d_cnt, mode, d_pre_exist, d_pre_out, ld_pre, d_pre_cnt, d_out, ld_out, n, C);
+  INSC_LAUNCH_CHECK();
+  return INSC_OK;
+}
+
+int insc_incre_conv_ssc(const float *d_in, int64_t ld_in, const float *d_pre_in, int64_t ld_pre, int64_t n_pre_rows,
+                        float *d_out, int64_t ld_out, const float *d_W, const float *d_Wp, const float *d_bias,
+                        const int32_t *d_nbr, const int32_t *d_nbr_pre, int64_t n, int Cin, int Cout, void *stream) {
+  INSC_REQUIRE(n >= 0 && n_pre_rows >= 0 && Cin > 0 && Cout > 0 && ld_in >= Cin && ld_pre >= Cin && ld_out >= Cout,
+               INSC_ERR_ARG, "insc_incre_conv_ssc: bad sizes");
+  if (n == 0) return INSC_OK;
+  INSC_REQUIRE(d_in && d_out && (d_W || d_Wp) && d_nbr && d_nbr_pre && (d_pre_in || n_pre_rows == 0), INSC_ERR_ARG,
+               "insc_incre_conv_ssc: null pointer");
+  hipStream_t s = (hipStream_t)stream;
+  // rules inside the frame's site set, on the residual features (CUDA/Convolution.cpp:264-268,283)
+  int rc = launch_conv(d_in, ld_in, n, d_out, ld_out, d_W, d_Wp, d_bias, d_nbr, nullptr, MAP_NBR, 27, nullptr, nullptr,
+                       n, Cin, Cout, nullptr, nullptr, s);
+  if (rc || n_pre_rows == 0) return rc;
+  // new sites gather the saved features of their neighbours in the saved set (:274,287)
+  BnEpilogue ep;
+  ep.res = d_out;
+  ep.ldr = ld_out;
+  return launch_conv(d_pre_in, ld_pre, n_pre_rows, d_out, ld_out, d_W, d_Wp, nullptr, d_nbr_pre, nullptr, MAP_NBR, 27,
+                     nullptr, nullptr, n, Cin, Cout, nullptr, nullptr, s, ep);
+}
+
+int insc_incre_bn_leaky(const float *d_in, int64_t ld_in, float *d_out, int64_t ld_out, const float *d_mean,
+                        const float *d_var, const float *d_gamma, const float *d_beta, float eps, float leakiness,
+                        const int32_t *d_pre_exist, const float *d_pre_in, int64_t ld_pre_in, const float *d_pre_out,
+                        int64_t ld_pre_out, int64_t n, int C, void *stream) {
+  INSC_REQUIRE(n >= 0 && C > 0 && ld_in >= C && ld_out >= C && ld_pre_in >= C && ld_pre_out >= C, INSC_ERR_ARG,
+               "insc_incre_bn_leaky: bad sizes");
+  if (n == 0) return INSC_OK;
+  INSC_REQUIRE(d_in && d_out && d_mean && d_var && d_pre_exist && d_pre_in && d_pre_out, INSC_ERR_ARG,
+               "insc_incre_bn_leaky: null pointer");
+  hipLaunchKernelGGL(incre_bn_kernel, dim3(grid_for(n * C, 256, 1 << 16)), dim3(256), 0, (hipStream_t)stream, d_in,
+                     ld_in, d_out, ld_out, d_mean, d_var, d_gamma, d_beta, eps, leakiness, d_pre_exist, d_pre_in,
+                     ld_pre_in, d_pre_out, ld_pre_out, n, C);
+  INSC_LAUNCH_CHECK();
+  return INSC_OK;
+}
+
+int insc_incre_deconv_down2(const float *d_in, int64_t ld_in, int64_t n_in_rows, const float *d_pre_in, int64_t ld_pre,
+                            int64_t n_pre_rows, float *d_out, int64_t ld_out, const float *d_W, const float *d_Wp,
+                            const float *d_bias, const int32_t *d_parent, const int32_t *d_offset,
+                            const int32_t *d_pre_exist_in, const int32_t *d_pre_exist_out, int64_t n_rows, int Cin,
+                            int Cout, void *stream) {
+  INSC_REQUIRE(n_rows >= 0 && n_in_rows >= 0 && n_pre_rows >= 0 && Cin > 0 && Cout > 0 && ld_in >= Cin &&
+                   ld_pre >= Cin && ld_out >= Cout,
+               INSC_ERR_ARG, "insc_incre_deconv_down2: bad sizes");
+  if (n_rows == 0) return INSC_OK;
+  INSC_REQUIRE(d_in && d_out && (d_W || d_Wp) && d_parent && d_offset && d_pre_exist_in && d_pre_exist_out &&
+                   (d_pre_in || n_pre_rows == 0),
+               INSC_ERR_ARG, "insc_incre_deconv_down2: null pointer");
+  hipStream_t s = (hipStream_t)stream;
+  int rc = launch_conv(d_in, ld_in, n_in_rows, d_out, ld_out, d_W, d_Wp, d_bias, d_parent, d_offset, MAP_PARENT, 8,
+                       nullptr, nullptr, n_rows, Cin, Cout, nullptr, nullptr, s);
+  if (rc || n_pre_rows == 0) return rc;
+  void *ws;
+  rc = workspace(WS_API, s, sizeof(int32_t) * (size_t)n_rows, &ws);
+  if (rc) return rc;
+  int32_t *parent2 = (int32_t *)ws;
+  hipLaunchKernelGGL(incre_parent_kernel, dim3(grid_for(n_rows, 256)), dim3(256), 0, s, d_parent, d_pre_exist_in,
+                     d_pre_exist_out, n_rows, n_in_rows, parent2);
+  INSC_LAUNCH_CHECK();
+  BnEpilogue ep;
+  ep.res = d_out;
+  ep.ldr = ld_out;
+  return launch_conv(d_pre_in, ld_pre, n_pre_rows, d_out, ld_out, d_W, d_Wp, nullptr, parent2, d_offset, MAP_PARENT, 8,
+                     nullptr, nullptr, n_rows, Cin, Cout, nullptr, nullptr, s, ep);
+}
+
+int insc_incre_output(const float *d_in, int64_t ld_in, const float *d_pre_in, int64_t ld_pre,
+                      const int32_t *d_pre_exist, const int32_t *d_site_of_point, int64_t P, int C, float *d_out,
+                      void *stream) {
+  INSC_REQUIRE(P >= 0 && C > 0 && ld_in >= C && ld_pre >= C, INSC_ERR_ARG, "insc_incre_output: bad sizes");
+  if (P == 0) return INSC_OK;
+  INSC_REQUIRE(d_in && d_pre_in && d_pre_exist && d_site_of_point && d_out, INSC_ERR_ARG,
+               "insc_incre_output: null pointer");
+  hipLaunchKernelGGL(incre_output_kernel, dim3(grid_for(P * C, 256, 1 << 16)), dim3(256), 0, (hipStream_t)stream, d_in,
+                     ld_in, d_pre_in, ld_pre, d_pre_exist, d_site_of_point, P, C, d_out);
+  INSC_LAUNCH_CHECK();
+  return INSC_OK;
+}
+
+}  // extern "C"

@@ -26,18 +26,6 @@ struct Vec<1> {
   static __device__ __forceinline__ void st(float *p, T v) { *p = v; }
 };
 
-__device__ __forceinline__ float leaky(float o, float leak) { return o * ((o > 0.0f) ? 1.0f : leak); }
-
-// per-channel scale / shift of inference batch norm; every kernel that normalises goes through
-// this one function so that fused and unfused paths give the same bits
-__device__ __forceinline__ void bn_coeffs(const float *__restrict__ mean, const float *__restrict__ var,
-                                          const float *__restrict__ gamma, const float *__restrict__ beta, float eps,
-                                          int c, float &w, float &b) {
-  const float invstd = 1.0f / sqrtf(var[c] + eps);
-  w = invstd * (gamma ? gamma[c] : 1.0f);
-  b = fmaf(-mean[c], w, beta ? beta[c] : 0.0f);
-}
-
 template <int V>
 __global__ __launch_bounds__(256) void bn_kernel(const float *__restrict__ in, int64_t ld_in, float *__restrict__ out,
                                                  int64_t ld_out, const float *__restrict__ mean,

@@ -159,6 +159,8 @@ class Metadata_3(object):
         self.in_sum = None
         self.in_cnt = None
         self.n_points = 0
+        self._pre_exist = {}  # residual frames: per spatial size, this frame's site -> saved site
+        self._nbr_pre = {}
 
     def __del__(self):
         try:
@@ -275,6 +277,39 @@ class Metadata_3(object):
             lib.insc_order_by_offset(ptr(order), ptr(d.offset.t), I64(fine.n), ptr(buf), stream_ptr())
             d.by_offset_n = fine.n
         return d.by_offset.t
+
+    def pre_exist_map(self, spatial_size, pre_m):
+        """int32 [n]: id of each of this site set's sites in `pre_m`'s site set of the same
+        spatial size, or -1 (getPreExistMaps, Metadata/Metadata.cpp:609-626)."""
+        k = _key(spatial_size)
+        hit = self._pre_exist.get(k)
+        sc = self.scale(k)
+        if hit is None or hit[0] is not pre_m or hit[1].numel() != sc.n:
+            pe = torch.empty(max(sc.n, 1), dtype=torch.int32, device=self.device)[:sc.n]
+            pre_sc = pre_m.scales.get(k)
+            if pre_sc is None or pre_sc.n == 0:
+                pe.fill_(-1)
+            elif sc.n:
+                lib.insc_grid_query(pre_sc.grid, lib.insc_grid_coords(sc.grid), I64(sc.n), ptr(pe), stream_ptr())
+            hit = self._pre_exist[k] = (pre_m, pe)
+        return hit[1]
+
+    def incre_ssc_map(self, spatial_size, pre_m):
+        """int32 [n,27] neighbours, in `pre_m`'s site set, of the sites that are new to it
+        (insc_incre_rulebook_ssc3)."""
+        k = _key(spatial_size)
+        hit = self._nbr_pre.get(k)
+        sc = self.scale(k)
+        if hit is None or hit[0] is not pre_m or hit[1].size(0) != sc.n:
+            nbr = torch.empty((max(sc.n, 1), 27), dtype=torch.int32, device=self.device)[:sc.n]
+            pre_sc = pre_m.scales.get(k)
+            if pre_sc is None or pre_sc.n == 0:
+                nbr.fill_(-1)
+            elif sc.n:
+                lib.insc_incre_rulebook_ssc3(sc.grid, pre_sc.grid, ptr(self.pre_exist_map(k, pre_m)), I64(sc.n),
+                                             ptr(nbr), stream_ptr())
+            hit = self._nbr_pre[k] = (pre_m, nbr)
+        return hit[1]
 
     def ssc_rulebook_for(self, sc):
         for k, v in self.scales.items():
@@ -506,6 +541,150 @@ def NetworkInNetwork_updateOutput(input_features, output_features, weight, bias)
         ensure_init(input_features.device.index)
         conv_rows(input_features, output_features, w, b, None, 1, None, None, n)
     return float(n) * w.size(0) * w.size(1)
+
+
+# =========================================================================================
+# residual frames: the reference's Incre_* operators (pybind.cpp:218-258).  `m` holds only the
+# frame's own points; `pre_m` and the pre_* feature matrices are the state saved by the last
+# full forward and are not modified.
+# =========================================================================================
+def _pre_rows(pre_m, size):
+    sc = pre_m.scales.get(_key(size))
+    return 0 if sc is None else sc.n
+
+
+def Incre_InputLayer_updateOutput(m, spatialSize, input_coords, input_features, output_features, batchSize, mode,
+                                  pre_m, pre_output_feats):
+    """cuda_Incre_InputLayer_updateOutput (CUDA/IOLayers.cpp:290-337)."""
+    input_features = _check_feats(input_features, "input_features")
+    if m is pre_m:
+        raise ValueError("a residual frame needs a Metadata of its own")
+    if pre_m.mode is not None and int(mode) != pre_m.mode:
+        raise ValueError("input mode differs from the saved frame's")
+    m.clear()
+    m._bind(input_features.device)
+    m.setInputSpatialSize(spatialSize)
+    m.mode = int(mode)
+    P, C = input_features.shape
+    if input_coords.size(0) != P:
+        raise ValueError("coords and features disagree on the number of rows")
+    sc = m.scale(spatialSize, create_capacity=max(int(1.25 * P), 4096))
+    _append_points(m, sc, input_coords, input_features)
+    _resize(output_features, sc.n, C, input_features)
+    if sc.n == 0:
+        return
+    if m.mode == 0:  # the reference hands the rows through unchanged in mode 0 (:320-322)
+        lib.insc_input_finish(ptr(m.in_sum.t), ptr(m.in_cnt.t), 0, ptr(output_features), I64(C), None, None,
+                              I64(sc.n), int(C), stream_ptr())
+        return
+    pre = _check_feats(pre_output_feats, "pre_output_feats")
+    if pre.size(1) != C or pre.size(0) < _pre_rows(pre_m, spatialSize):
+        raise ValueError("saved input-layer output does not match the saved site set")
+    pe = m.pre_exist_map(spatialSize, pre_m)
+    lib.insc_incre_input(ptr(m.in_sum.t), ptr(m.in_cnt.t), int(m.mode), ptr(pe), ptr(pre), I64(_ld(pre)),
+                         ptr(pre_m.in_cnt.t), ptr(output_features), I64(C), I64(sc.n), int(C), stream_ptr())
+
+
+def Incre_OutputLayer_updateOutput(m, input_features, output_features, pre_m, pre_input_feats):
+    """cuda_Incre_OutputLayer_updateOutput (CUDA/IOLayers.cpp:339-368): one row per point of the frame."""
+    input_features = _check_feats(input_features, "input_features")
+    pre = _check_feats(pre_input_feats, "pre_input_feats")
+    sop = m.site_of_point
+    P, C = sop.numel(), input_features.size(1)
+    if pre.size(1) != C or pre.size(0) < _pre_rows(pre_m, m.input_size):
+        raise ValueError("saved features do not match the saved site set")
+    _resize(output_features, P, C, input_features)
+    if P:
+        pe = m.pre_exist_map(m.input_size, pre_m)
+        lib.insc_incre_output(ptr(input_features), I64(_ld(input_features)), ptr(pre), I64(_ld(pre)), ptr(pe),
+                              ptr(sop), I64(P), int(C), ptr(output_features), stream_ptr())
+
+
+def Incre_SubmanifoldConvolution_updateOutput(inputSize, filterSize, m, input_features, output_features, weight, bias,
+                                              pre_m, pre_input_feats, count_muladds=True):
+    """cuda_Incre_SubmanifoldConvolution_updateOutput (CUDA/Convolution.cpp:221-303); returns the
+    multiply-adds of both rulebooks (count_muladds=False skips the count and its host round trip)."""
+    if _key(filterSize) != (3, 3, 3):
+        raise NotImplementedError("only 3x3x3 submanifold convolutions are provided")
+    input_features = _check_feats(input_features, "input_features")
+    pre = _check_feats(pre_input_feats, "pre_input_feats")
+    sc = m.ssc_rulebook(inputSize)
+    w, b = (weight if weight.is_contiguous() else weight.contiguous()), _opt(bias)
+    if input_features.size(0) != sc.n or input_features.size(1) != w.size(1) or w.size(0) != 27:
+        raise ValueError("feature / weight shapes do not match the active sites")
+    n_pre = _pre_rows(pre_m, inputSize)
+    if pre.size(1) != w.size(1) or pre.size(0) < n_pre:
+        raise ValueError("saved features do not match the saved site set")
+    _resize(output_features, sc.n, w.size(2), input_features)
+    if sc.n == 0:
+        return 0.0
+    nbr_pre = m.incre_ssc_map(inputSize, pre_m)
+    Cin, Cout = w.size(1), w.size(2)
+    lib.insc_incre_conv_ssc(ptr(input_features), I64(_ld(input_features)), ptr(pre), I64(_ld(pre)), I64(n_pre),
+                            ptr(output_features), I64(_ld(output_features)), ptr(w), ptr(packed_weight(w, 27)),
+                            ptr(b), ptr(sc.nbr.t), ptr(nbr_pre), I64(sc.n), int(Cin), int(Cout), stream_ptr())
+    if not count_muladds:
+        return 0.0
+    return float(m.n_ssc_rules(sc) + int((nbr_pre >= 0).sum().item())) * Cin * Cout
+
+
+def Incre_Convolution_updateOutput(inputSize, outputSize, filterSize, filterStride, m, input_features,
+                                   output_features, weight, bias):
+    """cuda_Incre_Convolution_updateOutput (CUDA/Convolution.cpp:83-113): the plain strided
+    convolution on the frame's own rulebook (linear, so exact on differences)."""
+    return Convolution_updateOutput(inputSize, outputSize, filterSize, filterStride, m, input_features,
+                                    output_features, weight, bias)
+
+
+def Incre_Deconvolution_updateOutput(inputSize, outputSize, filterSize, filterStride, m, input_features,
+                                     output_features, weight, bias, pre_m, pre_input_feats):
+    """cuda_Incre_Deconvolution_updateOutput (CUDA/Deconvolution.cpp:61-96): input is the coarse scale."""
+    _check_down(filterSize, filterStride)
+    input_features = _check_feats(input_features, "input_features")
+    pre = _check_feats(pre_input_feats, "pre_input_feats")
+    fine, coarse, d = m.down_rulebook(outputSize, inputSize)
+    w, b = (weight if weight.is_contiguous() else weight.contiguous()), _opt(bias)
+    if input_features.size(0) != coarse.n or input_features.size(1) != w.size(1) or w.size(0) != 8:
+        raise ValueError("feature / weight shapes do not match the active sites")
+    n_pre = _pre_rows(pre_m, inputSize)
+    if pre.size(1) != w.size(1) or pre.size(0) < n_pre:
+        raise ValueError("saved features do not match the saved site set")
+    _resize(output_features, fine.n, w.size(2), input_features)
+    if fine.n == 0:
+        return 0.0
+    pe_in = m.pre_exist_map(inputSize, pre_m)
+    pe_out = m.pre_exist_map(outputSize, pre_m)
+    lib.insc_incre_deconv_down2(ptr(input_features), I64(_ld(input_features)), I64(coarse.n), ptr(pre), I64(_ld(pre)),
+                                I64(n_pre), ptr(output_features), I64(_ld(output_features)), ptr(w),
+                                ptr(packed_weight(w, 8)), ptr(b), ptr(d.parent.t), ptr(d.offset.t), ptr(pe_in),
+                                ptr(pe_out), I64(fine.n), int(w.size(1)), int(w.size(2)), stream_ptr())
+    return float(fine.n) * w.size(1) * w.size(2)
+
+
+def Incre_BatchNormalization_updateOutput(input_features, output_features, saveMean, saveInvStd, runningMean,
+                                          runningVar, weight, bias, eps, momentum, train, leakiness, m, pre_m,
+                                          pre_output_feats, pre_input_feats, inputSize):
+    """cuda_Incre_BatchNormalization_updateOutput (CUDA/BatchNormalization.cpp:63-91), inference only."""
+    if train:
+        raise NotImplementedError("training-mode batch norm is outside the inference path")
+    input_features = _check_feats(input_features, "input_features")
+    pre_in = _check_feats(pre_input_feats, "pre_input_feats")
+    pre_out = _check_feats(pre_output_feats, "pre_output_feats")
+    n, C = input_features.shape
+    n_pre = _pre_rows(pre_m, inputSize)
+    if pre_in.size(1) != C or pre_out.size(1) != C or pre_in.size(0) < n_pre or pre_out.size(0) < n_pre:
+        raise ValueError("saved features do not match the saved site set")
+    if n != m.getNActive(inputSize):
+        raise ValueError("features do not match the active sites")
+    _resize(output_features, n, C, input_features)
+    if n:
+        pe = m.pre_exist_map(inputSize, pre_m)
+        mean, var, g, b = runningMean.detach(), runningVar.detach(), _opt(weight), _opt(bias)
+        lib.insc_incre_bn_leaky(ptr(input_features), I64(_ld(input_features)), ptr(output_features),
+                                I64(_ld(output_features)), ptr(mean), ptr(var), ptr(g), ptr(b),
+                                ctypes.c_float(eps), ctypes.c_float(leakiness),
+                                ptr(pe), ptr(pre_in), I64(_ld(pre_in)), ptr(pre_out), I64(_ld(pre_out)), I64(n),
+                                int(C), stream_ptr())
 
 
 def n_rulebook_bits():

@@ -22,3 +22,4 @@ from .networkArchitectures import UNet  # noqa: E402
 from .utils import (toLongTensor, optionalTensor, checkpoint_save, checkpoint_restore,  # noqa: E402
                     ssc_offset_permutation, convert_zmajor_state_dict)
 from .compiled import compile, CompiledNet  # noqa: E402
+from .incremental import set_mode as set_incremental_mode, get_mode as get_incremental_mode  # noqa: E402

@@ -71,6 +71,14 @@ _SIGS = {
     "insc_labels_count": [vp, ctypes.POINTER(c_i64), vp],
     "insc_labels_export": [vp, vp, vp, c_i64, vp],
     "insc_labels_finalize": [vp, vp, c_i64, vp],
+    "insc_incre_rulebook_ssc3": [vp, vp, vp, c_i64, vp, vp],
+    "insc_incre_input": [vp, vp, c_int, vp, vp, c_i64, vp, vp, c_i64, c_i64, c_int, vp],
+    "insc_incre_conv_ssc": [vp, c_i64, vp, c_i64, c_i64, vp, c_i64, vp, vp, vp, vp, vp, c_i64, c_int, c_int, vp],
+    "insc_incre_bn_leaky": [vp, c_i64, vp, c_i64, vp, vp, vp, vp, c_f32, c_f32, vp, vp, c_i64, vp, c_i64, c_i64,
+                            c_int, vp],
+    "insc_incre_deconv_down2": [vp, c_i64, c_i64, vp, c_i64, c_i64, vp, c_i64, vp, vp, vp, vp, vp, vp, vp, c_i64,
+                                c_int, c_int, vp],
+    "insc_incre_output": [vp, c_i64, vp, c_i64, vp, vp, c_i64, c_int, vp, vp],
     "insc_scan_exclusive_i32": [vp, vp, c_i64, vp, vp],
     "insc_sort_pairs_u64": [vp, vp, c_i64, c_int, vp],
 }

@@ -2,7 +2,7 @@
 import torch
 from torch.nn import Module, Parameter
 
-from . import SCN
+from . import SCN, incremental
 from .sparseConvNetTensor import SparseConvNetTensor
 from .utils import StateBuf, optionalTensor
 
@@ -34,7 +34,17 @@ class BatchNormalization(Module):
         if self.training:
             raise NotImplementedError("training-mode batch norm is outside the inference path; call .eval()")
         output = SparseConvNetTensor(None, input.metadata, input.spatial_size)
-        if not increment:
+        kind = incremental.kind(increment)
+        if kind == "residual":
+            out = input.features.new_empty((0, self.nPlanes))
+            SCN.Incre_BatchNormalization_updateOutput(
+                input.features, out, None, None, self.running_mean, self.running_var,
+                optionalTensor(self, 'weight'), optionalTensor(self, 'bias'), self.eps, self.momentum, False,
+                self.leakiness, output.metadata, self.save_output.metadata, self.save_output.features,
+                self.save_input.features, input.spatial_size)
+            output.features = out
+            return output
+        if kind is None:
             out = input.features.new_empty((0, self.nPlanes))
             SCN.BatchNormalization_updateOutput(
                 input.features, out, None, None, self.running_mean, self.running_var,
@@ -51,6 +61,8 @@ class BatchNormalization(Module):
                         float(self.eps), float(self.leakiness), rows, count, d.n_upper)
             output.features = out
             output.dirty = d
+        self.save_output = output
+        self.save_input = input
         return output
 
     def input_spatial_size(self, out_size):

@@ -127,6 +127,11 @@ class CompiledNet(object):
 
     def __call__(self, input, increment=False, all_points=None):
         coords, feats = input[0], input[1]
+        from . import incremental
+        if incremental.kind(increment) == "residual":
+            raise NotImplementedError("the compiled executor runs full and exact incremental frames; "
+                                      "residual frames go through the module tree")
+        increment = bool(increment)
         if all_points is None:
             all_points = (not increment) or self.output_layer.all_points
         c = coords.to(device=self.device, dtype=torch.int32).contiguous()

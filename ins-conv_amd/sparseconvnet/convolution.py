@@ -31,7 +31,14 @@ class Convolution(Module):
         output.spatial_size = (input.spatial_size - self.filter_size) // self.filter_stride + 1
         assert ((output.spatial_size - 1) * self.filter_stride + self.filter_size == input.spatial_size).all(), (
             input.spatial_size, output.spatial_size, self.filter_size, self.filter_stride)
-        if not increment:
+        kind = incremental.kind(increment)
+        if kind == "residual":
+            out = input.features.new_empty((0, self.nOut))
+            SCN.Incre_Convolution_updateOutput(
+                input.spatial_size, output.spatial_size, self.filter_size, self.filter_stride, input.metadata,
+                input.features, out, self.weight, optionalTensor(self, 'bias'))
+            output.features = out
+        elif kind is None:
             out = input.features.new_empty((0, self.nOut))
             sparseconvnet.forward_pass_multiplyAdd_count += SCN.Convolution_updateOutput(
                 input.spatial_size, output.spatial_size, self.filter_size, self.filter_stride, input.metadata,

@@ -28,7 +28,15 @@ class Deconvolution(Module):
         assert input.features.nelement() == 0 or input.features.size(1) == self.nIn
         output = SparseConvNetTensor(None, input.metadata, None)
         output.spatial_size = (input.spatial_size - 1) * self.filter_stride + self.filter_size
-        if not increment:
+        kind = incremental.kind(increment)
+        if kind == "residual":
+            out = input.features.new_empty((0, self.nOut))
+            SCN.Incre_Deconvolution_updateOutput(
+                input.spatial_size, output.spatial_size, self.filter_size, self.filter_stride, input.metadata,
+                input.features, out, self.weight, optionalTensor(self, 'bias'), self.save_meta,
+                self.save_input_feats)
+            output.features = out
+        elif kind is None:
             out = input.features.new_empty((0, self.nOut))
             sparseconvnet.forward_pass_multiplyAdd_count += SCN.Deconvolution_updateOutput(
                 input.spatial_size, output.spatial_size, self.filter_size, self.filter_stride, input.metadata,
@@ -48,6 +56,7 @@ class Deconvolution(Module):
                             down.parent.t, down.offset.t, rows, count, d.n_upper)
             output.features = out
             output.dirty = d
+            self.save_input_feats = input.features
         return output
 
     def __repr__(self):

@@ -13,6 +13,11 @@ Every one of these maps only grows a set, so a set derived from another contains
 The reference's incremental path does not dilate (CUDA/Convolution.cpp:221-303) and is an
 approximation; recomputing exactly the dirty rows from cached inputs makes an incremental
 frame equal to a full forward over all points seen so far.
+
+Both kinds of incremental forward are provided.  `increment=True` selects the default kind
+(set_mode), `increment="exact"` / `increment="residual"` name one: "exact" is the dirty-set
+path above, "residual" the reference's own (features of a frame are differences to the state
+saved by the last full or exact forward, SCN.Incre_*; the saved state is left untouched).
 """
 import ctypes
 import itertools
@@ -23,6 +28,29 @@ from ._lib import lib, ptr, stream_ptr
 
 I64 = ctypes.c_int64
 _ids = itertools.count()
+_KINDS = ("exact", "residual")
+_mode = "exact"
+
+
+def set_mode(mode):
+    """Kind of incremental forward that `increment=True` stands for: "exact" or "residual"."""
+    global _mode
+    if mode not in _KINDS:
+        raise ValueError("incremental mode must be one of %s" % (_KINDS,))
+    _mode = mode
+
+
+def get_mode():
+    return _mode
+
+
+def kind(increment):
+    """None for a full forward, else "exact" or "residual"."""
+    if isinstance(increment, str):
+        if increment not in _KINDS:
+            raise ValueError("increment must be a bool or one of %s" % (_KINDS,))
+        return increment
+    return _mode if increment else None
 
 
 class DirtySet(object):

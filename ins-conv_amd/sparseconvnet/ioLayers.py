@@ -25,7 +25,9 @@ class InputLayer(Module):
 
     forward(input, increment=True) appends the given points to the sites of the last full
     forward and marks the touched sites dirty; the output then holds the features of ALL
-    sites, with only the dirty rows recomputed downstream.
+    sites, with only the dirty rows recomputed downstream.  With increment="residual" (or
+    incremental.set_mode("residual")) the frame is processed the reference's way instead: a
+    site set of its own, features as differences to the saved state.
     """
 
     def __init__(self, dimension, spatial_size, mode=3, normal_guide_scale=10240):
@@ -45,7 +47,18 @@ class InputLayer(Module):
         assert len(input) >= 2, len(input)
         coords, feats = input[0], input[1]
         batch_size = input[2] if len(input) > 2 else 0
-        if not increment:
+        kind = incremental.kind(increment)
+        if kind == "residual":
+            # the frame gets a site set of its own; the saved output stays as it is (ioLayers.py:70-80)
+            prev = self.save_output
+            output = SparseConvNetTensor(metadata=Metadata(self.dimension), spatial_size=self.spatial_size)
+            output.metadata._bind(feats.device)
+            out = feats.new_empty((0, feats.size(1)))
+            SCN.Incre_InputLayer_updateOutput(output.metadata, self.spatial_size, coords, feats, out, batch_size,
+                                              self.mode, prev.metadata, prev.features)
+            output.features = out
+            return output
+        if kind is None:
             output = SparseConvNetTensor(metadata=Metadata(self.dimension), spatial_size=self.spatial_size)
             m = output.metadata
             m._bind(feats.device)
@@ -94,6 +107,10 @@ class OutputLayer(Module):
     def forward(self, input, increment=False):
         m = input.metadata
         f = input.features
+        if incremental.kind(increment) == "residual":
+            out = f.new_empty((0, f.size(1)))
+            SCN.Incre_OutputLayer_updateOutput(m, f, out, self.save_meta, self.save_input_feats)
+            return out
         sop = m.site_of_all_points if (not increment or self.all_points) else m.site_of_point
         out = torch.empty((sop.numel(), f.size(1)), dtype=f.dtype, device=f.device)
         if sop.numel():

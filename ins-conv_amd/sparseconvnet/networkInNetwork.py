@@ -4,7 +4,7 @@ from torch.nn import Module, Parameter
 
 import sparseconvnet
 
-from . import SCN
+from . import SCN, incremental
 from .sparseConvNetTensor import SparseConvNetTensor
 from .utils import StateBuf, optionalTensor
 
@@ -23,7 +23,12 @@ class NetworkInNetwork(Module):
     def forward(self, input, increment=False):
         assert input.features.nelement() == 0 or input.features.size(1) == self.nIn, (self.nIn, input.features.shape)
         output = SparseConvNetTensor(None, input.metadata, input.spatial_size)
-        if not increment:
+        kind = incremental.kind(increment)
+        if kind == "residual":  # linear: the plain operator on the frame's rows (networkInNetwork.py:72-81)
+            out = input.features.new_empty((0, self.nOut))
+            SCN.NetworkInNetwork_updateOutput(input.features, out, self.weight, optionalTensor(self, 'bias'))
+            output.features = out
+        elif kind is None:
             out = input.features.new_empty((0, self.nOut))
             sparseconvnet.forward_pass_multiplyAdd_count += SCN.NetworkInNetwork_updateOutput(
                 input.features, out, self.weight, optionalTensor(self, 'bias'))

@@ -27,7 +27,14 @@ class SubmanifoldConvolution(Module):
     def forward(self, input, increment=False):
         assert input.features.nelement() == 0 or input.features.size(1) == self.nIn, (self.nIn, self.nOut, input)
         output = SparseConvNetTensor(None, input.metadata, input.spatial_size)
-        if not increment:
+        kind = incremental.kind(increment)
+        if kind == "residual":
+            out = input.features.new_empty((0, self.nOut))
+            SCN.Incre_SubmanifoldConvolution_updateOutput(
+                input.spatial_size, self.filter_size, input.metadata, input.features, out, self.weight,
+                optionalTensor(self, 'bias'), self.save_meta, self.save_input_feats, count_muladds=False)
+            output.features = out
+        elif kind is None:
             out = input.features.new_empty((0, self.nOut))
             sparseconvnet.forward_pass_multiplyAdd_count += SCN.SubmanifoldConvolution_updateOutput(
                 input.spatial_size, self.filter_size, input.metadata, input.features, out, self.weight,
@@ -46,6 +53,7 @@ class SubmanifoldConvolution(Module):
                           27, rows, count, d.n_upper)
             output.features = out
             output.dirty = d
+            self.save_input_feats = input.features
         return output
 
     def __repr__(self):

@@ -18,7 +18,11 @@ class JoinTable(torch.nn.Sequential):
         output = SparseConvNetTensor(None, input[0].metadata, input[0].spatial_size)
         n = input[0].features.size(0)
         C = sum(i.features.size(1) for i in input)
-        if increment:
+        kind = incremental.kind(increment)
+        if kind == "residual":  # a frame's rows only; the cached output is left alone
+            increment = False
+            out = torch.empty((n, C), dtype=torch.float32, device=input[0].features.device)
+        elif increment:
             d = input[0].dirty
             for i in input[1:]:
                 d = incremental.union(d, i.dirty)
@@ -53,7 +57,11 @@ class AddTable(torch.nn.Sequential):
         n, C = input[0].features.shape
         rows = count = None
         n_rows = n
-        if increment:
+        kind = incremental.kind(increment)
+        if kind == "residual":
+            increment = False
+            out = torch.empty((n, C), dtype=torch.float32, device=input[0].features.device)
+        elif increment:
             d = input[0].dirty
             for i in input[1:]:
                 d = incremental.union(d, i.dirty)

@@ -161,6 +161,125 @@ def nin_forward(feats, W, bias=None):
 
 
 # --------------------------------------------------------------------------------------
+# residual frames: the reference's Incre_* operators, restated with numpy.
+# A frame has a site set of its own (site_coords of the frame's points); pre_* is the state
+# saved by the last full forward.  pre_exist[i] = id of the frame's site i in the saved site
+# set, or -1 (getPreExistMaps, Metadata/Metadata.cpp:609-626).
+# Pinned in tests/test_oracle_incre.py by the identity every operator must satisfy on its own:
+# saved value + residual == the operator applied to the merged scene, at the frame's sites.
+# --------------------------------------------------------------------------------------
+def incre_pre_exist(pre_coords, coords):
+    return grid_query(pre_coords, coords)
+
+
+def incre_input_forward(feats, site_of_point, count, mode, pre_exist, pre_out, pre_count):
+    """InputLayer_inc_fp_ (CUDA/IOLayers.cu:81-105), rule rows as built by inputLayerRules
+    (Metadata/IOLayersRules.h:104-129): modes 1/2 keep one row, 3/4 all rows of a voxel."""
+    f = _f(feats)
+    N, C = len(count), f.shape[1]
+    out = np.zeros((N, C), np.float32)
+    if mode == 0:  # rows handed through (CUDA/IOLayers.cpp:320-322)
+        out[site_of_point] = f
+        return out
+    rows = [[] for _ in range(N)]
+    for p, s in enumerate(site_of_point):
+        rows[s].append(p)
+    for i in range(N):
+        r = rows[i]
+        if mode == 1:
+            r = r[:1]
+        elif mode == 2:
+            r = r[-1:]
+        pe = int(pre_exist[i])
+        na = len(r)
+        pn = 0 if pe < 0 else (int(pre_count[pe]) if mode >= 3 else 1)
+        m = np.float32(1.0) / np.float32(na + pn) if (mode == 4 and na > 0) else np.float32(1.0)
+        acc = np.zeros(C, np.float32)
+        for p in r:
+            acc = acc + m * f[p]
+        if pe >= 0:
+            acc = acc + _f(pre_out)[pe] * (np.float32(pn) * m - np.float32(1.0))
+        out[i] = acc
+    return out
+
+
+def incre_output_forward(feats, site_of_point, pre_exist, pre_in):
+    """InputLayer_inc_bp_ (CUDA/IOLayers.cu:122-141): residual + saved value per point."""
+    f, pin = _f(feats), _f(pre_in)
+    sop = np.asarray(site_of_point)
+    out = f[sop].copy()
+    pe = np.asarray(pre_exist)[sop]
+    has = pe >= 0
+    out[has] += pin[pe[has]]
+    return out
+
+
+def incre_ssc_rules(coords, pre_coords, pre_exist):
+    """Rules of IncreSubmanifoldBuildObject (CUDA/SubmanifoldRules_cuda.cpp:233-472): for every
+    site of the frame that the saved set does not hold, its 27 neighbours looked up in the saved
+    set -> (counts[27], pairs[R,2]) with pairs = (saved site, frame site), the 27 lists back to back."""
+    c = _c4(coords)
+    new = np.nonzero(np.asarray(pre_exist) < 0)[0]
+    counts = np.zeros(27, np.int32)
+    lists = []
+    for k in range(27):
+        d = np.array([k // 9 - 1, (k // 3) % 3 - 1, k % 3 - 1, 0], np.int32)
+        q = c[new] + d
+        ok = (q[:, :3] >= 0).all(1) & (q[:, :3] < 65536).all(1)
+        hit = np.full(len(new), -1, np.int32)
+        if ok.any():
+            hit[ok] = grid_query(pre_coords, q[ok])
+        sel = hit >= 0
+        counts[k] = sel.sum()
+        lists.append(np.stack([hit[sel], new[sel].astype(np.int32)], 1))
+    pairs = np.concatenate(lists, 0) if lists else np.zeros((0, 2), np.int32)
+    return counts, np.ascontiguousarray(pairs, np.int32)
+
+
+def incre_ssc_forward(feats, pre_in, W, bias, rules, rules_pre, n):
+    """cuda_Incre_SubmanifoldConvolution_updateOutput (CUDA/Convolution.cpp:221-303): the frame's
+    own rules on the residual features, then the rules of incre_ssc_rules on the saved input."""
+    out, _ = conv_forward(feats, W, bias, rules[1], rules[0], n)
+    if len(rules_pre[1]):
+        extra, _ = conv_forward(pre_in, W, None, rules_pre[1], rules_pre[0], n)
+        out = out + extra
+    return out.astype(np.float32)
+
+
+def incre_bn_forward(feats, mean, var, gamma, beta, eps, leakiness, pre_exist, pre_in, pre_out):
+    """Incre_BatchNormalization_f_test (CUDA/BatchNormalization.cu:112-150)."""
+    f = _f(feats)
+    C = f.shape[1]
+    g = _f(gamma) if gamma is not None else np.ones(C, np.float32)
+    bt = _f(beta) if beta is not None else np.zeros(C, np.float32)
+    w = (np.power(_f(var) + np.float32(eps), np.float32(-0.5)) * g).astype(np.float32)
+    b = (bt - _f(mean) * w).astype(np.float32)
+    o = (w * f + b).astype(np.float32)
+    pe = np.asarray(pre_exist)
+    has = pe >= 0
+    t = o.copy()
+    t[has] = o[has] + _f(pre_in)[pe[has]] * w
+    y = np.where(t > 0, t, t * np.float32(leakiness)).astype(np.float32)
+    y[has] -= _f(pre_out)[pe[has]]
+    return y
+
+
+def incre_deconv_forward(feats, pre_in, W, bias, parent, offset, pre_exist_in, pre_exist_out):
+    """dDeconvolution_incre_KMxKN_forwardA (CUDA/Deconvolution.cu:84-150): the saved coarse
+    feature joins in when the coarse site existed and the fine site is new."""
+    f, W = _f(feats), _f(W)
+    parent, offset = np.asarray(parent), np.asarray(offset)
+    x = f[parent].copy()
+    pe_c = np.asarray(pre_exist_in)[parent]
+    add = (pe_c >= 0) & (np.asarray(pre_exist_out) < 0)
+    x[add] += _f(pre_in)[pe_c[add]]
+    out = np.einsum("ni,nio->no", x.astype(np.float64), W[offset].astype(np.float64)).astype(np.float32)
+    if bias is not None:
+        out = out + _f(bias)
+    return out.astype(np.float32)
+
+
+# --------------------------------------------------------------------------------------
 # canonical forms used to compare integer structures bit-exactly
 # --------------------------------------------------------------------------------------
 def canonical_sites(site_coords):
