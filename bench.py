@@ -82,7 +82,7 @@ def ssc_workload(device, channels=(32, 64)):
     return step, info, (xs[0], stacks[0])
 
 
-def conv_roofline(device, reps=30):
+def conv_roofline(device, reps=30, warm=200):
     """Average duration of the 32-channel submanifold convolution kernel at 500k voxels and the
     roofline figures derived from it."""
     import torch
@@ -97,7 +97,7 @@ def conv_roofline(device, reps=30):
     out = torch.empty((sc.n, conv.nOut), device=device)
     w = conv.weight
     plan = m.ssc_plan(sc)  # built once per rulebook, like the neighbour map and the order
-    for _ in range(3):
+    for _ in range(warm):  # long enough for the clocks to leave their idle state
         SCN.ssc_rows_planned(x.features, out, w, None, sc, plan)
     torch.cuda.synchronize()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -115,11 +115,11 @@ def conv_roofline(device, reps=30):
     achieved = bytes_alg / t / 1e9
     return {
         "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-        "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": 653.0e6,
+        "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": 639.1e6,
         "kernel": "conv_wlds_kernel (SSC 3^3, 32->32, filter in LDS, persistent blocks; 500k sites, %d rules)" % n_rules,
         "avg_us": round(t * 1e6, 1), "algorithmic_bytes": int(bytes_alg),
         "traffic_note": "HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE (x1.999, copy-kernel calibration) + "
-                        "WRITE_SIZE (x1.000): 578.8 MB + 74.2 MB, profiles/conv_wlds_ssc32_500k.txt",
+                        "WRITE_SIZE (x1.000): 541.3 MB + 97.8 MB, profiles/conv_wlds_ssc32_500k.txt",
         "mfma_tflops": round(flops / t / 1e12, 2), "mfma_frac": round(flops / t / 1e12 / MFMA_FP32_PEAK_TFLOPS, 4),
         "ssc_msites_per_s": round(sc.n / t / 1e6, 1),
     }
@@ -352,7 +352,7 @@ def main():
         for _ in range(5):
             SCN.copy_rows(a, b, None, None, a.size(0))
         torch.cuda.synchronize()
-        print(json.dumps({"roofline": conv_roofline(device, reps=10)}))
+        print(json.dumps({"roofline": conv_roofline(device, reps=10, warm=3)}))
         return
 
     extra = {}
@@ -391,7 +391,7 @@ def main():
         extra = {"median_ms": round(float(np.median(per_frame)), 3),
                  "p95_ms": round(float(np.percentile(per_frame, 95)), 3),
                  "last_frame_ms": round(per_frame[-1], 3), "first_timed_frame_ms": round(per_frame[0], 3)}
-        cpu = None if args.no_cpu_baseline else cpu_baseline_unet()
+        cpu_fn = cpu_baseline_unet
     elif args.workload == "unet":
         import scenes
 
@@ -413,7 +413,7 @@ def main():
         value, metric, unit, hib = round(ms, 3), "full U-Net forward ms (150k vox)", "ms", False
         config = {"workload": "cfg4: full U-Net forward (grid + rulebooks + all layers), 150k voxels / 165k points",
                   "sites_per_level": net.sites_per_level()[:7]}
-        cpu = None if args.no_cpu_baseline else cpu_baseline_unet()
+        cpu_fn = cpu_baseline_unet
     else:
         W = 3 if args.warmup is None else args.warmup
         K = 20 if args.steps is None else args.steps
@@ -431,7 +431,7 @@ def main():
         metric, unit, hib = "SSC Msites/s", "Msites/s", True
         config = {"workload": "cfg3: 4x[SSC(3)+BN+ReLU] at 500k voxels, C=32 then C=64 (8 convs/step)",
                   "sites": info["sites"], "rules": info["rules"]}
-        cpu = None if args.no_cpu_baseline else cpu_baseline_ssc()
+        cpu_fn = cpu_baseline_ssc
 
     out = {
         "metric": metric, "value": value, "unit": unit, "n_gpus": 1, "steps": K, "warmup": W,
@@ -441,8 +441,10 @@ def main():
     out.update(extra)
     out["roofline"] = conv_roofline(device)
     out["kernels"] = kernel_table(device)
-    if cpu is not None:
-        out["cpu_baseline"] = cpu
+    # the CPU leg comes last: the GPU idles during it, and a measurement taken right after would
+    # start at idle clocks
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_fn()
     print(json.dumps(out))
 
 

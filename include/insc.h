@@ -252,6 +252,9 @@ int insc_net_op_add(insc_net *net, int a, int b, int out);
 /* Freeze the program; out_tensor feeds the output layer; capacity_sites is reserved at scale 0
  * (half of it at each coarser scale; everything grows on demand). */
 int insc_net_finalize(insc_net *net, int out_tensor, int64_t capacity_sites, void *stream);
+/* Before insc_net_finalize: also keep the input of every batch norm, which residual frames
+ * (insc_net_forward_residual) read and which the fused layers would otherwise not store. */
+int insc_net_enable_residual(insc_net *net);
 /* Re-pack the weights after the caller changed them in place. */
 int insc_net_refresh_weights(insc_net *net, void *stream);
 /* One frame: d_coords int32 [P,coord_cols] (x,y,z[,batch]), d_feats float32 [P,in_channels].
@@ -261,6 +264,15 @@ int insc_net_refresh_weights(insc_net *net, void *stream);
  * Returns when the frame has completed. */
 int insc_net_forward(insc_net *net, const int32_t *d_coords, int coord_cols, const float *d_feats, int64_t P,
                      int increment, float *d_out, int out_all, int64_t *h_n_sites, void *stream);
+/* One residual frame: the reference's own incremental forward (demo.py:26-38 with
+ * increment=True; Incre_* operators, pybind.cpp:218-258) as one call.  The frame's points form a
+ * site set of their own, features are differences to the state saved by the last
+ * insc_net_forward, and that state is not modified.  d_out (nullable): [P,C], saved value +
+ * residual for every point of the frame (cuda_Incre_OutputLayer_updateOutput,
+ * CUDA/IOLayers.cpp:339-368).  h_n_sites (nullable): sites of the frame at the input scale.
+ * Returns once the frame's site counts are known; the layers may still be running on the stream. */
+int insc_net_forward_residual(insc_net *net, const int32_t *d_coords, int coord_cols, const float *d_feats, int64_t P,
+                              float *d_out, int64_t *h_n_sites, void *stream);
 int insc_net_tensor_view(insc_net *net, int tensor, float **d_ptr, int64_t *ld, int64_t *rows, int *channels);
 int insc_net_counts(insc_net *net, int64_t *h_sites_per_level, int64_t *h_points);
 /* Phase timing (the reference brackets the same phases with easy_profiler blocks,

@@ -33,8 +33,10 @@ int hip_fail(hipError_t e, const char *what, const char *file, int line);
 // it only ever grows, so steady-state calls allocate nothing.  Work using an arena is
 // ordered by its stream.
 // Arena 0 belongs to the scan primitive, arena 1 to the sort primitive, arena 2 to the
-// API-level function that is running (none of which calls another arena-2 user).
-enum { WS_SCAN = 0, WS_SORT = 1, WS_API = 2, WS_CONV = 3, WS_LABELS = 4 };
+// API-level function that is running (none of which calls another arena-2 user; the convolution
+// launcher packs weights there when the caller brings none), arena 5 to the residual-frame
+// operators, which call that launcher.
+enum { WS_SCAN = 0, WS_SORT = 1, WS_API = 2, WS_CONV = 3, WS_LABELS = 4, WS_INCRE = 5 };
 int workspace(int which, hipStream_t stream, size_t bytes, void **out);
 int device_cus();
 // `count` int32 counters per (device, stream), zero at kernel start; users leave them at zero
@@ -93,6 +95,11 @@ int launch_bn(const float *in, int64_t ld_in, float *out, int64_t ld_out, const 
 int launch_add(const float *a, int64_t ld_a, const float *b, int64_t ld_b, float *out, int64_t ld_out,
                const int32_t *rows, const int32_t *d_n_rows, int64_t n_rows, int C, const uint8_t *row_mask,
                hipStream_t s, BnEpilogue ep = BnEpilogue());
+// batch norm of a residual frame (incre.hip); w, b: precomputed scale / shift or null
+int launch_incre_bn(const float *in, int64_t ld_in, float *out, int64_t ld_out, const float *mean, const float *var,
+                    const float *gamma, const float *beta, float eps, float leak, const float *w, const float *b,
+                    const int32_t *pre_exist, const float *pre_in, int64_t ld_pin, const float *pre_out,
+                    int64_t ld_pout, int64_t n, int C, hipStream_t s);
 int launch_input_finish(const float *sum, const int32_t *cnt, int mode, float *out, int64_t ld_out,
                         const int32_t *rows, const int32_t *d_n_rows, int64_t n_rows, int C,
                         const uint8_t *row_mask, hipStream_t s);

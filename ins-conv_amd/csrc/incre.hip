@@ -43,7 +43,9 @@ __global__ __launch_bounds__(256) void incre_bn_kernel(const float *__restrict__
                                                        float *__restrict__ out, int64_t ld_out,
                                                        const float *__restrict__ mean, const float *__restrict__ var,
                                                        const float *__restrict__ gamma, const float *__restrict__ beta,
-                                                       float eps, float leak, const int32_t *__restrict__ pre_exist,
+                                                       float eps, float leak, const float *__restrict__ wv,
+                                                       const float *__restrict__ bv,
+                                                       const int32_t *__restrict__ pre_exist,
                                                        const float *__restrict__ pre_in, int64_t ld_pin,
                                                        const float *__restrict__ pre_out, int64_t ld_pout, int64_t n,
                                                        int C) {
@@ -51,7 +53,12 @@ __global__ __launch_bounds__(256) void incre_bn_kernel(const float *__restrict__
     const int64_t row = e / C;
     const int c = (int)(e - row * C);
     float w, b;
-    bn_coeffs(mean, var, gamma, beta, eps, c, w, b);
+    if (wv) {  // scale / shift already formed (bn_scale_shift: the same two numbers)
+      w = wv[c];
+      b = bv[c];
+    } else {
+      bn_coeffs(mean, var, gamma, beta, eps, c, w, b);
+    }
     const float o = fmaf(in[row * ld_in + c], w, b);
     const int pe = pre_exist[row];
     float y;
@@ -95,6 +102,17 @@ __global__ __launch_bounds__(256) void incre_output_kernel(const float *__restri
     }
     out[e] = v;
   }
+}
+
+int launch_incre_bn(const float *in, int64_t ld_in, float *out, int64_t ld_out, const float *mean, const float *var,
+                    const float *gamma, const float *beta, float eps, float leak, const float *w, const float *b,
+                    const int32_t *pre_exist, const float *pre_in, int64_t ld_pin, const float *pre_out,
+                    int64_t ld_pout, int64_t n, int C, hipStream_t s) {
+  if (n == 0) return INSC_OK;
+  hipLaunchKernelGGL(incre_bn_kernel, dim3(grid_for(n * C, 256, 1 << 16)), dim3(256), 0, s, in, ld_in, out, ld_out,
+                     mean, var, gamma, beta, eps, leak, w, b, pre_exist, pre_in, ld_pin, pre_out, ld_pout, n, C);
+  INSC_LAUNCH_CHECK();
+  return INSC_OK;
 }
 
 }  // namespace insc
@@ -147,11 +165,8 @@ int insc_incre_bn_leaky(const float *d_in, int64_t ld_in, float *d_out, int64_t 
   if (n == 0) return INSC_OK;
   INSC_REQUIRE(d_in && d_out && d_mean && d_var && d_pre_exist && d_pre_in && d_pre_out, INSC_ERR_ARG,
                "insc_incre_bn_leaky: null pointer");
-  hipLaunchKernelGGL(incre_bn_kernel, dim3(grid_for(n * C, 256, 1 << 16)), dim3(256), 0, (hipStream_t)stream, d_in,
-                     ld_in, d_out, ld_out, d_mean, d_var, d_gamma, d_beta, eps, leakiness, d_pre_exist, d_pre_in,
-                     ld_pre_in, d_pre_out, ld_pre_out, n, C);
-  INSC_LAUNCH_CHECK();
-  return INSC_OK;
+  return launch_incre_bn(d_in, ld_in, d_out, ld_out, d_mean, d_var, d_gamma, d_beta, eps, leakiness, nullptr, nullptr,
+                         d_pre_exist, d_pre_in, ld_pre_in, d_pre_out, ld_pre_out, n, C, (hipStream_t)stream);
 }
 
 int insc_incre_deconv_down2(const float *d_in, int64_t ld_in, int64_t n_in_rows, const float *d_pre_in, int64_t ld_pre,
@@ -171,7 +186,7 @@ int insc_incre_deconv_down2(const float *d_in, int64_t ld_in, int64_t n_in_rows,
                        nullptr, nullptr, n_rows, Cin, Cout, nullptr, nullptr, s);
   if (rc || n_pre_rows == 0) return rc;
   void *ws;
-  rc = workspace(WS_API, s, sizeof(int32_t) * (size_t)n_rows, &ws);
+  rc = workspace(WS_INCRE, s, sizeof(int32_t) * (size_t)n_rows, &ws);
   if (rc) return rc;
   int32_t *parent2 = (int32_t *)ws;
   hipLaunchKernelGGL(incre_parent_kernel, dim3(grid_for(n_rows, 256)), dim3(256), 0, s, d_parent, d_pre_exist_in,

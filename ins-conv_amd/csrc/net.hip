@@ -76,9 +76,27 @@ struct DirtyNode {
 
 }  // namespace insc
 
+namespace insc {
+// Everything a residual frame needs besides the saved state: the frame's own site set (fresh
+// grids and maps at every scale), its links to the saved one, and feature matrices sized for
+// the frame.  Built anew by every residual frame; nothing in it outlives the frame.
+struct ResidualFrame {
+  std::vector<Level> levels;            // grid, nbr, parent, offset, child of the frame's sites
+  std::vector<int32_t *> pre_exist;     // [cap] id in the saved site set of the scale, or -1
+  std::vector<int32_t *> nbr_pre;       // [cap,27] saved neighbours of the sites new to the saved set
+  std::vector<Buffer> buffers;          // same layout as the program's buffers, rows = sites of the frame
+  std::vector<int> ld;                  // row stride of every buffer (0: unused)
+  int64_t cap = 0;                      // sites every scale can hold
+  float *in_sum = nullptr;
+  int32_t *in_cnt = nullptr, *chain_head = nullptr, *chain_next = nullptr, *sop = nullptr;
+};
+}  // namespace insc
+
 struct insc_net {
   int n_levels = 0, in_channels = 0, mode = 4;
   bool finalized = false, have_state = false;
+  bool keep_raw = false;  // keep the input of every batch norm (residual frames read it)
+  insc::ResidualFrame rf;
   std::vector<insc::Level> levels;
   std::vector<insc::Buffer> buffers;
   std::vector<insc::Tensor> tensors;
@@ -540,6 +558,21 @@ int insc_net_destroy(insc_net *net) {
     if (op.bn_w) (void)hipFree(op.bn_w);
     if (op.bn_b) (void)hipFree(op.bn_b);
   }
+  for (Level &L : net->rf.levels) {
+    if (L.grid) insc_grid_destroy(L.grid);
+    void *ps[] = {L.nbr, L.parent, L.offset, L.child};
+    for (void *p : ps)
+      if (p) (void)hipFree(p);
+  }
+  for (int32_t *p : net->rf.pre_exist)
+    if (p) (void)hipFree(p);
+  for (int32_t *p : net->rf.nbr_pre)
+    if (p) (void)hipFree(p);
+  for (Buffer &B : net->rf.buffers)
+    if (B.p) (void)hipFree(B.p);
+  void *rps[] = {net->rf.in_sum, net->rf.in_cnt, net->rf.chain_head, net->rf.chain_next, net->rf.sop};
+  for (void *p : rps)
+    if (p) (void)hipFree(p);
   void *ps[] = {net->in_sum, net->in_cnt, net->chain_head, net->chain_next, net->site_of_point, net->mask_arena};
   for (void *p : ps)
     if (p) (void)hipFree(p);
@@ -737,7 +770,7 @@ int insc_net_finalize(insc_net *net, int out_tensor, int64_t capacity_sites, voi
       if (!can || A.fused_bn >= 0 || producer[bn.in0] > i) continue;
       A.fused_bn = i;
       bn.fused = true;
-      A.write_raw = readers[bn.in0] > 1;
+      A.write_raw = readers[bn.in0] > 1 || net->keep_raw;
       if (!A.write_raw) {
         Tensor &T = net->tensors[bn.in0];
         Buffer &B = net->buffers[T.buf];
@@ -959,6 +992,255 @@ int insc_net_forward(insc_net *net, const int32_t *d_coords, int coord_cols, con
   INSC_HIP(hipStreamSynchronize(s));  // the counts are known already; the call returns when the frame is done
   net->ev_valid = net->profiling;
   if (h_n_sites) *h_n_sites = net->levels[0].n;
+  return INSC_OK;
+}
+
+/* Ask for residual frames (insc_net_forward_residual) before insc_net_finalize: the input of
+ * every batch norm is then kept although its producer computes the batch norm itself. */
+int insc_net_enable_residual(insc_net *net) {
+  INSC_REQUIRE(net && !net->finalized, INSC_ERR_STATE, "insc_net_enable_residual: net is null or already finalized");
+  net->keep_raw = true;
+  return INSC_OK;
+}
+
+}  // extern "C"
+
+namespace insc {
+
+static void free_dev(void *p) {
+  if (p) (void)hipFree(p);
+}
+
+// (re)allocate the frame's structures for `cap` sites per scale; nothing is preserved
+static int rframe_reserve(insc_net *net, int64_t need, hipStream_t s) {
+  ResidualFrame &R = net->rf;
+  const int L = net->n_levels;
+  if (R.levels.empty()) {
+    R.levels.resize(L);
+    R.pre_exist.assign(L, nullptr);
+    R.nbr_pre.assign(L, nullptr);
+    R.buffers.resize(net->buffers.size());
+    R.ld.assign(net->buffers.size(), 0);
+    for (size_t b = 0; b < net->buffers.size(); b++) R.buffers[b].level = net->buffers[b].level;
+    // the program's buffers may have lost matrices nothing reads in a fused frame; here every
+    // tensor is written, so strides come from the tensors: widest column range per buffer
+    for (const Tensor &T : net->tensors) R.ld[T.buf] = std::max(R.ld[T.buf], T.col0 + T.C);
+    for (size_t b = 0; b < net->buffers.size(); b++) R.buffers[b].ld = R.ld[b];
+  }
+  if (need <= R.cap) return INSC_OK;
+  INSC_HIP(hipStreamSynchronize(s));
+  const int64_t cap = (std::max<int64_t>(need + need / 2, 4096) + 31) / 32 * 32;
+  int rc;
+  for (int l = 0; l < L; l++) {
+    Level &Lv = R.levels[l];
+    if (Lv.grid) insc_grid_destroy(Lv.grid);
+    Lv.grid = nullptr;
+    if ((rc = insc_grid_create(cap, &Lv.grid))) return rc;
+    free_dev(Lv.nbr);
+    free_dev(Lv.parent);
+    free_dev(Lv.offset);
+    free_dev(Lv.child);
+    free_dev(R.pre_exist[l]);
+    free_dev(R.nbr_pre[l]);
+    Lv.parent = Lv.offset = Lv.child = nullptr;
+    if ((rc = dev_alloc(&Lv.nbr, (size_t)cap * 27))) return rc;
+    if ((rc = dev_alloc(&R.pre_exist[l], (size_t)cap))) return rc;
+    if ((rc = dev_alloc(&R.nbr_pre[l], (size_t)cap * 27))) return rc;
+    if (l + 1 < L) {
+      if ((rc = dev_alloc(&Lv.parent, (size_t)cap))) return rc;
+      if ((rc = dev_alloc(&Lv.offset, (size_t)cap))) return rc;
+      if ((rc = dev_alloc(&Lv.child, (size_t)cap * 8))) return rc;
+      Lv.child_rows = cap;
+    }
+    Lv.cap = cap;
+  }
+  free_dev(R.in_sum);
+  free_dev(R.in_cnt);
+  free_dev(R.chain_head);
+  free_dev(R.chain_next);
+  free_dev(R.sop);
+  if ((rc = dev_alloc(&R.in_sum, (size_t)cap * net->in_channels))) return rc;
+  if ((rc = dev_alloc(&R.in_cnt, (size_t)cap))) return rc;
+  if ((rc = dev_alloc(&R.chain_head, (size_t)cap))) return rc;
+  if ((rc = dev_alloc(&R.chain_next, (size_t)cap))) return rc;
+  if ((rc = dev_alloc(&R.sop, (size_t)cap))) return rc;
+  if ((rc = fill_i32(R.chain_head, cap, -1, s))) return rc;  // the accumulation leaves it at -1
+  R.cap = cap;
+  return INSC_OK;
+}
+
+static int rframe_buffers(insc_net *net, hipStream_t s) {
+  ResidualFrame &R = net->rf;
+  for (size_t b = 0; b < R.buffers.size(); b++) {
+    Buffer &B = R.buffers[b];
+    const int64_t n = R.levels[B.level].n;
+    if (B.ld == 0 || n <= B.rows) continue;
+    INSC_HIP(hipStreamSynchronize(s));
+    free_dev(B.p);
+    B.p = nullptr;
+    const int64_t rows = std::max<int64_t>(n + n / 2, 256);
+    int rc = dev_alloc(&B.p, (size_t)rows * B.ld);
+    if (rc) return rc;
+    B.rows = rows;
+  }
+  return INSC_OK;
+}
+
+static float *rtensor_ptr(insc_net *net, int t) {
+  const Tensor &T = net->tensors[t];
+  return net->rf.buffers[T.buf].p + T.col0;
+}
+static int64_t rtensor_ld(insc_net *net, int t) { return net->rf.buffers[net->tensors[t].buf].ld; }
+
+// one layer of a residual frame: every op runs on its own (no fusions), on all rows of the frame
+static int run_op_residual(insc_net *net, const Op &op, hipStream_t s) {
+  ResidualFrame &R = net->rf;
+  const Tensor &To = net->tensors[op.out];
+  const Level &Lo = R.levels[To.level];
+  const int64_t n = Lo.n;
+  if (n == 0 || op.kind == OP_JOIN) return INSC_OK;
+  const float *in0 = rtensor_ptr(net, op.in0);
+  const int64_t ld0 = rtensor_ld(net, op.in0);
+  float *out = rtensor_ptr(net, op.out);
+  const int64_t ld_out = rtensor_ld(net, op.out);
+  const int li = net->tensors[op.in0].level;
+  const int64_t n_in = R.levels[li].n;
+  // the saved input of the layer and the saved site count of its scale
+  const float *pre0 = net->tensors[op.in0].kept ? tensor_ptr(net, op.in0) : nullptr;
+  const int64_t ldp0 = net->tensors[op.in0].kept ? tensor_ld(net, op.in0) : 0;
+  const int64_t n_pre_in = net->levels[li].n;
+  void *st = (void *)s;
+  switch (op.kind) {
+    case OP_SSC:
+      INSC_REQUIRE(pre0, INSC_ERR_STATE, "residual frame: the input of a convolution was not kept");
+      return insc_incre_conv_ssc(in0, ld0, pre0, ldp0, n_pre_in, out, ld_out, op.W, op.Wp, op.bias, Lo.nbr,
+                                 R.nbr_pre[To.level], n, op.Cin, op.Cout, st);
+    case OP_NIN:
+      return launch_conv(in0, ld0, n_in, out, ld_out, op.W, op.Wp, op.bias, nullptr, nullptr, MAP_IDENTITY, 1, nullptr,
+                         nullptr, n, op.Cin, op.Cout, nullptr, nullptr, s);
+    case OP_CONV:
+      return launch_conv(in0, ld0, n_in, out, ld_out, op.W, op.Wp, op.bias, R.levels[li].child, nullptr, MAP_NBR, 8,
+                         nullptr, nullptr, n, op.Cin, op.Cout, nullptr, nullptr, s);
+    case OP_DECONV:
+      INSC_REQUIRE(pre0, INSC_ERR_STATE, "residual frame: the input of a deconvolution was not kept");
+      return insc_incre_deconv_down2(in0, ld0, n_in, pre0, ldp0, n_pre_in, out, ld_out, op.W, op.Wp, op.bias, Lo.parent,
+                                     Lo.offset, R.pre_exist[li], R.pre_exist[To.level], n, op.Cin, op.Cout, st);
+    case OP_BN:
+      INSC_REQUIRE(pre0 && net->tensors[op.out].kept, INSC_ERR_STATE,
+                   "residual frame: the input of a batch norm was not kept (insc_net_enable_residual before finalize)");
+      return launch_incre_bn(in0, ld0, out, ld_out, op.mean, op.var, op.gamma, op.beta, op.eps, op.leak, op.bn_w,
+                             op.bn_b, R.pre_exist[To.level], pre0, ldp0, tensor_ptr(net, op.out),
+                             tensor_ld(net, op.out), n, op.Cout, s);
+    case OP_ADD:
+      return launch_add(in0, ld0, rtensor_ptr(net, op.in1), rtensor_ld(net, op.in1), out, ld_out, nullptr, nullptr, n,
+                        op.Cout, nullptr, s);
+    case OP_COPY:
+      return launch_add(in0, ld0, nullptr, 0, out, ld_out, nullptr, nullptr, n, op.Cout, nullptr, s);
+  }
+  set_error("run_op_residual: unknown op kind %d", op.kind);
+  return INSC_ERR_STATE;
+}
+
+}  // namespace insc
+
+extern "C" {
+
+/* One residual frame, the reference's own incremental mode (Incre_* operators; the module
+ * tree's increment="residual"): the frame's points form a site set of their own, features are
+ * differences to the state saved by the last full / exact incremental frame, and that state
+ * is left as it is.  d_out: [P, C] rows of the output tensor, saved value + residual, one per
+ * point of the frame.  h_n_sites (nullable): sites of the frame at the input scale.
+ * Needs insc_net_enable_residual before insc_net_finalize.  The call returns once the frame's
+ * site counts are known; the layers may still be running on the stream. */
+int insc_net_forward_residual(insc_net *net, const int32_t *d_coords, int coord_cols, const float *d_feats, int64_t P,
+                              float *d_out, int64_t *h_n_sites, void *stream) {
+  INSC_REQUIRE(net && net->finalized, INSC_ERR_STATE, "insc_net_forward_residual: net is not finalized");
+  INSC_REQUIRE(net->keep_raw, INSC_ERR_STATE,
+               "insc_net_forward_residual: call insc_net_enable_residual before insc_net_finalize");
+  INSC_REQUIRE(net->have_state, INSC_ERR_STATE, "insc_net_forward_residual: residual frame before any full frame");
+  INSC_REQUIRE(P >= 0 && (P == 0 || (d_coords && d_feats)) && (coord_cols == 3 || coord_cols == 4), INSC_ERR_ARG,
+               "insc_net_forward_residual: bad arguments");
+  if (h_n_sites) *h_n_sites = 0;
+  if (P == 0) return INSC_OK;
+  hipStream_t s = (hipStream_t)stream;
+  const int L = net->n_levels;
+  const int C0 = net->in_channels;
+  ResidualFrame &R = net->rf;
+  int rc;
+  if ((rc = rframe_reserve(net, P, s))) return rc;
+
+  // ---- the frame's own site set --------------------------------------------------------------
+  for (int l = 0; l < L; l++) {
+    Level &Lv = R.levels[l];
+    if ((rc = insc_grid_clear(Lv.grid, stream))) return rc;
+    if (l + 1 < L)
+      if ((rc = fill_i32(Lv.child, P * 8, -1, s))) return rc;  // a scale has at most P sites
+  }
+  INSC_HIP(hipMemsetAsync(R.in_sum, 0, sizeof(float) * (size_t)P * C0, s));
+  INSC_HIP(hipMemsetAsync(R.in_cnt, 0, sizeof(int32_t) * (size_t)P, s));
+  void *ws;
+  if ((rc = workspace(WS_API, s, sizeof(int32_t) * 4 * (size_t)P, &ws))) return rc;
+  int32_t *c4 = (int32_t *)ws;
+  const unsigned nb = grid_for(P, 256);
+  hipLaunchKernelGGL(coords_to_int4_kernel, dim3(nb), dim3(256), 0, s, d_coords, coord_cols, P, c4);
+  INSC_LAUNCH_CHECK();
+  if ((rc = grid_insert_nosync(R.levels[0].grid, c4, P, R.sop, s))) return rc;
+  hipLaunchKernelGGL(chain_push_kernel, dim3(nb), dim3(256), 0, s, R.sop, P, R.chain_head, R.chain_next);
+  hipLaunchKernelGGL(chain_sum_kernel, dim3(nb), dim3(256), 0, s, d_feats, C0, R.sop, P, R.chain_head, R.chain_next,
+                     R.in_sum, R.in_cnt, (uint8_t *)nullptr, (uint8_t *)nullptr, (const int32_t *)nullptr);
+  INSC_LAUNCH_CHECK();
+  if ((rc = ssc3_new_sites(R.levels[0].grid, R.levels[0].nbr, P, s))) return rc;
+  for (int l = 0; l + 1 < L; l++) {
+    Level &F = R.levels[l], &Cs = R.levels[l + 1];
+    if ((rc = down2_new_sites(F.grid, Cs.grid, P, F.parent, F.offset, F.child, s))) return rc;
+    if ((rc = ssc3_new_sites(Cs.grid, Cs.nbr, P, s))) return rc;
+  }
+  // the exact site counts size every later launch (one short host round trip, as in an exact frame)
+  for (int l = 0; l < L; l++) {
+    INSC_HIP(hipMemcpyAsync(net->h_counts + 2 * l, R.levels[l].grid->d_n, sizeof(int32_t), hipMemcpyDeviceToHost, s));
+    INSC_HIP(hipMemcpyAsync(net->h_counts + 2 * l + 1, R.levels[l].grid->d_err, sizeof(int32_t), hipMemcpyDeviceToHost,
+                            s));
+  }
+  INSC_HIP(hipStreamSynchronize(s));
+  for (int l = 0; l < L; l++) {
+    Level &Lv = R.levels[l];
+    Lv.n = Lv.n_upper = net->h_counts[2 * l];
+    Lv.grid->n_exact = Lv.grid->n_upper = Lv.n;
+    const int err = net->h_counts[2 * l + 1];
+    INSC_REQUIRE(!(err & 1), INSC_ERR_COORD,
+                 "insc_net_forward_residual: a coordinate is outside 0..65535 (batch 0..32767)");
+    INSC_REQUIRE(!(err & 2), INSC_ERR_CAPACITY, "insc_net_forward_residual: capacity of scale %d exceeded", l);
+  }
+  if ((rc = rframe_buffers(net, s))) return rc;
+  // ---- links to the saved site set -------------------------------------------------------------
+  for (int l = 0; l < L; l++) {
+    Level &Lv = R.levels[l];
+    if (Lv.n == 0) continue;
+    if ((rc = insc_grid_query(net->levels[l].grid, Lv.grid->coords, Lv.n, R.pre_exist[l], stream))) return rc;
+    if ((rc = insc_incre_rulebook_ssc3(Lv.grid, net->levels[l].grid, R.pre_exist[l], Lv.n, R.nbr_pre[l], stream)))
+      return rc;
+  }
+  // ---- input layer, layers, output layer -----------------------------------------------------------
+  const int64_t n0 = R.levels[0].n;
+  if (net->mode == 0) {
+    if ((rc = launch_input_finish(R.in_sum, R.in_cnt, 0, rtensor_ptr(net, 0), rtensor_ld(net, 0), nullptr, nullptr, n0,
+                                  C0, nullptr, s)))
+      return rc;
+  } else if ((rc = insc_incre_input(R.in_sum, R.in_cnt, net->mode, R.pre_exist[0], tensor_ptr(net, 0),
+                                    tensor_ld(net, 0), net->in_cnt, rtensor_ptr(net, 0), rtensor_ld(net, 0), n0, C0,
+                                    stream))) {
+    return rc;
+  }
+  for (const Op &op : net->ops)
+    if ((rc = run_op_residual(net, op, s))) return rc;
+  if (d_out) {
+    const Tensor &To = net->tensors[net->out_tensor];
+    if ((rc = insc_incre_output(rtensor_ptr(net, net->out_tensor), rtensor_ld(net, net->out_tensor),
+                                tensor_ptr(net, net->out_tensor), tensor_ld(net, net->out_tensor), R.pre_exist[0],
+                                R.sop, P, To.C, d_out, stream)))
+      return rc;
+  }
+  if (h_n_sites) *h_n_sites = n0;
   return INSC_OK;
 }
 

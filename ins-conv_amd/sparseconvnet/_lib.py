@@ -58,6 +58,8 @@ _SIGS = {
     "insc_net_finalize": [vp, c_int, c_i64, vp],
     "insc_net_refresh_weights": [vp, vp],
     "insc_net_forward": [vp, vp, c_int, vp, c_i64, c_int, vp, c_int, ctypes.POINTER(c_i64), vp],
+    "insc_net_enable_residual": [vp],
+    "insc_net_forward_residual": [vp, vp, c_int, vp, c_i64, vp, ctypes.POINTER(c_i64), vp],
     "insc_net_tensor_view": [vp, c_int, ctypes.POINTER(vp), ctypes.POINTER(c_i64), ctypes.POINTER(c_i64),
                              ctypes.POINTER(c_int)],
     "insc_net_counts": [vp, ctypes.POINTER(c_i64), ctypes.POINTER(c_i64)],

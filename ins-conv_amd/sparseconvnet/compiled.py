@@ -3,6 +3,7 @@
     net = scn.compile(sparse_model)          # Sequential starting with InputLayer, ending with OutputLayer
     feats = net([coords, features, batch], increment=False)     # same call shape as the module
     feats = net([new_coords, new_features, batch], increment=True)
+    net = scn.compile(sparse_model, residual=True)               # also allows increment="residual"
 
 The module path issues one C call per layer from Python; this path hands the whole frame to
 one C call, so an incremental frame costs a few hundred kernel launches and no Python work.
@@ -21,7 +22,7 @@ _KIND = {"ssc": 0, "conv": 2, "deconv": 3, "nin": 4}
 
 
 class CompiledNet(object):
-    def __init__(self, model, capacity_sites=1 << 18):
+    def __init__(self, model, capacity_sites=1 << 18, residual=False):
         import sparseconvnet as scn
 
         mods = list(model)
@@ -46,6 +47,9 @@ class CompiledNet(object):
             x = self._trace(m, x)
         self.out_tensor = x
         self.out_channels = self._chan[x]
+        self.residual = bool(residual)
+        if self.residual:
+            lib.insc_net_enable_residual(self.h)
         lib.insc_net_finalize(self.h, int(x), I64(int(capacity_sites)), stream_ptr())
 
     def __del__(self):
@@ -129,8 +133,7 @@ class CompiledNet(object):
         coords, feats = input[0], input[1]
         from . import incremental
         if incremental.kind(increment) == "residual":
-            raise NotImplementedError("the compiled executor runs full and exact incremental frames; "
-                                      "residual frames go through the module tree")
+            return self._residual(coords, feats)
         increment = bool(increment)
         if all_points is None:
             all_points = (not increment) or self.output_layer.all_points
@@ -146,6 +149,21 @@ class CompiledNet(object):
                              int(bool(all_points)), ctypes.byref(n), stream_ptr())
         self.n_sites = int(n.value)
         self._timed = getattr(self, "_profiling", False)
+        return out
+
+    def _residual(self, coords, feats):
+        """The reference's own incremental frame (SCN.Incre_* semantics) in one C call: rows of
+        the frame's points only; the saved state is not touched."""
+        if not self.residual:
+            raise RuntimeError("compile the model with residual=True to run residual frames")
+        c = coords.to(device=self.device, dtype=torch.int32).contiguous()
+        f = feats.detach().to(device=self.device, dtype=torch.float32).contiguous()
+        P = c.size(0)
+        out = torch.empty((P, self.out_channels), dtype=torch.float32, device=self.device)
+        n = I64(0)
+        lib.insc_net_forward_residual(self.h, ptr(c), int(c.size(1)), ptr(f), I64(P), ptr(out), ctypes.byref(n),
+                                      stream_ptr())
+        self.n_sites_frame = int(n.value)
         return out
 
     def profile(self, enable=True):
@@ -164,5 +182,5 @@ class CompiledNet(object):
         return [int(v) for v in a]
 
 
-def compile(model, capacity_sites=1 << 18):
-    return CompiledNet(model, capacity_sites)
+def compile(model, capacity_sites=1 << 18, residual=False):
+    return CompiledNet(model, capacity_sites, residual)

@@ -279,3 +279,40 @@ def test_increment_true_follows_set_mode():
     assert torch.equal(got, want)
     with pytest.raises(ValueError):
         model(_inp(*f1), increment="approximate")
+
+
+@pytest.mark.parametrize("levels,m", [(3, 16), (7, 32)])
+def test_compiled_residual_frames_equal_module_tree(levels, m):
+    """The executor's residual frame (one C call) against the module tree's: same kernels on the
+    same rows, so the same bits.  With residual=True the executor also keeps the inputs of the
+    batch norms; full and exact incremental frames must not change because of that, and a
+    residual frame must leave the saved state as it was."""
+    import sparseconvnet as scn
+    from netdefs import NaiveUNet
+
+    f0, f1, _ = _frames(35)
+    model = NaiveUNet(m=m, levels=levels, seed=12).cuda()
+    ref_model = copy.deepcopy(model)
+    net = scn.compile(model.sparseModel, capacity_sites=4096, residual=True)
+    plain = scn.compile(copy.deepcopy(model).sparseModel, capacity_sites=4096)
+    with torch.no_grad():
+        full = net(_inp(*f0), increment=False)
+        assert torch.equal(full, ref_model.sparseModel(_inp(*f0), False))
+        want = ref_model.sparseModel(_inp(*f1), "residual")
+        got = net(_inp(*f1), increment="residual")
+        assert got.shape == want.shape == (len(f1[0]), m)
+        assert torch.equal(got, want), "max diff %.3e" % (got - want).abs().max().item()
+        assert net.n_sites_frame == len(np.unique(f1[0], axis=0))
+        # a smaller frame right after a larger one (the frame's buffers are reused)
+        half = (f1[0][:700], f1[1][:700])
+        assert torch.equal(net(_inp(*half), increment="residual"), ref_model.sparseModel(_inp(*half), "residual"))
+        # the saved state is intact: an exact incremental frame equals a full forward over both
+        exact = net(_inp(*f1), increment=True, all_points=True)
+        both = ref_model.sparseModel(_inp(np.concatenate([f0[0], f1[0]]), np.concatenate([f0[1], f1[1]])), False)
+        assert torch.equal(exact, both)
+        # and residual frames now refer to the state after that exact frame
+        want2 = ref_model.sparseModel(_inp(*half), "residual")
+        assert torch.equal(net(_inp(*half), increment="residual"), want2)
+        with pytest.raises(RuntimeError):
+            plain(_inp(*f0), increment=False)
+            plain(_inp(*f1), increment="residual")
