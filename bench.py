@@ -391,6 +391,30 @@ def main():
         extra = {"median_ms": round(float(np.median(per_frame)), 3),
                  "p95_ms": round(float(np.percentile(per_frame, 95)), 3),
                  "last_frame_ms": round(per_frame[-1], 3), "first_timed_frame_ms": round(per_frame[0], 3)}
+        # For comparison: the reference's own incremental mode (residual features on the frame's
+        # sites only - an approximation), last frame of the sweep against the scene of all earlier
+        # frames.  Its saved state never changes, so the same frame is simply repeated.
+        import sparseconvnet as scn
+
+        last = W + K
+        rnet = scn.compile(model.sparseModel, capacity_sites=1 << 18, residual=True)
+        seen = to_dev(np.concatenate([p for p, _ in seq[:last]]), np.concatenate([c for _, c in seq[:last]]), device)
+        with torch.no_grad():
+            rnet(seen, increment=False)
+            for _ in range(3):
+                model.linear(rnet(frames[last], increment="residual"))
+            torch.cuda.synchronize()
+            rt = []
+            for _ in range(20):
+                t1 = time.perf_counter()
+                model.linear(rnet(frames[last], increment="residual"))
+                torch.cuda.synchronize()
+                rt.append((time.perf_counter() - t1) * 1e3)
+        extra["residual_frame_ms"] = round(float(np.median(rt)), 3)
+        extra["residual_frame_note"] = ("reference-style residual frame (Incre_* semantics, approximate), %d points "
+                                        "on the %d-voxel saved scene, median of 20"
+                                        % (len(seq[last][0]), rnet.sites_per_level()[0]))
+        del rnet
         cpu_fn = cpu_baseline_unet
     elif args.workload == "unet":
         import scenes

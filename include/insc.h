@@ -193,6 +193,21 @@ int insc_input_finish(const float *d_sum, const int32_t *d_cnt, int mode, float 
  * CUDA/IOLayers.cpp:123-145: InputLayer_bp_ with multiplier 1). */
 int insc_output_gather(const float *d_in, int64_t ld_in, const int32_t *d_site_of_point, int64_t P, int C,
                        float *d_out, void *stream);
+/* Size-2 stride-2 pooling to the next coarser scale over the child map of insc_rulebook_down2:
+ * mode 0 = MaxPooling_updateOutput (CUDA/MaxPooling.cpp:18-36; the output starts at zero, so the
+ * result is max(0, max over the children)), mode 1 = AveragePooling_updateOutput
+ * (CUDA/AveragePooling.cpp:19-39: sum over the children divided by the filter volume 8).  The
+ * reference's nFeaturesToDrop is a pointer offset on d_in.  UnPooling_updateOutput
+ * (CUDA/UnPooling.cpp:17-37), out_fine[i] = in_coarse[parent[i]], is insc_output_gather with the
+ * parent map in place of site_of_point. */
+int insc_pool_down2(const float *d_in, int64_t ld_in, const int32_t *d_child, int64_t n_coarse, int C, int mode,
+                    float *d_out, int64_t ld_out, void *stream);
+/* Dense [batch, C, X, Y, Z] float32 copy (zero where no site is active) of the feature matrix of
+ * the grid's first n sites (SparseToDense_updateOutput, CUDA/SparseToDense.cpp:16-41; cell offset
+ * as RectangularRegion::offset, Metadata/RectangularRegions.h:52-60).  Sites outside the box or
+ * the batch range are skipped. */
+int insc_sparse_to_dense(const insc_grid *g, const float *d_in, int64_t ld_in, int64_t n, int C, int64_t X, int64_t Y,
+                         int64_t Z, int batch, float *d_out, void *stream);
 
 /* ---------------------------------------------------------------------------------------
  * Dirty-site propagation for the incremental forward.  Masks are uint8 per site.

@@ -3,6 +3,7 @@
 // thread owns a fixed group of four channels and walks rows, so loads and stores are
 // 16-byte wide and coalesced along a row.
 #include "common.h"
+#include "grid.h"
 
 namespace insc {
 
@@ -208,6 +209,48 @@ __global__ __launch_bounds__(256) void input_finish_kernel(const float *__restri
   }
 }
 
+// Size-2 stride-2 pooling over the child map: one thread per (coarse site, channel).
+//   MODE 0: max over the children, starting from zero (MaxPooling_fp, CUDA/MaxPooling.cu:10-33,
+//           on an output that cuda_MaxPooling_updateOutput has zeroed)
+//   MODE 1: sum over the children of x/8 in ascending offset order (AveragePooling_fp,
+//           CUDA/AveragePooling.cu:10-33 with alpha = 1/filterVolume, one launch per offset)
+template <int MODE>
+__global__ __launch_bounds__(256) void pool_down2_kernel(const float *__restrict__ in, int64_t ld_in,
+                                                         const int32_t *__restrict__ child, int64_t n_coarse, int C,
+                                                         float *__restrict__ out, int64_t ld_out) {
+  for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < n_coarse * C; e += (int64_t)gridDim.x * 256) {
+    const int64_t row = e / C;
+    const int c = (int)(e - row * C);
+    float acc = 0.0f;
+#pragma unroll
+    for (int k = 0; k < 8; k++) {
+      const int f = child[row * 8 + k];
+      if (f < 0) continue;
+      const float x = in[(int64_t)f * ld_in + c];
+      if (MODE == 0)
+        acc = (acc < x) ? x : acc;
+      else
+        acc += 0.125f * x;
+    }
+    out[row * ld_out + c] = acc;
+  }
+}
+
+// Dense [batch, C, X, Y, Z] copy of a sparse feature matrix (SparseToDense_fp,
+// CUDA/SparseToDense.cu:9-30; cell offset as RectangularRegion::offset, last axis fastest).
+__global__ __launch_bounds__(256) void sparse_to_dense_kernel(const float *__restrict__ in, int64_t ld_in,
+                                                              const int32_t *__restrict__ coords, int64_t n, int C,
+                                                              int64_t X, int64_t Y, int64_t Z, int batch,
+                                                              float *__restrict__ out) {
+  for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < n * C; e += (int64_t)gridDim.x * 256) {
+    const int64_t row = e / C;
+    const int c = (int)(e - row * C);
+    const int4 p = reinterpret_cast<const int4 *>(coords)[row];
+    if (p.x >= X || p.y >= Y || p.z >= Z || p.w >= batch) continue;
+    out[(((int64_t)p.w * C + c) * X + p.x) * Y * Z + (int64_t)p.y * Z + p.z] = in[row * ld_in + c];
+  }
+}
+
 static inline bool vec4_ok(const void *p, int64_t ld) { return ((uintptr_t)p % 16 == 0) && (ld % 4 == 0); }
 
 int launch_bn(const float *d_in, int64_t ld_in, float *d_out, int64_t ld_out, const float *d_mean, const float *d_var,
@@ -344,6 +387,37 @@ int insc_output_gather(const float *d_in, int64_t ld_in, const int32_t *d_site_o
   if (P == 0) return INSC_OK;
   hipLaunchKernelGGL(gather_rows_kernel, dim3(grid_for(P * C, 256, 1 << 16)), dim3(256), 0, (hipStream_t)stream, d_in,
                      ld_in, d_site_of_point, P, C, d_out);
+  INSC_LAUNCH_CHECK();
+  return INSC_OK;
+}
+
+int insc_pool_down2(const float *d_in, int64_t ld_in, const int32_t *d_child, int64_t n_coarse, int C, int mode,
+                    float *d_out, int64_t ld_out, void *stream) {
+  INSC_REQUIRE(n_coarse >= 0 && C > 0 && ld_in >= C && ld_out >= C && (mode == 0 || mode == 1), INSC_ERR_ARG,
+               "insc_pool_down2: bad arguments");
+  if (n_coarse == 0) return INSC_OK;
+  INSC_REQUIRE(d_in && d_child && d_out, INSC_ERR_ARG, "insc_pool_down2: null pointer");
+  const dim3 g(grid_for(n_coarse * C, 256, 1 << 16));
+  if (mode == 0)
+    hipLaunchKernelGGL(pool_down2_kernel<0>, g, dim3(256), 0, (hipStream_t)stream, d_in, ld_in, d_child, n_coarse, C,
+                       d_out, ld_out);
+  else
+    hipLaunchKernelGGL(pool_down2_kernel<1>, g, dim3(256), 0, (hipStream_t)stream, d_in, ld_in, d_child, n_coarse, C,
+                       d_out, ld_out);
+  INSC_LAUNCH_CHECK();
+  return INSC_OK;
+}
+
+int insc_sparse_to_dense(const insc_grid *g, const float *d_in, int64_t ld_in, int64_t n, int C, int64_t X, int64_t Y,
+                         int64_t Z, int batch, float *d_out, void *stream) {
+  INSC_REQUIRE(g && n >= 0 && n <= g->capacity_sites && C > 0 && ld_in >= C && X > 0 && Y > 0 && Z > 0 && batch > 0,
+               INSC_ERR_ARG, "insc_sparse_to_dense: bad arguments");
+  INSC_REQUIRE(d_out && (n == 0 || d_in), INSC_ERR_ARG, "insc_sparse_to_dense: null pointer");
+  hipStream_t s = (hipStream_t)stream;
+  INSC_HIP(hipMemsetAsync(d_out, 0, sizeof(float) * (size_t)batch * C * X * Y * Z, s));
+  if (n == 0) return INSC_OK;
+  hipLaunchKernelGGL(sparse_to_dense_kernel, dim3(grid_for(n * C, 256, 1 << 16)), dim3(256), 0, s, d_in, ld_in,
+                     g->coords, n, C, X, Y, Z, batch, d_out);
   INSC_LAUNCH_CHECK();
   return INSC_OK;
 }

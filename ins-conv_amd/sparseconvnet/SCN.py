@@ -687,6 +687,73 @@ def Incre_BatchNormalization_updateOutput(input_features, output_features, saveM
                                 int(C), stream_ptr())
 
 
+# =========================================================================================
+# size-2 stride-2 pooling, unpooling and the dense copy (siblings of the strided convolution:
+# they share its rulebook)
+# =========================================================================================
+def _pool(mode, inputSize, outputSize, poolSize, poolStride, m, input_features, output_features, nFeaturesToDrop):
+    _check_down(poolSize, poolStride)
+    input_features = _check_feats(input_features, "input_features")
+    fine, coarse, d = m.down_rulebook(inputSize, outputSize)
+    drop = int(nFeaturesToDrop)
+    C = input_features.size(1) - drop
+    if input_features.size(0) != fine.n or C <= 0:
+        raise ValueError("features do not match the active sites / nFeaturesToDrop too large")
+    _resize(output_features, coarse.n, C, input_features)
+    if coarse.n:
+        src = input_features[:, drop:]
+        lib.insc_pool_down2(ptr(src), I64(_ld(input_features)), ptr(d.child.t), I64(coarse.n), int(C), int(mode),
+                            ptr(output_features), I64(C), stream_ptr())
+
+
+def MaxPooling_updateOutput(inputSize, outputSize, poolSize, poolStride, m, input_features, output_features,
+                            nFeaturesToDrop):
+    """cuda_MaxPooling_updateOutput (CUDA/MaxPooling.cpp:18-36), size 2 / stride 2."""
+    _pool(0, inputSize, outputSize, poolSize, poolStride, m, input_features, output_features, nFeaturesToDrop)
+
+
+def AveragePooling_updateOutput(inputSize, outputSize, poolSize, poolStride, m, input_features, output_features,
+                                nFeaturesToDrop):
+    """cuda_AveragePooling_updateOutput (CUDA/AveragePooling.cpp:19-39), size 2 / stride 2."""
+    _pool(1, inputSize, outputSize, poolSize, poolStride, m, input_features, output_features, nFeaturesToDrop)
+
+
+def UnPooling_updateOutput(inputSize, outputSize, poolSize, poolStride, m, input_features, output_features,
+                           nFeaturesToDrop):
+    """cuda_UnPooling_updateOutput (CUDA/UnPooling.cpp:17-37): input is the coarse scale; every
+    fine site copies its parent's row."""
+    _check_down(poolSize, poolStride)
+    input_features = _check_feats(input_features, "input_features")
+    fine, coarse, d = m.down_rulebook(outputSize, inputSize)
+    drop = int(nFeaturesToDrop)
+    C = input_features.size(1) - drop
+    if input_features.size(0) != coarse.n or C <= 0:
+        raise ValueError("features do not match the active sites / nFeaturesToDrop too large")
+    _resize(output_features, fine.n, C, input_features)
+    if fine.n:
+        src = input_features[:, drop:]
+        lib.insc_output_gather(ptr(src), I64(_ld(input_features)), ptr(d.parent.t), I64(fine.n), int(C),
+                               ptr(output_features), stream_ptr())
+
+
+def SparseToDense_updateOutput(inputSize, m, input_features, output_features, nPlanes):
+    """cuda_SparseToDense_updateOutput (CUDA/SparseToDense.cpp:16-41): [batch, nPlanes, X, Y, Z]."""
+    input_features = _check_feats(input_features, "input_features")
+    sc = m.scale(inputSize)
+    X, Y, Z = _key(inputSize)
+    C = input_features.size(1)
+    if input_features.size(0) != sc.n or C != int(nPlanes):
+        raise ValueError("features do not match the active sites / nPlanes")
+    batch = int(sc.coords_view()[:, 3].max().item()) + 1 if sc.n else 1
+    if output_features.device != input_features.device or output_features.dtype != input_features.dtype:
+        output_features.data = torch.empty((batch, C, X, Y, Z), dtype=input_features.dtype,
+                                           device=input_features.device)
+    else:
+        output_features.resize_(batch, C, X, Y, Z)
+    lib.insc_sparse_to_dense(sc.grid, ptr(input_features), I64(_ld(input_features)), I64(sc.n), int(C), I64(X), I64(Y),
+                             I64(Z), int(batch), ptr(output_features), stream_ptr())
+
+
 def n_rulebook_bits():
     return 32
 

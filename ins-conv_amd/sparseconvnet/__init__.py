@@ -18,6 +18,7 @@ from .convolution import Convolution  # noqa: E402
 from .deconvolution import Deconvolution  # noqa: E402
 from .batchNormalization import BatchNormalization, BatchNormReLU, BatchNormLeakyReLU  # noqa: E402
 from .networkInNetwork import NetworkInNetwork  # noqa: E402
+from .pooling import MaxPooling, AveragePooling, UnPooling, SparseToDense  # noqa: E402
 from .networkArchitectures import UNet  # noqa: E402
 from .utils import (toLongTensor, optionalTensor, checkpoint_save, checkpoint_restore,  # noqa: E402
                     ssc_offset_permutation, convert_zmajor_state_dict)

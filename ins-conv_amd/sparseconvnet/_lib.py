@@ -40,6 +40,8 @@ _SIGS = {
     "insc_input_accumulate": [vp, c_i64, c_int, vp, c_int, vp, vp, c_i64, vp],
     "insc_input_finish": [vp, vp, c_int, vp, c_i64, vp, vp, c_i64, c_int, vp],
     "insc_output_gather": [vp, c_i64, vp, c_i64, c_int, vp, vp],
+    "insc_pool_down2": [vp, c_i64, vp, c_i64, c_int, c_int, vp, c_i64, vp],
+    "insc_sparse_to_dense": [vp, vp, c_i64, c_i64, c_int, c_i64, c_i64, c_i64, c_int, vp, vp],
     "insc_fill_u8": [vp, c_i64, c_int, vp],
     "insc_fill_i32": [vp, c_i64, ctypes.c_int32, vp],
     "insc_dirty_mark": [vp, c_i64, vp, vp],

@@ -280,6 +280,44 @@ def incre_deconv_forward(feats, pre_in, W, bias, parent, offset, pre_exist_in, p
 
 
 # --------------------------------------------------------------------------------------
+# size-2 stride-2 pooling, unpooling, dense copy (numpy).  Pinned in tests/test_oracle_pool.py
+# against torch max_pool3d / avg_pool3d / nearest upsampling on dense tensors and against
+# torch.sparse_coo_tensor(...).to_dense().
+# --------------------------------------------------------------------------------------
+def max_pool_forward(feats, parent, n_coarse, drop=0):
+    """MaxPooling_ForwardPass on a zeroed output (CPU/MaxPooling.cpp:7-20, 38-57): max(0, children)."""
+    f = _f(feats)[:, drop:]
+    out = np.zeros((n_coarse, f.shape[1]), np.float32)
+    np.maximum.at(out, np.asarray(parent), f)
+    return out
+
+
+def avg_pool_forward(feats, parent, offset, n_coarse, drop=0):
+    """AveragePooling_ForwardPass (CPU/AveragePooling.cpp:7-21): sum over the children of x / 8, the
+    rules of offset 0 first, then 1, ... (one pass per offset)."""
+    f = _f(feats)[:, drop:]
+    out = np.zeros((n_coarse, f.shape[1]), np.float32)
+    parent, offset = np.asarray(parent), np.asarray(offset)
+    for k in range(8):
+        sel = offset == k
+        out[parent[sel]] += np.float32(0.125) * f[sel]  # one child per (parent, offset): no repeats
+    return out
+
+
+def unpool_forward(feats, parent, drop=0):
+    """UnPooling_ForwardPass (CPU/UnPooling.cpp:7-20): every fine site takes its parent's row."""
+    return _f(feats)[:, drop:][np.asarray(parent)].copy()
+
+
+def sparse_to_dense(feats, site_coords, size, batch):
+    """SparseToDense_ForwardPass (CPU/SparseToDense.cpp:7-19): [batch, C, X, Y, Z], zeros elsewhere."""
+    f, c = _f(feats), _c4(site_coords)
+    out = np.zeros((batch, f.shape[1]) + tuple(size), np.float32)
+    out[c[:, 3], :, c[:, 0], c[:, 1], c[:, 2]] = f
+    return out
+
+
+# --------------------------------------------------------------------------------------
 # canonical forms used to compare integer structures bit-exactly
 # --------------------------------------------------------------------------------------
 def canonical_sites(site_coords):
