@@ -115,11 +115,11 @@ def conv_roofline(device, reps=30, warm=200):
     achieved = bytes_alg / t / 1e9
     return {
         "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-        "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": 639.1e6,
+        "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": 639.8e6,
         "kernel": "conv_wlds_kernel (SSC 3^3, 32->32, filter in LDS, persistent blocks; 500k sites, %d rules)" % n_rules,
         "avg_us": round(t * 1e6, 1), "algorithmic_bytes": int(bytes_alg),
         "traffic_note": "HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE (x1.999, copy-kernel calibration) + "
-                        "WRITE_SIZE (x1.000): 541.3 MB + 97.8 MB, profiles/conv_wlds_ssc32_500k.txt",
+                        "WRITE_SIZE (x1.000): 541.9 MB + 97.8 MB, profiles/conv_wlds_ssc32_500k.txt",
         "mfma_tflops": round(flops / t / 1e12, 2), "mfma_frac": round(flops / t / 1e12 / MFMA_FP32_PEAK_TFLOPS, 4),
         "ssc_msites_per_s": round(sc.n / t / 1e6, 1),
     }
@@ -252,6 +252,34 @@ def unet_model(device):
     return model, scn.compile(model.sparseModel, capacity_sites=1 << 18)
 
 
+def residual_row(model, seq, frames, last, device):
+    """For comparison: the reference's own incremental mode (residual features on the frame's sites
+    only - an approximation), frame `last` of the sweep against the scene of all earlier frames.
+    Its saved state never changes, so the same frame is simply repeated."""
+    import numpy as np
+    import torch
+
+    import sparseconvnet as scn
+
+    rnet = scn.compile(model.sparseModel, capacity_sites=1 << 18, residual=True)
+    seen = to_dev(np.concatenate([p for p, _ in seq[:last]]), np.concatenate([c for _, c in seq[:last]]), device)
+    with torch.no_grad():
+        rnet(seen, increment=False)
+        for _ in range(3):
+            model.linear(rnet(frames[last], increment="residual"))
+        torch.cuda.synchronize()
+        rt = []
+        for _ in range(20):
+            t1 = time.perf_counter()
+            model.linear(rnet(frames[last], increment="residual"))
+            torch.cuda.synchronize()
+            rt.append((time.perf_counter() - t1) * 1e3)
+    return {"residual_frame_ms": round(float(np.median(rt)), 3),
+            "residual_frame_note": "reference-style residual frame (Incre_* semantics, approximate), %d points on "
+                                   "the %d-voxel saved scene, median of 20"
+                                   % (len(seq[last][0]), rnet.sites_per_level()[0])}
+
+
 def to_dev(pts, rgb, device):
     import numpy as np
     import torch
@@ -323,6 +351,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=None)
     ap.add_argument("--workload", default="incr", choices=["incr", "unet", "ssc"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-residual", action="store_true",
+                    help="skip the residual-frame comparison row of the incremental workload")
+    ap.add_argument("--residual-only", action="store_true",
+                    help="run only the residual-frame comparison row (short; used under rocprofv3)")
     ap.add_argument("--kernels-only", action="store_true",
                     help="print only the table of bandwidth-bound kernels")
     ap.add_argument("--roofline-only", action="store_true",
@@ -342,6 +374,14 @@ def main():
     if args.kernels_only:
         print(json.dumps({"kernels": kernel_table(device)}))
         return
+    if args.residual_only:
+        import scenes
+
+        seq = scenes.sweep_sequence()
+        model, _ = unet_model(device)
+        frames = [to_dev(p, c, device) for p, c in seq]
+        print(json.dumps(residual_row(model, seq, frames, len(seq) - 1, device)))
+        return
     if args.roofline_only:
         # plus a plain copy of known size (500k x 32 floats: 64 MB read, 64 MB written), the
         # yardstick the FETCH_SIZE / WRITE_SIZE counters of the same run are scaled by
@@ -352,7 +392,7 @@ def main():
         for _ in range(5):
             SCN.copy_rows(a, b, None, None, a.size(0))
         torch.cuda.synchronize()
-        print(json.dumps({"roofline": conv_roofline(device, reps=10, warm=3)}))
+        print(json.dumps({"roofline": conv_roofline(device)}))
         return
 
     extra = {}
@@ -391,30 +431,8 @@ def main():
         extra = {"median_ms": round(float(np.median(per_frame)), 3),
                  "p95_ms": round(float(np.percentile(per_frame, 95)), 3),
                  "last_frame_ms": round(per_frame[-1], 3), "first_timed_frame_ms": round(per_frame[0], 3)}
-        # For comparison: the reference's own incremental mode (residual features on the frame's
-        # sites only - an approximation), last frame of the sweep against the scene of all earlier
-        # frames.  Its saved state never changes, so the same frame is simply repeated.
-        import sparseconvnet as scn
-
-        last = W + K
-        rnet = scn.compile(model.sparseModel, capacity_sites=1 << 18, residual=True)
-        seen = to_dev(np.concatenate([p for p, _ in seq[:last]]), np.concatenate([c for _, c in seq[:last]]), device)
-        with torch.no_grad():
-            rnet(seen, increment=False)
-            for _ in range(3):
-                model.linear(rnet(frames[last], increment="residual"))
-            torch.cuda.synchronize()
-            rt = []
-            for _ in range(20):
-                t1 = time.perf_counter()
-                model.linear(rnet(frames[last], increment="residual"))
-                torch.cuda.synchronize()
-                rt.append((time.perf_counter() - t1) * 1e3)
-        extra["residual_frame_ms"] = round(float(np.median(rt)), 3)
-        extra["residual_frame_note"] = ("reference-style residual frame (Incre_* semantics, approximate), %d points "
-                                        "on the %d-voxel saved scene, median of 20"
-                                        % (len(seq[last][0]), rnet.sites_per_level()[0]))
-        del rnet
+        if not args.no_residual:
+            extra.update(residual_row(model, seq, frames, W + K, device))
         cpu_fn = cpu_baseline_unet
     elif args.workload == "unet":
         import scenes
