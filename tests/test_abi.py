@@ -71,3 +71,64 @@ def test_module_api_surface():
     assert n_ssc == 4 * 3 + 4 * 2  # 4 per level on the way down, 4 per non-bottom level on the way up
     w = scn.SubmanifoldConvolution(3, 16, 24, 3, False).weight
     assert tuple(w.shape) == (27, 16, 24)
+
+
+def test_scn_function_surface():
+    """The native-extension functions of the reference that this path covers
+    (sparseconvnet/SCN/pybind.cpp:153-258) exist with the reference's argument counts."""
+    import inspect
+
+    from sparseconvnet import SCN
+
+    expect = {
+        "InputLayer_updateOutput": 7, "OutputLayer_updateOutput": 3, "SubmanifoldConvolution_updateOutput": 8,
+        "Convolution_updateOutput": 9, "Deconvolution_updateOutput": 9, "BatchNormalization_updateOutput": 12,
+        "NetworkInNetwork_updateOutput": 4, "Incre_InputLayer_updateOutput": 9, "Incre_OutputLayer_updateOutput": 5,
+        "Incre_SubmanifoldConvolution_updateOutput": 9, "Incre_Convolution_updateOutput": 9,
+        "Incre_Deconvolution_updateOutput": 11, "Incre_BatchNormalization_updateOutput": 17,
+        "MaxPooling_updateOutput": 8, "AveragePooling_updateOutput": 8, "UnPooling_updateOutput": 8,
+        "SparseToDense_updateOutput": 5,
+    }
+    for name, n in expect.items():
+        params = [p for p in inspect.signature(getattr(SCN, name)).parameters.values()
+                  if p.default is inspect.Parameter.empty or p.name == "dilated_rate"]
+        assert len(params) == n, (name, [p.name for p in params])
+    for name in ("Metadata_3", "Result_3", "ResultOfWeight", "n_rulebook_bits"):
+        assert hasattr(SCN, name)
+
+
+def test_residual_entry_points_validate_before_touching_the_device():
+    from sparseconvnet import _lib
+
+    lib = _lib.cdll()
+    assert lib.insc_incre_input(None, None, 7, None, None, 0, None, None, 0, 1, 1, None) == -1
+    assert b"insc_incre_input" in lib.insc_last_error()
+    assert lib.insc_incre_bn_leaky(None, 1, None, 1, None, None, None, None, 0.0, 0.0, None, None, 1, None, 1, -1, 1,
+                                   None) == -1
+    assert lib.insc_incre_conv_ssc(None, 4, None, 4, 0, None, 4, None, None, None, None, None, 5, 4, 4, None) == -1
+    assert b"null pointer" in lib.insc_last_error()
+    assert lib.insc_pool_down2(None, 4, None, 3, 4, 2, None, 4, None) == -1
+    assert lib.insc_incre_rulebook_ssc3(None, None, None, 0, None, None) == -1
+    assert lib.insc_net_forward_residual(None, None, 3, None, 0, None, None, None) == -4
+    assert lib.insc_net_enable_residual(None) == -4
+
+
+def test_incremental_mode_switch():
+    import pytest
+
+    import sparseconvnet as scn
+    from sparseconvnet import incremental
+
+    assert scn.get_incremental_mode() == "exact"
+    assert incremental.kind(False) is None and incremental.kind(True) == "exact"
+    assert incremental.kind("residual") == "residual"
+    scn.set_incremental_mode("residual")
+    try:
+        assert incremental.kind(True) == "residual" and incremental.kind(0) is None
+        assert incremental.kind("exact") == "exact"
+    finally:
+        scn.set_incremental_mode("exact")
+    with pytest.raises(ValueError):
+        scn.set_incremental_mode("fast")
+    with pytest.raises(ValueError):
+        incremental.kind("yes")
