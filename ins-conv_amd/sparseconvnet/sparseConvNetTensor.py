@@ -1,48 +1,46 @@
-"""SparseConvNetTensor (reference: sparseconvnet/sparseConvNetTensor.py).
+"""SparseConvNetTensor: a feature matrix, the Metadata that says which sites its rows belong to,
+and the spatial size of the scale (reference: sparseconvnet/sparseConvNetTensor.py).
 
-`dirty` is an addition: during an incremental forward it names the rows of `features` that
-changed in this frame (None during a full forward).
+`dirty` is an addition: during an exact incremental forward it names the rows of `features`
+that changed in this frame (None otherwise).
 """
 
 
 class SparseConvNetTensor(object):
     def __init__(self, features=None, metadata=None, spatial_size=None):
-        self.features = features
-        self.metadata = metadata
-        self.spatial_size = spatial_size
+        self.features, self.metadata, self.spatial_size = features, metadata, spatial_size
         self.dirty = None
 
-    def get_spatial_locations(self, spatial_size=None):
-        "Coordinates and batch index for the active spatial locations"
-        if spatial_size is None:
-            spatial_size = self.spatial_size
-        return self.metadata.getSpatialLocations(spatial_size)
-
-    def to(self, device):
-        self.features = self.features.to(device)
+    def _with_features(self, fn):
+        self.features = fn(self.features)
         return self
 
-    def type(self, t=None):
-        if t:
-            self.features = self.features.type(t)
-            return self
-        return self.features.type()
+    # torch.Tensor-like movers; each works in place on `features` and returns self
+    def to(self, device):
+        return self._with_features(lambda f: f.to(device))
 
     def cuda(self):
-        self.features = self.features.cuda()
-        return self
+        return self._with_features(lambda f: f.cuda())
 
     def cpu(self):
-        self.features = self.features.cpu()
-        return self
+        return self._with_features(lambda f: f.cpu())
+
+    def type(self, t=None):
+        if not t:
+            return self.features.type()
+        return self._with_features(lambda f: f.type(t))
 
     def detach(self):
-        x = SparseConvNetTensor(self.features.detach(), self.metadata, self.spatial_size)
-        x.dirty = self.dirty
-        return x
+        out = SparseConvNetTensor(self.features.detach(), self.metadata, self.spatial_size)
+        out.dirty = self.dirty
+        return out
+
+    def get_spatial_locations(self, spatial_size=None):
+        """Long [N,4] (x, y, z, batch index) of the active sites, rows in feature order."""
+        size = self.spatial_size if spatial_size is None else spatial_size
+        return self.metadata.getSpatialLocations(size)
 
     def __repr__(self):
-        sl = self.get_spatial_locations() if self.metadata else None
-        return ('SparseConvNetTensor<<features=' + repr(self.features) + ',features.shape=' +
-                repr(self.features.shape) + ',batch_locations=' + repr(sl) + ',spatial size=' +
-                repr(self.spatial_size) + '>>')
+        where = self.get_spatial_locations() if self.metadata else None
+        return "SparseConvNetTensor<<features=%r,features.shape=%r,batch_locations=%r,spatial size=%r>>" % (
+            self.features, self.features.shape, where, self.spatial_size)

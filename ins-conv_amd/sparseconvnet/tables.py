@@ -1,4 +1,5 @@
-"""JoinTable / AddTable / ConcatTable (reference: sparseconvnet/tables.py:13-48)."""
+"""JoinTable / AddTable / ConcatTable (reference: sparseconvnet/tables.py:13-48) and the
+pass-through branch of a ConcatTable, Identity (sparseconvnet/identity.py)."""
 import torch
 
 from . import SCN, incremental
@@ -95,3 +96,14 @@ class ConcatTable(torch.nn.Sequential):
 
     def input_spatial_size(self, out_size):
         return self._modules['0'].input_spatial_size(out_size)
+
+
+class Identity(torch.nn.Module):
+    """The skip branch of a residual block or of a U-Net scale: hands its input on, whatever the
+    kind of forward."""
+
+    def forward(self, input, increment=False):
+        return input
+
+    def input_spatial_size(self, out_size):
+        return out_size
