@@ -518,6 +518,7 @@ __global__ __launch_bounds__((S == 1 ? CONV_WAVES : S) * 64) void conv_mfma_kern
 // ---------------------------------------------------------------------------------------
 constexpr int WL_WAVES = 12;
 constexpr int WL_DEPTH = 4;
+constexpr int WL_SCHED = 256;  // a block orders up to this many tiles of its own by cost
 
 __global__ __launch_bounds__(WL_WAVES * 64) void conv_wlds_kernel(
     const float *__restrict__ in, int64_t ld_in, float *__restrict__ out, int64_t ld_out,
@@ -529,6 +530,7 @@ __global__ __launch_bounds__(WL_WAVES * 64) void conv_wlds_kernel(
   __shared__ __attribute__((aligned(16))) float wl[K * 1024];
   __shared__ int nbl[WL_WAVES][TILE_M * K];
   __shared__ int next_turn;
+  __shared__ int cost_l[WL_SCHED], sched_l[WL_SCHED];
   const int64_t n = d_n_rows ? min((int64_t)*d_n_rows, n_rows) : n_rows;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int r = lane & 31, h = lane >> 5;
@@ -540,9 +542,37 @@ __global__ __launch_bounds__(WL_WAVES * 64) void conv_wlds_kernel(
     for (int i = threadIdx.x; i < K * 256; i += WL_WAVES * 64) dst[i] = src[i];
   }
   if (threadIdx.x == 0) next_turn = 0;
-  __syncthreads();
-
   const int64_t ntiles = (n + TILE_M - 1) / TILE_M;
+  // Blocks are dealt to the eight XCDs round robin (block b runs on XCD b % 8) and every XCD has an
+  // L2 of its own: rank the blocks XCD by XCD, so that the tiles an XCD works on at any time are
+  // neighbours in the processing order and share gathered rows in its L2.
+  const int G8 = gridDim.x >> 3;
+  const int brank = (gridDim.x & 7) == 0 ? (int)(blockIdx.x & 7) * G8 + (int)(blockIdx.x >> 3) : (int)blockIdx.x;
+  // The block of rank q owns the tiles q, q + gridDim.x, ...  With a tile plan it takes them most
+  // expensive first (cost = offsets the tile uses; ties in tile order): its wavefronts then finish
+  // within a cheap tile of each other instead of an average one.
+  const int my_tiles = ntiles > brank ? (int)((ntiles - brank + gridDim.x - 1) / gridDim.x) : 0;
+  const bool lpt = plan.map != nullptr && my_tiles > WL_WAVES && my_tiles <= WL_SCHED;
+  if (lpt) {
+    for (int j = threadIdx.x; j < my_tiles; j += WL_WAVES * 64) {
+      const int64_t tt = (int64_t)j * gridDim.x + brank;
+      cost_l[j] = (!tile_flags || tile_flags[tt]) ? __builtin_popcount(plan.tmask[tt]) : -1;
+    }
+  }
+  __syncthreads();
+  if (lpt) {
+    for (int j = threadIdx.x; j < my_tiles; j += WL_WAVES * 64) {
+      const int c = cost_l[j];
+      int rank = 0;
+      for (int i = 0; i < my_tiles; i++) {
+        const int ci = cost_l[i];
+        rank += (ci > c || (ci == c && i < j)) ? 1 : 0;
+      }
+      sched_l[rank] = j;
+    }
+    __syncthreads();
+  }
+
   int *nl = nbl[wave];
   const __amdgpu_buffer_rsrc_t rin = make_rsrc(in, in_bytes), rmap = make_rsrc(map0, map_bytes);
   // the outputs are addressed with 32-bit byte offsets as well; rows that do not exist get an
@@ -555,15 +585,16 @@ __global__ __launch_bounds__(WL_WAVES * 64) void conv_wlds_kernel(
   const float ew = (ep.out2 && col < Cout) ? ep.w[col] : 0.0f;
   const float eb = (ep.out2 && col < Cout) ? ep.b[col] : 0.0f;
 
-  // Block b owns the tiles b, b + gridDim.x, ...; its wavefronts draw them from a counter in LDS
+  // The wavefronts of a block draw its tiles from a counter in LDS
   // (tile costs differ by 3x: a fixed deal per wavefront leaves the slowest one far behind).
   // draw(): the next tile of this block that has work, or ntiles.
   auto draw = [&]() -> int64_t {
     for (;;) {
       int v = 0;
       if (lane == 0) v = atomicAdd(&next_turn, 1);
-      const int64_t t = (int64_t)__builtin_amdgcn_readfirstlane(v) * gridDim.x + blockIdx.x;
-      if (t >= ntiles) return ntiles;
+      const int turn = __builtin_amdgcn_readfirstlane(v);
+      if (turn >= my_tiles) return ntiles;
+      const int64_t t = (int64_t)(lpt ? sched_l[turn] : turn) * gridDim.x + brank;
       if (!tile_flags || tile_flags[t]) return t;
     }
   };
