@@ -1,0 +1,142 @@
+"""Edge cases of the path on the GPU: several scenes in one batch, sites on the border of the
+coordinate range, empty and duplicate-only increments, residual frames that share nothing or
+everything with the saved scene."""
+import copy
+
+import numpy as np
+import pytest
+import torch
+
+import scenes
+
+pytestmark = pytest.mark.gpu
+
+
+def _inp(pts, rgb, bs=1):
+    return [torch.from_numpy(pts.astype(np.int64)), torch.from_numpy(rgb).cuda(), bs]
+
+
+def _scene(seed, n=5000):
+    vox = scenes.indoor_scene(seed=seed, n=n, dims=(60, 50, 20), n_boxes=5, side_rng=(6, 14))
+    rgb = np.random.default_rng(seed).uniform(0, 1, (len(vox), 3)).astype(np.float32)
+    return vox, rgb
+
+
+def test_batch_of_scenes_equals_scenes_run_alone():
+    """Two scenes with batch indices 0 and 1 (overlapping coordinates): nothing may leak across the
+    batch index - each scene's logits equal those of the scene run alone, bit for bit - and the
+    whole batch matches the oracle."""
+    import oracle_net
+    from netdefs import NaiveUNet
+
+    (va, fa), (vb, fb) = _scene(41), _scene(42, 4000)
+    vb = vb.copy()
+    vb[:, 3] = 1
+    rng = np.random.default_rng(43)
+    perm = rng.permutation(len(va) + len(vb))
+    pts, rgb = np.concatenate([va, vb])[perm], np.concatenate([fa, fb])[perm]
+    model = NaiveUNet(m=16, levels=4, seed=13).cuda()
+    cpu = copy.deepcopy(model).cpu()
+    with torch.no_grad():
+        both = model.sparseModel(_inp(pts, rgb, 2))
+        alone_a = model.sparseModel(_inp(va, fa))
+        alone_b = model.sparseModel(_inp(vb[:, :3], fb))
+    inv = np.argsort(perm)
+    assert torch.equal(both[inv[:len(va)]], alone_a)
+    assert torch.equal(both[inv[len(va):]], alone_b)
+    ref = oracle_net.forward(cpu.sparseModel, [pts, rgb, 2])
+    scale = max(1.0, float(np.abs(ref).max()))
+    np.testing.assert_allclose(both.cpu().numpy(), ref, rtol=1e-4, atol=1e-5 * scale)
+
+
+def test_sites_on_the_border_of_the_coordinate_range(orc):
+    """Voxels at 0 and 65535: their neighbours outside the range do not exist (and must not alias
+    voxels on the other side)."""
+    from sparseconvnet import SCN
+
+    rng = np.random.default_rng(44)
+    lo = np.stack(np.meshgrid(np.arange(0, 6), np.arange(0, 6), np.arange(0, 3), indexing="ij"), -1).reshape(-1, 3)
+    hi = 65535 - lo
+    mid = np.array([[65535, 0, 7], [0, 65535, 7], [32768, 32768, 32768]])
+    pts = np.concatenate([lo, hi, mid]).astype(np.int32)
+    pts = np.concatenate([pts, np.zeros((len(pts), 1), np.int32)], 1)[rng.permutation(len(pts))]
+    f = rng.normal(size=(len(pts), 16)).astype(np.float32)
+    size = torch.LongTensor([65536] * 3)
+    m = SCN.Metadata_3()
+    feats = torch.empty(0, device="cuda")
+    SCN.InputLayer_updateOutput(m, size, torch.from_numpy(pts.astype(np.int64)), torch.from_numpy(f).cuda(), feats, 0, 0)
+    W = (rng.normal(size=(27, 16, 16)) * 0.1).astype(np.float32)
+    out = torch.empty(0, device="cuda")
+    SCN.SubmanifoldConvolution_updateOutput(size, torch.LongTensor([3, 3, 3]), m, feats, out,
+                                            torch.from_numpy(W).cuda(), torch.Tensor(), 1)
+    nbr, counts, pairs = orc.ssc_rules(pts)
+    assert (m.ssc_rulebook(size).nbr.t[:len(pts)].cpu().numpy() == nbr).all()
+    ref, _ = orc.conv_forward(f, W, None, pairs, counts, len(pts))
+    np.testing.assert_allclose(out.cpu().numpy(), ref, rtol=1e-4, atol=1e-5)
+    # the stride-2 scale of the corner voxels
+    out2 = torch.empty(0, device="cuda")
+    W2 = (rng.normal(size=(8, 16, 16)) * 0.2).astype(np.float32)
+    SCN.Convolution_updateOutput(size, torch.LongTensor([32768] * 3), torch.LongTensor([2] * 3),
+                                 torch.LongTensor([2] * 3), m, feats, out2, torch.from_numpy(W2).cuda(), torch.Tensor())
+    parent, off, cc = orc.down2_rules(pts)
+    c2, p2 = orc.down2_pairs(parent, off)
+    ref2, _ = orc.conv_forward(f, W2, None, p2, c2, len(cc))
+    np.testing.assert_allclose(out2.cpu().numpy(), ref2, rtol=1e-4, atol=1e-5)
+
+
+def test_empty_and_duplicate_only_increments():
+    """An increment of zero points, one that only repeats points already seen, and one that only
+    re-observes old voxels with new colours: the executor must stay equal to a full forward."""
+    import sparseconvnet as scn
+    from netdefs import NaiveUNet
+
+    vox, rgb = _scene(45)
+    model = NaiveUNet(m=16, levels=4, seed=14).cuda()
+    ref_model = copy.deepcopy(model)
+    net = scn.compile(model.sparseModel, capacity_sites=8192)
+    n0 = 3500
+    with torch.no_grad():
+        base = net(_inp(vox[:n0], rgb[:n0]), increment=False)
+        out = net(_inp(vox[:0], rgb[:0]), increment=True, all_points=True)
+        assert torch.equal(out, base)
+        assert net(_inp(vox[:0], rgb[:0]), increment=True).shape == (0, 16)
+        # the same points again: means unchanged, no new sites
+        out = net(_inp(vox[:500], rgb[:500]), increment=True, all_points=True)
+        allp, allf = np.concatenate([vox[:n0], vox[:500]]), np.concatenate([rgb[:n0], rgb[:500]])
+        assert torch.equal(out, ref_model.sparseModel(_inp(allp, allf)))
+        assert net.sites_per_level()[0] == n0
+        # old voxels, new colours
+        rng = np.random.default_rng(46)
+        idx = rng.integers(0, n0, 300)
+        f2 = rng.uniform(0, 1, (300, 3)).astype(np.float32)
+        out = net(_inp(vox[idx], f2), increment=True, all_points=True)
+        allp, allf = np.concatenate([allp, vox[idx]]), np.concatenate([allf, f2])
+        assert torch.equal(out, ref_model.sparseModel(_inp(allp, allf)))
+        # and finally new voxels
+        out = net(_inp(vox[n0:], rgb[n0:]), increment=True, all_points=True)
+        allp, allf = np.concatenate([allp, vox[n0:]]), np.concatenate([allf, rgb[n0:]])
+        assert torch.equal(out, ref_model.sparseModel(_inp(allp, allf)))
+
+
+def test_residual_frames_disjoint_from_and_inside_the_saved_scene():
+    """A residual frame far away from the saved scene is a plain forward over its own points; one
+    made only of saved voxels with unchanged colours has residual zero, so it returns the saved
+    rows."""
+    import sparseconvnet as scn
+    from netdefs import NaiveUNet
+
+    vox, rgb = _scene(47)
+    model = NaiveUNet(m=16, levels=4, seed=15).cuda()
+    ref_model = copy.deepcopy(model)
+    net = scn.compile(model.sparseModel, capacity_sites=8192, residual=True)
+    far = vox[:1500].copy()
+    far[:, :3] += 1500
+    with torch.no_grad():
+        saved = net(_inp(vox, rgb), increment=False)
+        got = net(_inp(far, rgb[:1500]), increment="residual")
+        alone = ref_model.sparseModel(_inp(far, rgb[:1500]))
+        assert torch.equal(got, alone)
+        # saved voxels, same colours, one point per voxel: mean unchanged -> residual 0
+        idx = np.random.default_rng(48).permutation(len(vox))[:1200]
+        got = net(_inp(vox[idx], rgb[idx]), increment="residual")
+    np.testing.assert_allclose(got.cpu().numpy(), saved[idx].cpu().numpy(), rtol=0, atol=2e-5)
