@@ -518,6 +518,7 @@ __global__ __launch_bounds__((S == 1 ? CONV_WAVES : S) * 64) void conv_mfma_kern
 // ---------------------------------------------------------------------------------------
 constexpr int WL_WAVES = 12;
 constexpr int WL_DEPTH = 4;
+constexpr int WL_MIN_TILES = 4096;  // smaller launches go to conv_mfma_kernel
 constexpr int WL_SCHED = 256;  // a block orders up to this many tiles of its own by cost
 
 __global__ __launch_bounds__(WL_WAVES * 64) void conv_wlds_kernel(
@@ -867,7 +868,11 @@ int launch_conv(const float *in, int64_t ld_in, int64_t in_rows, float *out, int
     const bool small_ids = in_rows < (1 << 24) && out_rows < (1 << 24) && ld_out * 4 < (1 << 24) &&
                            ep.ld2 * 4 < (1 << 24) && out_rows * ld_out * 4 < (int64_t)BUF_OOB &&
                            out_rows * ep.ld2 * 4 < (int64_t)BUF_OOB;
-    if (mode == MAP_NBR && K == 27 && Cin <= 32 && Cout <= 32 && map_bytes64 < (int64_t)BUF_OOB && small_ids) {
+    // (below some four thousand tiles the persistent kernel's start-up - every block copies the
+    // whole filter into LDS - costs more than it saves: 34 us against 21 us at 32k sites, even at
+    // 150k; both kernels give the same bits)
+    if (mode == MAP_NBR && K == 27 && Cin <= 32 && Cout <= 32 && map_bytes64 < (int64_t)BUF_OOB && small_ids &&
+        tiles >= WL_MIN_TILES) {
       const uint32_t map_bytes = (uint32_t)map_bytes64;
       // persistent blocks, a multiple of the XCD count, at most one per compute unit
       const int64_t want = cdiv(tiles, WL_WAVES);

@@ -53,6 +53,8 @@ int order_append_new_sites_sorted(const insc_grid *g, const int32_t *d_nbr, int3
                                   int64_t n_new_upper, hipStream_t s);
 int order_append_new_sites_by_offset(const insc_grid *g, const int32_t *d_offset, const int32_t *d_pos_in_order,
                                      int32_t *d_order, int32_t *d_pos, int64_t n_new_upper, hipStream_t s);
+// most sites the two sorted appends put in order (more keep their arrival order)
+int64_t order_sorted_max();
 // device pointer to the site count before the most recent insert
 static inline const int32_t *grid_n_prev_ptr(const insc_grid *g) { return g->d_n + 1; }
 

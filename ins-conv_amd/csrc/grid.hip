@@ -532,6 +532,8 @@ int order_append_new_sites(const insc_grid *g, int32_t *d_order, int32_t *d_pos,
   return INSC_OK;
 }
 
+int64_t order_sorted_max() { return SORT_NEW_MAX; }
+
 int order_append_new_sites_sorted(const insc_grid *g, const int32_t *d_nbr, int32_t *d_order, int32_t *d_pos,
                                   int64_t n_new_upper, hipStream_t s) {
   if (n_new_upper <= 0) return INSC_OK;

@@ -936,6 +936,15 @@ int insc_net_forward(insc_net *net, const int32_t *d_coords, int coord_cols, con
     for (int l = 0; l < L; l++) {
       Level &Lv = net->levels[l];
       if (Lv.n == 0) continue;
+      if (Lv.n <= order_sorted_max()) {
+        // a small scale: all its sites came with this frame's one insert, and the single-workgroup
+        // sorts of the incremental path order them in two launches instead of some fifty
+        if ((rc = order_append_new_sites_sorted(Lv.grid, Lv.nbr, Lv.order, Lv.pos, Lv.n, s))) return rc;
+        if (l + 1 < L)
+          if ((rc = order_append_new_sites_by_offset(Lv.grid, Lv.offset, Lv.pos, Lv.bo_order, Lv.bo_pos, Lv.n, s)))
+            return rc;
+        continue;
+      }
       if ((rc = insc_order_build(Lv.grid, Lv.nbr, 0, Lv.n, Lv.order, stream))) return rc;
       hipLaunchKernelGGL(invert_perm_kernel, dim3(grid_for(Lv.n, 256)), dim3(256), 0, s, Lv.order, Lv.n, Lv.pos);
       if (l + 1 < L) {

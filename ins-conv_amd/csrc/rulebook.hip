@@ -37,11 +37,13 @@ __device__ __forceinline__ uint64_t spread3(uint64_t v) {  // 12 bits -> every t
   return v;
 }
 
-// sort key: batch (7 bits) | Morton code of the 64^3 block (30 bits) | neighbour pattern (27 bits).
-// Sites with the same pattern inside a block end up in the same tiles, so a tile skips the
-// offsets none of its rows has; larger blocks give purer tiles (the gather locality they cost
-// matters less than the matrix-core work they save).  The order is a heuristic only: batches
-// beyond 127 share groups, which is harmless.
+// sort key, 40 bits (five 8-bit radix passes): batch parity | Morton code of the 64^3 block, four
+// bits per axis | neighbour pattern (27 bits).  Sites with the same pattern inside a block end up
+// in the same tiles, so a tile skips the offsets none of its rows has; larger blocks give purer
+// tiles (the gather locality they cost matters less than the matrix-core work they save).  The
+// order is a heuristic only: blocks 1024 voxels apart and batches of equal parity share groups,
+// which costs some locality and nothing else.
+constexpr int ORDER_KEY_BITS = 40;
 __global__ void order_key_kernel(const int32_t *__restrict__ coords, const int32_t *__restrict__ nbr, int64_t first,
                                  int64_t n, uint64_t *__restrict__ keys, int32_t *__restrict__ vals) {
   int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -50,9 +52,9 @@ __global__ void order_key_kernel(const int32_t *__restrict__ coords, const int32
   int4 c = reinterpret_cast<const int4 *>(coords)[i];
   uint32_t m = 0;
   for (int k = 0; k < 27; k++) m |= (nbr[i * 27 + k] >= 0 ? 1u : 0u) << k;
-  const uint64_t mort = spread3((uint64_t)(c.x >> 6)) | (spread3((uint64_t)(c.y >> 6)) << 1) |
-                        (spread3((uint64_t)(c.z >> 6)) << 2);
-  keys[t] = ((uint64_t)(c.w & 127) << 57) | ((mort & 0x3fffffffull) << 27) | (uint64_t)m;
+  const uint64_t mort = spread3((uint64_t)((c.x >> 6) & 15)) | (spread3((uint64_t)((c.y >> 6) & 15)) << 1) |
+                        (spread3((uint64_t)((c.z >> 6) & 15)) << 2);
+  keys[t] = ((uint64_t)(c.w & 1) << 39) | (mort << 27) | (uint64_t)m;
   vals[t] = (int)i;
 }
 
@@ -187,7 +189,7 @@ int insc_order_build(const insc_grid *g, const int32_t *d_nbr, int64_t first, in
   hipLaunchKernelGGL(order_key_kernel, dim3(grid_for(n, 256)), dim3(256), 0, s, insc_grid_coords(g), d_nbr, first, n,
                      keys, d_order + first);
   INSC_LAUNCH_CHECK();
-  return sort_pairs_u64(keys, d_order + first, n, 64, s);
+  return sort_pairs_u64(keys, d_order + first, n, ORDER_KEY_BITS, s);
 }
 
 int insc_order_by_offset(const int32_t *d_order, const int32_t *d_offset, int64_t n, int32_t *d_out, void *stream) {
