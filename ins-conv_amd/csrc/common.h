@@ -81,11 +81,12 @@ int build_tile_plan(const int32_t *nbr, const int32_t *order, const int32_t *d_n
                     int32_t *map, uint32_t *tmask, hipStream_t s);
 
 // in_rows: rows of the input matrix (bounds the gather).  out may be null when ep.out2 is set.
+// latency != 0 picks the launch shape for small row counts (residual frames).
 int launch_conv(const float *in, int64_t ld_in, int64_t in_rows, float *out, int64_t ld_out, const float *W,
                 const float *Wp, const float *bias, const int32_t *map0, const int32_t *map1, int mode, int K,
                 const int32_t *rows, const int32_t *d_n_rows, int64_t n_rows, int Cin, int Cout,
                 const uint8_t *tile_flags, const uint8_t *row_mask, hipStream_t s, BnEpilogue ep = BnEpilogue(),
-                TilePlan plan = TilePlan());
+                TilePlan plan = TilePlan(), int latency = 0);
 int64_t packed_floats(int K, int Cin, int Cout);
 int pack_weights(const float *W, int K, int Cin, int Cout, float *Wp, hipStream_t s);
 int launch_bn(const float *in, int64_t ld_in, float *out, int64_t ld_out, const float *mean, const float *var,

@@ -837,7 +837,8 @@ int pack_weights(const float *W, int K, int Cin, int Cout, float *Wp, hipStream_
 int launch_conv(const float *in, int64_t ld_in, int64_t in_rows, float *out, int64_t ld_out, const float *W,
                 const float *Wp, const float *bias, const int32_t *map0, const int32_t *map1, int mode, int K,
                 const int32_t *rows, const int32_t *d_n_rows, int64_t n_rows, int Cin, int Cout,
-                const uint8_t *tile_flags, const uint8_t *row_mask, hipStream_t s, BnEpilogue ep, TilePlan plan) {
+                const uint8_t *tile_flags, const uint8_t *row_mask, hipStream_t s, BnEpilogue ep, TilePlan plan,
+                int latency) {
   if (n_rows == 0) return INSC_OK;
   if (plan.map && (mode != MAP_NBR || K != 27 || plan.ld * 27 * 4 >= (int64_t)BUF_OOB || plan.ld < cdiv(n_rows, TILE_M) * TILE_M))
     plan = TilePlan();  // only the 3^3 map has a plan; an unusable one is ignored
@@ -872,7 +873,7 @@ int launch_conv(const float *in, int64_t ld_in, int64_t in_rows, float *out, int
     // whole filter into LDS - costs more than it saves: 34 us against 21 us at 32k sites, even at
     // 150k; both kernels give the same bits)
     if (mode == MAP_NBR && K == 27 && Cin <= 32 && Cout <= 32 && map_bytes64 < (int64_t)BUF_OOB && small_ids &&
-        tiles >= WL_MIN_TILES) {
+        tiles >= WL_MIN_TILES && !latency) {
       const uint32_t map_bytes = (uint32_t)map_bytes64;
       // persistent blocks, a multiple of the XCD count, at most one per compute unit
       const int64_t want = cdiv(tiles, WL_WAVES);
@@ -889,13 +890,21 @@ int launch_conv(const float *in, int64_t ld_in, int64_t in_rows, float *out, int
     //  wider layers sit at the coarse scales of a U-Net, which have few tiles: one output block
     //    per wavefront, and for 3^3 / 2^3 maps the items of a tile are dealt to S wavefronts
     //    (S grows with Cin: 2, 4, 8 for 3^3).
-    const bool split = Cin >= 64 && K > 1 && (mode == MAP_NBR || (mode == MAP_PARENT && Cin >= 96));
+    // latency != 0 (residual frames: a few thousand rows at most, so a launch lasts as long as
+    // its most expensive tile): the items of every 3^3 tile are dealt to four wavefronts whatever
+    // the width, and to more blocks for the wide layers.  Also a function of the layer shape only.
+    const bool lat = latency && mode == MAP_NBR && K == 27 && Cin >= 32;
+    const bool split = lat || (Cin >= 64 && K > 1 && (mode == MAP_NBR || (mode == MAP_PARENT && Cin >= 96)));
     const int NB0 = split ? 1 : conv_nb_per_group(Cout);
     const int nbtp = conv_nbt_padded(Cout);
     int S = 1;
     if (split) S = K == 27 ? (Cin >= 160 ? 8 : Cin >= 128 ? 4 : 2) : (Cin >= 96 ? 4 : 1);  // K == 8: conv and deconv
     const int NB = (S == 1 && Cin >= 96) ? 1 : NB0;
-    const int G = (split && K == 27) ? (Cin >= 160 ? 4 : Cin >= 128 ? 2 : 1) : 1;
+    int G = (split && K == 27) ? (Cin >= 160 ? 4 : Cin >= 128 ? 2 : 1) : 1;
+    if (lat) {
+      G = Cin >= 128 ? 4 : Cin >= 64 ? 2 : 1;
+      S = 4;
+    }
     if (G > 1) S = 4;
     const unsigned gx = (unsigned)(S == 1 ? cdiv(tiles, CONV_WAVES) : tiles);
     dim3 grid(gx, (unsigned)(NB == 1 ? nbt : nbtp / NB), (unsigned)G), block((S == 1 ? CONV_WAVES : S) * 64);

@@ -146,14 +146,14 @@ int insc_incre_conv_ssc(const float *d_in, int64_t ld_in, const float *d_pre_in,
   hipStream_t s = (hipStream_t)stream;
   // rules inside the frame's site set, on the residual features (CUDA/Convolution.cpp:264-268,283)
   int rc = launch_conv(d_in, ld_in, n, d_out, ld_out, d_W, d_Wp, d_bias, d_nbr, nullptr, MAP_NBR, 27, nullptr, nullptr,
-                       n, Cin, Cout, nullptr, nullptr, s);
+                       n, Cin, Cout, nullptr, nullptr, s, BnEpilogue(), TilePlan(), 1);
   if (rc || n_pre_rows == 0) return rc;
   // new sites gather the saved features of their neighbours in the saved set (:274,287)
   BnEpilogue ep;
   ep.res = d_out;
   ep.ldr = ld_out;
   return launch_conv(d_pre_in, ld_pre, n_pre_rows, d_out, ld_out, d_W, d_Wp, nullptr, d_nbr_pre, nullptr, MAP_NBR, 27,
-                     nullptr, nullptr, n, Cin, Cout, nullptr, nullptr, s, ep);
+                     nullptr, nullptr, n, Cin, Cout, nullptr, nullptr, s, ep, TilePlan(), 1);
 }
 
 int insc_incre_bn_leaky(const float *d_in, int64_t ld_in, float *d_out, int64_t ld_out, const float *d_mean,

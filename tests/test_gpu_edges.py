@@ -135,7 +135,10 @@ def test_residual_frames_disjoint_from_and_inside_the_saved_scene():
         saved = net(_inp(vox, rgb), increment=False)
         got = net(_inp(far, rgb[:1500]), increment="residual")
         alone = ref_model.sparseModel(_inp(far, rgb[:1500]))
-        assert torch.equal(got, alone)
+        # (not the same bits: a residual frame's convolutions use the launch shape for small row
+        # counts, which adds the terms of a row in another order)
+        scale = max(1.0, float(alone.abs().max()))
+        np.testing.assert_allclose(got.cpu().numpy(), alone.cpu().numpy(), rtol=1e-4, atol=1e-5 * scale)
         # saved voxels, same colours, one point per voxel: mean unchanged -> residual 0
         idx = np.random.default_rng(48).permutation(len(vox))[:1200]
         got = net(_inp(vox[idx], rgb[idx]), increment="residual")
