@@ -115,11 +115,11 @@ def conv_roofline(device, reps=30, warm=200):
     achieved = bytes_alg / t / 1e9
     return {
         "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-        "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": 552.4e6,
+        "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": 553.0e6,
         "kernel": "conv_wlds_kernel (SSC 3^3, 32->32, filter in LDS, persistent blocks; 500k sites, %d rules)" % n_rules,
         "avg_us": round(t * 1e6, 1), "algorithmic_bytes": int(bytes_alg),
         "traffic_note": "HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE (x1.999, copy-kernel calibration) + "
-                        "WRITE_SIZE (x1.000): 453.8 MB + 98.6 MB, profiles/conv_wlds_ssc32_500k.txt",
+                        "WRITE_SIZE (x1.000): 454.4 MB + 98.6 MB, profiles/conv_wlds_ssc32_500k.txt",
         "mfma_tflops": round(flops / t / 1e12, 2), "mfma_frac": round(flops / t / 1e12 / MFMA_FP32_PEAK_TFLOPS, 4),
         "ssc_msites_per_s": round(sc.n / t / 1e6, 1),
     }
@@ -431,6 +431,12 @@ def main():
         extra = {"median_ms": round(float(np.median(per_frame)), 3),
                  "p95_ms": round(float(np.percentile(per_frame, 95)), 3),
                  "last_frame_ms": round(per_frame[-1], 3), "first_timed_frame_ms": round(per_frame[0], 3)}
+        # rows the last timed frame recomputed: per scale, the smallest and the largest dirty set
+        # among the tensors of that scale, beside the scale's sites
+        sites = net.sites_per_level()
+        extra["dirty_rows_last_frame"] = [
+            {"scale": l, "sites": int(sites[l]), "min": min(r for _, r in sets), "max": max(r for _, r in sets)}
+            for l, sets in enumerate(net.dirty_rows()) if sets]
         if not args.no_residual:
             extra.update(residual_row(model, seq, frames, W + K, device))
         cpu_fn = cpu_baseline_unet

@@ -279,6 +279,12 @@ int insc_net_refresh_weights(insc_net *net, void *stream);
  * Returns when the frame has completed. */
 int insc_net_forward(insc_net *net, const int32_t *d_coords, int coord_cols, const float *d_feats, int64_t P,
                      int increment, float *d_out, int out_all, int64_t *h_n_sites, void *stream);
+/* The dirty sets of the last exact incremental frame (diagnostics; no counterpart in the
+ * reference, whose incremental frames do not propagate): for set i in program order,
+ * h_level[i] = its scale, h_kind[i] = 0 input, 1 dilated by a 3^3 layer, 2 parents, 3 children,
+ * 4 union, h_rows[i] = its number of rows.  *h_n_sets <= max_sets sets are reported.  Synchronises. */
+int insc_net_dirty_counts(insc_net *net, int max_sets, int *h_n_sets, int *h_level, int *h_kind, int64_t *h_rows,
+                          void *stream);
 /* One residual frame: the reference's own incremental forward (demo.py:26-38 with
  * increment=True; Incre_* operators, pybind.cpp:218-258) as one call.  The frame's points form a
  * site set of their own, features are differences to the state saved by the last

@@ -225,6 +225,21 @@ __global__ void dirty_union_kernel(const uint8_t *__restrict__ a, const uint8_t 
   if (tflag_bo) tflag_bo[bo_pos[i] >> 5] = 1;
 }
 
+// dirty rows of one set: one count per block, added up with an atomic per block
+__global__ __launch_bounds__(256) void count_mask_kernel(const uint8_t *__restrict__ mask, int64_t n,
+                                                         unsigned long long *__restrict__ out) {
+  __shared__ int part[256];
+  int c = 0;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) c += mask[i] ? 1 : 0;
+  part[threadIdx.x] = c;
+  __syncthreads();
+  for (int d = 128; d > 0; d >>= 1) {
+    if ((int)threadIdx.x < d) part[threadIdx.x] += part[threadIdx.x + d];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0 && part[0]) atomicAdd(out, (unsigned long long)part[0]);
+}
+
 __global__ void fill_bytes_kernel(uint4 *p, size_t n16) {
   size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   size_t stride = (size_t)gridDim.x * blockDim.x;
@@ -1279,6 +1294,39 @@ int insc_net_profile(insc_net *net, int enable, float *h_ms4) {
     for (int i = 0; i < 5; i++) INSC_HIP(hipEventCreate(&net->ev[i]));
   net->profiling = enable != 0;
   if (!enable) net->ev_valid = false;
+  return INSC_OK;
+}
+
+/* The dirty sets of the last exact incremental frame: for set i (program order; i < *h_n_sets
+ * <= max_sets) h_level[i] = its scale, h_kind[i] = how it is derived (0 input, 1 dilated by a 3^3
+ * layer, 2 parents, 3 children, 4 union) and h_rows[i] = its number of rows.  Synchronises. */
+int insc_net_dirty_counts(insc_net *net, int max_sets, int *h_n_sets, int *h_level, int *h_kind, int64_t *h_rows,
+                          void *stream) {
+  INSC_REQUIRE(net && net->finalized && h_n_sets && h_level && h_kind && h_rows && max_sets >= 0, INSC_ERR_ARG,
+               "insc_net_dirty_counts: bad arguments");
+  hipStream_t s = (hipStream_t)stream;
+  const int ns = std::min<int>(max_sets, (int)net->dirty.size());
+  *h_n_sets = ns;
+  if (ns == 0) return INSC_OK;
+  void *ws;
+  int rc = workspace(WS_API, s, sizeof(unsigned long long) * (size_t)ns, &ws);
+  if (rc) return rc;
+  unsigned long long *d = (unsigned long long *)ws;
+  INSC_HIP(hipMemsetAsync(d, 0, sizeof(unsigned long long) * (size_t)ns, s));
+  for (int i = 0; i < ns; i++) {
+    const DirtyNode &dn = net->dirty[i];
+    const int64_t n = net->levels[dn.level].n;
+    h_level[i] = dn.level;
+    h_kind[i] = dn.kind;
+    if (n > 0 && dn.mask) {
+      hipLaunchKernelGGL(count_mask_kernel, dim3(grid_for(n, 256, 1024)), dim3(256), 0, s, dn.mask, n, d + i);
+      INSC_LAUNCH_CHECK();
+    }
+  }
+  std::vector<unsigned long long> h((size_t)ns);
+  INSC_HIP(hipMemcpyAsync(h.data(), d, sizeof(unsigned long long) * (size_t)ns, hipMemcpyDeviceToHost, s));
+  INSC_HIP(hipStreamSynchronize(s));
+  for (int i = 0; i < ns; i++) h_rows[i] = (int64_t)h[(size_t)i];
   return INSC_OK;
 }
 

@@ -176,6 +176,20 @@ class CompiledNet(object):
         self._profiling, self._timed = bool(enable), False
         return out
 
+    def dirty_rows(self):
+        """Rows of every dirty set of the last exact incremental frame, per scale: a list (one entry
+        per scale) of lists of (kind, rows) in program order; kind is "input", "dilate", "parents",
+        "children" or "union"."""
+        n = ctypes.c_int(0)
+        cap = 512
+        lv, kd, rows = (ctypes.c_int * cap)(), (ctypes.c_int * cap)(), (I64 * cap)()
+        lib.insc_net_dirty_counts(self.h, cap, ctypes.byref(n), lv, kd, rows, stream_ptr())
+        names = ("input", "dilate", "parents", "children", "union")
+        out = [[] for _ in range(max(lv[:n.value], default=-1) + 1)]
+        for i in range(n.value):
+            out[lv[i]].append((names[kd[i]], int(rows[i])))
+        return out
+
     def sites_per_level(self):
         a = (I64 * 16)()
         lib.insc_net_counts(self.h, a, None)

@@ -58,3 +58,33 @@ def test_compiled_rejects_incremental_without_state():
     pts, rgb = _frames(2, seed=32)[0]
     with pytest.raises(InscError):
         net(_inp(pts, rgb), increment=True)
+
+
+def test_dirty_set_rows_of_a_frame():
+    """The dirty sets the executor reports: the input's set is the frame's touched voxels, every
+    derived set contains its source (sets only grow along the program), none exceeds its scale,
+    and at the finest scale they stay a fraction of the scene for a local increment."""
+    import sparseconvnet as scn
+    from netdefs import NaiveUNet
+
+    frames = _frames(3, seed=33)
+    model = NaiveUNet(m=16, levels=4, seed=2).cuda()
+    net = scn.compile(model.sparseModel)
+    with torch.no_grad():
+        net(_inp(*frames[0]), increment=False)
+        pts, rgb = frames[1]
+        net(_inp(pts, rgb), increment=True)
+    sets = net.dirty_rows()
+    sites = net.sites_per_level()
+    assert len(sets) == 4
+    assert sets[0][0][0] == "input"
+    touched = len(np.unique(np.asarray(pts)[:, :3], axis=0))
+    assert sets[0][0][1] == touched
+    for l, ss in enumerate(sets):
+        assert ss, "scale %d has no dirty set" % l
+        for kind, rows in ss:
+            assert 0 < rows <= sites[l], (l, kind, rows, sites[l])
+    rows0 = [r for _, r in sets[0]]
+    assert min(rows0) == touched and max(rows0) >= touched
+    # dilation by 3^3 layers grows a set; a frame here touches one end of the scene
+    assert [r for k, r in sets[0] if k == "dilate"][0] > touched
