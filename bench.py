@@ -193,6 +193,9 @@ def kernel_table(device, reps=20):
         rows.append({"kernel": name, "us": round(sec * 1e6, 1), "algorithmic_bytes": int(nbytes),
                      "GB/s": round(gbs, 1), "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4), "units": note})
 
+    # the box's own copy bandwidth at this size, as the reference point for the rows below
+    t = timed(lambda: y.copy_(x))
+    add("device-to-device copy (torch; reference point, not a kernel of the path)", t, NF * C * 8, "%d x %d" % (NF, C))
     t = timed(lambda: lib.insc_grid_insert(grid, ptr(c4), I64(P), ptr(sop), ctypes.byref(n_sites), st),
               pre=lambda: lib.insc_grid_clear(grid, st))
     add("hash grid insert (claim, scan, assign, resolve; incl. count read-back)", t, P * 32, "%d points -> %d sites" % (P, n_sites.value))

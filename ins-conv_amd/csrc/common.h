@@ -76,9 +76,10 @@ struct TilePlan {
   const int32_t *map = nullptr;
   int64_t ld = 0;
   const uint32_t *tmask = nullptr;
+  const int32_t *sched = nullptr;  // [ld / 32] tiles by falling cost, or null
 };
 int build_tile_plan(const int32_t *nbr, const int32_t *order, const int32_t *d_n, int64_t n_rows, int64_t ld,
-                    int32_t *map, uint32_t *tmask, hipStream_t s);
+                    int32_t *map, uint32_t *tmask, int32_t *sched, hipStream_t s);
 
 // in_rows: rows of the input matrix (bounds the gather).  out may be null when ep.out2 is set.
 // latency != 0 picks the launch shape for small row counts (residual frames).

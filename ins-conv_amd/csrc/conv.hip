@@ -12,6 +12,8 @@
 
 #include "common.h"
 
+#include <atomic>
+
 namespace insc {
 
 typedef float f16v __attribute__((ext_vector_type(16)));
@@ -220,7 +222,8 @@ __global__ __launch_bounds__((S == 1 ? CONV_WAVES : S) * 64) void conv_mfma_kern
   __shared__ float red[S > 1 ? S - 1 : 1][S > 1 ? 16 * 64 : 1];
   __shared__ unsigned wmask[S];
   const int64_t n = d_n_rows ? min((int64_t)*d_n_rows, n_rows) : n_rows;
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  // (the wavefront's number as a scalar: the item cursor below then runs on the scalar unit)
+  const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), lane = threadIdx.x & 63;
   const int r = lane & 31, h = lane >> 5;
   const int64_t t0 = (S == 1 ? (int64_t)blockIdx.x * WAVES + wave : (int64_t)blockIdx.x) * TILE_M;
   const int cb0 = blockIdx.y * NB;  // first output-channel block of this column group
@@ -479,15 +482,26 @@ __global__ __launch_bounds__((S == 1 ? CONV_WAVES : S) * 64) void conv_mfma_kern
   int rid[16];
 #pragma unroll
   for (int v = 0; v < 16; v++) rid[v] = __shfl(my_row, 8 * (v >> 2) + 4 * h + (v & 3), 64);
+  // (the values of the residual input are all fetched before the first store: a store may alias them
+  // as far as the compiler knows, and loads issued between the stores would wait one by one)
+  if (ep.res) {
+    float rv[NB][16];
+#pragma unroll
+    for (int v = 0; v < 16; v++) {
+      const float *rp = ep.res + (int64_t)(rid[v] < 0 ? 0 : rid[v]) * ep.ldr + cb0 * 32 + r;
+#pragma unroll
+      for (int b = 0; b < NB; b++) rv[b][v] = (rid[v] >= 0 && (cb0 + b) * 32 + r < Cout) ? rp[b * 32] : 0.0f;
+    }
+#pragma unroll
+    for (int v = 0; v < 16; v++) {
+#pragma unroll
+      for (int b = 0; b < NB; b++) acc[b][v] += rv[b][v];
+    }
+    __builtin_amdgcn_sched_barrier(0);  // (the sums stay above the stores)
+  }
 #pragma unroll
   for (int v = 0; v < 16; v++) {
     if (rid[v] < 0) continue;
-    if (ep.res) {
-      const float *rp = ep.res + (int64_t)rid[v] * ep.ldr + cb0 * 32 + r;
-#pragma unroll
-      for (int b = 0; b < NB; b++)
-        if ((cb0 + b) * 32 + r < Cout) acc[b][v] += rp[b * 32];
-    }
     if (out) {
       float *op = out + (int64_t)rid[v] * ld_out + cb0 * 32 + r;
 #pragma unroll
@@ -739,11 +753,17 @@ __global__ __launch_bounds__(WL_WAVES * 64) void conv_wlds_kernel(
 #pragma unroll
     for (int v = 0; v < 16; v++) rid[v] = __shfl(my_row, 8 * (v >> 2) + 4 * h + (v & 3), 64);
     const uint32_t col4 = (uint32_t)col * 4u;
+    // (the residual input is fetched before the first store, which may alias it as far as the
+    // compiler knows: loads issued between the stores would wait one by one)
+    float rv[16];
+#pragma unroll
+    for (int v = 0; v < 16; v++)
+      rv[v] = (ep.res && rid[v] >= 0 && col < Cout) ? ep.res[(int64_t)rid[v] * ep.ldr + col] : 0.0f;
 #pragma unroll
     for (int v = 0; v < 16; v++) {
       const bool ok = rid[v] >= 0 && col < Cout;
       float av = acc[v];  // (a bit cast applied to the vector element itself reads element 0)
-      if (ep.res && ok) av += ep.res[(int64_t)rid[v] * ep.ldr + col];
+      if (ep.res && ok) av += rv[v];
       if (out)
         __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(av), rout,
                                               (int)(ok ? __umul24((unsigned)rid[v], ldo4) + col4 : BUF_OOB), 0, 0);
@@ -764,6 +784,285 @@ __global__ __launch_bounds__(WL_WAVES * 64) void conv_wlds_kernel(
     for (int i = 0; i < NSTAGE; i++) st[i] = stn[i];
     tn = tnn;
     my_row_n = my_row_nn;
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// Wide 3^3 layers with many tiles: persistent blocks of S wavefronts.  A block works through
+// units (tile, output block) of a cost-ordered list (plan.sched: tiles by falling number of active
+// offsets); block b takes the units b, 2B-1-b, 2B+b, ... (every other round reversed, so a block
+// that starts with an expensive unit continues with a cheap one).  While a unit is computed the
+// neighbour-map slice, row ids and tile id of the next ones are in flight, so that no wavefront
+// ever waits for a launch, a map or a row id between two units - with one block per unit the
+// matrix cores idle through 5-10 us of such latencies per wavefront, and the units a compute unit
+// happens to receive differ by 2x in cost.
+// The S wavefronts deal the (offset, chunk) items of the unit exactly as conv_mfma_kernel<1, 27,
+// MAP_NBR, S> with one block per tile does, and the partial sums are added in the same order: both
+// kernels give the same bits.  All wavefronts share the final sum and the stores (8 * 4 / S rows each).
+// ---------------------------------------------------------------------------------------
+template <int S>
+__global__ __launch_bounds__(S * 64) __attribute__((amdgpu_waves_per_eu(3, 3))) void conv_pers_kernel(
+    const float *__restrict__ in, int64_t ld_in, float *__restrict__ out, int64_t ld_out,
+    const float *__restrict__ Wp, const float *__restrict__ bias, const int32_t *__restrict__ rows,
+    const int32_t *__restrict__ d_n_rows, int64_t n_rows, int Cin, int Cout, int nbt, int nbtp,
+    const uint8_t *__restrict__ tile_flags, uint32_t in_bytes, uint32_t wp_bytes, BnEpilogue ep, TilePlan plan) {
+  constexpr int K = 27;
+  constexpr int NSTAGE = (TILE_M * K + 64 * S - 1) / (64 * S);
+  constexpr int VPW = 16 / S;  // accumulator registers (groups of 4 rows x 2 half-waves) a wavefront finishes
+  __shared__ int nl[2][TILE_M * K];
+  __shared__ float red[2][S][16 * 64];
+  const int64_t n = d_n_rows ? min((int64_t)*d_n_rows, n_rows) : n_rows;
+  const int64_t ntiles = (n + TILE_M - 1) / TILE_M, units = ntiles * nbt;
+  const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), lane = threadIdx.x & 63;
+  const int r = lane & 31, h = lane >> 5;
+  const int nch = conv_nch(Cin);
+  const int64_t B = gridDim.x, b = blockIdx.x;
+  const __amdgpu_buffer_rsrc_t rplan = make_rsrc(plan.map, (uint32_t)(plan.ld * K * 4));
+  // unit j of this block: b, 2B - 1 - b, 2B + b, ...
+  auto unit_at = [&](int64_t j) -> int64_t { return j * B + ((j & 1) ? B - 1 - b : b); };
+  // Tile id, tile flag and offset mask of a unit are the same for every lane, but they are fetched
+  // with vector loads: scalar loads share their counter with the LDS reads of the item loop, which
+  // would then wait for them.
+  const __amdgpu_buffer_rsrc_t rsched = make_rsrc(plan.sched, (uint32_t)(ntiles * 4));
+  const __amdgpu_buffer_rsrc_t rtmask = make_rsrc(plan.tmask, (uint32_t)(ntiles * 4));
+  const __amdgpu_buffer_rsrc_t rflag = make_rsrc(tile_flags, tile_flags ? (uint32_t)ntiles : 0u);
+  auto tile_issue = [&](int64_t u) -> int {  // out of range: 0, never used
+    return __builtin_amdgcn_raw_buffer_load_b32(rsched, (int)(u < units ? (uint32_t)(u / nbt) * 4u : BUF_OOB), 0, 0);
+  };
+  auto stage_issue = [&](int tile, int (&st)[NSTAGE]) {
+#pragma unroll
+    for (int i = 0; i < NSTAGE; i++) {
+      const int e = (i * S + wave) * 64 + lane;  // e = k * 32 + row
+      const bool ok = tile >= 0 && e < TILE_M * K;  // (the value of a load sent out of range is never used)
+      const uint32_t voff = ok ? (uint32_t)((e >> 5) * (int)plan.ld + tile * TILE_M + (e & 31)) * 4u : BUF_OOB;
+      st[i] = __builtin_amdgcn_raw_buffer_load_b32(rplan, (int)voff, 0, 0);
+    }
+  };
+  auto row_of = [&](int tile) -> int {
+    const int64_t p = (int64_t)tile * TILE_M + r;
+    return (tile >= 0 && p < n) ? (rows ? rows[p] : (int)p) : -1;
+  };
+  auto flag_issue = [&](int tile) -> int {
+    return (int)__builtin_amdgcn_raw_buffer_load_b8(rflag, (int)(tile >= 0 ? (uint32_t)tile : BUF_OOB), 0, 0);
+  };
+  auto mask_issue = [&](int tile) -> int {
+    return __builtin_amdgcn_raw_buffer_load_b32(rtmask, (int)(tile >= 0 ? (uint32_t)tile * 4u : BUF_OOB), 0, 0);
+  };
+
+  const __amdgpu_buffer_rsrc_t rin = make_rsrc(in, in_bytes), rw = make_rsrc(Wp, wp_bytes);
+  const uint32_t ld4 = (uint32_t)ld_in * 4u, lane16 = (uint32_t)lane * 16u;
+  // outputs and the residual input are addressed with 32-bit byte offsets as well (the host checks
+  // the sizes); rows that do not exist get an out-of-range offset and the hardware drops the access
+  const __amdgpu_buffer_rsrc_t rout = make_rsrc(out, out ? BUF_OOB : 0u), rout2 = make_rsrc(ep.out2, ep.out2 ? BUF_OOB : 0u);
+  const __amdgpu_buffer_rsrc_t rres = make_rsrc(ep.res, ep.res ? BUF_OOB : 0u);
+  const __amdgpu_buffer_rsrc_t rbias = make_rsrc(bias, bias ? (uint32_t)Cout * 4u : 0u);
+  const __amdgpu_buffer_rsrc_t rew = make_rsrc(ep.w, ep.out2 ? (uint32_t)Cout * 4u : 0u);
+  const __amdgpu_buffer_rsrc_t reb = make_rsrc(ep.b, ep.out2 ? (uint32_t)Cout * 4u : 0u);
+  const uint32_t ldo4 = (uint32_t)ld_out * 4u, ldo24 = (uint32_t)ep.ld2 * 4u, ldr4 = (uint32_t)ep.ldr * 4u;
+  // Offsets of which this wavefront holds at least 1, 2, .. items (it takes, of offset k, the chunks
+  // ch0(k), ch0(k) + S, ... with ch0(k) = (wave - k * nch) mod S): the items of a tile with offset
+  // mask m are then counted with a few population counts.
+  constexpr int MAXQ = 4;  // nch <= MAXQ * S
+  unsigned kmask[MAXQ];
+#pragma unroll
+  for (int q = 0; q < MAXQ; q++) kmask[q] = 0;
+  for (int k = 0; k < K; k++) {
+    const int c0 = (wave - k * nch) & (S - 1);
+    const int cnt = c0 < nch ? (nch - c0 + S - 1) / S : 0;
+#pragma unroll
+    for (int q = 0; q < MAXQ; q++)
+      if (cnt > q) kmask[q] |= 1u << k;
+  }
+  // bias and the fused batch norm's scale / shift for this lane's column of output block ob (sent
+  // out of range, they read as zero)
+  auto col_issue = [&](int ob, float &bv, float &ew, float &eb) {
+    const uint32_t off = (uint32_t)(ob * 32 + r) * 4u;
+    bv = __uint_as_float((unsigned)__builtin_amdgcn_raw_buffer_load_b32(rbias, (int)(wave == 0 ? off : BUF_OOB), 0, 0));
+    ew = __uint_as_float((unsigned)__builtin_amdgcn_raw_buffer_load_b32(rew, (int)off, 0, 0));
+    eb = __uint_as_float((unsigned)__builtin_amdgcn_raw_buffer_load_b32(reb, (int)off, 0, 0));
+  };
+
+  // LDS copies of the map slice and of the partial sums are double buffered (parity par): one
+  // barrier per unit publishes the partial sums of this unit and the map slice of the next
+  // Pipeline over the units of this block: while unit j is computed, the map slice, row ids, flag
+  // and mask of unit j + 1 and the tile id of unit j + 2 are in flight.
+  int64_t j = 0, u = unit_at(0);
+  int tile_c = u < units ? __builtin_amdgcn_readfirstlane(tile_issue(u)) : -1;
+  int tile_n = unit_at(1) < units ? __builtin_amdgcn_readfirstlane(tile_issue(unit_at(1))) : -1;
+  int par = 0;
+  {
+    int st[NSTAGE];
+    stage_issue(tile_c, st);
+#pragma unroll
+    for (int i = 0; i < NSTAGE; i++) {
+      const int e = (i * S + wave) * 64 + lane;
+      if (e < TILE_M * K) nl[0][e] = st[i];
+    }
+  }
+  int my_row = row_of(tile_c);
+  bool live = tile_c >= 0 && (!tile_flags || __builtin_amdgcn_readfirstlane(flag_issue(tile_c)) != 0);
+  unsigned tmask_c = (unsigned)__builtin_amdgcn_readfirstlane(mask_issue(tile_c));
+  float bv, ew, eb;
+  col_issue((int)(u % nbt), bv, ew, eb);
+  __syncthreads();
+
+  while (u < units) {
+    const int ob = (int)(u % nbt);
+    const int64_t un = unit_at(j + 1), unn = unit_at(j + 2);
+    const int tile_nn_v = tile_issue(unn);
+    int stn[NSTAGE];
+    stage_issue(tile_n, stn);
+    const int my_row_n = row_of(tile_n);
+    const int flag_n_v = flag_issue(tile_n);
+    const int tmask_n_v = mask_issue(tile_n);
+    float bv_n, ew_n, eb_n;
+    col_issue((int)(un % nbt), bv_n, ew_n, eb_n);
+    const int *nlc = nl[par];
+    const int c = ob * 32 + r;
+    f16v acc;
+    int rid[VPW];
+    float rv[VPW];
+
+    if (live) {
+      // Items (active offset k, 32-channel chunk ch), dealt by (k * nch + ch) % S: wavefront w takes,
+      // of offset k, the chunks ch0(k), ch0(k) + S, ... with ch0(k) = (w - k * nch) mod S.
+      const unsigned rest = tmask_c & kmask[0];
+      int nitems = 0;
+#pragma unroll
+      for (int q = 0; q < MAXQ; q++) nitems += __builtin_popcount(tmask_c & kmask[q]);
+#pragma unroll
+      for (int v = 0; v < 16; v++) acc[v] = bv;
+
+      if (rest) {
+        struct Cursor {
+          int k, ch;
+          unsigned rest;
+        };
+        auto ch0 = [&](int k) -> int { return (wave - k * nch) & (S - 1); };
+        auto step = [&](const Cursor &cu) -> Cursor {
+          const bool wrap = cu.ch + S >= nch;
+          const int nk = cu.rest ? __builtin_ctz(cu.rest) : -1;
+          Cursor nx;
+          nx.ch = wrap ? ch0(nk) : cu.ch + S;
+          nx.k = wrap ? nk : cu.k;
+          nx.rest = wrap ? (cu.rest & (cu.rest - 1)) : cu.rest;
+          return nx;
+        };
+        Cursor first;
+        first.k = __builtin_ctz(rest);
+        first.ch = ch0(first.k);
+        first.rest = rest & (rest - 1);
+        auto gather = [&](const Cursor &cu) -> Frag {
+          const int kk = cu.k < 0 ? 0 : cu.k;
+          const int src = nlc[kk * TILE_M + r];
+          const bool on = cu.k >= 0 && src >= 0 && (h == 0 || Cin - cu.ch * 32 >= 32);
+          const uint32_t voff = on ? (uint32_t)src * ld4 + (uint32_t)(cu.ch * 128 + h * 64) : BUF_OOB;
+          Frag f;
+#pragma unroll
+          for (int q = 0; q < 4; q++) f.q[q] = buf_load16(rin, voff + 16u * q, 0);
+          return f;
+        };
+        auto wload = [&](const Cursor &cu) -> Frag {
+          const int tile = ((cu.k < 0 ? 0 : cu.k) * nch + cu.ch) * nbtp + ob;
+          const uint32_t soff = (uint32_t)__builtin_amdgcn_readfirstlane(tile * 4096);
+          const uint32_t voff = cu.k >= 0 ? lane16 : BUF_OOB;
+          Frag f;
+#pragma unroll
+          for (int q = 0; q < 4; q++) f.q[q] = buf_load16(rw, voff + 1024u * q, soff);
+          return f;
+        };
+        // the same ring of D items in flight as in conv_mfma_kernel
+        constexpr int D = INSC_CONV_DEPTH_SPLIT;
+        Frag g[D], bw[D];
+        Cursor ci = first;
+#pragma unroll
+        for (int d = 0; d < D - 1; d++) {
+          g[d] = gather(ci);
+          bw[d] = wload(ci);
+          ci = step(ci);
+        }
+        for (int t0i = 0; t0i < nitems; t0i += D) {
+#pragma unroll
+          for (int uu = 0; uu < D; uu++) {
+            g[(uu + D - 1) % D] = gather(ci);
+            bw[(uu + D - 1) % D] = wload(ci);
+            ci = step(ci);
+            const bool real = t0i + uu < nitems;
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_sched_barrier(0);
+            if (real) {
+#pragma unroll
+              for (int s2 = 0; s2 < 16; s2++)
+                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(frag_at(g[uu], s2), frag_at(bw[uu], s2), acc, 0, 0, 0);
+            }
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_sched_barrier(0);
+          }
+        }
+      }
+
+    }
+    // the next unit's slice of the map and its scalars (taken before the loads and stores of this
+    // unit's output are issued: a wait for them placed later would wait for those as well)
+#pragma unroll
+    for (int i = 0; i < NSTAGE; i++) {
+      const int e = (i * S + wave) * 64 + lane;
+      if (e < TILE_M * K) nl[par ^ 1][e] = stn[i];
+    }
+    const int tile_nn = unn < units ? __builtin_amdgcn_readfirstlane(tile_nn_v) : -1;
+    const bool live_n = tile_n >= 0 && (!tile_flags || __builtin_amdgcn_readfirstlane(flag_n_v) != 0);
+    const unsigned tmask_n = tile_n >= 0 ? (unsigned)__builtin_amdgcn_readfirstlane(tmask_n_v) : 0u;
+    if (live) {
+      // partial sums of all wavefronts through LDS
+#pragma unroll
+      for (int v = 0; v < 16; v++) red[par][wave][v * 64 + lane] = acc[v];
+      // rows this wavefront will store, and their residual input (in flight across the barrier)
+#pragma unroll
+      for (int q = 0; q < VPW; q++) {
+        const int v = wave * VPW + q;
+        rid[q] = __shfl(my_row, 8 * (v >> 2) + 4 * h + (v & 3), 64);
+        if (c >= Cout) rid[q] = -1;
+        rv[q] = __uint_as_float((unsigned)__builtin_amdgcn_raw_buffer_load_b32(
+            rres, (int)(rid[q] >= 0 ? __umul24((unsigned)rid[q], ldr4) + (uint32_t)c * 4u : BUF_OOB), 0, 0));
+      }
+    }
+    __syncthreads();
+    if (live) {
+      // wavefront w adds the partial sums, in wavefront order, for the accumulator registers
+      // w * VPW .. and stores those rows
+      float a[VPW];
+#pragma unroll
+      for (int q = 0; q < VPW; q++) {
+        const int v = wave * VPW + q;
+        a[q] = red[par][0][v * 64 + lane];
+#pragma unroll
+        for (int w = 1; w < S; w++) a[q] += red[par][w][v * 64 + lane];
+        if (ep.res) a[q] += rv[q];
+      }
+#pragma unroll
+      for (int q = 0; q < VPW; q++) {
+        const uint32_t c4 = (uint32_t)c * 4u;
+        if (out)
+          __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(a[q]), rout,
+                                                (int)(rid[q] >= 0 ? __umul24((unsigned)rid[q], ldo4) + c4 : BUF_OOB), 0, 0);
+        if (ep.out2) {
+          const float y = fmaf(a[q], ew, eb);  // fused batch norm + leaky ReLU
+          __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(y * ((y > 0.0f) ? 1.0f : ep.leak)), rout2,
+                                                (int)(rid[q] >= 0 ? __umul24((unsigned)rid[q], ldo24) + c4 : BUF_OOB), 0, 0);
+        }
+      }
+    }
+    j++;
+    u = un;
+    tile_c = tile_n;
+    tile_n = tile_nn;
+    my_row = my_row_n;
+    live = live_n;
+    tmask_c = tmask_n;
+    bv = bv_n;
+    ew = ew_n;
+    eb = eb_n;
+    par ^= 1;
   }
 }
 
@@ -806,12 +1105,40 @@ __global__ __launch_bounds__(256) void tile_plan_kernel(const int32_t *__restric
   if ((threadIdx.x & 31) == 0) tmask[p >> 5] = m;
 }
 
+// sched = the tiles by falling number of active offsets (a counting sort over the 28 classes by one
+// workgroup; the order inside a class is the order of arrival and has no influence on any result).
+__global__ __launch_bounds__(1024) void tile_sched_kernel(const uint32_t *__restrict__ tmask,
+                                                          const int32_t *__restrict__ d_n, int64_t n_rows,
+                                                          int32_t *__restrict__ sched) {
+  __shared__ int cnt[28], base[28];
+  const int64_t n = d_n ? min((int64_t)*d_n, n_rows) : n_rows;
+  const int64_t ntiles = (n + TILE_M - 1) / TILE_M;
+  if (threadIdx.x < 28) cnt[threadIdx.x] = 0;
+  __syncthreads();
+  for (int64_t t = threadIdx.x; t < ntiles; t += 1024) atomicAdd(&cnt[27 - __builtin_popcount(tmask[t] & 0x7FFFFFFu)], 1);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int a = 0;
+    for (int c = 0; c < 28; c++) {
+      base[c] = a;
+      a += cnt[c];
+      cnt[c] = 0;
+    }
+  }
+  __syncthreads();
+  for (int64_t t = threadIdx.x; t < ntiles; t += 1024) {
+    const int c = 27 - __builtin_popcount(tmask[t] & 0x7FFFFFFu);
+    sched[base[c] + atomicAdd(&cnt[c], 1)] = (int32_t)t;
+  }
+}
+
 int build_tile_plan(const int32_t *nbr, const int32_t *order, const int32_t *d_n, int64_t n_rows, int64_t ld,
-                    int32_t *map, uint32_t *tmask, hipStream_t s) {
+                    int32_t *map, uint32_t *tmask, int32_t *sched, hipStream_t s) {
   if (n_rows <= 0) return INSC_OK;
   const int64_t padded = cdiv(n_rows, TILE_M) * TILE_M;
   hipLaunchKernelGGL(tile_plan_kernel, dim3(grid_for(padded, 256)), dim3(256), 0, s, nbr, order, d_n, n_rows, ld, map,
                      tmask);
+  if (sched) hipLaunchKernelGGL(tile_sched_kernel, dim3(1), dim3(1024), 0, s, tmask, d_n, n_rows, sched);
   INSC_LAUNCH_CHECK();
   return INSC_OK;
 }
@@ -831,6 +1158,11 @@ int pack_weights(const float *W, int K, int Cin, int Cout, float *Wp, hipStream_
   INSC_LAUNCH_CHECK();
   return INSC_OK;
 }
+
+// Launches of a wide 3^3 layer with at least this many (tile, output block) units and a tile
+// schedule go to the persistent kernel (below, one block per unit has all of them resident at once
+// anyway).  Both kernels give the same bits; the bound only moves time.
+static std::atomic<int64_t> g_pers_min_units{512};
 
 // W: raw [K,Cin,Cout] weights (always needed by the generic kernel); Wp: packed weights or
 // null, in which case they are packed into scratch memory first.
@@ -898,7 +1230,7 @@ int launch_conv(const float *in, int64_t ld_in, int64_t in_rows, float *out, int
     const int NB0 = split ? 1 : conv_nb_per_group(Cout);
     const int nbtp = conv_nbt_padded(Cout);
     int S = 1;
-    if (split) S = K == 27 ? (Cin >= 160 ? 8 : Cin >= 128 ? 4 : 2) : (Cin >= 96 ? 4 : 1);  // K == 8: conv and deconv
+    if (split) S = K == 27 ? (Cin >= 160 ? 8 : 4) : (Cin >= 96 ? 4 : 1);  // K == 8: conv and deconv
     const int NB = (S == 1 && Cin >= 96) ? 1 : NB0;
     int G = (split && K == 27) ? (Cin >= 160 ? 4 : Cin >= 128 ? 2 : 1) : 1;
     if (lat) {
@@ -906,6 +1238,21 @@ int launch_conv(const float *in, int64_t ld_in, int64_t in_rows, float *out, int
       S = 4;
     }
     if (G > 1) S = 4;
+    if (mode == MAP_NBR && K == 27 && S == 4 && G == 1 && !lat && plan.map && plan.sched &&
+        tiles * nbt >= g_pers_min_units.load(std::memory_order_relaxed) &&
+        small_ids && ep.ldr * 4 < (1 << 24) && out_rows * ep.ldr * 4 < (int64_t)BUF_OOB) {
+      // persistent blocks, as many as fit on the device at once
+      static int per_cu = 0;
+      if (!per_cu) {
+        INSC_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, conv_pers_kernel<4>, 256, 0));
+        if (per_cu < 1) per_cu = 1;
+      }
+      const unsigned nblk = (unsigned)std::min<int64_t>((int64_t)device_cus() * per_cu, tiles * nbt);
+      hipLaunchKernelGGL(conv_pers_kernel<4>, dim3(nblk), dim3(256), 0, s, in, ld_in, out, ld_out, Wp, bias, rows,
+                         d_n_rows, n_rows, Cin, Cout, nbt, nbtp, tile_flags, in_bytes, wp_bytes, ep, plan);
+      INSC_LAUNCH_CHECK();
+      return INSC_OK;
+    }
     const unsigned gx = (unsigned)(S == 1 ? cdiv(tiles, CONV_WAVES) : tiles);
     dim3 grid(gx, (unsigned)(NB == 1 ? nbt : nbtp / NB), (unsigned)G), block((S == 1 ? CONV_WAVES : S) * 64);
     float *part = nullptr;
@@ -1009,6 +1356,12 @@ using namespace insc;
 
 extern "C" {
 
+int insc_conv_set_persistent_min_units(int64_t units) {
+  INSC_REQUIRE(units >= 1, INSC_ERR_ARG, "insc_conv_set_persistent_min_units: units must be >= 1");
+  g_pers_min_units.store(units, std::memory_order_relaxed);
+  return INSC_OK;
+}
+
 int64_t insc_conv_packed_floats(int K, int Cin, int Cout) {
   if (K <= 0 || Cin <= 0 || Cout <= 0) return 0;
   return packed_floats(K, Cin, Cout);
@@ -1061,17 +1414,18 @@ int insc_conv_nbr(const float *d_in, int64_t ld_in, int64_t n_in_rows, float *d_
 }
 
 int insc_plan_build(const int32_t *d_nbr, const int32_t *d_order, const int32_t *d_n_rows, int64_t n_rows,
-                    int64_t plan_ld, int32_t *d_plan, uint32_t *d_tmask, void *stream) {
+                    int64_t plan_ld, int32_t *d_plan, uint32_t *d_tmask, int32_t *d_sched, void *stream) {
   INSC_REQUIRE(n_rows >= 0 && plan_ld >= cdiv(n_rows, TILE_M) * TILE_M, INSC_ERR_ARG,
                "insc_plan_build: plan_ld must cover the rows rounded up to a multiple of 32");
   INSC_REQUIRE(n_rows == 0 || (d_nbr && d_plan && d_tmask), INSC_ERR_ARG, "insc_plan_build: null pointer");
-  return build_tile_plan(d_nbr, d_order, d_n_rows, n_rows, plan_ld, d_plan, d_tmask, (hipStream_t)stream);
+  return build_tile_plan(d_nbr, d_order, d_n_rows, n_rows, plan_ld, d_plan, d_tmask, d_sched, (hipStream_t)stream);
 }
 
 int insc_conv_ssc_plan(const float *d_in, int64_t ld_in, int64_t n_in_rows, float *d_out, int64_t ld_out,
                        const float *d_W, const float *d_Wp, const float *d_bias, const int32_t *d_nbr,
-                       const int32_t *d_plan, int64_t plan_ld, const uint32_t *d_tmask, const int32_t *d_order,
-                       const int32_t *d_n_rows, int64_t n_rows, int Cin, int Cout, void *stream) {
+                       const int32_t *d_plan, int64_t plan_ld, const uint32_t *d_tmask, const int32_t *d_sched,
+                       const int32_t *d_order, const int32_t *d_n_rows, int64_t n_rows, int Cin, int Cout,
+                       void *stream) {
   INSC_REQUIRE(n_rows >= 0 && Cin > 0 && Cout > 0 && n_in_rows >= 0, INSC_ERR_ARG, "insc_conv_ssc_plan: bad sizes");
   INSC_REQUIRE(ld_in >= Cin && ld_out >= Cout, INSC_ERR_ARG, "insc_conv_ssc_plan: row stride smaller than channel count");
   INSC_REQUIRE(n_rows == 0 || (d_in && d_out && (d_W || d_Wp) && d_nbr && d_plan && d_tmask), INSC_ERR_ARG,
@@ -1081,6 +1435,7 @@ int insc_conv_ssc_plan(const float *d_in, int64_t ld_in, int64_t n_in_rows, floa
   plan.map = d_plan;
   plan.ld = plan_ld;
   plan.tmask = d_tmask;
+  plan.sched = d_sched;
   return launch_conv(d_in, ld_in, n_in_rows, d_out, ld_out, d_W, d_Wp, d_bias, d_nbr, nullptr, MAP_NBR, 27, d_order,
                      d_n_rows, n_rows, Cin, Cout, nullptr, nullptr, (hipStream_t)stream, BnEpilogue(), plan);
 }

@@ -28,6 +28,7 @@ struct Level {
   int32_t *pos = nullptr;       // [cap] inverse of order
   int32_t *plan = nullptr;      // [27,cap] tile plan of the 3^3 map in processing order
   uint32_t *tmask = nullptr;    // [cap/32] offsets used per tile
+  int32_t *sched = nullptr;     // [cap/32] tiles by falling number of offsets used
   int32_t *parent = nullptr;    // [cap] site at the next coarser level
   int32_t *offset = nullptr;    // [cap] position inside the parent cell
   int32_t *child = nullptr;     // [cap_coarse,8] (owned by the FINE level's link)
@@ -339,6 +340,7 @@ static int level_reserve(insc_net *net, int l, int64_t cap, hipStream_t s) {
   if ((rc = dev_grow(&L.pos, (size_t)old, (size_t)cap, s))) return rc;
   if ((rc = dev_grow(&L.plan, 0, (size_t)cap * 27, s))) return rc;  // rebuilt every frame
   if ((rc = dev_grow(&L.tmask, 0, (size_t)cap / 32 + 1, s))) return rc;
+  if ((rc = dev_grow(&L.sched, 0, (size_t)cap / 32 + 1, s))) return rc;
   if (l + 1 < net->n_levels) {
     if ((rc = dev_grow(&L.parent, (size_t)old, (size_t)cap, s))) return rc;
     if ((rc = dev_grow(&L.offset, (size_t)old, (size_t)cap, s))) return rc;
@@ -461,6 +463,7 @@ static int run_op(insc_net *net, const Op &op, bool incremental, hipStream_t s) 
       plan.map = Lo.plan;
       plan.ld = Lo.cap;
       plan.tmask = Lo.tmask;
+      plan.sched = Lo.sched;
       return launch_conv(in0, ld0, rows0, out, ld_out, op.W, op.Wp, op.bias, Lo.nbr, nullptr, MAP_NBR, 27, Lo.order, d_n,
                          n_up, op.Cin, op.Cout, d ? d->tflag : nullptr, d ? d->mask : nullptr, s, ep, plan);
     }
@@ -562,7 +565,7 @@ int insc_net_destroy(insc_net *net) {
   (void)hipDeviceSynchronize();
   for (Level &L : net->levels) {
     if (L.grid) insc_grid_destroy(L.grid);
-    void *ps[] = {L.nbr, L.order, L.pos, L.plan, L.tmask, L.parent, L.offset, L.child, L.bo_order, L.bo_pos};
+    void *ps[] = {L.nbr, L.order, L.pos, L.plan, L.tmask, L.sched, L.parent, L.offset, L.child, L.bo_order, L.bo_pos};
     for (void *p : ps)
       if (p) (void)hipFree(p);
   }
@@ -980,7 +983,7 @@ int insc_net_forward(insc_net *net, const int32_t *d_coords, int coord_cols, con
   // tile plans of the 3^3 maps, shared by all the layers of a scale
   for (int l = 0; l < L; l++) {
     Level &Lv = net->levels[l];
-    if (Lv.n > 0 && (rc = build_tile_plan(Lv.nbr, Lv.order, Lv.grid->d_n, Lv.n, Lv.cap, Lv.plan, Lv.tmask, s))) return rc;
+    if (Lv.n > 0 && (rc = build_tile_plan(Lv.nbr, Lv.order, Lv.grid->d_n, Lv.n, Lv.cap, Lv.plan, Lv.tmask, Lv.sched, s))) return rc;
   }
 
   // ---- input layer output ------------------------------------------------------------------

@@ -92,7 +92,7 @@ class _Scale(object):
         self.nbr_n = 0
         self.order = _Buf(None, torch.int32, device)
         self.order_n = 0
-        self.plan = None  # tile plan of the 3^3 map in processing order: (map [27*ld] int32, tmask, ld)
+        self.plan = None  # tile plan of the 3^3 map in processing order: (map [27*ld] int32, tmask, ld, sched)
         self.plan_n = -1
         self.n_rules = None  # cached number of (in,out) pairs of the 3^3 rulebook
         self.n_rules_at = -1
@@ -230,9 +230,10 @@ class Metadata_3(object):
             if sc.plan is None or sc.plan[2] < ld:
                 cap = max(ld, 1024)
                 sc.plan = (torch.empty(27 * cap, dtype=torch.int32, device=sc.device),
-                           torch.empty(cap // 32 + 1, dtype=torch.int32, device=sc.device), cap)
+                           torch.empty(cap // 32 + 1, dtype=torch.int32, device=sc.device), cap,
+                           torch.empty(cap // 32 + 1, dtype=torch.int32, device=sc.device))
             lib.insc_plan_build(ptr(sc.nbr.t), ptr(sc.order.t), None, I64(sc.n), I64(sc.plan[2]), ptr(sc.plan[0]),
-                                ptr(sc.plan[1]), stream_ptr())
+                                ptr(sc.plan[1]), ptr(sc.plan[3]), stream_ptr())
             sc.plan_n = sc.n
         return sc.plan
 
@@ -372,7 +373,8 @@ def ssc_rows_planned(in_f, out_f, weight, bias, sc, plan):
     Cin, Cout = weight.size(-2), weight.size(-1)
     lib.insc_conv_ssc_plan(ptr(in_f), I64(_ld(in_f)), I64(in_f.size(0)), ptr(out_f), I64(_ld(out_f)), ptr(weight),
                            ptr(packed_weight(weight, 27)), ptr(bias), ptr(sc.nbr.t), ptr(plan[0]), I64(plan[2]),
-                           ptr(plan[1]), ptr(sc.order.t), None, I64(int(sc.n)), int(Cin), int(Cout), stream_ptr())
+                           ptr(plan[1]), ptr(plan[3]), ptr(sc.order.t), None, I64(int(sc.n)), int(Cin), int(Cout),
+                           stream_ptr())
 
 
 def deconv_rows(in_f, out_f, weight, bias, parent, offset, rows, count, n_rows):

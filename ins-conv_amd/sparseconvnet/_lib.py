@@ -31,8 +31,10 @@ _SIGS = {
     "insc_conv_nbr": [vp, c_i64, c_i64, vp, c_i64, vp, vp, vp, vp, c_int, vp, vp, c_i64, c_int, c_int,
                       ctypes.POINTER(ctypes.c_double), vp],
     "insc_conv_pack_weights": [vp, c_int, c_int, c_int, vp, vp],
-    "insc_plan_build": [vp, vp, vp, c_i64, c_i64, vp, vp, vp],
-    "insc_conv_ssc_plan": [vp, c_i64, c_i64, vp, c_i64, vp, vp, vp, vp, vp, c_i64, vp, vp, vp, c_i64, c_int, c_int, vp],
+    "insc_plan_build": [vp, vp, vp, c_i64, c_i64, vp, vp, vp, vp],
+    "insc_conv_ssc_plan": [vp, c_i64, c_i64, vp, c_i64, vp, vp, vp, vp, vp, c_i64, vp, vp, vp, vp, c_i64, c_int, c_int,
+                           vp],
+    "insc_conv_set_persistent_min_units": [c_i64],
     "insc_deconv_down2": [vp, c_i64, c_i64, vp, c_i64, vp, vp, vp, vp, vp, vp, vp, c_i64, c_int, c_int, vp],
     "insc_bn_leaky": [vp, c_i64, vp, c_i64, vp, vp, vp, vp, c_f32, c_f32, vp, vp, c_i64, c_int, vp],
     "insc_add": [vp, c_i64, vp, c_i64, vp, c_i64, vp, vp, c_i64, c_int, vp],

@@ -11,8 +11,19 @@ from test_gpu_incremental import _frames, _inp
 pytestmark = pytest.mark.gpu
 
 
+@pytest.fixture(params=[512, 1], ids=["default-launch-policy", "persistent-kernel-forced"])
+def persistent_min_units(request):
+    """The wide 3^3 layers of these small scenes stay below the persistent kernel's threshold; the
+    second run forces them onto it (fused batch norm / residual epilogues, dirty-tile flags)."""
+    from sparseconvnet._lib import lib
+
+    lib.insc_conv_set_persistent_min_units(request.param)
+    yield request.param
+    lib.insc_conv_set_persistent_min_units(512)
+
+
 @pytest.mark.parametrize("levels,m", [(3, 16), (7, 32)])
-def test_compiled_full_and_incremental(levels, m):
+def test_compiled_full_and_incremental(levels, m, persistent_min_units):
     import sparseconvnet as scn
     from netdefs import NaiveUNet
 

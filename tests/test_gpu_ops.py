@@ -79,6 +79,43 @@ def test_submanifold_convolution(S, orc, Cin, Cout, bias):
     np.testing.assert_allclose(out.cpu().numpy(), ref, rtol=RTOL, atol=ATOL)
 
 
+@pytest.mark.parametrize("Cin,Cout,bias", [(64, 64, False), (64, 32, True), (96, 96, False), (80, 48, True),
+                                            (112, 100, False)])
+def test_persistent_kernel_gives_the_bits_of_the_per_tile_kernel(S, orc, Cin, Cout, bias):
+    """Wide 3^3 layers (64..127 input channels) have two kernels: one block per (tile, output block),
+    and persistent blocks that walk a cost-ordered tile schedule.  They must agree bit for bit (an
+    incremental frame and a full frame may take different ones), and with the oracle to the float
+    tolerance."""
+    from sparseconvnet._lib import lib
+
+    pts = scenes.boxes_scene(seed=5, n=7000)
+    m, x, feats = setup_sites(S, pts, Cin, seed=Cin + 1)
+    sc = m.ssc_rulebook(SZ)
+    rng = np.random.default_rng(Cout + 3)
+    W = cu((rng.normal(size=(27, Cin, Cout)) * (2.0 / Cin / 27) ** 0.5).astype(np.float32))
+    b = rng.normal(size=Cout).astype(np.float32) if bias else None
+    bt = cu(b) if bias else None
+    a = torch.full((sc.n, Cout), 3.0, device="cuda")
+    c = torch.full((sc.n, Cout), -3.0, device="cuda")
+    try:
+        lib.insc_conv_set_persistent_min_units(1)
+        S.ssc_rows_planned(feats, a, W, bt, sc, m.ssc_plan(sc))
+        lib.insc_conv_set_persistent_min_units(1 << 40)
+        S.ssc_rows_planned(feats, c, W, bt, sc, m.ssc_plan(sc))
+    finally:
+        lib.insc_conv_set_persistent_min_units(512)
+    assert torch.equal(a, c)
+    sched = m.ssc_plan(sc)[3][:(sc.n + 31) // 32].cpu().numpy()
+    tmask = m.ssc_plan(sc)[1][:(sc.n + 31) // 32].cpu().numpy().astype(np.uint32)
+    assert sorted(sched.tolist()) == list(range(len(sched))), "the schedule is a permutation of the tiles"
+    cost = np.array([bin(int(v)).count("1") for v in tmask])[sched]
+    assert (np.diff(cost) <= 0).all(), "tiles by falling number of offsets in use"
+    _, osc, _ = orc.grid_build(pts)
+    _, counts, pairs = orc.ssc_rules(osc)
+    ref, _ = orc.conv_forward(feats.cpu().numpy(), W.cpu().numpy(), b, pairs, counts, len(osc))
+    np.testing.assert_allclose(a.cpu().numpy(), ref, rtol=RTOL, atol=ATOL)
+
+
 def test_submanifold_convolution_cfg1_vs_dense_conv3d(S):
     """Workload 1 against the library routine directly (no oracle in the loop)."""
     import torch.nn.functional as F
