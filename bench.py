@@ -125,6 +125,37 @@ def conv_roofline(device, reps=30, warm=200):
     }
 
 
+def wide_conv_row(device, C=64, reps=20, warm=60):
+    """The 64-channel submanifold convolution of workload 3 (500k voxels), which is bound by the
+    matrix cores rather than by HBM: us per launch and the fraction of the fp32 MFMA peak."""
+    import torch
+
+    from sparseconvnet import SCN
+
+    _, info, (x, stack) = ssc_workload(device, channels=(C,))
+    conv = stack[0]
+    m = x.metadata
+    sc = m.ssc_rulebook(x.spatial_size)
+    out = torch.empty((sc.n, conv.nOut), device=device)
+    plan = m.ssc_plan(sc)
+    for _ in range(warm):
+        SCN.ssc_rows_planned(x.features, out, conv.weight, None, sc, plan)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        SCN.ssc_rows_planned(x.features, out, conv.weight, None, sc, plan)
+    e1.record()
+    torch.cuda.synchronize()
+    t = e0.elapsed_time(e1) * 1e-3 / reps
+    flops = 2.0 * info["rules"] * C * C
+    bytes_alg = info["rules"] * (4 * C + 8) + sc.n * 4 * C + 27 * C * C * 4
+    return {"kernel": "conv_pers_kernel<4> (SSC 3^3, %d->%d, persistent blocks over the tile schedule; 500k sites)" % (C, C),
+            "bound": "mfma", "avg_us": round(t * 1e6, 1), "achieved": round(flops / t / 1e12, 2),
+            "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(flops / t / 1e12 / MFMA_FP32_PEAK_TFLOPS, 4),
+            "GB/s_on_algorithmic_bytes": round(bytes_alg / t / 1e9, 1)}
+
+
 # ---------------------------------------------------------------------------------------------
 # the bandwidth-bound kernels of the path, one C call each, against the HBM roofline
 # ---------------------------------------------------------------------------------------------
@@ -491,6 +522,7 @@ def main():
     }
     out.update(extra)
     out["roofline"] = conv_roofline(device)
+    out["wide_layer"] = wide_conv_row(device)
     out["kernels"] = kernel_table(device)
     # the CPU leg comes last: the GPU idles during it, and a measurement taken right after would
     # start at idle clocks
