@@ -146,10 +146,11 @@ int insc_conv_pack_weights(const float *d_W, int K, int Cin, int Cout, float *d_
  * its chunk rulebook, SubmanifoldRules_cuda.cpp:572-1112, plays this role for its kernel):
  * d_plan[k*plan_ld + p] = d_nbr[d_order[p]*27 + k] for p < n_rows and -1 up to the next multiple of
  * 32; d_tmask[t] = bit k set if some row of tile t (positions 32t..32t+31) has neighbour k.
- * d_sched (nullable) [t] = the tiles by falling number of neighbours in use, the order in which
- * the persistent kernel of wide layers takes them.
- * plan_ld >= n_rows rounded up to a multiple of 32; d_plan holds 27*plan_ld int32, d_tmask and
- * d_sched plan_ld/32 entries.  d_order NULL = identity.  Rebuild after the map or the order changed. */
+ * d_sched (nullable) = the tiles by falling number of neighbours in use (plan_ld/32 entries), then
+ * the groups of four consecutive tiles by falling number of neighbours any of the four uses: the
+ * orders in which the persistent kernels of wide layers take them.
+ * plan_ld >= n_rows rounded up to a multiple of 32; d_plan holds 27*plan_ld int32, d_tmask
+ * plan_ld/32 entries, d_sched plan_ld/32 + plan_ld/128 + 1.  d_order NULL = identity.  Rebuild after the map or the order changed. */
 int insc_plan_build(const int32_t *d_nbr, const int32_t *d_order, const int32_t *d_n_rows, int64_t n_rows,
                     int64_t plan_ld, int32_t *d_plan, uint32_t *d_tmask, int32_t *d_sched, void *stream);
 /* insc_conv_nbr for K = 27 over the rows d_order[0..n_rows) with their tile plan: same result
@@ -161,8 +162,11 @@ int insc_conv_ssc_plan(const float *d_in, int64_t ld_in, int64_t n_in_rows, floa
                        void *stream);
 /* A 3^3 layer of 64..127 input channels with a tile schedule runs on persistent blocks once it has
  * at least `units` (tile, 32-column output block) pairs (default 512); below, one block per pair.
- * Same bits either way: a tuning and test knob with no counterpart in the reference. */
+ * With at least `units` (four consecutive tiles, output block) pairs (default 896) it runs on the
+ * kernel whose blocks share the weight tiles through LDS.  Same bits in all three cases: tuning and
+ * test knobs with no counterpart in the reference. */
 int insc_conv_set_persistent_min_units(int64_t units);
+int insc_conv_set_shared_weights_min_units(int64_t units);
 /* Size-2 stride-2 deconvolution: out[i,:] = bias + in[parent[i],:] . W[offset[i]]
  * (Deconvolution_updateOutput, CUDA/Deconvolution.cpp:28-58: the convolution's rules with
  * the roles of input and output swapped). */

@@ -1066,6 +1066,283 @@ __global__ __launch_bounds__(S * 64) __attribute__((amdgpu_waves_per_eu(3, 3))) 
   }
 }
 
+// ---------------------------------------------------------------------------------------
+// Wide 3^3 layers with many tiles, second design: the bytes a compute unit pulls through its L1
+// bound these layers (8 KB per 16 MFMAs: a gathered chunk and a weight tile), so here the four
+// wavefronts of a block work on four consecutive tiles and walk the union of their offsets in
+// step: the weight tile of a step goes from L2 into LDS once per block (buffer loads that write
+// LDS directly, a quarter per wavefront) and is read from there by all four, and a wavefront
+// computes NB output blocks from one gathered chunk.  A wavefront owns its tile: no partial sums
+// cross wavefronts.  To give the bits of conv_mfma_kernel<1, 27, MAP_NBR, ST> it keeps that
+// kernel's ST partial sums - the items (k, ch) with (k * nch + ch) % ST == p, in ascending order,
+// bias in sum 0 - in ST accumulators per output block and adds them in order at the end.
+// Blocks are persistent over units (group of four tiles, NB output blocks) taken from the cost-
+// ordered group schedule as in conv_pers_kernel.
+// The two weight buffers and the two A slots alternate with the parity of the step, and the step
+// loop is unrolled by two so that each is a compile-time choice: the compiler then knows that a
+// read of one weight buffer cannot touch the load into the other that is still in flight (for a
+// single array it would wait for every outstanding load before each LDS read).
+// ---------------------------------------------------------------------------------------
+#define INSC_LDS_PTR(x) ((__attribute__((address_space(3))) void *)(x))
+template <int NB, int ST>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) void conv_wshare_kernel(
+    const float *__restrict__ in, int64_t ld_in, float *__restrict__ out, int64_t ld_out,
+    const float *__restrict__ Wp, const float *__restrict__ bias, const int32_t *__restrict__ rows,
+    const int32_t *__restrict__ d_n_rows, int64_t n_rows, int Cin, int Cout, int nbt, int nbtp,
+    const uint8_t *__restrict__ tile_flags, uint32_t in_bytes, uint32_t wp_bytes, BnEpilogue ep, TilePlan plan) {
+  constexpr int K = 27, WV = 4;
+  constexpr int NSTAGE = (TILE_M * K + 63) / 64;  // 14 loads of 64 entries; the last one half empty
+  __shared__ int nl[WV][NSTAGE * 64];
+  __shared__ float4 wl0[NB][256];
+  __shared__ float4 wl1[NB][256];
+  const int64_t n = d_n_rows ? min((int64_t)*d_n_rows, n_rows) : n_rows;
+  const int ntiles = (int)((n + TILE_M - 1) / TILE_M), ngroups = (ntiles + WV - 1) / WV;
+  const int nug = (nbt + NB - 1) / NB;  // units per group
+  const int64_t units = (int64_t)ngroups * nug;
+  const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), lane = threadIdx.x & 63;
+  const int r = lane & 31, h = lane >> 5;
+  const int nch = conv_nch(Cin);
+  const int64_t B = gridDim.x, b = blockIdx.x;
+  const __amdgpu_buffer_rsrc_t rplan = make_rsrc(plan.map, (uint32_t)(plan.ld * K * 4));
+  const __amdgpu_buffer_rsrc_t rsched = make_rsrc(plan.sched + (plan.ld + 31) / 32, (uint32_t)ngroups * 4u);  // group schedule
+  const __amdgpu_buffer_rsrc_t rtmask = make_rsrc(plan.tmask, (uint32_t)ntiles * 4u);
+  const __amdgpu_buffer_rsrc_t rflag = make_rsrc(tile_flags, tile_flags ? (uint32_t)ntiles : 0u);
+  const __amdgpu_buffer_rsrc_t rin = make_rsrc(in, in_bytes), rw = make_rsrc(Wp, wp_bytes);
+  const __amdgpu_buffer_rsrc_t rout = make_rsrc(out, out ? BUF_OOB : 0u), rout2 = make_rsrc(ep.out2, ep.out2 ? BUF_OOB : 0u);
+  const __amdgpu_buffer_rsrc_t rres = make_rsrc(ep.res, ep.res ? BUF_OOB : 0u);
+  const __amdgpu_buffer_rsrc_t rbias = make_rsrc(bias, bias ? (uint32_t)Cout * 4u : 0u);
+  const __amdgpu_buffer_rsrc_t rew = make_rsrc(ep.w, ep.out2 ? (uint32_t)Cout * 4u : 0u);
+  const __amdgpu_buffer_rsrc_t reb = make_rsrc(ep.b, ep.out2 ? (uint32_t)Cout * 4u : 0u);
+  const uint32_t ld4 = (uint32_t)ld_in * 4u, ldo4 = (uint32_t)ld_out * 4u, ldo24 = (uint32_t)ep.ld2 * 4u,
+                 ldr4 = (uint32_t)ep.ldr * 4u;
+  int *nlw = nl[wave];
+
+  auto unit_at = [&](int64_t j) -> int64_t { return j * B + ((j & 1) ? B - 1 - b : b); };
+  auto group_issue = [&](int64_t u) -> int {
+    return __builtin_amdgcn_raw_buffer_load_b32(rsched, (int)(u < units ? (uint32_t)(u / nug) * 4u : BUF_OOB), 0, 0);
+  };
+  // offset masks of the four tiles of a group (0 for a tile that does not exist or is not flagged):
+  // lanes 0..3 fetch one each, every wavefront the same four
+  auto masks_issue = [&](int g, int &mv, int &fv) {
+    const int t = g * WV + (lane & 3);
+    const bool ok = g >= 0 && t < ntiles;
+    mv = __builtin_amdgcn_raw_buffer_load_b32(rtmask, (int)(ok ? (uint32_t)t * 4u : BUF_OOB), 0, 0);
+    fv = tile_flags ? (int)__builtin_amdgcn_raw_buffer_load_b8(rflag, (int)(ok ? (uint32_t)t : BUF_OOB), 0, 0) : (ok ? 1 : 0);
+  };
+  // this wavefront's slice of the map, straight into LDS (entry e = k * 32 + row at nlw[e])
+  // (load i covers the offsets 2i and 2i + 1: one per half-wave; the lane's part of the address is the
+  // same for every i, the rest is a scalar)
+  auto stage_issue = [&](int tile) {
+    if (tile < 0) return;  // no such tile: its wavefront never reads the slice
+    const uint32_t base = (uint32_t)(h * (int)plan.ld + tile * TILE_M + r) * 4u;
+    const uint32_t pair = (uint32_t)plan.ld * 8u;
+#pragma unroll
+    for (int i = 0; i < NSTAGE; i++) {
+      const uint32_t voff = (2 * i + 1 < K || h == 0) ? base : BUF_OOB;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rplan, INSC_LDS_PTR(nlw + i * 64), 4, (int)voff, (int)(i * pair), 0, 0);
+    }
+  };
+  auto row_of = [&](int tile) -> int {
+    const int64_t p = (int64_t)tile * TILE_M + r;
+    return (tile >= 0 && p < n) ? (rows ? rows[p] : (int)p) : -1;
+  };
+  struct Step {
+    int k, ch;
+    unsigned rest;
+  };
+  auto step_next = [&](const Step &c) -> Step {  // past the end: k = -1
+    Step nx;
+    const bool wrap = c.ch + 1 >= nch;
+    const int nk = c.rest ? __builtin_ctz(c.rest) : -1;
+    nx.ch = wrap ? 0 : c.ch + 1;
+    nx.k = wrap ? nk : c.k;
+    nx.rest = wrap ? (c.rest & (c.rest - 1)) : c.rest;
+    return nx;
+  };
+
+  int64_t j = 0, u = unit_at(0);
+  int g_c = u < units ? __builtin_amdgcn_readfirstlane(group_issue(u)) : -1;
+  int g_n = unit_at(1) < units ? __builtin_amdgcn_readfirstlane(group_issue(unit_at(1))) : -1;
+  int mv_c, fv_c;
+  masks_issue(g_c, mv_c, fv_c);
+  int tile = g_c >= 0 && g_c * WV + wave < ntiles ? g_c * WV + wave : -1;
+  stage_issue(tile);
+  int my_row = row_of(tile);
+
+  while (u < units) {
+    const int ob0 = (int)(u % nug) * NB;
+    const int64_t un = unit_at(j + 1), unn = unit_at(j + 2);
+    const int g_nn_v = group_issue(unn);
+    int mv_n, fv_n;
+    masks_issue(g_n, mv_n, fv_n);
+    const int tile_n = g_n >= 0 && g_n * WV + wave < ntiles ? g_n * WV + wave : -1;
+    const int my_row_n = row_of(tile_n);
+    // masks of the group: mine and the union
+    unsigned mt[WV];
+#pragma unroll
+    for (int w = 0; w < WV; w++)
+      mt[w] = __builtin_amdgcn_readlane(fv_c, w) ? (unsigned)__builtin_amdgcn_readlane(mv_c, w) : 0u;
+    unsigned mine = 0, uni = 0;
+#pragma unroll
+    for (int w = 0; w < WV; w++) {
+      uni |= mt[w];
+      if (w == wave) mine = mt[w];
+    }
+    if (tile < 0) mine = 0;
+
+    if (uni) {
+      // bias and the fused batch norm's coefficients of this lane's columns
+      float bv[NB], ew[NB], eb[NB];
+#pragma unroll
+      for (int o = 0; o < NB; o++) {
+        const uint32_t off = (uint32_t)((ob0 + o) * 32 + r) * 4u;
+        bv[o] = __uint_as_float((unsigned)__builtin_amdgcn_raw_buffer_load_b32(rbias, (int)off, 0, 0));
+        ew[o] = __uint_as_float((unsigned)__builtin_amdgcn_raw_buffer_load_b32(rew, (int)off, 0, 0));
+        eb[o] = __uint_as_float((unsigned)__builtin_amdgcn_raw_buffer_load_b32(reb, (int)off, 0, 0));
+      }
+      f16v acc[ST][NB];  // partial sum p holds the items with (k * nch + ch) % ST == p; bias in sum 0
+#pragma unroll
+      for (int pp = 0; pp < ST; pp++) {
+#pragma unroll
+        for (int o = 0; o < NB; o++) {
+#pragma unroll
+          for (int v = 0; v < 16; v++) acc[pp][o][v] = pp == 0 ? bv[o] : 0.0f;
+        }
+      }
+      const int nsteps = __builtin_popcount(uni) * nch;
+      // weight tiles of a step -> LDS, a quarter (1 KB) per wavefront and output block
+      auto w_issue0 = [&](const Step &c) {
+#pragma unroll
+        for (int o = 0; o < NB; o++) {
+          const uint32_t soff = (uint32_t)(((c.k < 0 ? 0 : c.k) * nch + c.ch) * nbtp + ob0 + o) * 4096u;
+          const bool ok = c.k >= 0 && ob0 + o < nbt;
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, INSC_LDS_PTR(&wl0[o][wave * 64]), 16,
+                                                   (int)(ok ? (uint32_t)(wave * 1024 + lane * 16) : BUF_OOB), (int)soff, 0, 0);
+        }
+      };
+      auto w_issue1 = [&](const Step &c) {
+#pragma unroll
+        for (int o = 0; o < NB; o++) {
+          const uint32_t soff = (uint32_t)(((c.k < 0 ? 0 : c.k) * nch + c.ch) * nbtp + ob0 + o) * 4096u;
+          const bool ok = c.k >= 0 && ob0 + o < nbt;
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, INSC_LDS_PTR(&wl1[o][wave * 64]), 16,
+                                                   (int)(ok ? (uint32_t)(wave * 1024 + lane * 16) : BUF_OOB), (int)soff, 0, 0);
+        }
+      };
+      auto gather = [&](const Step &c) -> Frag {
+        const int kk = c.k < 0 ? 0 : c.k;
+        const int src = nlw[kk * TILE_M + r];
+        const bool on = c.k >= 0 && ((mine >> kk) & 1u) && src >= 0 && (h == 0 || Cin - c.ch * 32 >= 32);
+        const uint32_t voff = on ? (uint32_t)src * ld4 + (uint32_t)(c.ch * 128 + h * 64) : BUF_OOB;
+        Frag f;
+#pragma unroll
+        for (int q = 0; q < 4; q++) f.q[q] = buf_load16(rin, voff + 16u * q, 0);
+        return f;
+      };
+      auto compute = [&](const Step &c, const Frag &a, const float4 (*wl)[256]) {
+        if (c.k < 0 || !((mine >> c.k) & 1u)) return;  // (the same for every lane of the wavefront)
+        const int part = (c.k * nch + c.ch) & (ST - 1);
+#pragma unroll
+        for (int o = 0; o < NB; o++) {
+          if (ob0 + o >= nbt) break;
+          Frag bf;
+#pragma unroll
+          for (int q = 0; q < 4; q++) bf.q[q] = wl[o][q * 64 + lane];
+#pragma unroll
+          for (int pp = 0; pp < ST; pp++) {
+            if (part != pp) continue;  // (one copy of the MFMA block per partial sum: the accumulator is a compile-time choice)
+#pragma unroll
+            for (int s2 = 0; s2 < 16; s2++)
+              acc[pp][o] = __builtin_amdgcn_mfma_f32_32x32x2f32(frag_at(a, s2), frag_at(bf, s2), acc[pp][o], 0, 0, 0);
+          }
+        }
+      };
+      Step c0;  // step on the matrix cores
+      c0.k = __builtin_ctz(uni);
+      c0.ch = 0;
+      c0.rest = uni & (uni - 1);
+      Step c1 = step_next(c0);
+      __builtin_amdgcn_sched_barrier(0);
+      w_issue0(c0);
+      __builtin_amdgcn_sched_barrier(0);
+      Frag a0 = gather(c0), a1;
+      __builtin_amdgcn_sched_barrier(0);
+      // Before a barrier every wavefront waits until its own quarter of the step's weight tiles has
+      // landed in LDS: everything but the four gather loads issued after it (vmcnt(4); the order of
+      // the loads is pinned).
+      for (int s0 = 0; s0 < nsteps; s0 += 2) {
+        // even step: weights in wl0, chunk in a0
+        __builtin_amdgcn_s_waitcnt(0x0F74);
+        __syncthreads();  // W(s0) is complete for every wavefront, and nobody reads wl1 any more
+        __builtin_amdgcn_sched_barrier(0);
+        w_issue1(c1);
+        __builtin_amdgcn_sched_barrier(0);
+        a1 = gather(c1);
+        __builtin_amdgcn_sched_barrier(0);
+        compute(c0, a0, wl0);
+        c0 = step_next(c1);
+        // odd step: weights in wl1, chunk in a1
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_waitcnt(0x0F74);
+        __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+        w_issue0(c0);
+        __builtin_amdgcn_sched_barrier(0);
+        a0 = gather(c0);
+        __builtin_amdgcn_sched_barrier(0);
+        compute(c1, a1, wl1);
+        c1 = step_next(c0);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      __syncthreads();  // the weight buffers are free for the next unit
+
+      // this unit's rows; the next unit's map slice goes out first (nobody reads nl any more)
+      stage_issue(tile_n);
+      int rid[16];
+#pragma unroll
+      for (int v = 0; v < 16; v++) rid[v] = __shfl(my_row, 8 * (v >> 2) + 4 * h + (v & 3), 64);
+      if (mine) {
+#pragma unroll
+        for (int o = 0; o < NB; o++) {
+          const int cc = (ob0 + o) * 32 + r;
+          if (ob0 + o >= nbt) break;
+          float rv[16];
+#pragma unroll
+          for (int v = 0; v < 16; v++)
+            rv[v] = __uint_as_float((unsigned)__builtin_amdgcn_raw_buffer_load_b32(
+                rres, (int)((rid[v] >= 0 && cc < Cout) ? __umul24((unsigned)rid[v], ldr4) + (uint32_t)cc * 4u : BUF_OOB), 0, 0));
+#pragma unroll
+          for (int v = 0; v < 16; v++) {
+            const bool ok = rid[v] >= 0 && cc < Cout;
+            float a = acc[0][o][v];
+#pragma unroll
+            for (int pp = 1; pp < ST; pp++) a += acc[pp][o][v];
+            if (ep.res) a += rv[v];
+            if (out)
+              __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(a), rout,
+                                                    (int)(ok ? __umul24((unsigned)rid[v], ldo4) + (uint32_t)cc * 4u : BUF_OOB), 0, 0);
+            if (ep.out2) {
+              const float y = fmaf(a, ew[o], eb[o]);
+              __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(y * ((y > 0.0f) ? 1.0f : ep.leak)), rout2,
+                                                    (int)(ok ? __umul24((unsigned)rid[v], ldo24) + (uint32_t)cc * 4u : BUF_OOB), 0, 0);
+            }
+          }
+        }
+      }
+    } else {
+      stage_issue(tile_n);
+    }
+    j++;
+    u = un;
+    g_c = g_n;
+    g_n = unn < units ? __builtin_amdgcn_readfirstlane(g_nn_v) : -1;
+    mv_c = mv_n;
+    fv_c = fv_n;
+    tile = tile_n;
+    my_row = my_row_n;
+  }
+}
+
 __global__ void count_rules_kernel(const int32_t *__restrict__ map0, int K, const int32_t *__restrict__ rows,
                                    const int32_t *__restrict__ d_n_rows, int64_t n_rows,
                                    unsigned long long *__restrict__ total) {
@@ -1109,7 +1386,7 @@ __global__ __launch_bounds__(256) void tile_plan_kernel(const int32_t *__restric
 // workgroup; the order inside a class is the order of arrival and has no influence on any result).
 __global__ __launch_bounds__(1024) void tile_sched_kernel(const uint32_t *__restrict__ tmask,
                                                           const int32_t *__restrict__ d_n, int64_t n_rows,
-                                                          int32_t *__restrict__ sched) {
+                                                          int32_t *__restrict__ sched, int32_t *__restrict__ gsched) {
   __shared__ int cnt[28], base[28];
   const int64_t n = d_n ? min((int64_t)*d_n, n_rows) : n_rows;
   const int64_t ntiles = (n + TILE_M - 1) / TILE_M;
@@ -1130,6 +1407,32 @@ __global__ __launch_bounds__(1024) void tile_sched_kernel(const uint32_t *__rest
     const int c = 27 - __builtin_popcount(tmask[t] & 0x7FFFFFFu);
     sched[base[c] + atomicAdd(&cnt[c], 1)] = (int32_t)t;
   }
+  // the same for groups of four consecutive tiles, by the offsets any of the four uses; the group
+  // schedule follows the tile schedule at gsched
+  const int64_t ngroups = (ntiles + 3) / 4;
+  auto gmask = [&](int64_t g) -> unsigned {
+    unsigned m = 0;
+    for (int64_t t = g * 4; t < min(g * 4 + 4, ntiles); t++) m |= tmask[t];
+    return m & 0x7FFFFFFu;
+  };
+  __syncthreads();
+  if (threadIdx.x < 28) cnt[threadIdx.x] = 0;
+  __syncthreads();
+  for (int64_t g = threadIdx.x; g < ngroups; g += 1024) atomicAdd(&cnt[27 - __builtin_popcount(gmask(g))], 1);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int a = 0;
+    for (int c = 0; c < 28; c++) {
+      base[c] = a;
+      a += cnt[c];
+      cnt[c] = 0;
+    }
+  }
+  __syncthreads();
+  for (int64_t g = threadIdx.x; g < ngroups; g += 1024) {
+    const int c = 27 - __builtin_popcount(gmask(g));
+    gsched[base[c] + atomicAdd(&cnt[c], 1)] = (int32_t)g;
+  }
 }
 
 int build_tile_plan(const int32_t *nbr, const int32_t *order, const int32_t *d_n, int64_t n_rows, int64_t ld,
@@ -1138,7 +1441,8 @@ int build_tile_plan(const int32_t *nbr, const int32_t *order, const int32_t *d_n
   const int64_t padded = cdiv(n_rows, TILE_M) * TILE_M;
   hipLaunchKernelGGL(tile_plan_kernel, dim3(grid_for(padded, 256)), dim3(256), 0, s, nbr, order, d_n, n_rows, ld, map,
                      tmask);
-  if (sched) hipLaunchKernelGGL(tile_sched_kernel, dim3(1), dim3(1024), 0, s, tmask, d_n, n_rows, sched);
+  if (sched)
+    hipLaunchKernelGGL(tile_sched_kernel, dim3(1), dim3(1024), 0, s, tmask, d_n, n_rows, sched, sched + (ld + 31) / 32);
   INSC_LAUNCH_CHECK();
   return INSC_OK;
 }
@@ -1163,6 +1467,9 @@ int pack_weights(const float *W, int K, int Cin, int Cout, float *Wp, hipStream_
 // schedule go to the persistent kernel (below, one block per unit has all of them resident at once
 // anyway).  Both kernels give the same bits; the bound only moves time.
 static std::atomic<int64_t> g_pers_min_units{512};
+// ... and with at least this many (group of four tiles, output block) units to the kernel whose blocks
+// share the weight tiles through LDS (faster from about 60k sites at 64 channels; same bits again).
+static std::atomic<int64_t> g_shared_min_units{896};
 
 // W: raw [K,Cin,Cout] weights (always needed by the generic kernel); Wp: packed weights or
 // null, in which case they are packed into scratch memory first.
@@ -1238,9 +1545,23 @@ int launch_conv(const float *in, int64_t ld_in, int64_t in_rows, float *out, int
       S = 4;
     }
     if (G > 1) S = 4;
-    if (mode == MAP_NBR && K == 27 && S == 4 && G == 1 && !lat && plan.map && plan.sched &&
-        tiles * nbt >= g_pers_min_units.load(std::memory_order_relaxed) &&
-        small_ids && ep.ldr * 4 < (1 << 24) && out_rows * ep.ldr * 4 < (int64_t)BUF_OOB) {
+    const bool wide_planned = mode == MAP_NBR && K == 27 && S == 4 && G == 1 && !lat && plan.map && plan.sched &&
+                              small_ids && ep.ldr * 4 < (1 << 24) && out_rows * ep.ldr * 4 < (int64_t)BUF_OOB;
+    if (wide_planned && cdiv(tiles, 4) * nbt >= g_shared_min_units.load(std::memory_order_relaxed)) {
+      // blocks of four tiles that share the weight tiles through LDS
+      static int per_cu2 = 0;
+      if (!per_cu2) {
+        INSC_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu2, conv_wshare_kernel<1, 4>, 256, 0));
+        if (per_cu2 < 1) per_cu2 = 1;
+      }
+      const int64_t wunits = cdiv(tiles, 4) * nbt;
+      const unsigned nblk = (unsigned)std::min<int64_t>((int64_t)device_cus() * per_cu2, wunits);
+      hipLaunchKernelGGL((conv_wshare_kernel<1, 4>), dim3(nblk), dim3(256), 0, s, in, ld_in, out, ld_out, Wp, bias, rows,
+                         d_n_rows, n_rows, Cin, Cout, nbt, nbtp, tile_flags, in_bytes, wp_bytes, ep, plan);
+      INSC_LAUNCH_CHECK();
+      return INSC_OK;
+    }
+    if (wide_planned && tiles * nbt >= g_pers_min_units.load(std::memory_order_relaxed)) {
       // persistent blocks, as many as fit on the device at once
       static int per_cu = 0;
       if (!per_cu) {
@@ -1359,6 +1680,12 @@ extern "C" {
 int insc_conv_set_persistent_min_units(int64_t units) {
   INSC_REQUIRE(units >= 1, INSC_ERR_ARG, "insc_conv_set_persistent_min_units: units must be >= 1");
   g_pers_min_units.store(units, std::memory_order_relaxed);
+  return INSC_OK;
+}
+
+int insc_conv_set_shared_weights_min_units(int64_t units) {
+  INSC_REQUIRE(units >= 1, INSC_ERR_ARG, "insc_conv_set_shared_weights_min_units: units must be >= 1");
+  g_shared_min_units.store(units, std::memory_order_relaxed);
   return INSC_OK;
 }
 

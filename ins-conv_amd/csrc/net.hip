@@ -340,7 +340,7 @@ static int level_reserve(insc_net *net, int l, int64_t cap, hipStream_t s) {
   if ((rc = dev_grow(&L.pos, (size_t)old, (size_t)cap, s))) return rc;
   if ((rc = dev_grow(&L.plan, 0, (size_t)cap * 27, s))) return rc;  // rebuilt every frame
   if ((rc = dev_grow(&L.tmask, 0, (size_t)cap / 32 + 1, s))) return rc;
-  if ((rc = dev_grow(&L.sched, 0, (size_t)cap / 32 + 1, s))) return rc;
+  if ((rc = dev_grow(&L.sched, 0, (size_t)cap / 32 + (size_t)cap / 128 + 3, s))) return rc;  // tiles, then groups of 4
   if (l + 1 < net->n_levels) {
     if ((rc = dev_grow(&L.parent, (size_t)old, (size_t)cap, s))) return rc;
     if ((rc = dev_grow(&L.offset, (size_t)old, (size_t)cap, s))) return rc;

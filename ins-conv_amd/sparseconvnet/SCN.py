@@ -231,7 +231,7 @@ class Metadata_3(object):
                 cap = max(ld, 1024)
                 sc.plan = (torch.empty(27 * cap, dtype=torch.int32, device=sc.device),
                            torch.empty(cap // 32 + 1, dtype=torch.int32, device=sc.device), cap,
-                           torch.empty(cap // 32 + 1, dtype=torch.int32, device=sc.device))
+                           torch.empty(cap // 32 + cap // 128 + 3, dtype=torch.int32, device=sc.device))
             lib.insc_plan_build(ptr(sc.nbr.t), ptr(sc.order.t), None, I64(sc.n), I64(sc.plan[2]), ptr(sc.plan[0]),
                                 ptr(sc.plan[1]), ptr(sc.plan[3]), stream_ptr())
             sc.plan_n = sc.n

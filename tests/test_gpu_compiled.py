@@ -11,15 +11,19 @@ from test_gpu_incremental import _frames, _inp
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture(params=[512, 1], ids=["default-launch-policy", "persistent-kernel-forced"])
+@pytest.fixture(params=[(512, 896), (1, 1 << 40), (512, 1)],
+                ids=["default-launch-policy", "persistent-kernel-forced", "shared-weights-kernel-forced"])
 def persistent_min_units(request):
-    """The wide 3^3 layers of these small scenes stay below the persistent kernel's threshold; the
-    second run forces them onto it (fused batch norm / residual epilogues, dirty-tile flags)."""
+    """The wide 3^3 layers of these small scenes stay below the thresholds of the two persistent
+    kernels; the second and third run force them onto one and the other (fused batch norm / residual
+    epilogues, dirty-tile flags)."""
     from sparseconvnet._lib import lib
 
-    lib.insc_conv_set_persistent_min_units(request.param)
+    lib.insc_conv_set_persistent_min_units(request.param[0])
+    lib.insc_conv_set_shared_weights_min_units(request.param[1])
     yield request.param
     lib.insc_conv_set_persistent_min_units(512)
+    lib.insc_conv_set_shared_weights_min_units(896)
 
 
 @pytest.mark.parametrize("levels,m", [(3, 16), (7, 32)])

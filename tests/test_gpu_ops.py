@@ -81,11 +81,11 @@ def test_submanifold_convolution(S, orc, Cin, Cout, bias):
 
 @pytest.mark.parametrize("Cin,Cout,bias", [(64, 64, False), (64, 32, True), (96, 96, False), (80, 48, True),
                                             (112, 100, False)])
-def test_persistent_kernel_gives_the_bits_of_the_per_tile_kernel(S, orc, Cin, Cout, bias):
-    """Wide 3^3 layers (64..127 input channels) have two kernels: one block per (tile, output block),
-    and persistent blocks that walk a cost-ordered tile schedule.  They must agree bit for bit (an
-    incremental frame and a full frame may take different ones), and with the oracle to the float
-    tolerance."""
+def test_persistent_kernels_give_the_bits_of_the_per_tile_kernel(S, orc, Cin, Cout, bias):
+    """Wide 3^3 layers (64..127 input channels) have three kernels: one block per (tile, output
+    block), persistent blocks that walk a cost-ordered tile schedule, and persistent blocks of four
+    tiles that share the weight tiles through LDS.  They must agree bit for bit (an incremental frame
+    and a full frame may take different ones), and with the oracle to the float tolerance."""
     from sparseconvnet._lib import lib
 
     pts = scenes.boxes_scene(seed=5, n=7000)
@@ -97,19 +97,33 @@ def test_persistent_kernel_gives_the_bits_of_the_per_tile_kernel(S, orc, Cin, Co
     bt = cu(b) if bias else None
     a = torch.full((sc.n, Cout), 3.0, device="cuda")
     c = torch.full((sc.n, Cout), -3.0, device="cuda")
+    d = torch.full((sc.n, Cout), 5.0, device="cuda")
     try:
+        lib.insc_conv_set_shared_weights_min_units(1 << 40)
         lib.insc_conv_set_persistent_min_units(1)
         S.ssc_rows_planned(feats, a, W, bt, sc, m.ssc_plan(sc))
         lib.insc_conv_set_persistent_min_units(1 << 40)
         S.ssc_rows_planned(feats, c, W, bt, sc, m.ssc_plan(sc))
+        lib.insc_conv_set_shared_weights_min_units(1)
+        S.ssc_rows_planned(feats, d, W, bt, sc, m.ssc_plan(sc))
     finally:
         lib.insc_conv_set_persistent_min_units(512)
+        lib.insc_conv_set_shared_weights_min_units(896)
     assert torch.equal(a, c)
-    sched = m.ssc_plan(sc)[3][:(sc.n + 31) // 32].cpu().numpy()
-    tmask = m.ssc_plan(sc)[1][:(sc.n + 31) // 32].cpu().numpy().astype(np.uint32)
-    assert sorted(sched.tolist()) == list(range(len(sched))), "the schedule is a permutation of the tiles"
+    assert torch.equal(d, c)
+    nt = (sc.n + 31) // 32
+    plan = m.ssc_plan(sc)
+    sched = plan[3][:nt].cpu().numpy()
+    tmask = plan[1][:nt].cpu().numpy().astype(np.uint32)
+    assert sorted(sched.tolist()) == list(range(nt)), "the schedule is a permutation of the tiles"
     cost = np.array([bin(int(v)).count("1") for v in tmask])[sched]
     assert (np.diff(cost) <= 0).all(), "tiles by falling number of offsets in use"
+    ng = (nt + 3) // 4
+    gsched = plan[3][plan[2] // 32:plan[2] // 32 + ng].cpu().numpy()
+    assert sorted(gsched.tolist()) == list(range(ng)), "the group schedule is a permutation of the groups"
+    gmask = [int(np.bitwise_or.reduce(tmask[4 * g:4 * g + 4])) for g in range(ng)]
+    gcost = np.array([bin(v).count("1") for v in gmask])[gsched]
+    assert (np.diff(gcost) <= 0).all(), "groups by falling number of offsets in use"
     _, osc, _ = orc.grid_build(pts)
     _, counts, pairs = orc.ssc_rules(osc)
     ref, _ = orc.conv_forward(feats.cpu().numpy(), W.cpu().numpy(), b, pairs, counts, len(osc))
