@@ -19,6 +19,10 @@ namespace insc {
 
 enum OpKind { OP_SSC, OP_BN, OP_CONV, OP_DECONV, OP_NIN, OP_ADD, OP_COPY, OP_JOIN };
 enum DirtyKind { D_INPUT, D_DILATE, D_PARENTS, D_CHILDREN, D_UNION };
+// Scales this small are recomputed whole by incremental frames.  (128 tiles: every launch has all its
+// tiles resident at once, and with the eight 3^3 layers of such a scale and of each coarser one a
+// change anywhere reaches nearly every site of it anyway.)
+constexpr int64_t DIRTY_FULL_SITES = 4096;
 
 struct Level {
   insc_grid *grid = nullptr;
@@ -113,6 +117,7 @@ struct insc_net {
   int64_t points_cap = 0, n_points = 0, n_points_frame = 0;
   uint8_t *mask_arena = nullptr;
   size_t mask_arena_bytes = 0;
+  std::vector<size_t> arena_level_off;  // [n_levels + 1] where the sets of a scale start in the arena
   int32_t *h_counts = nullptr;  // pinned: per level count, error flags
   int out_tensor = -1;
   bool profiling = false;
@@ -241,10 +246,10 @@ __global__ __launch_bounds__(256) void count_mask_kernel(const uint8_t *__restri
   if (threadIdx.x == 0 && part[0]) atomicAdd(out, (unsigned long long)part[0]);
 }
 
-__global__ void fill_bytes_kernel(uint4 *p, size_t n16) {
+__global__ void fill_bytes_kernel(uint4 *p, size_t n16, unsigned v) {
   size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   size_t stride = (size_t)gridDim.x * blockDim.x;
-  for (; i < n16; i += stride) p[i] = make_uint4(0, 0, 0, 0);
+  for (; i < n16; i += stride) p[i] = make_uint4(v, v, v, v);
 }
 
 __global__ void gather_out_kernel(const float *__restrict__ in, int64_t ld_in, const int32_t *__restrict__ sop,
@@ -379,15 +384,22 @@ static int level_reserve(insc_net *net, int l, int64_t cap, hipStream_t s) {
     INSC_HIP(hipMalloc((void **)&net->mask_arena, bytes));
     net->mask_arena_bytes = bytes;
   }
+  // scale by scale, so that the sets of the scales from some scale on are one range of the arena
   size_t off = 0;
-  for (DirtyNode &d : net->dirty) {
-    const size_t c = (size_t)net->levels[d.level].cap;
-    const size_t mb = (c + 255) / 256 * 256, tb = (c / 32 + 1 + 255) / 256 * 256;
-    d.mask = net->mask_arena + off;
-    d.tflag = d.mask + mb;
-    d.tflag_bo = d.tflag + tb;
-    off += mb + 3 * tb;
+  net->arena_level_off.assign((size_t)net->n_levels + 1, 0);
+  for (int lv = 0; lv < net->n_levels; lv++) {
+    net->arena_level_off[(size_t)lv] = off;
+    for (DirtyNode &d : net->dirty) {
+      if (d.level != lv) continue;
+      const size_t c = (size_t)net->levels[d.level].cap;
+      const size_t mb = (c + 255) / 256 * 256, tb = (c / 32 + 1 + 255) / 256 * 256;
+      d.mask = net->mask_arena + off;
+      d.tflag = d.mask + mb;
+      d.tflag_bo = d.tflag + tb;
+      off += mb + 3 * tb;
+    }
   }
+  net->arena_level_off[(size_t)net->n_levels] = off;
   return INSC_OK;
 }
 
@@ -908,7 +920,7 @@ int insc_net_forward(insc_net *net, const int32_t *d_coords, int coord_cols, con
 
   if (inc && net->mask_arena_bytes) {
     hipLaunchKernelGGL(fill_bytes_kernel, dim3(1024), dim3(256), 0, s, (uint4 *)net->mask_arena,
-                       net->mask_arena_bytes / 16);
+                       net->mask_arena_bytes / 16, 0u);
     INSC_LAUNCH_CHECK();
   }
 
@@ -996,9 +1008,23 @@ int insc_net_forward(insc_net *net, const int32_t *d_coords, int coord_cols, con
   }
   // ---- dirty sets, then the layers ---------------------------------------------------------
   if (net->profiling) INSC_HIP(hipEventRecord(net->ev[1], s));
-  if (inc)
+  if (inc) {
+    // A scale of at most DIRTY_FULL_SITES sites is recomputed whole (every set of it and of the
+    // coarser scales is "all rows": one fill instead of one launch per set); recomputing a clean row
+    // reproduces its bits.
+    int l_full = L;
+    for (int l = L - 1; l >= 0 && net->levels[l].n <= DIRTY_FULL_SITES; l--) l_full = l;
+    if (l_full < L && !net->arena_level_off.empty()) {
+      const size_t b0 = net->arena_level_off[(size_t)l_full], b1 = net->arena_level_off[(size_t)L];
+      if (b1 > b0) {
+        hipLaunchKernelGGL(fill_bytes_kernel, dim3(64), dim3(256), 0, s, (uint4 *)(net->mask_arena + b0), (b1 - b0) / 16,
+                           0x01010101u);
+        INSC_LAUNCH_CHECK();
+      }
+    }
     for (int i = 0; i < (int)net->dirty.size(); i++)
-      if ((rc = run_dirty_node(net, i, s))) return rc;
+      if (net->dirty[i].level < l_full && (rc = run_dirty_node(net, i, s))) return rc;
+  }
   if (net->profiling) INSC_HIP(hipEventRecord(net->ev[2], s));
   for (const Op &op : net->ops)
     if ((rc = run_op(net, op, inc, s))) return rc;
