@@ -130,6 +130,36 @@ def test_persistent_kernels_give_the_bits_of_the_per_tile_kernel(S, orc, Cin, Co
     np.testing.assert_allclose(a.cpu().numpy(), ref, rtol=RTOL, atol=ATOL)
 
 
+@pytest.mark.parametrize("n", [1, 20, 33, 130, 1025])
+def test_persistent_kernels_on_tiny_and_ragged_scenes(S, n):
+    """One site, one tile, two tiles, a group of four tiles with a partial fifth, a partial last tile:
+    all three kernels of a 64->64 layer give the same bits."""
+    from sparseconvnet._lib import lib
+
+    rng = np.random.default_rng(n)
+    side = max(2, int(round((3 * n) ** (1 / 3))))  # a third of the cube's voxels
+    vox = np.unique(rng.integers(0, side, (8 * n + 8, 3)), axis=0)
+    pts = (vox[rng.permutation(len(vox))[:n]] + 100).astype(np.int64)
+    assert len(pts) == n
+    m, x, feats = setup_sites(S, pts, 64, seed=n)
+    sc = m.ssc_rulebook(SZ)
+    W = cu((rng.normal(size=(27, 64, 64)) * 0.05).astype(np.float32))
+    outs = []
+    try:
+        for pers, shared in [(1 << 40, 1 << 40), (1, 1 << 40), (1 << 40, 1)]:
+            lib.insc_conv_set_persistent_min_units(pers)
+            lib.insc_conv_set_shared_weights_min_units(shared)
+            o = torch.full((sc.n, 64), float(len(outs)), device="cuda")
+            S.ssc_rows_planned(feats, o, W, None, sc, m.ssc_plan(sc))
+            outs.append(o)
+    finally:
+        lib.insc_conv_set_persistent_min_units(512)
+        lib.insc_conv_set_shared_weights_min_units(896)
+    assert torch.equal(outs[0], outs[1])
+    assert torch.equal(outs[0], outs[2])
+    assert torch.isfinite(outs[0]).all() and outs[0].abs().max().item() > 0
+
+
 def test_submanifold_convolution_cfg1_vs_dense_conv3d(S):
     """Workload 1 against the library routine directly (no oracle in the loop)."""
     import torch.nn.functional as F
