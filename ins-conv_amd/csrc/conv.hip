@@ -1539,7 +1539,9 @@ int launch_conv(const float *in, int64_t ld_in, int64_t in_rows, float *out, int
     int S = 1;
     if (split) S = K == 27 ? (Cin >= 160 ? 8 : 4) : (Cin >= 96 ? 4 : 1);  // K == 8: conv and deconv
     const int NB = (S == 1 && Cin >= 96) ? 1 : NB0;
-    int G = (split && K == 27) ? (Cin >= 160 ? 4 : Cin >= 128 ? 2 : 1) : 1;
+    // (the split across blocks is for scales with few tiles; in a U-Net the width grows with the depth,
+    // and a layer that narrows to at most 96 channels sits at a fine scale with many tiles)
+    int G = (split && K == 27 && Cout > 96) ? (Cin >= 160 ? 4 : Cin >= 128 ? 2 : 1) : 1;
     if (lat) {
       G = Cin >= 128 ? 4 : Cin >= 64 ? 2 : 1;
       S = 4;
