@@ -46,6 +46,19 @@ def test_error_reporting_without_gpu():
     assert b"insc_scan_exclusive_i32" in lib.insc_last_error()
     assert lib.insc_conv_packed_floats(27, 32, 32) == 27 * 1024
     assert lib.insc_conv_packed_floats(27, 48, 224) == 27 * 2 * 8 * 1024
+    # the thresholds between the kernels of wide 3^3 layers: host state only
+    import ctypes
+
+    for name in ("insc_conv_set_persistent_min_units", "insc_conv_set_shared_weights_min_units"):
+        fn = getattr(lib, name)
+        fn.argtypes, fn.restype = [ctypes.c_int64], ctypes.c_int
+        assert fn(0) == -1 and name.encode() in lib.insc_last_error()
+        assert fn(512 if "persistent" in name else 896) == 0
+    # a plan whose leading dimension does not cover the rows is refused before any launch
+    lib.insc_plan_build.restype = ctypes.c_int
+    lib.insc_plan_build.argtypes = [ctypes.c_void_p] * 3 + [ctypes.c_int64] * 2 + [ctypes.c_void_p] * 4
+    assert lib.insc_plan_build(None, None, None, 100, 96, None, None, None, None) == -1
+    assert b"plan_ld" in lib.insc_last_error()
 
 
 def test_module_api_surface():
