@@ -1528,7 +1528,7 @@ int launch_conv(const float *in, int64_t ld_in, int64_t in_rows, float *out, int
     //    reused across them);
     //  wider layers sit at the coarse scales of a U-Net, which have few tiles: one output block
     //    per wavefront, and for 3^3 / 2^3 maps the items of a tile are dealt to S wavefronts
-    //    (S grows with Cin: 2, 4, 8 for 3^3).
+    //    (four for 3^3) in each of G blocks.
     // latency != 0 (residual frames: a few thousand rows at most, so a launch lasts as long as
     // its most expensive tile): the items of every 3^3 tile are dealt to four wavefronts whatever
     // the width, and to more blocks for the wide layers.  Also a function of the layer shape only.
