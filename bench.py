@@ -150,7 +150,7 @@ def wide_conv_row(device, C=64, reps=20, warm=60):
     t = e0.elapsed_time(e1) * 1e-3 / reps
     flops = 2.0 * info["rules"] * C * C
     bytes_alg = info["rules"] * (4 * C + 8) + sc.n * 4 * C + 27 * C * C * 4
-    return {"kernel": "conv_wshare_kernel<1, 4> (SSC 3^3, %d->%d, persistent blocks of four tiles sharing weight tiles through LDS; 500k sites)" % (C, C),
+    return {"kernel": "conv_wshare_kernel<2, 4> (SSC 3^3, %d->%d, persistent blocks of four tiles sharing weight tiles through LDS, two output blocks per gathered chunk; 500k sites)" % (C, C),
             "bound": "mfma", "avg_us": round(t * 1e6, 1), "achieved": round(flops / t / 1e12, 2),
             "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(flops / t / 1e12 / MFMA_FP32_PEAK_TFLOPS, 4),
             "GB/s_on_algorithmic_bytes": round(bytes_alg / t / 1e9, 1)}

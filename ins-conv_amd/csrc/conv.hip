@@ -1085,7 +1085,7 @@ __global__ __launch_bounds__(S * 64) __attribute__((amdgpu_waves_per_eu(3, 3))) 
 // ---------------------------------------------------------------------------------------
 #define INSC_LDS_PTR(x) ((__attribute__((address_space(3))) void *)(x))
 template <int NB, int ST>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) void conv_wshare_kernel(
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NB * ST > 4 ? 2 : 3, NB * ST > 4 ? 2 : 3))) void conv_wshare_kernel(
     const float *__restrict__ in, int64_t ld_in, float *__restrict__ out, int64_t ld_out,
     const float *__restrict__ Wp, const float *__restrict__ bias, const int32_t *__restrict__ rows,
     const int32_t *__restrict__ d_n_rows, int64_t n_rows, int Cin, int Cout, int nbt, int nbtp,
@@ -1551,6 +1551,21 @@ int launch_conv(const float *in, int64_t ld_in, int64_t in_rows, float *out, int
                               small_ids && ep.ldr * 4 < (1 << 24) && out_rows * ep.ldr * 4 < (int64_t)BUF_OOB;
     if (wide_planned && cdiv(tiles, 4) * nbt >= g_shared_min_units.load(std::memory_order_relaxed)) {
       // blocks of four tiles that share the weight tiles through LDS
+      // with enough units left, two output blocks per gathered chunk (eight accumulators: two
+      // wavefronts per SIMD instead of three, but a third fewer bytes per MFMA)
+      if (nbt >= 2 && cdiv(tiles, 4) * cdiv(nbt, 2) * 3 >= g_shared_min_units.load(std::memory_order_relaxed) * 2) {
+        static int per_cu4 = 0;
+        if (!per_cu4) {
+          INSC_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu4, conv_wshare_kernel<2, 4>, 256, 0));
+          if (per_cu4 < 1) per_cu4 = 1;
+        }
+        const int64_t wunits = cdiv(tiles, 4) * cdiv(nbt, 2);
+        const unsigned nblk = (unsigned)std::min<int64_t>((int64_t)device_cus() * per_cu4, wunits);
+        hipLaunchKernelGGL((conv_wshare_kernel<2, 4>), dim3(nblk), dim3(256), 0, s, in, ld_in, out, ld_out, Wp, bias, rows,
+                           d_n_rows, n_rows, Cin, Cout, nbt, nbtp, tile_flags, in_bytes, wp_bytes, ep, plan);
+        INSC_LAUNCH_CHECK();
+        return INSC_OK;
+      }
       static int per_cu2 = 0;
       if (!per_cu2) {
         INSC_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu2, conv_wshare_kernel<1, 4>, 256, 0));

@@ -104,7 +104,14 @@ def test_persistent_kernels_give_the_bits_of_the_per_tile_kernel(S, orc, Cin, Co
         S.ssc_rows_planned(feats, a, W, bt, sc, m.ssc_plan(sc))
         lib.insc_conv_set_persistent_min_units(1 << 40)
         S.ssc_rows_planned(feats, c, W, bt, sc, m.ssc_plan(sc))
-        lib.insc_conv_set_shared_weights_min_units(1)
+        lib.insc_conv_set_shared_weights_min_units(1)  # two output blocks per gathered chunk where there are two
+        S.ssc_rows_planned(feats, d, W, bt, sc, m.ssc_plan(sc))
+        assert torch.equal(d, c)
+        # one output block per unit: enough units for that, too few for pairs of output blocks (with
+        # three output blocks the pairs always qualify as well)
+        groups, nbt = ((sc.n + 31) // 32 + 3) // 4, (Cout + 31) // 32
+        lib.insc_conv_set_shared_weights_min_units(groups * nbt)
+        d.fill_(9.0)
         S.ssc_rows_planned(feats, d, W, bt, sc, m.ssc_plan(sc))
     finally:
         lib.insc_conv_set_persistent_min_units(512)
