@@ -80,6 +80,19 @@ struct TilePlan {
 };
 int build_tile_plan(const int32_t *nbr, const int32_t *order, const int32_t *d_n, int64_t n_rows, int64_t ld,
                     int32_t *map, uint32_t *tmask, int32_t *sched, hipStream_t s);
+// the same for up to 16 maps in two launches (a map with n_rows == 0 is skipped)
+struct TilePlanJob {
+  const int32_t *nbr, *order, *d_n;
+  int64_t n_rows, ld;
+  int32_t *map;
+  uint32_t *tmask;
+  int32_t *sched;
+};
+struct TilePlanBatch {
+  TilePlanJob job[16];
+  int n;
+};
+int build_tile_plans(const TilePlanBatch &b, hipStream_t s);
 
 // in_rows: rows of the input matrix (bounds the gather).  out may be null when ep.out2 is set.
 // latency != 0 picks the launch shape for small row counts (residual frames).

@@ -1361,10 +1361,9 @@ __global__ void count_rules_kernel(const int32_t *__restrict__ map0, int K, cons
 // map[k * ld + p] = nbr[order[p]][k] for p < n, -1 up to the end of the last tile; tmask[t] = OR of
 // the offsets the rows of tile t have.  One thread per position; the writes of one offset are
 // coalesced across the wavefront.
-__global__ __launch_bounds__(256) void tile_plan_kernel(const int32_t *__restrict__ nbr,
-                                                        const int32_t *__restrict__ order,
-                                                        const int32_t *__restrict__ d_n, int64_t n_rows, int64_t ld,
-                                                        int32_t *__restrict__ map, uint32_t *__restrict__ tmask) {
+__device__ __forceinline__ void tile_plan_body(const int32_t *__restrict__ nbr, const int32_t *__restrict__ order,
+                                               const int32_t *__restrict__ d_n, int64_t n_rows, int64_t ld,
+                                               int32_t *__restrict__ map, uint32_t *__restrict__ tmask) {
   const int64_t n = d_n ? min((int64_t)*d_n, n_rows) : n_rows;
   const int64_t padded = (n + TILE_M - 1) / TILE_M * TILE_M;
   const int64_t p = (int64_t)blockIdx.x * 256 + threadIdx.x;
@@ -1381,12 +1380,23 @@ __global__ __launch_bounds__(256) void tile_plan_kernel(const int32_t *__restric
   for (int d = 16; d > 0; d >>= 1) m |= (unsigned)__shfl_xor((int)m, d, 64);
   if ((threadIdx.x & 31) == 0) tmask[p >> 5] = m;
 }
+__global__ __launch_bounds__(256) void tile_plan_kernel(const int32_t *__restrict__ nbr,
+                                                        const int32_t *__restrict__ order,
+                                                        const int32_t *__restrict__ d_n, int64_t n_rows, int64_t ld,
+                                                        int32_t *__restrict__ map, uint32_t *__restrict__ tmask) {
+  tile_plan_body(nbr, order, d_n, n_rows, ld, map, tmask);
+}
+// the plans of several maps (the scales of a network) in one launch: blockIdx.y picks the map
+__global__ __launch_bounds__(256) void tile_plan_batch_kernel(TilePlanBatch b) {
+  const TilePlanJob &j = b.job[blockIdx.y];
+  tile_plan_body(j.nbr, j.order, j.d_n, j.n_rows, j.ld, j.map, j.tmask);
+}
 
 // sched = the tiles by falling number of active offsets (a counting sort over the 28 classes by one
 // workgroup; the order inside a class is the order of arrival and has no influence on any result).
-__global__ __launch_bounds__(1024) void tile_sched_kernel(const uint32_t *__restrict__ tmask,
-                                                          const int32_t *__restrict__ d_n, int64_t n_rows,
-                                                          int32_t *__restrict__ sched, int32_t *__restrict__ gsched) {
+__device__ __forceinline__ void tile_sched_body(const uint32_t *__restrict__ tmask, const int32_t *__restrict__ d_n,
+                                                int64_t n_rows, int32_t *__restrict__ sched,
+                                                int32_t *__restrict__ gsched) {
   __shared__ int cnt[28], base[28];
   const int64_t n = d_n ? min((int64_t)*d_n, n_rows) : n_rows;
   const int64_t ntiles = (n + TILE_M - 1) / TILE_M;
@@ -1433,6 +1443,29 @@ __global__ __launch_bounds__(1024) void tile_sched_kernel(const uint32_t *__rest
     const int c = 27 - __builtin_popcount(gmask(g));
     gsched[base[c] + atomicAdd(&cnt[c], 1)] = (int32_t)g;
   }
+}
+__global__ __launch_bounds__(1024) void tile_sched_kernel(const uint32_t *__restrict__ tmask,
+                                                          const int32_t *__restrict__ d_n, int64_t n_rows,
+                                                          int32_t *__restrict__ sched, int32_t *__restrict__ gsched) {
+  tile_sched_body(tmask, d_n, n_rows, sched, gsched);
+}
+__global__ __launch_bounds__(1024) void tile_sched_batch_kernel(TilePlanBatch b) {
+  const TilePlanJob &j = b.job[blockIdx.x];
+  if (j.sched) tile_sched_body(j.tmask, j.d_n, j.n_rows, j.sched, j.sched + (j.ld + 31) / 32);
+}
+
+int build_tile_plans(const TilePlanBatch &b, hipStream_t s) {
+  int64_t most = 0;
+  bool any_sched = false;
+  for (int i = 0; i < b.n; i++) {
+    most = std::max(most, cdiv(b.job[i].n_rows, TILE_M) * TILE_M);
+    any_sched = any_sched || b.job[i].sched;
+  }
+  if (b.n <= 0 || most <= 0) return INSC_OK;
+  hipLaunchKernelGGL(tile_plan_batch_kernel, dim3(grid_for(most, 256), (unsigned)b.n), dim3(256), 0, s, b);
+  if (any_sched) hipLaunchKernelGGL(tile_sched_batch_kernel, dim3((unsigned)b.n), dim3(1024), 0, s, b);
+  INSC_LAUNCH_CHECK();
+  return INSC_OK;
 }
 
 int build_tile_plan(const int32_t *nbr, const int32_t *order, const int32_t *d_n, int64_t n_rows, int64_t ld,

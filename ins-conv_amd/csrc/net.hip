@@ -993,9 +993,15 @@ int insc_net_forward(insc_net *net, const int32_t *d_coords, int coord_cols, con
   }
 
   // tile plans of the 3^3 maps, shared by all the layers of a scale
-  for (int l = 0; l < L; l++) {
-    Level &Lv = net->levels[l];
-    if (Lv.n > 0 && (rc = build_tile_plan(Lv.nbr, Lv.order, Lv.grid->d_n, Lv.n, Lv.cap, Lv.plan, Lv.tmask, Lv.sched, s))) return rc;
+  {
+    TilePlanBatch batch;
+    batch.n = 0;
+    for (int l = 0; l < L; l++) {
+      Level &Lv = net->levels[l];
+      if (Lv.n <= 0) continue;
+      batch.job[batch.n++] = TilePlanJob{Lv.nbr, Lv.order, Lv.grid->d_n, Lv.n, Lv.cap, Lv.plan, Lv.tmask, Lv.sched};
+    }
+    if ((rc = build_tile_plans(batch, s))) return rc;
   }
 
   // ---- input layer output ------------------------------------------------------------------
