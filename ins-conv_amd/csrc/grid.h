@@ -53,6 +53,16 @@ int order_append_new_sites_sorted(const insc_grid *g, const int32_t *d_nbr, int3
                                   int64_t n_new_upper, hipStream_t s);
 int order_append_new_sites_by_offset(const insc_grid *g, const int32_t *d_offset, const int32_t *d_pos_in_order,
                                      int32_t *d_order, int32_t *d_pos, int64_t n_new_upper, hipStream_t s);
+// the three per-grid steps above for several grids (the scales of a network, at most 16) in one
+// launch each; every grid acts on the sites of its own most recent insert
+int ssc3_new_sites_batch(const insc_grid *const *grids, int32_t *const *d_nbr, int n, int64_t n_new_upper,
+                         hipStream_t s);
+int order_append_new_sites_sorted_batch(const insc_grid *const *grids, const int32_t *const *d_nbr,
+                                        int32_t *const *d_order, int32_t *const *d_pos, int n, int64_t n_new_upper,
+                                        hipStream_t s);
+int order_append_new_sites_by_offset_batch(const insc_grid *const *grids, const int32_t *const *d_offset,
+                                           const int32_t *const *d_pos_in_order, int32_t *const *d_order,
+                                           int32_t *const *d_pos, int n, int64_t n_new_upper, hipStream_t s);
 // most sites the two sorted appends put in order (more keep their arrival order)
 int64_t order_sorted_max();
 // device pointer to the site count before the most recent insert

@@ -281,9 +281,9 @@ __global__ void down2_child_kernel(const int32_t *__restrict__ parent, const int
 }
 
 // ---- variants over the sites added by the last insert, [d_n[1], d_n[0]) --------------------
-__global__ void ssc3_nbr_new_kernel(const Slot *__restrict__ table, int64_t mask,
-                                    const int32_t *__restrict__ site_coords, const int32_t *__restrict__ d_n,
-                                    int32_t *__restrict__ nbr) {
+__device__ __forceinline__ void ssc3_nbr_new_body(const Slot *__restrict__ table, int64_t mask,
+                                                  const int32_t *__restrict__ site_coords,
+                                                  const int32_t *__restrict__ d_n, int32_t *__restrict__ nbr) {
   const int64_t first = d_n[1], n = (int64_t)d_n[0] - first;
   int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (t >= n * 27) return;
@@ -298,6 +298,25 @@ __global__ void ssc3_nbr_new_kernel(const Slot *__restrict__ table, int64_t mask
     r = grid_find(table, mask, pack_key(x, y, z, c.w));
   nbr[o * 27 + k] = r;
   if (r >= 0 && r < first) nbr[(int64_t)r * 27 + (26 - k)] = (int)o;
+}
+__global__ void ssc3_nbr_new_kernel(const Slot *__restrict__ table, int64_t mask,
+                                    const int32_t *__restrict__ site_coords, const int32_t *__restrict__ d_n,
+                                    int32_t *__restrict__ nbr) {
+  ssc3_nbr_new_body(table, mask, site_coords, d_n, nbr);
+}
+// the same for several grids (the scales of a network) in one launch: blockIdx.y picks the grid
+struct NewSitesJob {
+  const Slot *table;
+  int64_t mask;
+  const int32_t *coords, *d_n;
+  int32_t *nbr;
+};
+struct NewSitesBatch {
+  NewSitesJob job[16];
+};
+__global__ void ssc3_nbr_new_batch_kernel(NewSitesBatch b) {
+  const NewSitesJob &j = b.job[blockIdx.y];
+  ssc3_nbr_new_body(j.table, j.mask, j.coords, j.d_n, j.nbr);
 }
 
 __global__ void down2_coords_new_kernel(const int32_t *__restrict__ fine_coords, const int32_t *__restrict__ d_n,
@@ -463,13 +482,12 @@ __device__ __forceinline__ uint64_t spread3_10(uint64_t v) {  // 10 bits -> ever
   return v;
 }
 template <int MODE>
-__global__ __launch_bounds__(1024) void order_append_sorted_kernel(const int32_t *__restrict__ d_n,
-                                                                   const int32_t *__restrict__ coords,
-                                                                   const int32_t *__restrict__ nbr,
-                                                                   const int32_t *__restrict__ offset,
-                                                                   const int32_t *__restrict__ aux,
-                                                                   int32_t *__restrict__ order,
-                                                                   int32_t *__restrict__ pos) {
+__device__ __forceinline__ void order_append_sorted_body(const int32_t *__restrict__ d_n,
+                                                         const int32_t *__restrict__ coords,
+                                                         const int32_t *__restrict__ nbr,
+                                                         const int32_t *__restrict__ offset,
+                                                         const int32_t *__restrict__ aux, int32_t *__restrict__ order,
+                                                         int32_t *__restrict__ pos) {
   // one 64-bit word per new site: sort key in the upper 51 bits, index of the site among the
   // new ones in the lower 13
   __shared__ uint64_t key[SORT_NEW_MAX];
@@ -524,6 +542,29 @@ __global__ __launch_bounds__(1024) void order_append_sorted_kernel(const int32_t
     if (pos) pos[v] = first + i;
   }
 }
+template <int MODE>
+__global__ __launch_bounds__(1024) void order_append_sorted_kernel(const int32_t *__restrict__ d_n,
+                                                                   const int32_t *__restrict__ coords,
+                                                                   const int32_t *__restrict__ nbr,
+                                                                   const int32_t *__restrict__ offset,
+                                                                   const int32_t *__restrict__ aux,
+                                                                   int32_t *__restrict__ order,
+                                                                   int32_t *__restrict__ pos) {
+  order_append_sorted_body<MODE>(d_n, coords, nbr, offset, aux, order, pos);
+}
+// one workgroup per grid
+struct OrderJob {
+  const int32_t *d_n, *coords, *nbr, *offset, *aux;
+  int32_t *order, *pos;
+};
+struct OrderBatch {
+  OrderJob job[16];
+};
+template <int MODE>
+__global__ __launch_bounds__(1024) void order_append_sorted_batch_kernel(OrderBatch b) {
+  const OrderJob &j = b.job[blockIdx.x];
+  order_append_sorted_body<MODE>(j.d_n, j.coords, j.nbr, j.offset, j.aux, j.order, j.pos);
+}
 
 int order_append_new_sites(const insc_grid *g, int32_t *d_order, int32_t *d_pos, int64_t n_new_upper, hipStream_t s) {
   if (n_new_upper <= 0) return INSC_OK;
@@ -533,6 +574,51 @@ int order_append_new_sites(const insc_grid *g, int32_t *d_order, int32_t *d_pos,
 }
 
 int64_t order_sorted_max() { return SORT_NEW_MAX; }
+
+int ssc3_new_sites_batch(const insc_grid *const *grids, int32_t *const *d_nbr, int n, int64_t n_new_upper,
+                         hipStream_t s) {
+  if (n <= 0 || n_new_upper <= 0) return INSC_OK;
+  if (n > 16) {
+    set_error("ssc3_new_sites_batch: at most 16 grids");
+    return INSC_ERR_ARG;
+  }
+  NewSitesBatch b;
+  for (int i = 0; i < n; i++) b.job[i] = NewSitesJob{grids[i]->table, grids[i]->n_slots - 1, grids[i]->coords, grids[i]->d_n, d_nbr[i]};
+  hipLaunchKernelGGL(ssc3_nbr_new_batch_kernel, dim3(grid_for(n_new_upper * 27, 256, 1ll << 30), (unsigned)n), dim3(256),
+                     0, s, b);
+  INSC_LAUNCH_CHECK();
+  return INSC_OK;
+}
+
+int order_append_new_sites_sorted_batch(const insc_grid *const *grids, const int32_t *const *d_nbr,
+                                        int32_t *const *d_order, int32_t *const *d_pos, int n, int64_t n_new_upper,
+                                        hipStream_t s) {
+  if (n <= 0 || n_new_upper <= 0) return INSC_OK;
+  if (n > 16) {
+    set_error("order_append_new_sites_sorted_batch: at most 16 grids");
+    return INSC_ERR_ARG;
+  }
+  OrderBatch b;
+  for (int i = 0; i < n; i++) b.job[i] = OrderJob{grids[i]->d_n, grids[i]->coords, d_nbr[i], nullptr, nullptr, d_order[i], d_pos[i]};
+  hipLaunchKernelGGL(order_append_sorted_batch_kernel<0>, dim3((unsigned)n), dim3(1024), 0, s, b);
+  INSC_LAUNCH_CHECK();
+  return INSC_OK;
+}
+
+int order_append_new_sites_by_offset_batch(const insc_grid *const *grids, const int32_t *const *d_offset,
+                                           const int32_t *const *d_pos_in_order, int32_t *const *d_order,
+                                           int32_t *const *d_pos, int n, int64_t n_new_upper, hipStream_t s) {
+  if (n <= 0 || n_new_upper <= 0) return INSC_OK;
+  if (n > 16) {
+    set_error("order_append_new_sites_by_offset_batch: at most 16 grids");
+    return INSC_ERR_ARG;
+  }
+  OrderBatch b;
+  for (int i = 0; i < n; i++) b.job[i] = OrderJob{grids[i]->d_n, nullptr, nullptr, d_offset[i], d_pos_in_order[i], d_order[i], d_pos[i]};
+  hipLaunchKernelGGL(order_append_sorted_batch_kernel<1>, dim3((unsigned)n), dim3(1024), 0, s, b);
+  INSC_LAUNCH_CHECK();
+  return INSC_OK;
+}
 
 int order_append_new_sites_sorted(const insc_grid *g, const int32_t *d_nbr, int32_t *d_order, int32_t *d_pos,
                                   int64_t n_new_upper, hipStream_t s) {

@@ -935,10 +935,39 @@ int insc_net_forward(insc_net *net, const int32_t *d_coords, int coord_cols, con
     INSC_LAUNCH_CHECK();
     Level &L0 = net->levels[0];
     if ((rc = grid_insert_nosync(L0.grid, c4, P, sop, s))) return rc;
-    if ((rc = ssc3_new_sites(L0.grid, L0.nbr, P, s))) return rc;
-    if ((rc = inc ? order_append_new_sites_sorted(L0.grid, L0.nbr, L0.order, L0.pos, P, s)
-                  : order_append_new_sites(L0.grid, L0.order, L0.pos, P, s)))
-      return rc;
+    // ---- coarser scales: the new sites of a scale are the parents of the new sites below ---
+    for (int l = 0; l + 1 < L; l++) {
+      Level &F = net->levels[l], &Cs = net->levels[l + 1];
+      if ((rc = down2_new_sites(F.grid, Cs.grid, P, F.parent, F.offset, F.child, s))) return rc;
+    }
+    // ---- neighbour maps and processing orders of the new sites, all scales per launch ------
+    const insc_grid *grids[16];
+    int32_t *nbrs[16], *orders[16], *poss[16], *bo_orders[16], *bo_poss[16];
+    const int32_t *cnbrs[16], *offsets[16], *cposs[16];
+    for (int l = 0; l < L; l++) {
+      Level &Lv = net->levels[l];
+      grids[l] = Lv.grid;
+      nbrs[l] = Lv.nbr;
+      cnbrs[l] = Lv.nbr;
+      orders[l] = Lv.order;
+      poss[l] = Lv.pos;
+      cposs[l] = Lv.pos;
+      offsets[l] = Lv.offset;
+      bo_orders[l] = Lv.bo_order;
+      bo_poss[l] = Lv.bo_pos;
+    }
+    if ((rc = ssc3_new_sites_batch(grids, nbrs, L, P, s))) return rc;
+    if (inc) {
+      if ((rc = order_append_new_sites_sorted_batch(grids, cnbrs, orders, poss, L, P, s))) return rc;
+      if ((rc = order_append_new_sites_by_offset_batch(grids, offsets, cposs, bo_orders, bo_poss, L - 1, P, s))) return rc;
+    } else {
+      for (int l = 0; l < L; l++) {
+        Level &Lv = net->levels[l];
+        if ((rc = order_append_new_sites(Lv.grid, Lv.order, Lv.pos, P, s))) return rc;
+        if (l + 1 < L && (rc = order_append_new_sites(Lv.grid, Lv.bo_order, Lv.bo_pos, P, s))) return rc;
+      }
+    }
+    // ---- input scale: accumulate the points' features per site ----------------------------
     DirtyNode &din = net->dirty[net->tensors[0].dirty];
     const unsigned nb = grid_for(P, 256);
     hipLaunchKernelGGL(chain_push_kernel, dim3(nb), dim3(256), 0, s, sop, P, net->chain_head, net->chain_next);
@@ -946,18 +975,6 @@ int insc_net_forward(insc_net *net, const int32_t *d_coords, int coord_cols, con
                        net->chain_next, net->in_sum, net->in_cnt, inc ? din.mask : nullptr,
                        inc ? din.tflag : nullptr, L0.pos);
     INSC_LAUNCH_CHECK();
-    // ---- coarser scales --------------------------------------------------------------------
-    for (int l = 0; l + 1 < L; l++) {
-      Level &F = net->levels[l], &Cs = net->levels[l + 1];
-      if ((rc = down2_new_sites(F.grid, Cs.grid, P, F.parent, F.offset, F.child, s))) return rc;
-      if ((rc = inc ? order_append_new_sites_by_offset(F.grid, F.offset, F.pos, F.bo_order, F.bo_pos, P, s)
-                    : order_append_new_sites(F.grid, F.bo_order, F.bo_pos, P, s)))
-        return rc;
-      if ((rc = ssc3_new_sites(Cs.grid, Cs.nbr, P, s))) return rc;
-      if ((rc = inc ? order_append_new_sites_sorted(Cs.grid, Cs.nbr, Cs.order, Cs.pos, P, s)
-                    : order_append_new_sites(Cs.grid, Cs.order, Cs.pos, P, s)))
-        return rc;
-    }
   }
   if (!inc) {
     // A full frame may synchronise: learn the exact counts, then build the processing orders
