@@ -118,6 +118,7 @@ struct insc_net {
   uint8_t *mask_arena = nullptr;
   size_t mask_arena_bytes = 0;
   std::vector<size_t> arena_level_off;  // [n_levels + 1] where the sets of a scale start in the arena
+  std::vector<uint8_t> dirty_full;      // per set, last incremental frame: known to hold every row (no mask kept)
   int32_t *h_counts = nullptr;  // pinned: per level count, error flags
   int out_tensor = -1;
   bool profiling = false;
@@ -444,7 +445,8 @@ static int run_op(insc_net *net, const Op &op, bool incremental, hipStream_t s) 
   if (op.fused) return INSC_OK;
   const Tensor &To = net->tensors[op.out];
   const Level &Lo = net->levels[To.level];
-  const DirtyNode *d = incremental ? &net->dirty[To.dirty] : nullptr;
+  // (a set known to hold every row needs no flags: the layer runs as in a full frame)
+  const DirtyNode *d = incremental && !net->dirty_full[(size_t)To.dirty] ? &net->dirty[To.dirty] : nullptr;
   const int32_t *d_n = Lo.grid->d_n;
   const int64_t n_up = Lo.n_upper;
   // a convolution that also forms the sum of its residual block writes what the OP_ADD would
@@ -1032,21 +1034,23 @@ int insc_net_forward(insc_net *net, const int32_t *d_coords, int coord_cols, con
   // ---- dirty sets, then the layers ---------------------------------------------------------
   if (net->profiling) INSC_HIP(hipEventRecord(net->ev[1], s));
   if (inc) {
-    // A scale of at most DIRTY_FULL_SITES sites is recomputed whole (every set of it and of the
-    // coarser scales is "all rows": one fill instead of one launch per set); recomputing a clean row
-    // reproduces its bits.
+    // A scale of at most DIRTY_FULL_SITES sites is recomputed whole: every set of it and of the
+    // coarser scales is "all rows" (recomputing a clean row reproduces its bits).  Being all rows
+    // is inherited along the program - the children of all coarse sites are all fine sites, a
+    // union with everything is everything, ... - so the decoder's sets at the finer scales are
+    // known to be full as well.  Such sets cost no launch and keep no mask.
     int l_full = L;
     for (int l = L - 1; l >= 0 && net->levels[l].n <= DIRTY_FULL_SITES; l--) l_full = l;
-    if (l_full < L && !net->arena_level_off.empty()) {
-      const size_t b0 = net->arena_level_off[(size_t)l_full], b1 = net->arena_level_off[(size_t)L];
-      if (b1 > b0) {
-        hipLaunchKernelGGL(fill_bytes_kernel, dim3(64), dim3(256), 0, s, (uint4 *)(net->mask_arena + b0), (b1 - b0) / 16,
-                           0x01010101u);
-        INSC_LAUNCH_CHECK();
-      }
+    net->dirty_full.assign(net->dirty.size(), 0);
+    for (size_t i = 0; i < net->dirty.size(); i++) {  // (a set's sources come before it)
+      const DirtyNode &dn = net->dirty[i];
+      bool full = dn.level >= l_full;
+      if (dn.src0 >= 0 && net->dirty_full[(size_t)dn.src0]) full = true;
+      if (dn.src1 >= 0 && net->dirty_full[(size_t)dn.src1]) full = true;
+      net->dirty_full[i] = full ? 1 : 0;
     }
     for (int i = 0; i < (int)net->dirty.size(); i++)
-      if (net->dirty[i].level < l_full && (rc = run_dirty_node(net, i, s))) return rc;
+      if (!net->dirty_full[(size_t)i] && (rc = run_dirty_node(net, i, s))) return rc;
   }
   if (net->profiling) INSC_HIP(hipEventRecord(net->ev[2], s));
   for (const Op &op : net->ops)
@@ -1370,6 +1374,7 @@ int insc_net_dirty_counts(insc_net *net, int max_sets, int *h_n_sets, int *h_lev
     const int64_t n = net->levels[dn.level].n;
     h_level[i] = dn.level;
     h_kind[i] = dn.kind;
+    if (i < (int)net->dirty_full.size() && net->dirty_full[(size_t)i]) continue;  // every row: filled in below
     if (n > 0 && dn.mask) {
       hipLaunchKernelGGL(count_mask_kernel, dim3(grid_for(n, 256, 1024)), dim3(256), 0, s, dn.mask, n, d + i);
       INSC_LAUNCH_CHECK();
@@ -1378,7 +1383,9 @@ int insc_net_dirty_counts(insc_net *net, int max_sets, int *h_n_sets, int *h_lev
   std::vector<unsigned long long> h((size_t)ns);
   INSC_HIP(hipMemcpyAsync(h.data(), d, sizeof(unsigned long long) * (size_t)ns, hipMemcpyDeviceToHost, s));
   INSC_HIP(hipStreamSynchronize(s));
-  for (int i = 0; i < ns; i++) h_rows[i] = (int64_t)h[(size_t)i];
+  for (int i = 0; i < ns; i++)
+    h_rows[i] = (i < (int)net->dirty_full.size() && net->dirty_full[(size_t)i]) ? net->levels[net->dirty[i].level].n
+                                                                                : (int64_t)h[(size_t)i];
   return INSC_OK;
 }
 
