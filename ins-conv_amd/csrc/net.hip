@@ -117,7 +117,6 @@ struct insc_net {
   int64_t points_cap = 0, n_points = 0, n_points_frame = 0;
   uint8_t *mask_arena = nullptr;
   size_t mask_arena_bytes = 0;
-  std::vector<size_t> arena_level_off;  // [n_levels + 1] where the sets of a scale start in the arena
   std::vector<uint8_t> dirty_full;      // per set, last incremental frame: known to hold every row (no mask kept)
   int32_t *h_counts = nullptr;  // pinned: per level count, error flags
   int out_tensor = -1;
@@ -247,10 +246,10 @@ __global__ __launch_bounds__(256) void count_mask_kernel(const uint8_t *__restri
   if (threadIdx.x == 0 && part[0]) atomicAdd(out, (unsigned long long)part[0]);
 }
 
-__global__ void fill_bytes_kernel(uint4 *p, size_t n16, unsigned v) {
+__global__ void fill_bytes_kernel(uint4 *p, size_t n16) {
   size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   size_t stride = (size_t)gridDim.x * blockDim.x;
-  for (; i < n16; i += stride) p[i] = make_uint4(v, v, v, v);
+  for (; i < n16; i += stride) p[i] = make_uint4(0, 0, 0, 0);
 }
 
 __global__ void gather_out_kernel(const float *__restrict__ in, int64_t ld_in, const int32_t *__restrict__ sop,
@@ -385,22 +384,15 @@ static int level_reserve(insc_net *net, int l, int64_t cap, hipStream_t s) {
     INSC_HIP(hipMalloc((void **)&net->mask_arena, bytes));
     net->mask_arena_bytes = bytes;
   }
-  // scale by scale, so that the sets of the scales from some scale on are one range of the arena
   size_t off = 0;
-  net->arena_level_off.assign((size_t)net->n_levels + 1, 0);
-  for (int lv = 0; lv < net->n_levels; lv++) {
-    net->arena_level_off[(size_t)lv] = off;
-    for (DirtyNode &d : net->dirty) {
-      if (d.level != lv) continue;
-      const size_t c = (size_t)net->levels[d.level].cap;
-      const size_t mb = (c + 255) / 256 * 256, tb = (c / 32 + 1 + 255) / 256 * 256;
-      d.mask = net->mask_arena + off;
-      d.tflag = d.mask + mb;
-      d.tflag_bo = d.tflag + tb;
-      off += mb + 3 * tb;
-    }
+  for (DirtyNode &d : net->dirty) {
+    const size_t c = (size_t)net->levels[d.level].cap;
+    const size_t mb = (c + 255) / 256 * 256, tb = (c / 32 + 1 + 255) / 256 * 256;
+    d.mask = net->mask_arena + off;
+    d.tflag = d.mask + mb;
+    d.tflag_bo = d.tflag + tb;
+    off += mb + 3 * tb;
   }
-  net->arena_level_off[(size_t)net->n_levels] = off;
   return INSC_OK;
 }
 
@@ -922,7 +914,7 @@ int insc_net_forward(insc_net *net, const int32_t *d_coords, int coord_cols, con
 
   if (inc && net->mask_arena_bytes) {
     hipLaunchKernelGGL(fill_bytes_kernel, dim3(1024), dim3(256), 0, s, (uint4 *)net->mask_arena,
-                       net->mask_arena_bytes / 16, 0u);
+                       net->mask_arena_bytes / 16);
     INSC_LAUNCH_CHECK();
   }
 
