@@ -1261,11 +1261,19 @@ int insc_net_forward_residual(insc_net *net, const int32_t *d_coords, int coord_
   hipLaunchKernelGGL(chain_sum_kernel, dim3(nb), dim3(256), 0, s, d_feats, C0, R.sop, P, R.chain_head, R.chain_next,
                      R.in_sum, R.in_cnt, (uint8_t *)nullptr, (uint8_t *)nullptr, (const int32_t *)nullptr);
   INSC_LAUNCH_CHECK();
-  if ((rc = ssc3_new_sites(R.levels[0].grid, R.levels[0].nbr, P, s))) return rc;
   for (int l = 0; l + 1 < L; l++) {
     Level &F = R.levels[l], &Cs = R.levels[l + 1];
     if ((rc = down2_new_sites(F.grid, Cs.grid, P, F.parent, F.offset, F.child, s))) return rc;
-    if ((rc = ssc3_new_sites(Cs.grid, Cs.nbr, P, s))) return rc;
+  }
+  {
+    // the neighbour maps of all scales in one launch
+    const insc_grid *grids[16];
+    int32_t *nbrs[16];
+    for (int l = 0; l < L; l++) {
+      grids[l] = R.levels[l].grid;
+      nbrs[l] = R.levels[l].nbr;
+    }
+    if ((rc = ssc3_new_sites_batch(grids, nbrs, L, P, s))) return rc;
   }
   // the exact site counts size every later launch (one short host round trip, as in an exact frame)
   for (int l = 0; l < L; l++) {
