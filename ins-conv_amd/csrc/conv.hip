@@ -227,10 +227,9 @@ __global__ __launch_bounds__((S == 1 ? CONV_WAVES : S) * 64) void conv_mfma_kern
   const int r = lane & 31, h = lane >> 5;
   // (with a tile schedule the blocks of a split launch take the tiles by falling cost: blocks go to the
   // compute units round robin, so every unit then holds a mix of expensive and cheap tiles)
-  const bool by_cost = S > 1 && MODE == MAP_NBR && K == 27 && plan.map != nullptr && plan.sched != nullptr &&
-                       (int64_t)blockIdx.x * TILE_M < n;
-  const int64_t t0 = (S == 1 ? (int64_t)blockIdx.x * WAVES + wave
-                             : (int64_t)(by_cost ? plan.sched[blockIdx.x] : (int)blockIdx.x)) * TILE_M;
+  const int64_t slot = S == 1 ? (int64_t)blockIdx.x * WAVES + wave : (int64_t)blockIdx.x;
+  const bool by_cost = MODE == MAP_NBR && K == 27 && plan.map != nullptr && plan.sched != nullptr && slot * TILE_M < n;
+  const int64_t t0 = (by_cost ? (int64_t)plan.sched[slot] : slot) * TILE_M;
   const int cb0 = blockIdx.y * NB;  // first output-channel block of this column group
   const int nch = conv_nch(Cin);
   // the items of a tile are dealt to S wavefronts in each of G = gridDim.z blocks
