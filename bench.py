@@ -115,11 +115,11 @@ def conv_roofline(device, reps=30, warm=200):
     achieved = bytes_alg / t / 1e9
     return {
         "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-        "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": 550.7e6,
+        "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": 551.6e6,
         "kernel": "conv_wlds_kernel (SSC 3^3, 32->32, filter in LDS, persistent blocks; 500k sites, %d rules)" % n_rules,
         "avg_us": round(t * 1e6, 1), "algorithmic_bytes": int(bytes_alg),
         "traffic_note": "HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE (x1.999, copy-kernel calibration) + "
-                        "WRITE_SIZE (x1.000): 452.1 MB + 98.6 MB, profiles/conv_wlds_ssc32_500k.txt",
+                        "WRITE_SIZE (x1.000): 453.0 MB + 98.6 MB, profiles/conv_wlds_ssc32_500k.txt",
         "mfma_tflops": round(flops / t / 1e12, 2), "mfma_frac": round(flops / t / 1e12 / MFMA_FP32_PEAK_TFLOPS, 4),
         "ssc_msites_per_s": round(sc.n / t / 1e6, 1),
     }
