@@ -24,7 +24,7 @@ import sys
 import time
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
-for p in (ROOT, os.path.join(ROOT, "tests"), os.path.join(ROOT, "ins-conv_amd")):
+for p in (ROOT, os.path.join(ROOT, "ins-conv_amd")):
     if p not in sys.path:
         sys.path.insert(0, p)
 
@@ -55,7 +55,7 @@ def ssc_workload(device, channels=(32, 64)):
     import numpy as np
     import torch
 
-    import scenes
+    from workloads import scenes
     import sparseconvnet as scn
 
     vox = scenes.indoor_scene(seed=3, n=500000)
@@ -168,7 +168,7 @@ def kernel_table(device, reps=20):
     import numpy as np
     import torch
 
-    import scenes
+    from workloads import scenes
     from sparseconvnet._lib import lib, ptr, stream_ptr
 
     I64 = ctypes.c_int64
@@ -280,7 +280,7 @@ def kernel_table(device, reps=20):
 # ---------------------------------------------------------------------------------------------
 def unet_model(device):
     import sparseconvnet as scn
-    from netdefs import NaiveUNet
+    from workloads.netdefs import NaiveUNet
 
     model = NaiveUNet(m=32, levels=7, seed=4).to(device)
     return model, scn.compile(model.sparseModel, capacity_sites=1 << 18)
@@ -327,9 +327,9 @@ def cpu_baseline_unet():
     import numpy as np
     import torch
 
-    import oracle_net
-    import scenes
-    from netdefs import NaiveUNet
+    from oracle import oracle_net
+    from workloads import scenes
+    from workloads.netdefs import NaiveUNet
     from oracle import oracle as orc
 
     pts, rgb, _ = scenes.unet_scene()
@@ -349,7 +349,7 @@ def cpu_baseline_unet():
 def cpu_baseline_ssc(n_sample=100000):
     import numpy as np
 
-    import scenes
+    from workloads import scenes
     from oracle import oracle as orc
 
     vox = scenes.indoor_scene(seed=3, n=500000)[:n_sample]
@@ -409,7 +409,7 @@ def main():
         print(json.dumps({"kernels": kernel_table(device)}))
         return
     if args.residual_only:
-        import scenes
+        from workloads import scenes
 
         seq = scenes.sweep_sequence()
         model, _ = unet_model(device)
@@ -431,7 +431,7 @@ def main():
 
     extra = {}
     if args.workload == "incr":
-        import scenes
+        from workloads import scenes
 
         seq = scenes.sweep_sequence()
         W = 9 if args.warmup is None else args.warmup
@@ -475,7 +475,7 @@ def main():
             extra.update(residual_row(model, seq, frames, W + K, device))
         cpu_fn = cpu_baseline_unet
     elif args.workload == "unet":
-        import scenes
+        from workloads import scenes
 
         W = 3 if args.warmup is None else args.warmup
         K = 20 if args.steps is None else args.steps

@@ -167,6 +167,10 @@ int insc_conv_ssc_plan(const float *d_in, int64_t ld_in, int64_t n_in_rows, floa
  * test knobs with no counterpart in the reference. */
 int insc_conv_set_persistent_min_units(int64_t units);
 int insc_conv_set_shared_weights_min_units(int64_t units);
+/* A 3^3 layer with at most 32 input and 32 output channels runs, from `tiles` 32-row tiles up
+ * (default 4096, i.e. 131k sites), on persistent blocks that keep the whole filter in LDS; below,
+ * one wavefront per tile.  Same bits in both cases: a tuning and test knob like the two above. */
+int insc_conv_set_filter_lds_min_tiles(int64_t tiles);
 /* Size-2 stride-2 deconvolution: out[i,:] = bias + in[parent[i],:] . W[offset[i]]
  * (Deconvolution_updateOutput, CUDA/Deconvolution.cpp:28-58: the convolution's rules with
  * the roles of input and output swapped). */

@@ -536,7 +536,7 @@ __global__ __launch_bounds__((S == 1 ? CONV_WAVES : S) * 64) void conv_mfma_kern
 // ---------------------------------------------------------------------------------------
 constexpr int WL_WAVES = 12;
 constexpr int WL_DEPTH = 4;
-constexpr int WL_MIN_TILES = 4096;  // smaller launches go to conv_mfma_kernel
+constexpr int WL_MIN_TILES = 4096;  // smaller launches go to conv_mfma_kernel (default of the knob below)
 constexpr int WL_SCHED = 256;  // a block orders up to this many tiles of its own by cost
 
 __global__ __launch_bounds__(WL_WAVES * 64) void conv_wlds_kernel(
@@ -1507,6 +1507,10 @@ static std::atomic<int64_t> g_pers_min_units{512};
 // ... and with at least this many (group of four tiles, output block) units to the kernel whose blocks
 // share the weight tiles through LDS (faster from about 60k sites at 64 channels; same bits again).
 static std::atomic<int64_t> g_shared_min_units{896};
+// Narrow 3^3 layers (Cin, Cout <= 32) with at least this many 32-row tiles run on the persistent
+// kernel that keeps the whole filter in LDS; smaller ones on the one-wavefront-per-tile kernel.
+// Same bits either way.
+static std::atomic<int64_t> g_wl_min_tiles{WL_MIN_TILES};
 
 // W: raw [K,Cin,Cout] weights (always needed by the generic kernel); Wp: packed weights or
 // null, in which case they are packed into scratch memory first.
@@ -1549,7 +1553,7 @@ int launch_conv(const float *in, int64_t ld_in, int64_t in_rows, float *out, int
     // whole filter into LDS - costs more than it saves: 34 us against 21 us at 32k sites, even at
     // 150k; both kernels give the same bits)
     if (mode == MAP_NBR && K == 27 && Cin <= 32 && Cout <= 32 && map_bytes64 < (int64_t)BUF_OOB && small_ids &&
-        tiles >= WL_MIN_TILES && !latency) {
+        tiles >= g_wl_min_tiles.load(std::memory_order_relaxed) && !latency) {
       const uint32_t map_bytes = (uint32_t)map_bytes64;
       // persistent blocks, a multiple of the XCD count, at most one per compute unit
       const int64_t want = cdiv(tiles, WL_WAVES);
@@ -1740,6 +1744,12 @@ int insc_conv_set_persistent_min_units(int64_t units) {
 int insc_conv_set_shared_weights_min_units(int64_t units) {
   INSC_REQUIRE(units >= 1, INSC_ERR_ARG, "insc_conv_set_shared_weights_min_units: units must be >= 1");
   g_shared_min_units.store(units, std::memory_order_relaxed);
+  return INSC_OK;
+}
+
+int insc_conv_set_filter_lds_min_tiles(int64_t tiles) {
+  INSC_REQUIRE(tiles >= 1, INSC_ERR_ARG, "insc_conv_set_filter_lds_min_tiles: tiles must be >= 1");
+  g_wl_min_tiles.store(tiles, std::memory_order_relaxed);
   return INSC_OK;
 }
 

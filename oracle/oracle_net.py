@@ -6,7 +6,7 @@ reference's CPU path, on numpy arrays.  Used to check whole-network results of t
 """
 import numpy as np
 
-from oracle import oracle as orc
+from . import oracle as orc
 
 
 class OTensor(object):

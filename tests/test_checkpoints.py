@@ -6,12 +6,12 @@ import os
 import numpy as np
 import torch
 
-import scenes
+from workloads import scenes
 
 
 def test_checkpoint_round_trip(tmp_path):
     import sparseconvnet as scn
-    from netdefs import NaiveUNet
+    from workloads.netdefs import NaiveUNet
 
     a, b = NaiveUNet(m=8, levels=3, seed=1), NaiveUNet(m=8, levels=3, seed=2)
     exp = str(tmp_path / "exp")

@@ -29,7 +29,7 @@ def persistent_min_units(request):
 @pytest.mark.parametrize("levels,m", [(3, 16), (7, 32)])
 def test_compiled_full_and_incremental(levels, m, persistent_min_units):
     import sparseconvnet as scn
-    from netdefs import NaiveUNet
+    from workloads.netdefs import NaiveUNet
 
     frames = _frames(6, seed=31)
     model = NaiveUNet(m=m, levels=levels, seed=9).cuda()
@@ -65,7 +65,7 @@ def test_compiled_full_and_incremental(levels, m, persistent_min_units):
 
 def test_compiled_rejects_incremental_without_state():
     import sparseconvnet as scn
-    from netdefs import NaiveUNet
+    from workloads.netdefs import NaiveUNet
     from sparseconvnet._lib import InscError
 
     model = NaiveUNet(m=16, levels=2, seed=1).cuda()
@@ -80,7 +80,7 @@ def test_dirty_set_rows_of_a_frame():
     derived set contains its source (sets only grow along the program), none exceeds its scale,
     and at the finest scale they stay a fraction of the scene for a local increment."""
     import sparseconvnet as scn
-    from netdefs import NaiveUNet
+    from workloads.netdefs import NaiveUNet
 
     frames = _frames(3, seed=33)
     model = NaiveUNet(m=16, levels=4, seed=2).cuda()

@@ -7,7 +7,7 @@ import numpy as np
 import pytest
 import torch
 
-import scenes
+from workloads import scenes
 
 pytestmark = pytest.mark.gpu
 
@@ -26,8 +26,8 @@ def test_batch_of_scenes_equals_scenes_run_alone():
     """Two scenes with batch indices 0 and 1 (overlapping coordinates): nothing may leak across the
     batch index - each scene's logits equal those of the scene run alone, bit for bit - and the
     whole batch matches the oracle."""
-    import oracle_net
-    from netdefs import NaiveUNet
+    from oracle import oracle_net
+    from workloads.netdefs import NaiveUNet
 
     (va, fa), (vb, fb) = _scene(41), _scene(42, 4000)
     vb = vb.copy()
@@ -88,7 +88,7 @@ def test_empty_and_duplicate_only_increments():
     """An increment of zero points, one that only repeats points already seen, and one that only
     re-observes old voxels with new colours: the executor must stay equal to a full forward."""
     import sparseconvnet as scn
-    from netdefs import NaiveUNet
+    from workloads.netdefs import NaiveUNet
 
     vox, rgb = _scene(45)
     model = NaiveUNet(m=16, levels=4, seed=14).cuda()
@@ -123,7 +123,7 @@ def test_residual_frames_disjoint_from_and_inside_the_saved_scene():
     made only of saved voxels with unchanged colours has residual zero, so it returns the saved
     rows."""
     import sparseconvnet as scn
-    from netdefs import NaiveUNet
+    from workloads.netdefs import NaiveUNet
 
     vox, rgb = _scene(47)
     model = NaiveUNet(m=16, levels=4, seed=15).cuda()

@@ -9,7 +9,7 @@ import numpy as np
 import pytest
 import torch
 
-import scenes
+from workloads import scenes
 
 pytestmark = pytest.mark.gpu
 SZ = torch.LongTensor([4096, 4096, 4096])
@@ -126,7 +126,7 @@ def test_workload5_sweep_ends_equal_to_a_full_forward():
     forward over every point in arrival order: the features of all points must be equal bit for
     bit, and the phase timer must report a plausible frame."""
     import sparseconvnet as scn
-    from netdefs import NaiveUNet
+    from workloads.netdefs import NaiveUNet
 
     seq = scenes.sweep_sequence()
     model = NaiveUNet(m=32, levels=7, seed=4).cuda()

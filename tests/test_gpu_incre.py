@@ -8,7 +8,7 @@ import numpy as np
 import pytest
 import torch
 
-import scenes
+from workloads import scenes
 
 pytestmark = pytest.mark.gpu
 RTOL, ATOL = 1e-4, 1e-5
@@ -209,9 +209,9 @@ def _inp(pts, rgb):
 def test_residual_frame_network_vs_oracle(levels, m):
     """Whole network: frame 0 full, frame 1 with increment="residual", against the oracle's
     residual network; then the saved state must be what the full forward left."""
-    import oracle_net
+    from oracle import oracle_net
     import sparseconvnet as scn
-    from netdefs import NaiveUNet
+    from workloads.netdefs import NaiveUNet
 
     f0, f1, _ = _frames(31)
     model = NaiveUNet(m=m, levels=levels, seed=9).cuda()
@@ -243,7 +243,7 @@ def test_residual_frame_covering_scene_equals_full_forward():
     """A frame that observes every saved voxel again is exact (every operator is exact on the
     frame's sites): logits(residual) == logits(full forward over both frames) within float
     tolerance, at 150k-scale channel widths but a small scene."""
-    from netdefs import NaiveUNet
+    from workloads.netdefs import NaiveUNet
 
     _, _, (vox, base) = _frames(32)
     rng = np.random.default_rng(33)
@@ -263,7 +263,7 @@ def test_residual_frame_covering_scene_equals_full_forward():
 
 def test_increment_true_follows_set_mode():
     import sparseconvnet as scn
-    from netdefs import NaiveUNet
+    from workloads.netdefs import NaiveUNet
 
     f0, f1, _ = _frames(34)
     model = NaiveUNet(m=16, levels=3, seed=11).cuda()
@@ -288,7 +288,7 @@ def test_compiled_residual_frames_equal_module_tree(levels, m):
     batch norms; full and exact incremental frames must not change because of that, and a
     residual frame must leave the saved state as it was."""
     import sparseconvnet as scn
-    from netdefs import NaiveUNet
+    from workloads.netdefs import NaiveUNet
 
     f0, f1, _ = _frames(35)
     model = NaiveUNet(m=m, levels=levels, seed=12).cuda()

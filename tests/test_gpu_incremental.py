@@ -11,7 +11,7 @@ import numpy as np
 import pytest
 import torch
 
-import scenes
+from workloads import scenes
 
 pytestmark = pytest.mark.gpu
 
@@ -45,7 +45,7 @@ def _inp(pts, rgb):
 @pytest.mark.parametrize("levels,m", [(3, 16), (5, 32)])
 def test_incremental_equals_full_recompute(levels, m):
     import sparseconvnet as scn
-    from netdefs import NaiveUNet
+    from workloads.netdefs import NaiveUNet
 
     frames = _frames(5, seed=21)
     model = NaiveUNet(m=m, levels=levels, seed=7).cuda()
@@ -70,7 +70,7 @@ def test_incremental_equals_full_recompute(levels, m):
 
 
 def test_incremental_default_output_is_the_increment_rows():
-    from netdefs import NaiveUNet
+    from workloads.netdefs import NaiveUNet
 
     frames = _frames(3, seed=22)
     model = NaiveUNet(m=16, levels=3, seed=8).cuda()

@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 import torch
 
-import scenes
+from workloads import scenes
 
 pytestmark = pytest.mark.gpu
 RTOL, ATOL = 1e-4, 1e-5

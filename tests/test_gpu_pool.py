@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 import torch
 
-import scenes
+from workloads import scenes
 
 pytestmark = pytest.mark.gpu
 SZ = torch.LongTensor([128, 128, 128])

@@ -4,7 +4,7 @@ import numpy as np
 import pytest
 import torch
 
-import scenes
+from workloads import scenes
 
 pytestmark = pytest.mark.gpu
 
@@ -30,8 +30,8 @@ def _check(a, b, what):
 
 @pytest.mark.parametrize("levels,m", [(3, 16), (7, 32)])
 def test_unet_full_forward_matches_oracle(levels, m):
-    import oracle_net
-    from netdefs import NaiveUNet
+    from oracle import oracle_net
+    from workloads.netdefs import NaiveUNet
 
     pts, rgb = _scene(6000, seed=11)
     model = NaiveUNet(m=m, levels=levels, seed=4).cuda()
@@ -47,7 +47,7 @@ def test_unet_full_forward_matches_oracle(levels, m):
 
 
 def test_unet_is_deterministic():
-    from netdefs import NaiveUNet
+    from workloads.netdefs import NaiveUNet
 
     pts, rgb = _scene(5000, seed=12)
     model = NaiveUNet(m=16, levels=4, seed=5).cuda()

@@ -226,9 +226,9 @@ def test_incre_input_other_modes_by_hand(orc):
 def test_residual_net_exact_when_frame_covers_scene(orc, levels):
     """Every operator is exact on the frame's sites, so a frame that observes every saved voxel
     again (plus new ones) must reproduce a full forward over all points of both frames."""
-    import oracle_net
-    import scenes
-    from netdefs import NaiveUNet
+    from oracle import oracle_net
+    from workloads import scenes
+    from workloads.netdefs import NaiveUNet
 
     vox = scenes.boxes_scene(seed=11, n=1500, grid=48, n_boxes=3, lo_rng=(4, 24), size_rng=(8, 18))
     rng = np.random.default_rng(12)

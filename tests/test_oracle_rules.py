@@ -6,7 +6,7 @@ dropped neighbour, wrong parity bit)."""
 import numpy as np
 import pytest
 
-import scenes
+from workloads import scenes
 
 
 def small_scene(seed, n=1500, grid=24):

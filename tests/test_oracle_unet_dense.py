@@ -99,9 +99,9 @@ def _U(p, x, masks, level, planes, reps):
 
 @pytest.mark.parametrize("levels,m", [(3, 4), (4, 3)])
 def test_oracle_network_vs_dense_torch_model(levels, m):
-    import oracle_net
-    import scenes
-    from netdefs import NaiveUNet
+    from oracle import oracle_net
+    from workloads import scenes
+    from workloads.netdefs import NaiveUNet
 
     vox = scenes.boxes_scene(seed=21, n=2500, grid=G, n_boxes=3, lo_rng=(2, 12), size_rng=(8, 18))
     rng = np.random.default_rng(22)
