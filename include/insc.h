@@ -63,6 +63,9 @@ int insc_grid_clear(insc_grid *g, void *stream);
 int insc_grid_reserve(insc_grid *g, int64_t capacity_sites, void *stream);
 /* Insert P coordinates (duplicates allowed).  d_site_of_point[p] receives the site of row p.
  * h_n_sites (nullable, host) receives the site count after the insert (synchronises).
+ * A coordinate outside the representable range gets site -1 and the next synchronising call on
+ * the grid returns INSC_ERR_COORD once; every other row of the call is inserted and the grid stays
+ * usable.
  * Replaces HashInputPointClouds + InsertAndCompactPointCloud (CUDPPWrapper.hpp:668-686,
  * 766-796; kernels CUDPPWrapper.cu:72-100,212-231). */
 int insc_grid_insert(insc_grid *g, const int32_t *d_coords4, int64_t P, int32_t *d_site_of_point, int64_t *h_n_sites,
@@ -287,11 +290,21 @@ int insc_net_finalize(insc_net *net, int out_tensor, int64_t capacity_sites, voi
 int insc_net_enable_residual(insc_net *net);
 /* Re-pack the weights after the caller changed them in place. */
 int insc_net_refresh_weights(insc_net *net, void *stream);
+/* Ops added so far (joins included); the op added last has index insc_net_op_count() - 1. */
+int insc_net_op_count(const insc_net *net);
+/* Point op `op` at parameters that moved (e.g. the caller's framework re-allocated them when a
+ * checkpoint was restored): d_W / d_bias for a convolution op, d_mean / d_var / d_gamma / d_beta for
+ * a batch norm; same shapes as when the op was added.  Follow with insc_net_refresh_weights.
+ * No counterpart in the reference, whose modules pass their tensors on every call. */
+int insc_net_rebind_op(insc_net *net, int op, const float *d_W, const float *d_bias, const float *d_mean,
+                       const float *d_var, const float *d_gamma, const float *d_beta);
 /* One frame: d_coords int32 [P,coord_cols] (x,y,z[,batch]), d_feats float32 [P,in_channels].
  * increment == 0 forgets all state and runs a full forward; increment != 0 appends the points
  * and recomputes only the rows they affect.  d_out (nullable) receives one row of the output
  * tensor per point of this frame (out_all == 0) or per point since the last full frame.
- * Returns when the frame has completed. */
+ * Returns when the frame has completed.  A frame is all or nothing: if any of its coordinates is
+ * outside the representable range the call returns INSC_ERR_COORD and the state is that of the
+ * previous frame (after a full frame that failed: no state; the next frame must be a full one). */
 int insc_net_forward(insc_net *net, const int32_t *d_coords, int coord_cols, const float *d_feats, int64_t P,
                      int increment, float *d_out, int out_all, int64_t *h_n_sites, void *stream);
 /* The dirty sets of the last exact incremental frame (diagnostics; no counterpart in the

@@ -370,6 +370,12 @@ static int grid_sync_errors(insc_grid *g, hipStream_t s, const char *who) {
   INSC_HIP(hipStreamSynchronize(s));
   g->n_exact = h[0];
   g->n_upper = h[0];
+  if (h[1]) {
+    // reported once: the rows at fault got site -1, every other row of the call was handled, and
+    // the grid stays usable
+    INSC_HIP(hipMemsetAsync(g->d_err, 0, sizeof(int32_t), s));
+    INSC_HIP(hipStreamSynchronize(s));
+  }
   if (h[1] & 1) {
     set_error("%s: a coordinate is outside 0..65535 (batch 0..32767)", who);
     return INSC_ERR_COORD;

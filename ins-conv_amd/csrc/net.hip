@@ -119,6 +119,8 @@ struct insc_net {
   size_t mask_arena_bytes = 0;
   std::vector<uint8_t> dirty_full;      // per set, last incremental frame: known to hold every row (no mask kept)
   int32_t *h_counts = nullptr;  // pinned: per level count, error flags
+  int32_t *d_bad = nullptr;     // number of the last frame that held a coordinate out of range
+  int32_t frame_id = 0;         // frames are numbered from 1
   int out_tensor = -1;
   bool profiling = false;
   hipEvent_t ev[5] = {nullptr, nullptr, nullptr, nullptr, nullptr};
@@ -262,11 +264,25 @@ __global__ void gather_out_kernel(const float *__restrict__ in, int64_t ld_in, c
   }
 }
 
-__global__ void coords_to_int4_kernel(const int32_t *__restrict__ in, int cols, int64_t P, int32_t *__restrict__ out) {
+// A frame is all or nothing: the first pass raises *bad if any coordinate of the frame cannot be
+// represented, the second pass then turns EVERY point of the frame into one the insert skips, so
+// that no grid, map or running sum changes and the host can report the error after the frame's one
+// round trip.  The flag holds the number of the last frame that raised it (frames are numbered from 1),
+// so it never needs clearing.
+__global__ void coords_check_kernel(const int32_t *__restrict__ in, int cols, int64_t P, int32_t *__restrict__ bad,
+                                    int32_t frame) {
   int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (p >= P) return;
   const int32_t *c = in + p * cols;
-  reinterpret_cast<int4 *>(out)[p] = make_int4(c[0], c[1], c[2], cols > 3 ? c[3] : 0);
+  if (!coord_ok(c[0], c[1], c[2], cols > 3 ? c[3] : 0)) bad[0] = frame;
+}
+__global__ void coords_to_int4_kernel(const int32_t *__restrict__ in, int cols, int64_t P, int32_t *__restrict__ out,
+                                      const int32_t *__restrict__ bad, int32_t frame) {
+  int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (p >= P) return;
+  const int32_t *c = in + p * cols;
+  reinterpret_cast<int4 *>(out)[p] =
+      (bad && bad[0] == frame) ? make_int4(COORD_SKIP, 0, 0, 0) : make_int4(c[0], c[1], c[2], cols > 3 ? c[3] : 0);
 }
 
 // -----------------------------------------------------------------------------------------
@@ -408,6 +424,7 @@ static int points_reserve(insc_net *net, int64_t need, hipStream_t s) {
 
 static int sync_counts(insc_net *net, hipStream_t s, const char *who) {
   const int L = net->n_levels;
+  INSC_HIP(hipMemcpyAsync(net->h_counts + 2 * L, net->d_bad, sizeof(int32_t), hipMemcpyDeviceToHost, s));
   for (int l = 0; l < L; l++) {
     INSC_HIP(hipMemcpyAsync(net->h_counts + 2 * l, net->levels[l].grid->d_n, sizeof(int32_t),
                             hipMemcpyDeviceToHost, s));
@@ -419,6 +436,13 @@ static int sync_counts(insc_net *net, hipStream_t s, const char *who) {
     Level &Lv = net->levels[l];
     Lv.n = Lv.n_upper = net->h_counts[2 * l];
     Lv.grid->n_exact = Lv.grid->n_upper = Lv.n;
+  }
+  if (net->h_counts[2 * L] == net->frame_id) {
+    // (nothing of the frame was inserted: the state is that of the previous frame)
+    set_error("%s: a coordinate is outside 0..65535 (batch 0..32767); the frame was dropped", who);
+    return INSC_ERR_COORD;
+  }
+  for (int l = 0; l < L; l++) {
     const int err = net->h_counts[2 * l + 1];
     if (err & 1) {
       set_error("%s: a coordinate is outside 0..65535 (batch 0..32767)", who);
@@ -562,6 +586,8 @@ int insc_net_create(int n_levels, int in_channels, int mode, insc_net **out) {
   t.buf = 0;
   net->tensors.push_back(t);
   INSC_HIP(hipHostMalloc((void **)&net->h_counts, sizeof(int32_t) * 64, hipHostMallocDefault));
+  INSC_HIP(hipMalloc((void **)&net->d_bad, 256));
+  INSC_HIP(hipMemset(net->d_bad, 0, 256));
   *out = net;
   return INSC_OK;
 }
@@ -597,7 +623,7 @@ int insc_net_destroy(insc_net *net) {
   void *rps[] = {net->rf.in_sum, net->rf.in_cnt, net->rf.chain_head, net->rf.chain_next, net->rf.sop};
   for (void *p : rps)
     if (p) (void)hipFree(p);
-  void *ps[] = {net->in_sum, net->in_cnt, net->chain_head, net->chain_next, net->site_of_point, net->mask_arena};
+  void *ps[] = {net->in_sum, net->in_cnt, net->chain_head, net->chain_next, net->site_of_point, net->mask_arena, net->d_bad};
   for (void *p : ps)
     if (p) (void)hipFree(p);
   if (net->h_counts) (void)hipHostFree(net->h_counts);
@@ -868,6 +894,29 @@ int insc_net_refresh_weights(insc_net *net, void *stream) {
   return INSC_OK;
 }
 
+int insc_net_op_count(const insc_net *net) { return net ? (int)net->ops.size() : 0; }
+
+int insc_net_rebind_op(insc_net *net, int op, const float *d_W, const float *d_bias, const float *d_mean,
+                       const float *d_var, const float *d_gamma, const float *d_beta) {
+  INSC_REQUIRE(net && op >= 0 && op < (int)net->ops.size(), INSC_ERR_ARG, "insc_net_rebind_op: no op %d", op);
+  Op &o = net->ops[op];
+  if (o.kind == OP_SSC || o.kind == OP_CONV || o.kind == OP_DECONV || o.kind == OP_NIN) {
+    INSC_REQUIRE(d_W, INSC_ERR_ARG, "insc_net_rebind_op: op %d is a convolution and needs d_W", op);
+    o.W = d_W;
+    o.bias = d_bias;
+  } else if (o.kind == OP_BN) {
+    INSC_REQUIRE(d_mean && d_var, INSC_ERR_ARG, "insc_net_rebind_op: op %d is a batch norm and needs d_mean, d_var", op);
+    o.mean = d_mean;
+    o.var = d_var;
+    o.gamma = d_gamma;
+    o.beta = d_beta;
+  } else {
+    set_error("insc_net_rebind_op: op %d has no parameters", op);
+    return INSC_ERR_ARG;
+  }
+  return INSC_OK;
+}
+
 /* One frame.  d_coords: int32 [P, coord_cols] (x,y,z[,batch]); d_feats: float32 [P,in_channels].
  * increment == 0: forget all state and run a full forward over these points.
  * increment != 0: append the points to the scene of the previous frames and recompute only
@@ -888,6 +937,7 @@ int insc_net_forward(insc_net *net, const int32_t *d_coords, int coord_cols, con
   const int C0 = net->in_channels;
   int rc;
   const bool inc = increment != 0;
+  net->frame_id = net->frame_id == INT32_MAX ? 1 : net->frame_id + 1;
 
   if (!inc) {
     for (int l = 0; l < L; l++) {
@@ -925,7 +975,10 @@ int insc_net_forward(insc_net *net, const int32_t *d_coords, int coord_cols, con
     void *ws;
     if ((rc = workspace(WS_API, s, sizeof(int32_t) * 4 * (size_t)P, &ws))) return rc;
     int32_t *c4 = (int32_t *)ws;
-    hipLaunchKernelGGL(coords_to_int4_kernel, dim3(grid_for(P, 256)), dim3(256), 0, s, d_coords, coord_cols, P, c4);
+    hipLaunchKernelGGL(coords_check_kernel, dim3(grid_for(P, 256)), dim3(256), 0, s, d_coords, coord_cols, P, net->d_bad,
+                       net->frame_id);
+    hipLaunchKernelGGL(coords_to_int4_kernel, dim3(grid_for(P, 256)), dim3(256), 0, s, d_coords, coord_cols, P, c4,
+                       net->d_bad, net->frame_id);
     INSC_LAUNCH_CHECK();
     Level &L0 = net->levels[0];
     if ((rc = grid_insert_nosync(L0.grid, c4, P, sop, s))) return rc;
@@ -1254,7 +1307,8 @@ int insc_net_forward_residual(insc_net *net, const int32_t *d_coords, int coord_
   if ((rc = workspace(WS_API, s, sizeof(int32_t) * 4 * (size_t)P, &ws))) return rc;
   int32_t *c4 = (int32_t *)ws;
   const unsigned nb = grid_for(P, 256);
-  hipLaunchKernelGGL(coords_to_int4_kernel, dim3(nb), dim3(256), 0, s, d_coords, coord_cols, P, c4);
+  hipLaunchKernelGGL(coords_to_int4_kernel, dim3(nb), dim3(256), 0, s, d_coords, coord_cols, P, c4,
+                     (const int32_t *)nullptr, 0);
   INSC_LAUNCH_CHECK();
   if ((rc = grid_insert_nosync(R.levels[0].grid, c4, P, R.sop, s))) return rc;
   hipLaunchKernelGGL(chain_push_kernel, dim3(nb), dim3(256), 0, s, R.sop, P, R.chain_head, R.chain_next);

@@ -437,9 +437,11 @@ def _append_points(m, sc, input_coords, input_features):
     P, C = input_features.shape
     n_before = sc.n
     c4 = _coords4(input_coords, m.device)
+    # checked before anything is inserted, so that a bad frame leaves the site set as it was
+    if P and bool(((c4[:, :3] < 0) | (c4[:, :3] > 65535)).any().item() or (c4[:, 3] < 0).any().item()
+                  or (c4[:, 3] > 32767).any().item()):
+        raise InscError(-5, "a coordinate is outside 0..65535 (batch 0..32767); nothing was inserted")
     sop = m.insert(sc, c4)
-    if bool((sop < 0).any().item()):
-        raise InscError(-5, "a coordinate is outside 0..65535")
     if m.in_sum is None:
         m.in_sum = _Buf(C, torch.float32, m.device, fill=0.0)
         m.in_cnt = _Buf(None, torch.int32, m.device, fill=0)

@@ -63,6 +63,7 @@ _SIGS = {
     "insc_net_op_add": [vp, c_int, c_int, c_int],
     "insc_net_finalize": [vp, c_int, c_i64, vp],
     "insc_net_refresh_weights": [vp, vp],
+    "insc_net_rebind_op": [vp, c_int, vp, vp, vp, vp, vp, vp],
     "insc_net_forward": [vp, vp, c_int, vp, c_i64, c_int, vp, c_int, ctypes.POINTER(c_i64), vp],
     "insc_net_enable_residual": [vp],
     "insc_net_forward_residual": [vp, vp, c_int, vp, c_i64, vp, ctypes.POINTER(c_i64), vp],
@@ -100,6 +101,7 @@ _OTHER = {
     "insc_grid_count_ptr": (vp, [vp]),
     "insc_grid_capacity": (c_i64, [vp]),
     "insc_conv_packed_floats": (c_i64, [c_int, c_int, c_int]),
+    "insc_net_op_count": (c_int, [vp]),
 }
 
 EXPORTS = sorted(list(_SIGS) + list(_OTHER))

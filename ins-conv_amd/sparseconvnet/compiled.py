@@ -8,7 +8,11 @@
 The module path issues one C call per layer from Python; this path hands the whole frame to
 one C call, so an incremental frame costs a few hundred kernel launches and no Python work.
 Results are bit-identical to the module path.  Parameters are read in place (device
-pointers); after modifying weights call `refresh()`.
+pointers).  Whatever touches every parameter of the model - `.to()` / `.cpu()` + `.cuda()`
+(new storage), `load_state_dict` / `checkpoint_restore` (new values) - is noticed at the next
+call and the executor is pointed at the current tensors and re-packs its weights; after editing
+single parameters in place call `refresh()`.  JoinTable takes two inputs (the U-Net's skip
+connection); wider joins run on the module path only.
 """
 import ctypes
 
@@ -40,6 +44,7 @@ class CompiledNet(object):
         self.h = ctypes.c_void_p()
         lib.insc_net_create(levels, int(self.in_channels), int(self.input_layer.mode), ctypes.byref(self.h))
         self._keep = []  # tensors whose storage the executor points into
+        self._bound = []  # (op index, module) of every op with parameters
         self._level = {0: 0}
         self._chan = {0: self.in_channels}
         x = 0
@@ -51,6 +56,7 @@ class CompiledNet(object):
         if self.residual:
             lib.insc_net_enable_residual(self.h)
         lib.insc_net_finalize(self.h, int(x), I64(int(capacity_sites)), stream_ptr())
+        self._sig = self._signature(False)
 
     def __del__(self):
         try:
@@ -73,8 +79,35 @@ class CompiledNet(object):
         t = t.detach()
         if not t.is_contiguous():
             raise ValueError("parameters must be contiguous")
+        if t.device != self.device:
+            raise ValueError("a parameter is on %s, the compiled net on %s" % (t.device, self.device))
         self._keep.append(t)
         return ptr(t)
+
+    @staticmethod
+    def _params(m):
+        """The tensors op parameters are read from, in the order of insc_net_rebind_op."""
+        import sparseconvnet as scn
+
+        bias = getattr(m, "bias", None)
+        if isinstance(m, scn.BatchNormalization):
+            return (None, None, m.running_mean, m.running_var, getattr(m, "weight", None), bias)
+        return (m.weight, bias, None, None, None, None)
+
+    def _bind_op(self, m):
+        self._bound.append((int(lib.insc_net_op_count(self.h)) - 1, m))
+
+    def _signature(self, full):
+        """(address, version) of the bound tensors: all of them, or the first and last op's only."""
+        ops = self._bound if full or len(self._bound) < 2 else (self._bound[0], self._bound[-1])
+        return tuple((t.data_ptr(), t._version) for _, m in ops for t in self._params(m) if t is not None)
+
+    def _rebind(self):
+        self._keep = []
+        for op, m in self._bound:
+            lib.insc_net_rebind_op(self.h, op, *[self._dev(t) for t in self._params(m)])
+        lib.insc_net_refresh_weights(self.h, stream_ptr())
+        self._sig = self._signature(False)
 
     def _trace(self, m, x):
         import sparseconvnet as scn
@@ -106,6 +139,7 @@ class CompiledNet(object):
             lib.insc_net_op_bn(self.h, x, o, self._dev(m.running_mean), self._dev(m.running_var),
                                self._dev(getattr(m, "weight", None)), self._dev(bias), ctypes.c_float(m.eps),
                                ctypes.c_float(m.leakiness))
+            self._bind_op(m)
             return o
         if isinstance(m, scn.SubmanifoldConvolution):
             if SCN._key(m.filter_size) != (3, 3, 3) or m.dilated_rate != 1:
@@ -123,15 +157,19 @@ class CompiledNet(object):
             raise NotImplementedError("no executor op for %s" % type(m).__name__)
         o = self._new(self._level[x] + dl, m.nOut)
         lib.insc_net_op_conv(self.h, _KIND[kind], x, o, self._dev(m.weight), self._dev(bias))
+        self._bind_op(m)
         return o
 
     # ---- running --------------------------------------------------------------------------
     def refresh(self):
-        lib.insc_net_refresh_weights(self.h, stream_ptr())
+        """Point the executor at the model's current parameter tensors and re-pack the weights."""
+        self._rebind()
 
     def __call__(self, input, increment=False, all_points=None):
         coords, feats = input[0], input[1]
         from . import incremental
+        if self._signature(False) != self._sig:  # the model was moved or reloaded since the last call
+            self._rebind()
         if incremental.kind(increment) == "residual":
             return self._residual(coords, feats)
         increment = bool(increment)

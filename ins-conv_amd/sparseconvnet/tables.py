@@ -72,7 +72,9 @@ class AddTable(torch.nn.Sequential):
             out = self._state.grow(n, keep=min(n, self._state.buf.size(0)))
         else:
             out = self._state.new(n, C, input[0].features)
-        if n:
+        if n and len(input) == 1:  # a sum of one term (the reference sums any number of inputs >= 1)
+            SCN.copy_rows(input[0].features, out, rows, count, n_rows)
+        elif n:
             SCN.add_rows(input[0].features, input[1].features, out, rows, count, n_rows)
             for i in input[2:]:
                 SCN.add_rows(out, i.features, out, rows, count, n_rows)

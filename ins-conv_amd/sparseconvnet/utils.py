@@ -52,40 +52,50 @@ class StateBuf(object):
 # checkpoints (sparseconvnet/utils.py:201-233) and weights trained elsewhere
 # ---------------------------------------------------------------------------------------------
 def is_power2(num):
-    return num != 0 and ((num & (num - 1)) == 0)
+    return num > 0 and bin(num).count("1") == 1
+
+
+def _checkpoint_file(exp_name, name2, epoch, digits=4):
+    return "%s-%0*d-%s.pth" % (exp_name, digits, epoch, name2)
 
 
 def checkpoint_save(model, exp_name, name2, epoch, use_cuda=True):
-    """state_dict to '<exp_name>-<epoch:04d>-<name2>.pth'; the previous epoch's file is removed
-    unless its number is a power of two (utils.py:222-233)."""
-    f = exp_name + "-%04d-" % epoch + name2 + ".pth"
+    """Writes the state_dict to '<exp_name>-<epoch:04d>-<name2>.pth' and drops the file of epoch - 1
+    unless that number is a power of two, so a long run keeps a logarithmic trail
+    (reference: sparseconvnet/utils.py:222-233; same file names, same pruning rule).  The
+    tensors are written from host memory; with use_cuda the model goes back to the GPU."""
     model.cpu()
-    torch.save(model.state_dict(), f)
+    torch.save(model.state_dict(), _checkpoint_file(exp_name, name2, epoch))
     if use_cuda:
         model.cuda()
-    epoch = epoch - 1
-    f = exp_name + "-%04d-" % epoch + name2 + ".pth"
-    if os.path.isfile(f) and not is_power2(epoch):
-        os.remove(f)
+    stale = _checkpoint_file(exp_name, name2, epoch - 1)
+    if not is_power2(epoch - 1) and os.path.isfile(stale):
+        os.remove(stale)
 
 
 def checkpoint_restore(model, exp_name, name2, use_cuda=True, epoch=0):
-    """Load the given epoch, or the latest '<exp_name>-*-<name2>.pth'; returns the next epoch
-    number (utils.py:201-218).  Files are read with weights_only=True (tensors only)."""
+    """Loads epoch `epoch`, or with epoch == 0 the newest '<exp_name>-*-<name2>.pth', into the
+    model and returns the number of the epoch to run next; without any file the model is left as
+    it is and 1 is returned (reference: sparseconvnet/utils.py:201-218).  Files are read with
+    weights_only=True: tensors only, nothing in the file is executed."""
+    path = None
+    if epoch > 0:
+        # the reference asks for nine digits here although it writes four; accept both
+        for digits in (9, 4):
+            if os.path.isfile(_checkpoint_file(exp_name, name2, epoch, digits)):
+                path = _checkpoint_file(exp_name, name2, epoch, digits)
+                break
+        if path is None:
+            raise AssertionError("no checkpoint %s" % _checkpoint_file(exp_name, name2, epoch))
+    else:
+        found = sorted(glob.glob(exp_name + "-*-" + name2 + ".pth"))
+        if found:
+            path = found[-1]
+            epoch = int(path[len(exp_name) + 1:len(path) - len(name2) - 5])
     if use_cuda:
         model.cpu()
-    if epoch > 0:
-        f = exp_name + "-%09d-" % epoch + name2 + ".pth"  # the reference's pattern for an explicit epoch
-        if not os.path.isfile(f):
-            f = exp_name + "-%04d-" % epoch + name2 + ".pth"  # what checkpoint_save writes
-        assert os.path.isfile(f), f
-        model.load_state_dict(torch.load(f, weights_only=True))
-    else:
-        fs = sorted(glob.glob(exp_name + "-*-" + name2 + ".pth"))
-        if len(fs) > 0:
-            f = fs[-1]
-            model.load_state_dict(torch.load(f, weights_only=True))
-            epoch = int(f[len(exp_name) + 1:-len(name2) - 5])
+    if path is not None:
+        model.load_state_dict(torch.load(path, weights_only=True))
     if use_cuda:
         model.cuda()
     return epoch + 1

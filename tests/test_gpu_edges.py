@@ -143,3 +143,71 @@ def test_residual_frames_disjoint_from_and_inside_the_saved_scene():
         idx = np.random.default_rng(48).permutation(len(vox))[:1200]
         got = net(_inp(vox[idx], rgb[idx]), increment="residual")
     np.testing.assert_allclose(got.cpu().numpy(), saved[idx].cpu().numpy(), rtol=0, atol=2e-5)
+
+
+def test_a_frame_with_a_bad_coordinate_is_dropped_whole():
+    """One coordinate outside the representable range: the executor and the module tree reject the
+    frame and keep the state of the previous frame, so that the next valid frame still equals a
+    full forward over the valid points; after a full frame that fails, an incremental frame is
+    refused until a full frame succeeded."""
+    import sparseconvnet as scn
+    from sparseconvnet._lib import InscError
+    from workloads.netdefs import NaiveUNet
+
+    vox, rgb = _scene(49)
+    model = NaiveUNet(m=16, levels=4, seed=16).cuda()
+    ref_model = copy.deepcopy(model)
+    mod_model = copy.deepcopy(model)
+    for mod in mod_model.modules():
+        if isinstance(mod, scn.OutputLayer):
+            mod.all_points = True
+    net = scn.compile(model.sparseModel, capacity_sites=8192)
+    n0, n1 = 3000, 4000
+    bad = vox[n0:n1].copy()
+    bad[17, 1] = 70000
+    neg = vox[n0:n1].copy()
+    neg[3, 2] = -1
+    with torch.no_grad():
+        net(_inp(vox[:n0], rgb[:n0]), increment=False)
+        mod_model.sparseModel(_inp(vox[:n0], rgb[:n0]), False)
+        for frame in (bad, neg):
+            with pytest.raises(InscError) as e:
+                net(_inp(frame, rgb[n0:n1]), increment=True)
+            assert e.value.code == -5
+            with pytest.raises(InscError):
+                mod_model.sparseModel(_inp(frame, rgb[n0:n1]), True)
+        assert net.sites_per_level()[0] == n0
+        out = net(_inp(vox[n0:], rgb[n0:]), increment=True, all_points=True)
+        out_mod = mod_model.sparseModel(_inp(vox[n0:], rgb[n0:]), True)
+        ref = ref_model.sparseModel(_inp(vox, rgb))
+        assert torch.equal(out, ref)
+        assert torch.equal(out_mod, ref)
+        # a full frame that fails leaves no state behind
+        with pytest.raises(InscError):
+            net(_inp(bad, rgb[n0:n1]), increment=False)
+        with pytest.raises(InscError) as e:
+            net(_inp(vox[:10], rgb[:10]), increment=True)
+        assert e.value.code == -4
+        assert torch.equal(net(_inp(vox, rgb), increment=False), ref)
+
+
+def test_grid_reports_a_bad_coordinate_once_and_stays_usable():
+    import ctypes
+
+    from sparseconvnet._lib import InscError, ensure_init, lib, ptr, stream_ptr
+
+    ensure_init(0)
+    I64 = ctypes.c_int64
+    g = ctypes.c_void_p()
+    lib.insc_grid_create(I64(4096), ctypes.byref(g))
+    c = torch.tensor([[1, 2, 3, 0], [70000, 0, 0, 0], [4, 5, 6, 0], [1, 2, 3, 0]], dtype=torch.int32, device="cuda")
+    sop = torch.empty(4, dtype=torch.int32, device="cuda")
+    n = I64(0)
+    with pytest.raises(InscError) as e:
+        lib.insc_grid_insert(g, ptr(c), I64(4), ptr(sop), ctypes.byref(n), stream_ptr())
+    assert e.value.code == -5
+    assert sop.tolist() == [0, -1, 1, 0]
+    c2 = torch.tensor([[9, 9, 9, 0], [4, 5, 6, 0]], dtype=torch.int32, device="cuda")
+    lib.insc_grid_insert(g, ptr(c2), I64(2), ptr(sop), ctypes.byref(n), stream_ptr())
+    assert n.value == 3 and sop[:2].tolist() == [2, 1]
+    lib.insc_grid_destroy(g)

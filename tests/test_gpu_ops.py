@@ -137,6 +137,46 @@ def test_persistent_kernels_give_the_bits_of_the_per_tile_kernel(S, orc, Cin, Co
     np.testing.assert_allclose(a.cpu().numpy(), ref, rtol=RTOL, atol=ATOL)
 
 
+@pytest.mark.parametrize("Cin,Cout,bias", [(16, 16, False), (16, 16, True), (32, 32, False), (32, 32, True),
+                                            (16, 32, True), (32, 20, False)])
+def test_filter_in_lds_kernel_against_oracle_and_per_tile_kernel(S, orc, Cin, Cout, bias):
+    """Narrow 3^3 layers (Cin, Cout <= 32) have two kernels: one wavefront per tile, and - from 4096
+    tiles up by default - persistent blocks that keep the whole filter in LDS (the kernel the
+    HBM-roofline figure is quoted on).  Here the threshold is lowered so that the 20k-voxel scene of
+    workload 1 runs on the second one, planned and unplanned staging, and the result is compared with
+    the CPU oracle (1e-4 / 1e-5) and bit for bit with the first kernel."""
+    from sparseconvnet._lib import lib
+
+    pts = scenes.boxes_scene(seed=1, n=20000)
+    m, x, feats = setup_sites(S, pts, Cin, seed=Cin + 7)
+    sc = m.ssc_rulebook(SZ)
+    rng = np.random.default_rng(Cout + 11)
+    W = cu((rng.normal(size=(27, Cin, Cout)) * (2.0 / Cin / 27) ** 0.5).astype(np.float32))
+    b = rng.normal(size=Cout).astype(np.float32) if bias else None
+    bt = cu(b) if bias else None
+    per_tile = torch.full((sc.n, Cout), 3.0, device="cuda")
+    lds_planned = torch.full((sc.n, Cout), -3.0, device="cuda")
+    lds_unplanned = torch.full((sc.n, Cout), 5.0, device="cuda")
+    lds_permuted = torch.full((sc.n, Cout), 7.0, device="cuda")
+    perm = torch.randperm(sc.n, generator=torch.Generator().manual_seed(Cin)).to(torch.int32).cuda()
+    try:
+        lib.insc_conv_set_filter_lds_min_tiles(1 << 40)
+        S.ssc_rows_planned(feats, per_tile, W, bt, sc, m.ssc_plan(sc))
+        lib.insc_conv_set_filter_lds_min_tiles(1)
+        S.ssc_rows_planned(feats, lds_planned, W, bt, sc, m.ssc_plan(sc))
+        S.conv_rows(feats, lds_unplanned, W, bt, sc.nbr.t, 27, sc.order.t, None, sc.n)
+        S.conv_rows(feats, lds_permuted, W, bt, sc.nbr.t, 27, perm, None, sc.n)
+    finally:
+        lib.insc_conv_set_filter_lds_min_tiles(4096)
+    assert torch.equal(lds_planned, per_tile)
+    assert torch.equal(lds_unplanned, per_tile)
+    assert torch.equal(lds_permuted, per_tile)
+    _, osc, _ = orc.grid_build(pts)
+    _, counts, pairs = orc.ssc_rules(osc)
+    ref, _ = orc.conv_forward(feats.cpu().numpy(), W.cpu().numpy(), b, pairs, counts, len(osc))
+    np.testing.assert_allclose(lds_planned.cpu().numpy(), ref, rtol=RTOL, atol=ATOL)
+
+
 @pytest.mark.parametrize("n", [1, 20, 33, 130, 1025])
 def test_persistent_kernels_on_tiny_and_ragged_scenes(S, n):
     """One site, one tile, two tiles, a group of four tiles with a partial fifth, a partial last tile:
