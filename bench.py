@@ -1,17 +1,24 @@
 #!/usr/bin/env python3
 """Benchmark of the incremental sparse-convolution inference path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload incr|unet|ssc]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload incr|unet|ssc|cfg1|cfg2]
 
 Prints ONE JSON line.  A step is one pass of the hot path over one batch of seeded synthetic
 input that is already resident in HBM when the timed region starts:
   incr (default): workload 5 - one incremental U-Net frame of the 50-frame sensor sweep
-         (3k-8k new voxels + 1k-2k re-observed voxels per frame, growing to 150k voxels);
-         frame 0 (full forward) and the first W incremental frames are untimed, the next K
-         incremental frames are timed back to back.  value = mean ms per frame.
+         (3k-8k new voxels + 1k-2k re-observed voxels per frame, growing to 150k voxels).
+         The LAST K incremental frames of the sweep are timed back to back, whatever K is, so
+         that the timed region ends on the 150 000-voxel scene the metric names; frame 0 (full
+         forward) and the 49 - K frames before them are untimed (W is a lower bound on those).
+         value = mean ms per frame; frame_at_150k_ms = the last frame alone.
   unet : workload 4 - full U-Net forward over the 150k-voxel scene (165k points).
   ssc  : workload 3 - 4 x [SubmanifoldConvolution(3) + BatchNormReLU] at 500k active voxels,
          once at 32 channels and once at 64 (8 convolutions per step); value = Msites/s.
+  cfg1 : workload 1 - one SubmanifoldConvolution(3) 16->16 on 20k voxels in 128^3: HIP us per
+         call, the CPU oracle's ms, largest absolute / relative error between the two.
+  cfg2 : workload 2 - hash grid insert of 200k voxels in 1024^3 (+10 % repeated points), query,
+         3^3 rulebook and stride-2 rulebook: Minserts/s, Mqueries/s, GB/s, and whether every
+         integer structure equals the CPU oracle's bit for bit (computed in the same run).
 `roofline` is measured live on the dominant kernel, the submanifold gather-GEMM-scatter, at
 the size the roofline target is stated for (500k voxels, 32 channels), with events on the
 launch stream.  `cpu_baseline` times the CPU oracle (a restatement of the reference's CPU
@@ -30,6 +37,38 @@ for p in (ROOT, os.path.join(ROOT, "ins-conv_amd")):
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 MFMA_FP32_PEAK_TFLOPS = 157.3
+
+
+def profile_records(name):
+    """Machine-readable lines of a counter summary under profiles/: every line of the form
+    `TRAFFIC key=value key=value ...` as a dict.  None if the summary is not there."""
+    path = os.path.join(ROOT, "profiles", name)
+    if not os.path.isfile(path):
+        return None
+    out = []
+    with open(path) as f:
+        for line in f:
+            w = line.split()
+            if w and w[0] == "TRAFFIC":
+                out.append(dict(kv.split("=", 1) for kv in w[1:]))
+    return out
+
+
+def profiled_traffic(name, kernel):
+    """HBM bytes per launch of `kernel` as recorded in profiles/<name> (FETCH_SIZE + WRITE_SIZE,
+    each scaled by the copy-kernel calibration of the same run).  The summary must be about this
+    kernel: a stale file fails loudly instead of lending its number to another kernel."""
+    recs = profile_records(name)
+    if recs is None:
+        return None, "profiles/%s not found" % name
+    hit = [r for r in recs if r.get("kernel") == kernel]
+    if len(hit) != 1:
+        raise SystemExit("bench.py: profiles/%s holds no TRAFFIC record for kernel %s" % (name, kernel))
+    r = hit[0]
+    fetch, write = float(r["fetch_bytes"]), float(r["write_bytes"])
+    return fetch + write, ("HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by what the "
+                           "same counter reads for a plain copy of known size: %.1f MB fetched + %.1f MB written, "
+                           "profiles/%s" % (fetch / 1e6, write / 1e6, name))
 
 
 # ---------------------------------------------------------------------------------------------
@@ -113,13 +152,13 @@ def conv_roofline(device, reps=30, warm=200):
     bytes_alg = n_rules * (4 * Cin + 8) + sc.n * 4 * Cout + 27 * Cin * Cout * 4
     flops = 2.0 * n_rules * Cin * Cout
     achieved = bytes_alg / t / 1e9
+    traffic, traffic_note = profiled_traffic("conv_wlds_ssc32_500k.txt", "insc::conv_wlds_kernel")
     return {
         "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-        "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": 551.6e6,
+        "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
         "kernel": "conv_wlds_kernel (SSC 3^3, 32->32, filter in LDS, persistent blocks; 500k sites, %d rules)" % n_rules,
         "avg_us": round(t * 1e6, 1), "algorithmic_bytes": int(bytes_alg),
-        "traffic_note": "HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE (x1.999, copy-kernel calibration) + "
-                        "WRITE_SIZE (x1.000): 453.0 MB + 98.6 MB, profiles/conv_wlds_ssc32_500k.txt",
+        "traffic_note": traffic_note,
         "mfma_tflops": round(flops / t / 1e12, 2), "mfma_frac": round(flops / t / 1e12 / MFMA_FP32_PEAK_TFLOPS, 4),
         "ssc_msites_per_s": round(sc.n / t / 1e6, 1),
     }
@@ -378,12 +417,189 @@ def cpu_baseline_ssc(n_sample=100000):
     }
 
 
+# ---------------------------------------------------------------------------------------------
+# workloads 1 and 2: one convolution against the CPU oracle; the integer structures
+# ---------------------------------------------------------------------------------------------
+def cfg1_workload(device, K, W):
+    """One SubmanifoldConvolution(3), 16 -> 16, on the 20k-voxel box scene in 128^3."""
+    import numpy as np
+    import torch
+
+    import sparseconvnet as scn
+    from oracle import oracle as orc
+    from sparseconvnet import SCN
+    from workloads import scenes
+
+    vox = scenes.boxes_scene(seed=1, n=20000)
+    rng = np.random.default_rng(1)
+    f = rng.normal(size=(len(vox), 16)).astype(np.float32)
+    Wt = (rng.normal(size=(27, 16, 16)) * (2.0 / 16 / 27) ** 0.5).astype(np.float32)
+    size = torch.LongTensor([128, 128, 128])
+    x = scn.InputLayer(3, size, mode=4)([torch.from_numpy(vox.astype(np.int64)), torch.from_numpy(f).to(device), 1])
+    m = x.metadata
+    sc = m.ssc_rulebook(size)
+    plan = m.ssc_plan(sc)
+    w = torch.from_numpy(Wt).to(device)
+    out = torch.empty((sc.n, 16), device=device)
+    for _ in range(W):
+        SCN.ssc_rows_planned(x.features, out, w, None, sc, plan)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(K):
+        SCN.ssc_rows_planned(x.features, out, w, None, sc, plan)
+    e1.record()
+    torch.cuda.synchronize()
+    t = e0.elapsed_time(e1) * 1e-3 / K
+    # the oracle on the same sites (same numbering: first appearance), timed on the host cores
+    _, osc, _ = orc.grid_build(vox)
+    _, counts, pairs = orc.ssc_rules(osc)
+    orc.conv_forward(f, Wt, None, pairs, counts, len(osc))
+    best = 1e30
+    for _ in range(5):
+        t0 = time.perf_counter()
+        ref, _ = orc.conv_forward(f, Wt, None, pairs, counts, len(osc))
+        best = min(best, time.perf_counter() - t0)
+    got = out.cpu().numpy()
+    err = np.abs(got - ref)
+    rel = err / np.maximum(np.abs(ref), 1e-3)
+    n_rules = int(counts.sum())
+    info = {"hip_us": round(t * 1e6, 2), "oracle_ms": round(best * 1e3, 3), "oracle_threads": orc.num_threads(),
+            "max_abs_err": float(err.max()), "max_rel_err": float(rel.max()),
+            "max_rel_err_note": "relative to max(|reference|, 1e-3)",
+            "within_1e-4_rel_1e-5_abs": bool((err <= 1e-5 + 1e-4 * np.abs(ref)).all()),
+            "sites": int(sc.n), "rules": n_rules}
+    return t, info
+
+
+def cfg2_workload(device, K, W):
+    """Hash grid + rulebooks of the 200k-voxel scene in 1024^3, timed per C call and compared with the
+    CPU oracle bit for bit in the same run."""
+    import ctypes
+
+    import numpy as np
+    import torch
+
+    from oracle import oracle as orc
+    from sparseconvnet._lib import lib, ptr, stream_ptr
+    from workloads import scenes
+
+    I64 = ctypes.c_int64
+    st = stream_ptr()
+    rng = np.random.default_rng(2)
+    vox = scenes.planes_boxes_scene(seed=2, n=200000).astype(np.int32)
+    pts = np.concatenate([vox, vox[rng.integers(0, len(vox), len(vox) // 10)]])
+    pts = np.ascontiguousarray(pts[rng.permutation(len(pts))][:, :4])
+    P, N = len(pts), len(vox)
+    c4 = torch.from_numpy(pts).to(device)
+    sop = torch.empty(P, dtype=torch.int32, device=device)
+    q = torch.empty(P, dtype=torch.int32, device=device)
+    grid, coarse = ctypes.c_void_p(), ctypes.c_void_p()
+    lib.insc_grid_create(I64(2 * N), ctypes.byref(grid))
+    lib.insc_grid_create(I64(N), ctypes.byref(coarse))
+    n_sites = I64(0)
+    nbr = torch.empty((N, 27), dtype=torch.int32, device=device)
+    parent = torch.empty(N, dtype=torch.int32, device=device)
+    offset = torch.empty(N, dtype=torch.int32, device=device)
+    child = torch.empty((N, 8), dtype=torch.int32, device=device)
+
+    def timed(fn, pre=None):
+        for _ in range(W):
+            if pre:
+                pre()
+            fn()
+        torch.cuda.synchronize()
+        total = 0.0
+        for _ in range(K):
+            if pre:
+                pre()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            fn()
+            e1.record()
+            torch.cuda.synchronize()
+            total += e0.elapsed_time(e1)
+        return total * 1e-3 / K
+
+    t_ins = timed(lambda: lib.insc_grid_insert(grid, ptr(c4), I64(P), ptr(sop), ctypes.byref(n_sites), st),
+                  pre=lambda: lib.insc_grid_clear(grid, st))
+    t_qry = timed(lambda: lib.insc_grid_query(grid, ptr(c4), I64(P), ptr(q), st))
+    t_ssc = timed(lambda: lib.insc_rulebook_ssc3(grid, I64(0), I64(N), ptr(nbr), 0, st))
+
+    def down_pre():
+        lib.insc_grid_clear(coarse, st)
+        child.fill_(-1)
+
+    t_dn = timed(lambda: lib.insc_rulebook_down2(grid, coarse, I64(0), I64(N), ptr(parent), ptr(offset), ptr(child),
+                                                 I64(N), st), pre=down_pre)
+    nc = I64(0)
+    lib.insc_grid_size(coarse, ctypes.byref(nc), st)
+    # bit-exactness against the oracle (ids are comparable as they are: both number by first appearance)
+    o_sop, o_sc, _ = orc.grid_build(pts)
+    o_nbr, _, _ = orc.ssc_rules(o_sc)
+    o_parent, o_off, o_cc = orc.down2_rules(o_sc)
+    coords = torch.empty((N, 4), dtype=torch.int32, device=device)
+    ccoords = torch.empty((nc.value, 4), dtype=torch.int32, device=device)
+    hip = ctypes.CDLL("libamdhip64.so")
+    torch.cuda.synchronize()
+    ok_copy = hip.hipMemcpy(ctypes.c_void_p(coords.data_ptr()), ctypes.c_void_p(lib.insc_grid_coords(grid)),
+                            ctypes.c_size_t(N * 16), 3) == 0
+    ok_copy = ok_copy and hip.hipMemcpy(ctypes.c_void_p(ccoords.data_ptr()),
+                                        ctypes.c_void_p(lib.insc_grid_coords(coarse)),
+                                        ctypes.c_size_t(nc.value * 16), 3) == 0
+    checks = {
+        "site_of_point": bool(np.array_equal(sop.cpu().numpy(), o_sop)),
+        "query": bool(np.array_equal(q.cpu().numpy(), o_sop)),
+        "site_coords": bool(ok_copy and np.array_equal(coords.cpu().numpy(), o_sc)),
+        "ssc_neighbour_map": bool(np.array_equal(nbr.cpu().numpy(), o_nbr)),
+        "down2_parent": bool(np.array_equal(parent.cpu().numpy(), o_parent)),
+        "down2_offset": bool(np.array_equal(offset.cpu().numpy(), o_off)),
+        "coarse_coords": bool(ok_copy and np.array_equal(ccoords.cpu().numpy(), o_cc)),
+    }
+    lib.insc_grid_destroy(grid)
+    lib.insc_grid_destroy(coarse)
+    ssc_bytes = N * (16 + 27 * 8 + 27 * 4)
+    info = {"points": P, "sites": int(n_sites.value), "coarse_sites": int(nc.value),
+            "insert_us": round(t_ins * 1e6, 1), "Minserts_per_s": round(P / t_ins / 1e6, 1),
+            "insert_GB/s": round(P * 32 / t_ins / 1e9, 1),
+            "query_us": round(t_qry * 1e6, 1), "Mqueries_per_s": round(P / t_qry / 1e6, 1),
+            "query_GB/s": round(P * 28 / t_qry / 1e9, 1),
+            "ssc_rulebook_us": round(t_ssc * 1e6, 1), "ssc_rulebook_GB/s": round(ssc_bytes / t_ssc / 1e9, 1),
+            "ssc_rulebook_frac_of_hbm_peak": round(ssc_bytes / t_ssc / 1e9 / HBM_PEAK_GBS, 4),
+            "down2_rulebook_us": round(t_dn * 1e6, 1), "down2_rulebook_GB/s": round(N * 36 / t_dn / 1e9, 1),
+            "bit_exact": bool(all(checks.values())), "bit_exact_checks": checks}
+    return t_ins + t_qry + t_ssc + t_dn, info
+
+
+def cpu_baseline_cfg2():
+    import numpy as np
+
+    from oracle import oracle as orc
+    from workloads import scenes
+
+    rng = np.random.default_rng(2)
+    vox = scenes.planes_boxes_scene(seed=2, n=200000).astype(np.int32)
+    pts = np.concatenate([vox, vox[rng.integers(0, len(vox), len(vox) // 10)]])
+    pts = np.ascontiguousarray(pts[rng.permutation(len(pts))][:, :4])
+    best = 1e30
+    for _ in range(3):
+        t0 = time.perf_counter()
+        _, sc, _ = orc.grid_build(pts)
+        orc.ssc_rules(sc)
+        orc.down2_rules(sc)
+        best = min(best, time.perf_counter() - t0)
+    return {"value": round(len(pts) / best / 1e6, 3), "unit": "Mpoints/s", "cores": orc.num_threads(), "kind": "port",
+            "sample": "the whole workload: grid build of %d points + 3^3 rulebook + stride-2 rulebook, best of 3"
+                      % len(pts)}
+
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=None)
     ap.add_argument("--warmup", type=int, default=None)
-    ap.add_argument("--workload", default="incr", choices=["incr", "unet", "ssc"])
+    ap.add_argument("--workload", default="incr", choices=["incr", "unet", "ssc", "cfg1", "cfg2"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-residual", action="store_true",
                     help="skip the residual-frame comparison row of the incremental workload")
@@ -434,37 +650,47 @@ def main():
         from workloads import scenes
 
         seq = scenes.sweep_sequence()
-        W = 9 if args.warmup is None else args.warmup
-        K = len(seq) - 1 - W if args.steps is None else args.steps
-        if W + K > len(seq) - 1 or K < 1:
-            sys.exit("bench.py: the sweep has %d incremental frames; need warmup + steps <= %d"
-                     % (len(seq) - 1, len(seq) - 1))
+        n_inc = len(seq) - 1  # incremental frames of the sweep (frame 0 is the full forward)
+        W = 5 if args.warmup is None else args.warmup
+        K = 20 if args.steps is None else args.steps
+        if K < 1 or K > 40 or W < 0 or W + K > n_inc:
+            sys.exit("bench.py: the sweep has %d incremental frames and the LAST --steps of them are timed (the "
+                     "scene must have grown to 150k voxels): need 1 <= steps <= 40 and warmup + steps <= %d"
+                     % (n_inc, n_inc))
+        first = n_inc - K + 1  # first timed frame; frames 1 .. first - 1 (at least W of them) are untimed
         model, net = unet_model(device)
         frames = [to_dev(p, c, device) for p, c in seq]
         with torch.no_grad():
             # the logits of a frame's points = Linear(features of those points)
             net(frames[0], increment=False)
-            for f in range(1, 1 + W):
+            for f in range(1, first):
                 model.linear(net(frames[f], increment=True))
             torch.cuda.synchronize()
+            sites_at_start = net.n_sites
             per_frame = []
             t0 = time.perf_counter()
-            for f in range(1 + W, 1 + W + K):
+            for f in range(first, n_inc + 1):
                 t1 = time.perf_counter()
                 model.linear(net(frames[f], increment=True))
                 torch.cuda.synchronize()
                 per_frame.append((time.perf_counter() - t1) * 1e3)
             dt = time.perf_counter() - t0
+        if net.n_sites != 150000:
+            sys.exit("bench.py: the sweep ended on %d voxels, not on the 150 000 the metric names" % net.n_sites)
         ms = dt * 1e3 / K
         value, metric, unit, hib = round(ms, 3), "incremental frame latency ms (UNet, 150k vox)", "ms", False
-        config = {"workload": "cfg5: incremental U-Net frames %d..%d of the 50-frame sweep (m=32, 7 levels, "
-                              "InputLayer mode 4 .. OutputLayer + Linear(32,20)); scene grows to 150k voxels"
-                              % (1 + W, W + K),
-                  "points_per_frame_mean": int(np.mean([len(seq[f][0]) for f in range(1 + W, 1 + W + K)])),
-                  "sites_at_end": net.n_sites, "sites_per_level_at_end": net.sites_per_level()[:7]}
-        extra = {"median_ms": round(float(np.median(per_frame)), 3),
+        config = {"workload": "cfg5: the last %d incremental U-Net frames (%d..%d) of the 50-frame sweep (m=32, 7 "
+                              "levels, InputLayer mode 4 .. OutputLayer + Linear(32,20)); frames 0..%d untimed; the "
+                              "scene grows from %d to 150 000 voxels over the timed frames"
+                              % (K, first, n_inc, first - 1, sites_at_start),
+                  "points_per_frame_mean": int(np.mean([len(seq[f][0]) for f in range(first, n_inc + 1)])),
+                  "points_last_frame": int(len(seq[n_inc][0])),
+                  "sites_at_start": sites_at_start, "sites_at_end": net.n_sites,
+                  "sites_per_level_at_end": net.sites_per_level()[:7]}
+        extra = {"frame_at_150k_ms": round(per_frame[-1], 3),
+                 "median_ms": round(float(np.median(per_frame)), 3),
                  "p95_ms": round(float(np.percentile(per_frame, 95)), 3),
-                 "last_frame_ms": round(per_frame[-1], 3), "first_timed_frame_ms": round(per_frame[0], 3)}
+                 "first_timed_frame_ms": round(per_frame[0], 3)}
         # rows the last timed frame recomputed: per scale, the smallest and the largest dirty set
         # among the tensors of that scale, beside the scale's sites
         sites = net.sites_per_level()
@@ -472,7 +698,7 @@ def main():
             {"scale": l, "sites": int(sites[l]), "min": min(r for _, r in sets), "max": max(r for _, r in sets)}
             for l, sets in enumerate(net.dirty_rows()) if sets]
         if not args.no_residual:
-            extra.update(residual_row(model, seq, frames, W + K, device))
+            extra.update(residual_row(model, seq, frames, n_inc, device))
         cpu_fn = cpu_baseline_unet
     elif args.workload == "unet":
         from workloads import scenes
@@ -496,6 +722,27 @@ def main():
         config = {"workload": "cfg4: full U-Net forward (grid + rulebooks + all layers), 150k voxels / 165k points",
                   "sites_per_level": net.sites_per_level()[:7]}
         cpu_fn = cpu_baseline_unet
+    elif args.workload == "cfg1":
+        W = 50 if args.warmup is None else args.warmup
+        K = 200 if args.steps is None else args.steps
+        t, info = cfg1_workload(device, K, W)
+        ms = t * 1e3
+        value, metric, unit, hib = round(info["sites"] / t / 1e6, 1), "SSC Msites/s", "Msites/s", True
+        config = {"workload": "cfg1: one SubmanifoldConvolution(3) 16->16 on 20 000 voxels (faces of 8 boxes in 128^3)"}
+        extra = {"cfg1": info}
+        cpu_fn = lambda: {"value": round(info["sites"] / (info["oracle_ms"] * 1e-3) / 1e6, 3), "unit": "Msites/s",
+                          "cores": info["oracle_threads"], "kind": "port",
+                          "sample": "the whole workload (one convolution over the 20k-voxel scene), best of 5"}
+    elif args.workload == "cfg2":
+        W = 2 if args.warmup is None else args.warmup
+        K = 20 if args.steps is None else args.steps
+        t, info = cfg2_workload(device, K, W)
+        ms = t * 1e3
+        value, metric, unit, hib = info["Minserts_per_s"], "hash grid Minserts/s", "Minserts/s", True
+        config = {"workload": "cfg2: hash grid insert of 200 000 voxels in 1024^3 (+10 % repeated points), query, 3^3 "
+                              "rulebook, stride-2 size-2 rulebook; one step = the four calls"}
+        extra = {"cfg2": info}
+        cpu_fn = cpu_baseline_cfg2
     else:
         W = 3 if args.warmup is None else args.warmup
         K = 20 if args.steps is None else args.steps
@@ -521,6 +768,11 @@ def main():
         "dtype": "f32", "data": "synthetic", "config": config,
     }
     out.update(extra)
+    if args.workload in ("cfg1", "cfg2"):  # small side workloads: the roofline rows belong to the main ones
+        if not args.no_cpu_baseline:
+            out["cpu_baseline"] = cpu_fn()
+        print(json.dumps(out))
+        return
     out["roofline"] = conv_roofline(device)
     out["wide_layer"] = wide_conv_row(device)
     out["kernels"] = kernel_table(device)
