@@ -70,6 +70,17 @@ int insc_grid_reserve(insc_grid *g, int64_t capacity_sites, void *stream);
  * 766-796; kernels CUDPPWrapper.cu:72-100,212-231). */
 int insc_grid_insert(insc_grid *g, const int32_t *d_coords4, int64_t P, int32_t *d_site_of_point, int64_t *h_n_sites,
                      void *stream);
+/* insc_grid_insert for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid it).  No counterpart in the reference.  Same result
+ * as insc_grid_insert, with two limits: at most 16384 points per call (INSC_ERR_CAPACITY beyond),
+ * and the grid is never grown - the host-side bound "sites so far + P" must fit the capacity
+ * (INSC_ERR_CAPACITY otherwise; reserve beforehand).  It calls no hipMalloc / hipFree: the per-row
+ * scratch is a 64 KB array in the library's device image, one per GPU, shared by all calls on that
+ * GPU - calls that overlap on one GPU (different streams or threads) race; calls on one stream do
+ * not.  Nothing in the scratch has to survive or be cleared between calls.  With h_n_sites == NULL
+ * the call only enqueues two kernels; with it, it copies the count back and synchronises. */
+int insc_grid_insert_noalloc(insc_grid *g, const int32_t *d_coords4, int64_t P, int32_t *d_site_of_point,
+                             int64_t *h_n_sites, void *stream);
 /* d_site[q] = site id of coordinate q, or -1.  Replaces Multival retrieve +
  * _dMultivalHashGetValue (CUDPPWrapper.cu:144-160), whose miss value is 0xFFFFFFFF. */
 int insc_grid_query(const insc_grid *g, const int32_t *d_coords4, int64_t Q, int32_t *d_site, void *stream);

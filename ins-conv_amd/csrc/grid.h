@@ -63,6 +63,9 @@ int order_append_new_sites_sorted_batch(const insc_grid *const *grids, const int
 int order_append_new_sites_by_offset_batch(const insc_grid *const *grids, const int32_t *const *d_offset,
                                            const int32_t *const *d_pos_in_order, int32_t *const *d_order,
                                            int32_t *const *d_pos, int n, int64_t n_new_upper, hipStream_t s);
+// looks up, for the current device, the address of the scratch array of insc_grid_insert_noalloc
+// (called by insc_init; the entry point does it itself on a device that was never initialised)
+int grid_noalloc_setup();
 // most sites the two sorted appends put in order (more keep their arrival order)
 int64_t order_sorted_max();
 // device pointer to the site count before the most recent insert

@@ -7,6 +7,8 @@
 //
 // Numbering: a site's id is its rank among first occurrences in the inserted list, offset by
 // the count before the call - deterministic and append-only.
+#include <mutex>
+
 #include "common.h"
 #include "grid.h"
 
@@ -581,6 +583,40 @@ int order_append_new_sites(const insc_grid *g, int32_t *d_order, int32_t *d_pos,
 
 int64_t order_sorted_max() { return SORT_NEW_MAX; }
 
+// ---- insert without allocation -------------------------------------------------------------
+// Scratch of insc_grid_insert_noalloc: the slot every row of the call claimed (what the grid's own,
+// growable slot_of_point buffer holds for insc_grid_insert).  One copy of the array lives on every
+// device the library's code is loaded on, at its own address; the name below is only the host's
+// handle for hipGetSymbolAddress and is never passed to a kernel.  Every entry a call reads was
+// written by the same call's first kernel, so nothing has to be cleared between calls.
+constexpr int NOALLOC_MAX_POINTS = FINISH_SMALL_MAX;
+static __device__ __align__(256) int32_t scratch[NOALLOC_MAX_POINTS];
+constexpr int MAX_DEVICES = 64;
+static int32_t *g_scratch_ptr[MAX_DEVICES] = {nullptr};
+static std::mutex g_scratch_mu;
+
+// address of `scratch` on the current device, looked up once per device
+static int scratch_on_current_device(int32_t **out) {
+  int dev = -1;
+  INSC_HIP(hipGetDevice(&dev));
+  INSC_REQUIRE(dev >= 0 && dev < MAX_DEVICES, INSC_ERR_STATE, "device %d is beyond the %d this library keeps scratch for",
+               dev, MAX_DEVICES);
+  std::lock_guard<std::mutex> lk(g_scratch_mu);
+  if (!g_scratch_ptr[dev]) {
+    int32_t *p = nullptr;
+    INSC_HIP(hipGetSymbolAddress((void **)&p, HIP_SYMBOL(scratch)));
+    INSC_REQUIRE(p, INSC_ERR_HIP, "hipGetSymbolAddress gave no address for the insert scratch on device %d", dev);
+    g_scratch_ptr[dev] = p;
+  }
+  *out = g_scratch_ptr[dev];
+  return INSC_OK;
+}
+
+int grid_noalloc_setup() {
+  int32_t *p;
+  return scratch_on_current_device(&p);
+}
+
 int ssc3_new_sites_batch(const insc_grid *const *grids, int32_t *const *d_nbr, int n, int64_t n_new_upper,
                          hipStream_t s) {
   if (n <= 0 || n_new_upper <= 0) return INSC_OK;
@@ -751,6 +787,45 @@ int insc_grid_insert(insc_grid *g, const int32_t *d_coords4, int64_t P, int32_t 
   }
   if (h_n_sites) {
     int rc = grid_sync_errors(g, s, "insc_grid_insert");
+    if (rc) return rc;
+    *h_n_sites = g->n_exact;
+  }
+  return INSC_OK;
+}
+
+int insc_grid_insert_noalloc(insc_grid *g, const int32_t *d_coords4, int64_t P, int32_t *d_site_of_point,
+                             int64_t *h_n_sites, void *stream) {
+  INSC_REQUIRE(g, INSC_ERR_ARG, "insc_grid_insert_noalloc: grid is null");
+  INSC_REQUIRE(P >= 0, INSC_ERR_ARG, "insc_grid_insert_noalloc: P=%lld is negative", (long long)P);
+  INSC_REQUIRE(P <= NOALLOC_MAX_POINTS, INSC_ERR_CAPACITY,
+               "insc_grid_insert_noalloc: %lld points exceed the %d one call takes (split the list, or use "
+               "insc_grid_insert, which may allocate)",
+               (long long)P, NOALLOC_MAX_POINTS);
+  INSC_REQUIRE(P == 0 || (d_coords4 && d_site_of_point), INSC_ERR_ARG, "insc_grid_insert_noalloc: null pointer");
+  hipStream_t s = (hipStream_t)stream;
+  if (P > 0) {
+    int dev = -1;
+    INSC_HIP(hipGetDevice(&dev));
+    INSC_REQUIRE(dev == g->device, INSC_ERR_STATE, "insc_grid_insert_noalloc: the grid lives on device %d, current is %d",
+                 g->device, dev);
+    int32_t *slot_of_point = nullptr;
+    int rc = scratch_on_current_device(&slot_of_point);
+    if (rc) return rc;
+    // this entry point never grows the grid: the host-side bound (every row a new site) must fit
+    INSC_REQUIRE(g->n_upper + P <= g->capacity_sites, INSC_ERR_CAPACITY,
+                 "insc_grid_insert_noalloc: up to %lld sites + %lld points may exceed the capacity of %lld; call "
+                 "insc_grid_reserve first (or insc_grid_size to tighten the bound after inserts with repeats)",
+                 (long long)g->n_upper, (long long)P, (long long)g->capacity_sites);
+    hipLaunchKernelGGL(grid_claim_kernel, dim3(grid_for(P, 256)), dim3(256), 0, s, g->table, g->n_slots - 1, d_coords4,
+                       P, slot_of_point, g->d_err);
+    hipLaunchKernelGGL(grid_finish_small_kernel, dim3(1), dim3(1024), 0, s, g->table, d_coords4, slot_of_point, (int)P,
+                       g->d_n, g->coords, g->capacity_sites, g->d_err, d_site_of_point);
+    INSC_LAUNCH_CHECK();
+    g->n_upper += P;
+    g->n_exact = -1;
+  }
+  if (h_n_sites) {
+    int rc = grid_sync_errors(g, s, "insc_grid_insert_noalloc");
     if (rc) return rc;
     *h_n_sites = g->n_exact;
   }

@@ -7,6 +7,7 @@
 #include <utility>
 
 #include "common.h"
+#include "grid.h"
 
 namespace insc {
 
@@ -127,7 +128,7 @@ int insc_init(int device) {
   INSC_REQUIRE(strncmp(prop.gcnArchName, "gfx950", 6) == 0, INSC_ERR_STATE,
                "insc_init: device %d is %s; this library holds gfx950 code only", device, prop.gcnArchName);
   g_device = device;
-  return INSC_OK;
+  return grid_noalloc_setup();
 }
 
 const char *insc_last_error(void) { return g_err; }
