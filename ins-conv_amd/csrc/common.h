@@ -92,7 +92,11 @@ struct TilePlanBatch {
   TilePlanJob job[16];
   int n;
 };
+// (a job with nbr == null keeps its map and only has its schedule rebuilt)
 int build_tile_plans(const TilePlanBatch &b, hipStream_t s);
+// the columns of the sites added by the last insert (positions from d_n[1] on), for plans whose
+// older part is up to date; a job with map == null is skipped
+int tile_plan_append_batch(const TilePlanBatch &b, int64_t n_new_upper, hipStream_t s);
 
 // in_rows: rows of the input matrix (bounds the gather).  out may be null when ep.out2 is set.
 // latency != 0 picks the launch shape for small row counts (residual frames).

@@ -1393,7 +1393,45 @@ __global__ __launch_bounds__(256) void tile_plan_kernel(const int32_t *__restric
 // the plans of several maps (the scales of a network) in one launch: blockIdx.y picks the map
 __global__ __launch_bounds__(256) void tile_plan_batch_kernel(TilePlanBatch b) {
   const TilePlanJob &j = b.job[blockIdx.y];
+  if (!j.nbr) return;  // this plan is up to date: only its schedule is wanted
   tile_plan_body(j.nbr, j.order, j.d_n, j.n_rows, j.ld, j.map, j.tmask);
+}
+
+// The columns of the sites added by the last insert, appended to a plan that holds the older
+// sites already: positions [first, end of the last tile) of every offset row (first = site count
+// before the insert; positions follow the processing order, in which new sites come last).  The
+// offset masks of the tiles they open have been cleared beforehand; the mask of a tile is the OR
+// over its rows.  One thread per (position, offset).
+__global__ __launch_bounds__(256) void tile_plan_append_batch_kernel(TilePlanBatch b) {
+  const TilePlanJob &j = b.job[blockIdx.y];
+  if (!j.map) return;
+  const int64_t first = j.d_n[1], n = j.d_n[0];
+  // one wavefront per tile, from the tile that holds position `first` on; lane = (row of the tile,
+  // parity of the offset)
+  const int lane = threadIdx.x & 63, r = lane & 31, h = lane >> 5;
+  const int64_t tile = first / TILE_M + (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (tile * TILE_M >= n) return;
+  const int64_t p = tile * TILE_M + r;
+  const bool mine = p >= first;  // (older positions of the first tile keep their entries)
+  const int site = (mine && p < n) ? (j.order ? j.order[p] : (int)p) : -1;
+  unsigned m = 0;
+  for (int k = h; k < 28; k += 2) {
+    const int v = (site >= 0 && k < 27) ? j.nbr[(int64_t)site * 27 + k] : -1;
+    if (mine && k < 27) j.map[(int64_t)k * j.ld + p] = v;
+    const unsigned long long bal = __ballot(v >= 0);
+    if ((unsigned)bal) m |= 1u << k;
+    if ((unsigned)(bal >> 32)) m |= 1u << (k + 1);
+  }
+  if (lane == 0 && m) atomicOr(&j.tmask[tile], m);
+}
+
+int tile_plan_append_batch(const TilePlanBatch &b, int64_t n_new_upper, hipStream_t s) {
+  if (b.n <= 0 || n_new_upper <= 0) return INSC_OK;
+  // (the new sites touch at most n_new_upper / 32 + 2 tiles; four tiles per block)
+  hipLaunchKernelGGL(tile_plan_append_batch_kernel, dim3(grid_for(n_new_upper / TILE_M + 2, 4), (unsigned)b.n), dim3(256),
+                     0, s, b);
+  INSC_LAUNCH_CHECK();
+  return INSC_OK;
 }
 
 // sched = the tiles by falling number of active offsets (a counting sort over the 28 classes by one
@@ -1462,11 +1500,11 @@ int build_tile_plans(const TilePlanBatch &b, hipStream_t s) {
   int64_t most = 0;
   bool any_sched = false;
   for (int i = 0; i < b.n; i++) {
-    most = std::max(most, cdiv(b.job[i].n_rows, TILE_M) * TILE_M);
+    if (b.job[i].nbr) most = std::max(most, cdiv(b.job[i].n_rows, TILE_M) * TILE_M);
     any_sched = any_sched || b.job[i].sched;
   }
-  if (b.n <= 0 || most <= 0) return INSC_OK;
-  hipLaunchKernelGGL(tile_plan_batch_kernel, dim3(grid_for(most, 256), (unsigned)b.n), dim3(256), 0, s, b);
+  if (b.n <= 0) return INSC_OK;
+  if (most > 0) hipLaunchKernelGGL(tile_plan_batch_kernel, dim3(grid_for(most, 256), (unsigned)b.n), dim3(256), 0, s, b);
   if (any_sched) hipLaunchKernelGGL(tile_sched_batch_kernel, dim3((unsigned)b.n), dim3(1024), 0, s, b);
   INSC_LAUNCH_CHECK();
   return INSC_OK;

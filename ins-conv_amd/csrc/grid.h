@@ -55,17 +55,46 @@ int order_append_new_sites_by_offset(const insc_grid *g, const int32_t *d_offset
                                      int32_t *d_order, int32_t *d_pos, int64_t n_new_upper, hipStream_t s);
 // the three per-grid steps above for several grids (the scales of a network, at most 16) in one
 // launch each; every grid acts on the sites of its own most recent insert
+// plans (nullable; per grid, plan null = none): tile plans to keep up to date with the map - the
+// entries of older sites that gain a neighbour are patched and the offset masks of the tiles the new
+// sites open are cleared; the new sites' own columns follow with tile_plan_append_batch
+struct PlanRef {
+  int32_t *plan;
+  uint32_t *tmask;
+  const int32_t *pos;
+  int64_t ld;
+};
 int ssc3_new_sites_batch(const insc_grid *const *grids, int32_t *const *d_nbr, int n, int64_t n_new_upper,
-                         hipStream_t s);
+                         hipStream_t s, const PlanRef *plans = nullptr);
 int order_append_new_sites_sorted_batch(const insc_grid *const *grids, const int32_t *const *d_nbr,
                                         int32_t *const *d_order, int32_t *const *d_pos, int n, int64_t n_new_upper,
                                         hipStream_t s);
 int order_append_new_sites_by_offset_batch(const insc_grid *const *grids, const int32_t *const *d_offset,
                                            const int32_t *const *d_pos_in_order, int32_t *const *d_order,
                                            int32_t *const *d_pos, int n, int64_t n_new_upper, hipStream_t s);
+// The inserts of a whole frame in one launch (at most frame_insert_max_points() points): the points
+// go into lv[0].grid, the sites that adds (halved) into lv[1].grid and so on, with the parent /
+// offset / child link of every scale to the next coarser one filled in for the new sites.  Every
+// grid then reports the sites of this insert as its newest ([d_n[1], d_n[0])).  d_coords: int32
+// [P, cols] (cols 3 or 4).  If any coordinate is out of range nothing is inserted anywhere, *d_bad
+// = frame, and every row of d_sop is -1.  h_counts (nullable, host memory the device can write):
+// receives per scale the site count and error flags, then at [2 * n_levels] `frame` for a dropped frame else 0.
+struct FrameInsertLevel {
+  insc_grid *grid;
+  int32_t *parent, *offset, *child;
+};
+int frame_insert_levels(const FrameInsertLevel *lv, int n_levels, const int32_t *d_coords, int cols, int64_t P,
+                        int32_t *d_bad, int32_t frame, int32_t *d_sop, int32_t *h_counts, hipStream_t s);
+int64_t frame_insert_max_points();
 // looks up, for the current device, the address of the scratch array of insc_grid_insert_noalloc
 // (called by insc_init; the entry point does it itself on a device that was never initialised)
 int grid_noalloc_setup();
+// both appends for several grids in ONE launch (d_offset[i] null: the grid has no coarser scale above
+// it and only gets the first order)
+int order_append_new_sites_both_batch(const insc_grid *const *grids, const int32_t *const *d_nbr,
+                                      const int32_t *const *d_offset, int32_t *const *d_order, int32_t *const *d_pos,
+                                      int32_t *const *d_bo_order, int32_t *const *d_bo_pos, int n, int64_t n_new_upper,
+                                      hipStream_t s);
 // most sites the two sorted appends put in order (more keep their arrival order)
 int64_t order_sorted_max();
 // device pointer to the site count before the most recent insert

@@ -283,11 +283,22 @@ __global__ void down2_child_kernel(const int32_t *__restrict__ parent, const int
 }
 
 // ---- variants over the sites added by the last insert, [d_n[1], d_n[0]) --------------------
+// With a tile plan (plan, tmask, pos, ld: the map transposed into processing order, see
+// build_tile_plan) the plan is kept up to date as well: the entry of every older site that gains a
+// neighbour is patched, and the offset masks of the tiles the new sites will open are cleared (their
+// columns follow once the new sites have their positions, tile_plan_append).
 __device__ __forceinline__ void ssc3_nbr_new_body(const Slot *__restrict__ table, int64_t mask,
                                                   const int32_t *__restrict__ site_coords,
-                                                  const int32_t *__restrict__ d_n, int32_t *__restrict__ nbr) {
+                                                  const int32_t *__restrict__ d_n, int32_t *__restrict__ nbr,
+                                                  int32_t *__restrict__ plan = nullptr,
+                                                  uint32_t *__restrict__ tmask = nullptr,
+                                                  const int32_t *__restrict__ pos = nullptr, int64_t ld = 0) {
   const int64_t first = d_n[1], n = (int64_t)d_n[0] - first;
   int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (plan) {
+    const int64_t tile = (first + 31) / 32 + t;
+    if (tile < (first + n + 31) / 32) tmask[tile] = 0;
+  }
   if (t >= n * 27) return;
   int64_t o = first + t / 27;
   int k = (int)(t % 27);
@@ -299,7 +310,14 @@ __device__ __forceinline__ void ssc3_nbr_new_body(const Slot *__restrict__ table
   else if (coord_ok(x, y, z, c.w))
     r = grid_find(table, mask, pack_key(x, y, z, c.w));
   nbr[o * 27 + k] = r;
-  if (r >= 0 && r < first) nbr[(int64_t)r * 27 + (26 - k)] = (int)o;
+  if (r >= 0 && r < first) {
+    nbr[(int64_t)r * 27 + (26 - k)] = (int)o;
+    if (plan) {
+      const int pr = pos[r];
+      plan[(int64_t)(26 - k) * ld + pr] = (int)o;
+      atomicOr(&tmask[pr >> 5], 1u << (26 - k));
+    }
+  }
 }
 __global__ void ssc3_nbr_new_kernel(const Slot *__restrict__ table, int64_t mask,
                                     const int32_t *__restrict__ site_coords, const int32_t *__restrict__ d_n,
@@ -312,13 +330,17 @@ struct NewSitesJob {
   int64_t mask;
   const int32_t *coords, *d_n;
   int32_t *nbr;
+  int32_t *plan;  // optional tile plan to keep up to date
+  uint32_t *tmask;
+  const int32_t *pos;
+  int64_t ld;
 };
 struct NewSitesBatch {
   NewSitesJob job[16];
 };
 __global__ void ssc3_nbr_new_batch_kernel(NewSitesBatch b) {
   const NewSitesJob &j = b.job[blockIdx.y];
-  ssc3_nbr_new_body(j.table, j.mask, j.coords, j.d_n, j.nbr);
+  ssc3_nbr_new_body(j.table, j.mask, j.coords, j.d_n, j.nbr, j.plan, j.tmask, j.pos, j.ld);
 }
 
 __global__ void down2_coords_new_kernel(const int32_t *__restrict__ fine_coords, const int32_t *__restrict__ d_n,
@@ -495,10 +517,9 @@ __device__ __forceinline__ void order_append_sorted_body(const int32_t *__restri
                                                          const int32_t *__restrict__ nbr,
                                                          const int32_t *__restrict__ offset,
                                                          const int32_t *__restrict__ aux, int32_t *__restrict__ order,
-                                                         int32_t *__restrict__ pos) {
-  // one 64-bit word per new site: sort key in the upper 51 bits, index of the site among the
-  // new ones in the lower 13
-  __shared__ uint64_t key[SORT_NEW_MAX];
+                                                         int32_t *__restrict__ pos, uint64_t *key) {
+  // key: SORT_NEW_MAX 64-bit words of LDS, one per new site: sort key in the upper 51 bits, index of
+  // the site among the new ones in the lower 13
   const int first = d_n[1], n = d_n[0] - first;
   const int tid = threadIdx.x;
   if (n <= 0) return;
@@ -558,7 +579,8 @@ __global__ __launch_bounds__(1024) void order_append_sorted_kernel(const int32_t
                                                                    const int32_t *__restrict__ aux,
                                                                    int32_t *__restrict__ order,
                                                                    int32_t *__restrict__ pos) {
-  order_append_sorted_body<MODE>(d_n, coords, nbr, offset, aux, order, pos);
+  __shared__ uint64_t key[SORT_NEW_MAX];
+  order_append_sorted_body<MODE>(d_n, coords, nbr, offset, aux, order, pos, key);
 }
 // one workgroup per grid
 struct OrderJob {
@@ -570,8 +592,27 @@ struct OrderBatch {
 };
 template <int MODE>
 __global__ __launch_bounds__(1024) void order_append_sorted_batch_kernel(OrderBatch b) {
+  __shared__ uint64_t key[SORT_NEW_MAX];
   const OrderJob &j = b.job[blockIdx.x];
-  order_append_sorted_body<MODE>(j.d_n, j.coords, j.nbr, j.offset, j.aux, j.order, j.pos);
+  order_append_sorted_body<MODE>(j.d_n, j.coords, j.nbr, j.offset, j.aux, j.order, j.pos, key);
+}
+// both orders of a scale by one workgroup: the processing order of the 3^3 layers, then - where the
+// scale has a coarser one above it - the order grouped by the position inside the parent cell, which
+// sorts by the position in the first
+struct OrderBothJob {
+  const int32_t *d_n, *coords, *nbr, *offset;  // offset null: no second order
+  int32_t *order, *pos, *bo_order, *bo_pos;
+};
+struct OrderBothBatch {
+  OrderBothJob job[16];
+};
+__global__ __launch_bounds__(1024) void order_append_both_batch_kernel(OrderBothBatch b) {
+  __shared__ uint64_t key[SORT_NEW_MAX];
+  const OrderBothJob &j = b.job[blockIdx.x];
+  order_append_sorted_body<0>(j.d_n, j.coords, j.nbr, nullptr, nullptr, j.order, j.pos, key);
+  if (!j.offset) return;
+  __syncthreads();  // the positions written above are read below, and the keys are reused
+  order_append_sorted_body<1>(j.d_n, nullptr, nullptr, j.offset, j.pos, j.bo_order, j.bo_pos, key);
 }
 
 int order_append_new_sites(const insc_grid *g, int32_t *d_order, int32_t *d_pos, int64_t n_new_upper, hipStream_t s) {
@@ -582,6 +623,237 @@ int order_append_new_sites(const insc_grid *g, int32_t *d_order, int32_t *d_pos,
 }
 
 int64_t order_sorted_max() { return SORT_NEW_MAX; }
+
+// ---- the inserts of a whole frame, all scales at once ----------------------------------------
+// The reference inserts scale by scale: the sites a frame adds at one scale are halved and inserted
+// at the next coarser one, a chain in which every step waits for the ids of the step before.  The
+// chain is not needed: a site that is new at scale l has only new sites below it, so the order in
+// which that chain numbers the new sites of scale l - first appearance among the new sites of scale
+// l - 1 in id order - is the order of the smallest ROW of the frame's point list that falls into
+// each new cell.  So every scale takes the frame's points themselves (coordinates >> l) and ranks
+// its new cells by their smallest row, all scales at the same time, in three launches for up to
+// FINISH_SMALL_MAX points: claim (one thread per row and scale; a row that finds its cell already
+// numbered is done - at the coarse scales that is nearly every row), finish (one workgroup per
+// scale ranks the winners in row order and hands out the ids), link (parent / offset / child
+// between the scales).  A frame is all or nothing: if some coordinate is out of range, finish takes
+// the frame's claims out of the tables again (they sit in slots that were empty before, so the
+// tables are then exactly what they were) and nothing is numbered.
+// Values that other rows of the frame may have changed are read past the L1 (atomic loads): the
+// claims are atomics performed in L2.
+struct FrameLevelDev {
+  Slot *table;
+  int64_t mask, capacity;
+  int32_t *coords, *d_n, *d_err;
+  int32_t *parent, *offset, *child;  // link to the next coarser scale (null at the coarsest)
+};
+struct FrameInsertArgs {
+  FrameLevelDev lv[16];
+  int n_levels;
+};
+__device__ __forceinline__ int table_val(const Slot *table, int64_t s) {
+  return __hip_atomic_load(&table[s].val, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+constexpr uint32_t REC_SITE = 0x80000000u;  // rec = REC_SITE | id: the cell was numbered before this frame
+constexpr uint32_t REC_NONE = 0xFFFFFFFFu;  // no slot: bad coordinate, or the table is full
+__device__ __forceinline__ int4 frame_point(const int32_t *__restrict__ coords_in, int cols, int p, int l) {
+  const int32_t *c = coords_in + (int64_t)p * cols;
+  return make_int4(c[0] >> l, c[1] >> l, c[2] >> l, cols > 3 ? c[3] : 0);
+}
+// rec[l * P + p]: what row p found at scale l - REC_SITE | id, the slot it claimed, or REC_NONE
+__global__ __launch_bounds__(256) void frame_claim_kernel(FrameInsertArgs a, const int32_t *__restrict__ coords_in,
+                                                          int cols, int P, int32_t *__restrict__ bad, int32_t frame,
+                                                          uint32_t *__restrict__ rec) {
+  const int l = blockIdx.y;
+  const FrameLevelDev &L = a.lv[l];
+  const int p = blockIdx.x * 256 + threadIdx.x;
+  if (p >= P) return;
+  const int32_t *c0 = coords_in + (int64_t)p * cols;
+  if (!coord_ok(c0[0], c0[1], c0[2], cols > 3 ? c0[3] : 0)) {
+    if (l == 0) bad[0] = frame;
+    rec[(int64_t)l * P + p] = REC_NONE;
+    return;
+  }
+  const int4 c = frame_point(coords_in, cols, p, l);
+  const uint64_t key = pack_key(c.x, c.y, c.z, c.w);
+  int64_t s = home_slot(key, L.mask);
+  uint32_t r = REC_NONE;
+  for (int64_t probe = 0; probe <= L.mask && probe < MAX_PROBES; probe++) {
+    const int4 raw = *reinterpret_cast<const int4 *>(&L.table[s]);  // key (two words), val, pad
+    unsigned long long k = ((unsigned long long)(unsigned)raw.y << 32) | (unsigned)raw.x;
+    if (k == key && raw.z >= 0 && raw.z < VAL_PENDING) {  // numbered before this frame
+      r = REC_SITE | (uint32_t)raw.z;
+      break;
+    }
+    if (k == INSC_EMPTY_KEY) k = atomicCAS(&L.table[s].key, INSC_EMPTY_KEY, (unsigned long long)key);
+    if (k == INSC_EMPTY_KEY || k == key) {
+      r = (uint32_t)s;
+      atomicMin(&L.table[s].val, VAL_PENDING + p);
+      break;
+    }
+    s = (s + 1) & L.mask;
+  }
+  if (r == REC_NONE) atomicOr(L.d_err, 2);
+  rec[(int64_t)l * P + p] = r;
+}
+
+// site[l * P + p] = site of row p at scale l
+__global__ __launch_bounds__(1024) void frame_finish_kernel(FrameInsertArgs a, const int32_t *__restrict__ coords_in,
+                                                            int cols, int P, const int32_t *__restrict__ bad,
+                                                            int32_t frame, int32_t *__restrict__ sop,
+                                                            int32_t *__restrict__ site, const uint32_t *__restrict__ rec,
+                                                            int32_t *h_counts) {
+  __shared__ int wave_total[16];
+  const int l = blockIdx.x;
+  const FrameLevelDev &L = a.lv[l];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int per = (P + 1023) / 1024, p0 = tid * per;
+  const int n_before = L.d_n[0];
+  site += (int64_t)l * P;
+  rec += (int64_t)l * P;
+  uint32_t rr[16];
+#pragma unroll
+  for (int j = 0; j < 16; j++) rr[j] = (j < per && p0 + j < P) ? rec[p0 + j] : REC_NONE;
+  if (bad[0] == frame) {
+    // the frame is dropped: its claims leave the table, no row gets a site
+#pragma unroll
+    for (int j = 0; j < 16; j++) {
+      if (j >= per || p0 + j >= P) continue;
+      if (rr[j] != REC_NONE && !(rr[j] & REC_SITE)) {
+        __hip_atomic_store(&L.table[rr[j]].val, VAL_UNSET, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(&L.table[rr[j]].key, INSC_EMPTY_KEY, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+      site[p0 + j] = -1;
+      if (l == 0) sop[p0 + j] = -1;
+    }
+    if (tid == 0) {
+      L.d_n[1] = n_before;
+      if (h_counts) {
+        h_counts[2 * l] = n_before;
+        h_counts[2 * l + 1] = 0;
+        if (l == 0) h_counts[2 * a.n_levels] = frame;
+      }
+    }
+    return;
+  }
+  // winners, ranked in row order
+  int tv[16];
+#pragma unroll
+  for (int j = 0; j < 16; j++) tv[j] = (rr[j] != REC_NONE && !(rr[j] & REC_SITE)) ? table_val(L.table, (int64_t)rr[j]) : -1;
+  unsigned win = 0;
+  int cnt = 0;
+#pragma unroll
+  for (int j = 0; j < 16; j++) {
+    if (tv[j] == VAL_PENDING + p0 + j) {
+      win |= 1u << j;
+      cnt++;
+    }
+  }
+  int incl = cnt;
+  for (int d = 1; d < 64; d <<= 1) {
+    const int v = __shfl_up(incl, d, 64);
+    if (lane >= d) incl += v;
+  }
+  if (lane == 63) wave_total[wave] = incl;
+  __syncthreads();
+  int base = n_before + incl - cnt, total = 0;
+  for (int w = 0; w < 16; w++) {
+    if (w < wave) base += wave_total[w];
+    total += wave_total[w];
+  }
+  // winners publish their id and record the new site
+#pragma unroll
+  for (int j = 0; j < 16; j++) {
+    if (!((win >> j) & 1u)) continue;
+    const int id = base++;
+    if (id >= L.capacity) {
+      atomicOr(L.d_err, 2);
+      continue;
+    }
+    const int4 c = frame_point(coords_in, cols, p0 + j, l);
+    __hip_atomic_store(&L.table[rr[j]].val, id, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    reinterpret_cast<int4 *>(L.coords)[id] = c;
+    if (L.offset) L.offset[id] = (c.x & 1) * 4 + (c.y & 1) * 2 + (c.z & 1);
+  }
+  __syncthreads();
+  // every row learns its site
+#pragma unroll
+  for (int j = 0; j < 16; j++) tv[j] = (rr[j] != REC_NONE && !(rr[j] & REC_SITE)) ? table_val(L.table, (int64_t)rr[j]) : -1;
+#pragma unroll
+  for (int j = 0; j < 16; j++) {
+    const int p = p0 + j;
+    if (j >= per || p >= P) continue;
+    const int v = rr[j] == REC_NONE ? -1 : (rr[j] & REC_SITE) ? (int)(rr[j] & ~REC_SITE) : tv[j];
+    const int st = (v >= 0 && v < VAL_PENDING) ? v : -1;
+    site[p] = st;
+    if (l == 0) sop[p] = st;
+  }
+  if (total > L.capacity - n_before) total = (int)(L.capacity - n_before);  // (the error flag is up)
+  if (tid == 0) {
+    L.d_n[1] = n_before;
+    L.d_n[0] = n_before + total;
+    if (h_counts) {
+      h_counts[2 * l] = n_before + total;
+      h_counts[2 * l + 1] = __hip_atomic_load(L.d_err, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (l == 0) h_counts[2 * a.n_levels] = 0;
+    }
+  }
+}
+
+// the links of the new sites of scale blockIdx.y to the scale above: every row that fell into a new
+// cell writes that cell's parent (rows of one cell write the same values)
+__global__ void frame_link_kernel(FrameInsertArgs a, int P, const int32_t *__restrict__ site) {
+  const int l = blockIdx.y;
+  const FrameLevelDev &F = a.lv[l];
+  const int p = blockIdx.x * blockDim.x + threadIdx.x;
+  if (p >= P) return;
+  const int i = site[(int64_t)l * P + p];
+  if (i < F.d_n[1]) return;  // not a site of this frame (or no site at all)
+  const int par = site[(int64_t)(l + 1) * P + p];
+  F.parent[i] = par;
+  if (par >= 0 && F.child) F.child[(int64_t)par * 8 + F.offset[i]] = i;
+}
+
+int frame_insert_levels(const FrameInsertLevel *lv, int n_levels, const int32_t *d_coords, int cols, int64_t P,
+                        int32_t *d_bad, int32_t frame, int32_t *d_sop, int32_t *h_counts, hipStream_t s) {
+  if (P <= 0) return INSC_OK;
+  if (n_levels < 1 || n_levels > 16 || P > FINISH_SMALL_MAX) {
+    set_error("frame_insert_levels: %d scales, %lld points (at most 16 scales, %d points)", n_levels, (long long)P,
+              FINISH_SMALL_MAX);
+    return INSC_ERR_ARG;
+  }
+  FrameInsertArgs a;
+  a.n_levels = n_levels;
+  for (int l = 0; l < n_levels; l++) {
+    insc_grid *g = lv[l].grid;
+    if (g->n_upper + P > g->capacity_sites) {
+      set_error("frame_insert_levels: %lld sites + %lld points exceed the capacity %lld of scale %d", (long long)g->n_upper,
+                (long long)P, (long long)g->capacity_sites, l);
+      return INSC_ERR_CAPACITY;
+    }
+    a.lv[l] = FrameLevelDev{g->table, g->n_slots - 1, g->capacity_sites, g->coords, g->d_n, g->d_err,
+                            lv[l].parent, lv[l].offset, lv[l].child};
+  }
+  void *ws;
+  int rc = workspace(WS_API, s, (size_t)P * n_levels * 2 * sizeof(int32_t) + 256, &ws);
+  if (rc) return rc;
+  int32_t *site = (int32_t *)ws;
+  uint32_t *rec = (uint32_t *)(site + P * n_levels);
+  hipLaunchKernelGGL(frame_claim_kernel, dim3(grid_for(P, 256), (unsigned)n_levels), dim3(256), 0, s, a, d_coords, cols,
+                     (int)P, d_bad, frame, rec);
+  hipLaunchKernelGGL(frame_finish_kernel, dim3((unsigned)n_levels), dim3(1024), 0, s, a, d_coords, cols, (int)P,
+                     (const int32_t *)d_bad, frame, d_sop, site, (const uint32_t *)rec, h_counts);
+  if (n_levels > 1)
+    hipLaunchKernelGGL(frame_link_kernel, dim3(grid_for(P, 256), (unsigned)(n_levels - 1)), dim3(256), 0, s, a, (int)P,
+                       (const int32_t *)site);
+  INSC_LAUNCH_CHECK();
+  for (int l = 0; l < n_levels; l++) {
+    lv[l].grid->n_upper += P;
+    lv[l].grid->n_exact = -1;
+  }
+  return INSC_OK;
+}
+
+int64_t frame_insert_max_points() { return FINISH_SMALL_MAX; }
 
 // ---- insert without allocation -------------------------------------------------------------
 // Scratch of insc_grid_insert_noalloc: the slot every row of the call claimed (what the grid's own,
@@ -618,14 +890,22 @@ int grid_noalloc_setup() {
 }
 
 int ssc3_new_sites_batch(const insc_grid *const *grids, int32_t *const *d_nbr, int n, int64_t n_new_upper,
-                         hipStream_t s) {
+                         hipStream_t s, const PlanRef *plans) {
   if (n <= 0 || n_new_upper <= 0) return INSC_OK;
   if (n > 16) {
     set_error("ssc3_new_sites_batch: at most 16 grids");
     return INSC_ERR_ARG;
   }
   NewSitesBatch b;
-  for (int i = 0; i < n; i++) b.job[i] = NewSitesJob{grids[i]->table, grids[i]->n_slots - 1, grids[i]->coords, grids[i]->d_n, d_nbr[i]};
+  for (int i = 0; i < n; i++) {
+    b.job[i] = NewSitesJob{grids[i]->table, grids[i]->n_slots - 1, grids[i]->coords, grids[i]->d_n, d_nbr[i], nullptr, nullptr, nullptr, 0};
+    if (plans && plans[i].plan) {
+      b.job[i].plan = plans[i].plan;
+      b.job[i].tmask = plans[i].tmask;
+      b.job[i].pos = plans[i].pos;
+      b.job[i].ld = plans[i].ld;
+    }
+  }
   hipLaunchKernelGGL(ssc3_nbr_new_batch_kernel, dim3(grid_for(n_new_upper * 27, 256, 1ll << 30), (unsigned)n), dim3(256),
                      0, s, b);
   INSC_LAUNCH_CHECK();
@@ -658,6 +938,23 @@ int order_append_new_sites_by_offset_batch(const insc_grid *const *grids, const 
   OrderBatch b;
   for (int i = 0; i < n; i++) b.job[i] = OrderJob{grids[i]->d_n, nullptr, nullptr, d_offset[i], d_pos_in_order[i], d_order[i], d_pos[i]};
   hipLaunchKernelGGL(order_append_sorted_batch_kernel<1>, dim3((unsigned)n), dim3(1024), 0, s, b);
+  INSC_LAUNCH_CHECK();
+  return INSC_OK;
+}
+
+int order_append_new_sites_both_batch(const insc_grid *const *grids, const int32_t *const *d_nbr,
+                                      const int32_t *const *d_offset, int32_t *const *d_order, int32_t *const *d_pos,
+                                      int32_t *const *d_bo_order, int32_t *const *d_bo_pos, int n, int64_t n_new_upper,
+                                      hipStream_t s) {
+  if (n <= 0 || n_new_upper <= 0) return INSC_OK;
+  if (n > 16) {
+    set_error("order_append_new_sites_both_batch: at most 16 grids");
+    return INSC_ERR_ARG;
+  }
+  OrderBothBatch b;
+  for (int i = 0; i < n; i++)
+    b.job[i] = OrderBothJob{grids[i]->d_n, grids[i]->coords, d_nbr[i], d_offset[i], d_order[i], d_pos[i], d_bo_order[i], d_bo_pos[i]};
+  hipLaunchKernelGGL(order_append_both_batch_kernel, dim3((unsigned)n), dim3(1024), 0, s, b);
   INSC_LAUNCH_CHECK();
   return INSC_OK;
 }

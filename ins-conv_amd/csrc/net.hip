@@ -42,6 +42,7 @@ struct Level {
   int64_t n = 0;                // exact count after the last completed frame
   int64_t n_upper = 0;          // bound valid during the frame being enqueued
   int64_t new_upper = 0;        // bound on sites added in this frame
+  bool plan_valid = false;      // the tile plan holds every site of the last completed frame
 };
 
 struct Buffer {
@@ -125,6 +126,7 @@ struct insc_net {
   bool profiling = false;
   hipEvent_t ev[5] = {nullptr, nullptr, nullptr, nullptr, nullptr};
   bool ev_valid = false;
+  hipEvent_t ev_counts = nullptr;  // the frame's inserts are done: the site counts lie in h_counts
 };
 
 namespace insc {
@@ -359,7 +361,8 @@ static int level_reserve(insc_net *net, int l, int64_t cap, hipStream_t s) {
   if ((rc = dev_grow(&L.nbr, (size_t)old * 27, (size_t)cap * 27, s))) return rc;
   if ((rc = dev_grow(&L.order, (size_t)old, (size_t)cap, s))) return rc;
   if ((rc = dev_grow(&L.pos, (size_t)old, (size_t)cap, s))) return rc;
-  if ((rc = dev_grow(&L.plan, 0, (size_t)cap * 27, s))) return rc;  // rebuilt every frame
+  if ((rc = dev_grow(&L.plan, 0, (size_t)cap * 27, s))) return rc;  // contents dropped: rebuilt by the next frame
+  L.plan_valid = false;
   if ((rc = dev_grow(&L.tmask, 0, (size_t)cap / 32 + 1, s))) return rc;
   if ((rc = dev_grow(&L.sched, 0, (size_t)cap / 32 + (size_t)cap / 128 + 3, s))) return rc;  // tiles, then groups of 4
   if (l + 1 < net->n_levels) {
@@ -422,6 +425,9 @@ static int points_reserve(insc_net *net, int64_t need, hipStream_t s) {
   return INSC_OK;
 }
 
+// the site counts and error flags of all scales, as they lie in net->h_counts
+static int apply_counts(insc_net *net, const char *who);
+
 static int sync_counts(insc_net *net, hipStream_t s, const char *who) {
   const int L = net->n_levels;
   INSC_HIP(hipMemcpyAsync(net->h_counts + 2 * L, net->d_bad, sizeof(int32_t), hipMemcpyDeviceToHost, s));
@@ -432,6 +438,11 @@ static int sync_counts(insc_net *net, hipStream_t s, const char *who) {
                             hipMemcpyDeviceToHost, s));
   }
   INSC_HIP(hipStreamSynchronize(s));
+  return apply_counts(net, who);
+}
+
+static int apply_counts(insc_net *net, const char *who) {
+  const int L = net->n_levels;
   for (int l = 0; l < L; l++) {
     Level &Lv = net->levels[l];
     Lv.n = Lv.n_upper = net->h_counts[2 * l];
@@ -586,6 +597,7 @@ int insc_net_create(int n_levels, int in_channels, int mode, insc_net **out) {
   t.buf = 0;
   net->tensors.push_back(t);
   INSC_HIP(hipHostMalloc((void **)&net->h_counts, sizeof(int32_t) * 64, hipHostMallocDefault));
+  INSC_HIP(hipEventCreateWithFlags(&net->ev_counts, hipEventDisableTiming));
   INSC_HIP(hipMalloc((void **)&net->d_bad, 256));
   INSC_HIP(hipMemset(net->d_bad, 0, 256));
   *out = net;
@@ -629,6 +641,7 @@ int insc_net_destroy(insc_net *net) {
   if (net->h_counts) (void)hipHostFree(net->h_counts);
   for (hipEvent_t e : net->ev)
     if (e) (void)hipEventDestroy(e);
+  if (net->ev_counts) (void)hipEventDestroy(net->ev_counts);
   delete net;
   return INSC_OK;
 }
@@ -970,22 +983,37 @@ int insc_net_forward(insc_net *net, const int32_t *d_coords, int coord_cols, con
 
   if (net->profiling) INSC_HIP(hipEventRecord(net->ev[0], s));
   int32_t *sop = net->site_of_point + net->n_points;
+  // An incremental frame of moderate size inserts at all scales in one launch, which also leaves
+  // the new site counts in host memory; the host picks them up further down, while the GPU is busy
+  // with the neighbour maps and orders of the new sites.
+  const bool fused_insert = inc && P > 0 && P <= frame_insert_max_points();
   if (P > 0) {
-    // ---- input scale: insert, accumulate --------------------------------------------------
-    void *ws;
-    if ((rc = workspace(WS_API, s, sizeof(int32_t) * 4 * (size_t)P, &ws))) return rc;
-    int32_t *c4 = (int32_t *)ws;
-    hipLaunchKernelGGL(coords_check_kernel, dim3(grid_for(P, 256)), dim3(256), 0, s, d_coords, coord_cols, P, net->d_bad,
-                       net->frame_id);
-    hipLaunchKernelGGL(coords_to_int4_kernel, dim3(grid_for(P, 256)), dim3(256), 0, s, d_coords, coord_cols, P, c4,
-                       net->d_bad, net->frame_id);
-    INSC_LAUNCH_CHECK();
     Level &L0 = net->levels[0];
-    if ((rc = grid_insert_nosync(L0.grid, c4, P, sop, s))) return rc;
-    // ---- coarser scales: the new sites of a scale are the parents of the new sites below ---
-    for (int l = 0; l + 1 < L; l++) {
-      Level &F = net->levels[l], &Cs = net->levels[l + 1];
-      if ((rc = down2_new_sites(F.grid, Cs.grid, P, F.parent, F.offset, F.child, s))) return rc;
+    if (fused_insert) {
+      FrameInsertLevel fl[16];
+      for (int l = 0; l < L; l++) {
+        Level &Lv = net->levels[l];
+        fl[l] = FrameInsertLevel{Lv.grid, Lv.parent, Lv.offset, Lv.child};
+      }
+      if ((rc = frame_insert_levels(fl, L, d_coords, coord_cols, P, net->d_bad, net->frame_id, sop, net->h_counts, s)))
+        return rc;
+      INSC_HIP(hipEventRecord(net->ev_counts, s));
+    } else {
+      // ---- input scale: insert ----------------------------------------------------------------
+      void *ws;
+      if ((rc = workspace(WS_API, s, sizeof(int32_t) * 4 * (size_t)P, &ws))) return rc;
+      int32_t *c4 = (int32_t *)ws;
+      hipLaunchKernelGGL(coords_check_kernel, dim3(grid_for(P, 256)), dim3(256), 0, s, d_coords, coord_cols, P, net->d_bad,
+                         net->frame_id);
+      hipLaunchKernelGGL(coords_to_int4_kernel, dim3(grid_for(P, 256)), dim3(256), 0, s, d_coords, coord_cols, P, c4,
+                         net->d_bad, net->frame_id);
+      INSC_LAUNCH_CHECK();
+      if ((rc = grid_insert_nosync(L0.grid, c4, P, sop, s))) return rc;
+      // ---- coarser scales: the new sites of a scale are the parents of the new sites below ---
+      for (int l = 0; l + 1 < L; l++) {
+        Level &F = net->levels[l], &Cs = net->levels[l + 1];
+        if ((rc = down2_new_sites(F.grid, Cs.grid, P, F.parent, F.offset, F.child, s))) return rc;
+      }
     }
     // ---- neighbour maps and processing orders of the new sites, all scales per launch ------
     const insc_grid *grids[16];
@@ -1003,10 +1031,24 @@ int insc_net_forward(insc_net *net, const int32_t *d_coords, int coord_cols, con
       bo_orders[l] = Lv.bo_order;
       bo_poss[l] = Lv.bo_pos;
     }
-    if ((rc = ssc3_new_sites_batch(grids, nbrs, L, P, s))) return rc;
+    // (an incremental frame keeps the tile plans of its scales up to date instead of rebuilding them:
+    // entries of older sites are patched along with the map, the new sites' columns are appended
+    // once they have their positions)
+    PlanRef prefs[16];
+    TilePlanBatch app;
+    app.n = L;
+    for (int l = 0; l < L; l++) {
+      Level &Lv = net->levels[l];
+      const bool keep = inc && Lv.plan_valid;
+      prefs[l] = keep ? PlanRef{Lv.plan, Lv.tmask, Lv.pos, Lv.cap} : PlanRef{nullptr, nullptr, nullptr, 0};
+      app.job[l] = TilePlanJob{Lv.nbr, Lv.order, Lv.grid->d_n, 0, Lv.cap, keep ? Lv.plan : nullptr, Lv.tmask, nullptr};
+    }
+    if ((rc = ssc3_new_sites_batch(grids, nbrs, L, P, s, prefs))) return rc;
     if (inc) {
-      if ((rc = order_append_new_sites_sorted_batch(grids, cnbrs, orders, poss, L, P, s))) return rc;
-      if ((rc = order_append_new_sites_by_offset_batch(grids, offsets, cposs, bo_orders, bo_poss, L - 1, P, s))) return rc;
+      offsets[L - 1] = nullptr;  // the coarsest scale has no order by position inside a parent cell
+      if ((rc = order_append_new_sites_both_batch(grids, cnbrs, offsets, orders, poss, bo_orders, bo_poss, L, P, s)))
+        return rc;
+      if ((rc = tile_plan_append_batch(app, P, s))) return rc;
     } else {
       for (int l = 0; l < L; l++) {
         Level &Lv = net->levels[l];
@@ -1053,7 +1095,12 @@ int insc_net_forward(insc_net *net, const int32_t *d_coords, int coord_cols, con
     // (tens of microseconds) buys launches sized to the real number of tiles.  With the bound
     // "every new point is a new site at every scale" a coarse scale of 70 sites would be
     // launched for thousands, and idle blocks cost more than the convolution itself.
-    if ((rc = sync_counts(net, s, "insc_net_forward"))) return rc;
+    if (fused_insert) {
+      INSC_HIP(hipEventSynchronize(net->ev_counts));
+      if ((rc = apply_counts(net, "insc_net_forward"))) return rc;
+    } else if ((rc = sync_counts(net, s, "insc_net_forward"))) {
+      return rc;
+    }
   }
 
   // tile plans of the 3^3 maps, shared by all the layers of a scale
@@ -1063,7 +1110,10 @@ int insc_net_forward(insc_net *net, const int32_t *d_coords, int coord_cols, con
     for (int l = 0; l < L; l++) {
       Level &Lv = net->levels[l];
       if (Lv.n <= 0) continue;
-      batch.job[batch.n++] = TilePlanJob{Lv.nbr, Lv.order, Lv.grid->d_n, Lv.n, Lv.cap, Lv.plan, Lv.tmask, Lv.sched};
+      // (a plan kept up to date by this incremental frame only needs its tile schedule redone)
+      const bool keep = inc && Lv.plan_valid;
+      batch.job[batch.n++] = TilePlanJob{keep ? nullptr : Lv.nbr, Lv.order, Lv.grid->d_n, Lv.n, Lv.cap, Lv.plan, Lv.tmask, Lv.sched};
+      Lv.plan_valid = true;
     }
     if ((rc = build_tile_plans(batch, s))) return rc;
   }
