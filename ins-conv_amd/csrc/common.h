@@ -100,11 +100,13 @@ int tile_plan_append_batch(const TilePlanBatch &b, int64_t n_new_upper, hipStrea
 
 // in_rows: rows of the input matrix (bounds the gather).  out may be null when ep.out2 is set.
 // latency != 0 picks the launch shape for small row counts (residual frames).
+// expect_rows (0: n_rows): how many rows the launch will probably find in *d_n_rows, when that is
+// far below the bound n_rows - it only picks among kernels that give the same bits.
 int launch_conv(const float *in, int64_t ld_in, int64_t in_rows, float *out, int64_t ld_out, const float *W,
                 const float *Wp, const float *bias, const int32_t *map0, const int32_t *map1, int mode, int K,
                 const int32_t *rows, const int32_t *d_n_rows, int64_t n_rows, int Cin, int Cout,
                 const uint8_t *tile_flags, const uint8_t *row_mask, hipStream_t s, BnEpilogue ep = BnEpilogue(),
-                TilePlan plan = TilePlan(), int latency = 0);
+                TilePlan plan = TilePlan(), int latency = 0, int64_t expect_rows = 0);
 int64_t packed_floats(int K, int Cin, int Cout);
 int pack_weights(const float *W, int K, int Cin, int Cout, float *Wp, hipStream_t s);
 int launch_bn(const float *in, int64_t ld_in, float *out, int64_t ld_out, const float *mean, const float *var,

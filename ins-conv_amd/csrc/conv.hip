@@ -733,20 +733,53 @@ __global__ __launch_bounds__(WL_WAVES * 64) void conv_wlds_kernel(
         kq[d] = next_k();
         g[d] = gather(kq[d]);
       }
+      // The loads of the item D - 1 ahead and the weight tile of the next item are issued in the
+      // shadow of this item's MFMAs (a dependent MFMA issues every 64 cycles; whatever sits between
+      // two of them is free), in four slices pinned by scheduling barriers.
+      Frag bw[2];
+      bw[0] = wread(kq[0]);
       for (int i0 = 0; i0 < nitems; i0 += D) {
 #pragma unroll
         for (int u = 0; u < D; u++) {
-          kq[(u + D - 1) % D] = next_k();
-          g[(u + D - 1) % D] = gather(kq[(u + D - 1) % D]);
-          const Frag bf = wread(kq[u]);
-          asm volatile("" ::: "memory");
+          const bool real = i0 + u < nitems;
+          const Frag &bf = bw[u % 2];
           __builtin_amdgcn_sched_barrier(0);
-          if (i0 + u < nitems) {
+          if (real) {
 #pragma unroll
-            for (int s = 0; s < 16; s++)
+            for (int s = 0; s < 4; s++)
               acc = __builtin_amdgcn_mfma_f32_32x32x2f32(frag_at(g[u], s), frag_at(bf, s), acc, 0, 0, 0);
           }
-          asm volatile("" ::: "memory");
+          __builtin_amdgcn_sched_barrier(0);
+          const int kn = next_k();
+          kq[(u + D - 1) % D] = kn;
+          const int src = nl[planned ? (kn < 0 ? 0 : kn) * TILE_M + r : r * K + (kn < 0 ? 0 : kn)];
+          __builtin_amdgcn_sched_barrier(0);
+          if (real) {
+#pragma unroll
+            for (int s = 4; s < 8; s++)
+              acc = __builtin_amdgcn_mfma_f32_32x32x2f32(frag_at(g[u], s), frag_at(bf, s), acc, 0, 0, 0);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+          {
+            const bool on = kn >= 0 && src >= 0 && half_on;
+            const uint32_t voff = on ? (uint32_t)src * ld4 + (uint32_t)(h * 64) : BUF_OOB;
+#pragma unroll
+            for (int q = 0; q < 4; q++) g[(u + D - 1) % D].q[q] = buf_load16(rin, voff + 16u * q, 0);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+          if (real) {
+#pragma unroll
+            for (int s = 8; s < 12; s++)
+              acc = __builtin_amdgcn_mfma_f32_32x32x2f32(frag_at(g[u], s), frag_at(bf, s), acc, 0, 0, 0);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+          bw[(u + 1) % 2] = wread(kq[(u + 1) % D]);
+          __builtin_amdgcn_sched_barrier(0);
+          if (real) {
+#pragma unroll
+            for (int s = 12; s < 16; s++)
+              acc = __builtin_amdgcn_mfma_f32_32x32x2f32(frag_at(g[u], s), frag_at(bf, s), acc, 0, 0, 0);
+          }
           __builtin_amdgcn_sched_barrier(0);
         }
       }
@@ -1556,8 +1589,9 @@ int launch_conv(const float *in, int64_t ld_in, int64_t in_rows, float *out, int
                 const float *Wp, const float *bias, const int32_t *map0, const int32_t *map1, int mode, int K,
                 const int32_t *rows, const int32_t *d_n_rows, int64_t n_rows, int Cin, int Cout,
                 const uint8_t *tile_flags, const uint8_t *row_mask, hipStream_t s, BnEpilogue ep, TilePlan plan,
-                int latency) {
+                int latency, int64_t expect_rows) {
   if (n_rows == 0) return INSC_OK;
+  if (expect_rows <= 0 || expect_rows > n_rows) expect_rows = n_rows;
   if (plan.map && (mode != MAP_NBR || K != 27 || plan.ld * 27 * 4 >= (int64_t)BUF_OOB || plan.ld < cdiv(n_rows, TILE_M) * TILE_M))
     plan = TilePlan();  // only the 3^3 map has a plan; an unusable one is ignored
   if (conv_uses_mfma(in, ld_in, Cin, K)) {
@@ -1591,7 +1625,7 @@ int launch_conv(const float *in, int64_t ld_in, int64_t in_rows, float *out, int
     // whole filter into LDS - costs more than it saves: 34 us against 21 us at 32k sites, even at
     // 150k; both kernels give the same bits)
     if (mode == MAP_NBR && K == 27 && Cin <= 32 && Cout <= 32 && map_bytes64 < (int64_t)BUF_OOB && small_ids &&
-        tiles >= g_wl_min_tiles.load(std::memory_order_relaxed) && !latency) {
+        cdiv(expect_rows, TILE_M) >= g_wl_min_tiles.load(std::memory_order_relaxed) && !latency) {
       const uint32_t map_bytes = (uint32_t)map_bytes64;
       // persistent blocks, a multiple of the XCD count, at most one per compute unit
       const int64_t want = cdiv(tiles, WL_WAVES);

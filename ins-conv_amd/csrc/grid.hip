@@ -552,6 +552,10 @@ __device__ __forceinline__ void order_append_sorted_body(const int32_t *__restri
     key[i] = k;
   }
   __syncthreads();
+  // Bitonic sort.  A pass of stride j <= 64 stays inside the 128 keys that the 64 pairs of one
+  // wavefront cover, so runs of such passes are ordered by the wavefront itself (LDS accesses of a
+  // wavefront complete in order); only passes of a larger stride, and the change from one kind to
+  // the other, need the whole workgroup to meet.
   for (int k = 2; k <= N; k <<= 1) {
     for (int j = k >> 1; j > 0; j >>= 1) {
       for (int p = tid; p < (N >> 1); p += 1024) {
@@ -562,9 +566,17 @@ __device__ __forceinline__ void order_append_sorted_body(const int32_t *__restri
           key[x] = a;
         }
       }
-      __syncthreads();
+      const int jn = j > 1 ? (j >> 1) : k;  // stride of the pass that follows (k: first pass of the next stage)
+      if (j > 64 || jn > 64) {
+        __syncthreads();
+      } else {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      }
     }
   }
+  __syncthreads();
   for (int i = tid; i < n; i += 1024) {
     const int v = first + (int)(key[i] & 8191);
     order[first + i] = v;

@@ -23,6 +23,8 @@ enum DirtyKind { D_INPUT, D_DILATE, D_PARENTS, D_CHILDREN, D_UNION };
 // tiles resident at once, and with the eight 3^3 layers of such a scale and of each coarser one a
 // change anywhere reaches nearly every site of it anyway.)
 constexpr int64_t DIRTY_FULL_SITES = 4096;
+// Scales from this size on may run a layer over a list of dirty rows instead of over flagged tiles.
+constexpr int64_t COMPACT_MIN_SITES = 32768;
 
 struct Level {
   insc_grid *grid = nullptr;
@@ -78,6 +80,17 @@ struct DirtyNode {
   uint8_t *tflag = nullptr;      // [cap/32+1] one byte per 32-row tile of the level's order
   uint8_t *tflag_bo = nullptr;   // same for the by-offset order (only if some deconvolution needs it)
   std::set<int> ancestors;
+  // A set that stays small against its scale is also kept as a list of its rows (in processing
+  // order), so that a layer works on tiles made of dirty rows only instead of on every tile that
+  // holds one: depth = 3^3 layers between the frame's points and this set at the input scale (-1:
+  // the set does not qualify), crows / ccount = the list and its length (ccount lies in the mask
+  // arena and is zero when a frame starts), compact = this frame uses the list.
+  int depth = -1;
+  int32_t *crows = nullptr;
+  int32_t *ccount = nullptr;
+  int64_t crows_cap = 0;
+  bool compact = false;
+  int64_t expect_rows = 0;  // estimate of the set's size in this frame
 };
 
 }  // namespace insc
@@ -233,6 +246,45 @@ __global__ void dirty_union_kernel(const uint8_t *__restrict__ a, const uint8_t 
   mask_out[i] = 1;
   tflag[pos[i] >> 5] = 1;
   if (tflag_bo) tflag_bo[bo_pos[i] >> 5] = 1;
+}
+
+// rows = the sites of the processing order whose mask byte is set.  A block compacts a run of
+// 1024 positions, keeping their order, and claims room for them with one atomic: the runs come out
+// in any order (no result depends on the order of a row list).  *count must be zero beforehand.
+__global__ __launch_bounds__(256) void dirty_compact_rows_kernel(const uint8_t *__restrict__ mask,
+                                                                 const int32_t *__restrict__ order,
+                                                                 const int32_t *__restrict__ d_n, int64_t n_upper,
+                                                                 int32_t *__restrict__ rows, int32_t *count) {
+  __shared__ int wave_total[4];
+  __shared__ int base_s;
+  const int64_t n = min((int64_t)*d_n, n_upper);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int64_t p0 = (int64_t)blockIdx.x * 1024 + tid * 4;
+  int site[4], cnt = 0;
+#pragma unroll
+  for (int j = 0; j < 4; j++) {
+    site[j] = p0 + j < n ? order[p0 + j] : -1;
+    if (site[j] >= 0 && !mask[site[j]]) site[j] = -1;
+    cnt += site[j] >= 0 ? 1 : 0;
+  }
+  int incl = cnt;
+  for (int d = 1; d < 64; d <<= 1) {
+    const int v = __shfl_up(incl, d, 64);
+    if (lane >= d) incl += v;
+  }
+  if (lane == 63) wave_total[wave] = incl;
+  __syncthreads();
+  int before = incl - cnt, total = 0;
+  for (int w = 0; w < 4; w++) {
+    if (w < wave) before += wave_total[w];
+    total += wave_total[w];
+  }
+  if (tid == 0) base_s = total ? atomicAdd(count, total) : 0;
+  __syncthreads();
+  int at = base_s + before;
+#pragma unroll
+  for (int j = 0; j < 4; j++)
+    if (site[j] >= 0) rows[at++] = site[j];
 }
 
 // dirty rows of one set: one count per block, added up with an atomic per block
@@ -410,7 +462,15 @@ static int level_reserve(insc_net *net, int l, int64_t cap, hipStream_t s) {
     d.mask = net->mask_arena + off;
     d.tflag = d.mask + mb;
     d.tflag_bo = d.tflag + tb;
+    d.ccount = (int32_t *)(d.tflag_bo + tb);
     off += mb + 3 * tb;
+    if (d.depth >= 0 && d.crows_cap < (int64_t)c) {
+      INSC_HIP(hipStreamSynchronize(s));
+      if (d.crows) INSC_HIP(hipFree(d.crows));
+      d.crows = nullptr;
+      INSC_HIP(hipMalloc((void **)&d.crows, sizeof(int32_t) * c));
+      d.crows_cap = (int64_t)c;
+    }
   }
   return INSC_OK;
 }
@@ -500,6 +560,9 @@ static int run_op(insc_net *net, const Op &op, bool incremental, hipStream_t s) 
   const int64_t rows0 = net->buffers[net->tensors[op.in0].buf].rows;
   switch (op.kind) {
     case OP_SSC: {
+      if (d && d->compact)  // tiles made of the set's rows only (no tile plan: its positions are the full order's)
+        return launch_conv(in0, ld0, rows0, out, ld_out, op.W, op.Wp, op.bias, Lo.nbr, nullptr, MAP_NBR, 27, d->crows,
+                           d->ccount, n_up, op.Cin, op.Cout, nullptr, d->mask, s, ep, TilePlan(), 0, d->expect_rows);
       TilePlan plan;
       plan.map = Lo.plan;
       plan.ld = Lo.cap;
@@ -615,6 +678,8 @@ int insc_net_destroy(insc_net *net) {
   }
   for (Buffer &B : net->buffers)
     if (B.p) (void)hipFree(B.p);
+  for (DirtyNode &d : net->dirty)
+    if (d.crows) (void)hipFree(d.crows);
   for (Op &op : net->ops) {
     if (op.Wp) (void)hipFree(op.Wp);
     if (op.bn_w) (void)hipFree(op.bn_w);
@@ -806,6 +871,13 @@ int insc_net_finalize(insc_net *net, int out_tensor, int64_t capacity_sites, voi
         if (rc) return rc;
       }
     }
+  }
+  // sets at the input scale that are reached from the frame's points through 3^3 layers only
+  for (DirtyNode &d : net->dirty) {
+    if (d.kind == D_INPUT)
+      d.depth = 0;
+    else if (d.kind == D_DILATE && d.level == 0 && d.src0 >= 0 && net->dirty[(size_t)d.src0].depth >= 0)
+      d.depth = net->dirty[(size_t)d.src0].depth + 1;
   }
   // Fold each batch norm into the kernel that produces its input (one fewer pass over the rows
   // and one fewer launch); the producer keeps writing its raw result only if something else
@@ -1144,8 +1216,23 @@ int insc_net_forward(insc_net *net, const int32_t *d_coords, int coord_cols, con
       if (dn.src1 >= 0 && net->dirty_full[(size_t)dn.src1]) full = true;
       net->dirty_full[i] = full ? 1 : 0;
     }
-    for (int i = 0; i < (int)net->dirty.size(); i++)
-      if (!net->dirty_full[(size_t)i] && (rc = run_dirty_node(net, i, s))) return rc;
+    // A set is also listed row by row when it is expected to stay well below its scale: from the
+    // sweeps measured, d 3^3 layers turn P touched voxels into about P * (6 d - 2) dirty rows.
+    // Either way every dirty row is recomputed and no other row is written: same results.
+    for (int i = 0; i < (int)net->dirty.size(); i++) {
+      DirtyNode &dn = net->dirty[(size_t)i];
+      const Level &Lv = net->levels[dn.level];
+      dn.expect_rows = P * (6 * dn.depth - 2);
+      dn.compact = !net->dirty_full[(size_t)i] && dn.depth >= 1 && dn.crows && Lv.n_upper >= COMPACT_MIN_SITES &&
+                   dn.expect_rows * 2 <= Lv.n_upper;
+      if (net->dirty_full[(size_t)i]) continue;
+      if ((rc = run_dirty_node(net, i, s))) return rc;
+      if (dn.compact) {
+        hipLaunchKernelGGL(dirty_compact_rows_kernel, dim3(grid_for(Lv.n_upper, 1024)), dim3(256), 0, s, dn.mask, Lv.order,
+                           Lv.grid->d_n, Lv.n_upper, dn.crows, dn.ccount);
+        INSC_LAUNCH_CHECK();
+      }
+    }
   }
   if (net->profiling) INSC_HIP(hipEventRecord(net->ev[2], s));
   for (const Op &op : net->ops)
