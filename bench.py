@@ -609,6 +609,10 @@ def main():
                     help="print only the table of bandwidth-bound kernels")
     ap.add_argument("--roofline-only", action="store_true",
                     help="run only the dominant-kernel measurement (short; used under rocprofv3)")
+    ap.add_argument("--wide-only", action="store_true",
+                    help="run only the 64-channel layer at 500k voxels (short; used under rocprofv3)")
+    ap.add_argument("--no-extras", action="store_true",
+                    help="skip the roofline, wide-layer and kernel-table rows (used under rocprofv3)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU; --gpus %d is not supported (no collectives, no sharding)"
@@ -631,6 +635,9 @@ def main():
         model, _ = unet_model(device)
         frames = [to_dev(p, c, device) for p, c in seq]
         print(json.dumps(residual_row(model, seq, frames, len(seq) - 1, device)))
+        return
+    if args.wide_only:
+        print(json.dumps({"wide_layer": wide_conv_row(device)}))
         return
     if args.roofline_only:
         # plus a plain copy of known size (500k x 32 floats: 64 MB read, 64 MB written), the
@@ -773,9 +780,10 @@ def main():
             out["cpu_baseline"] = cpu_fn()
         print(json.dumps(out))
         return
-    out["roofline"] = conv_roofline(device)
-    out["wide_layer"] = wide_conv_row(device)
-    out["kernels"] = kernel_table(device)
+    if not args.no_extras:
+        out["roofline"] = conv_roofline(device)
+        out["wide_layer"] = wide_conv_row(device)
+        out["kernels"] = kernel_table(device)
     # the CPU leg comes last: the GPU idles during it, and a measurement taken right after would
     # start at idle clocks
     if not args.no_cpu_baseline:

@@ -135,6 +135,8 @@ struct insc_net {
   int32_t *h_counts = nullptr;  // pinned: per level count, error flags
   int32_t *d_bad = nullptr;     // number of the last frame that held a coordinate out of range
   int32_t frame_id = 0;         // frames are numbered from 1
+  const int32_t *frame_sop = nullptr;  // site of every point of the frame being enqueued
+  int64_t frame_P = 0;
   int out_tensor = -1;
   bool profiling = false;
   hipEvent_t ev[5] = {nullptr, nullptr, nullptr, nullptr, nullptr};
@@ -205,6 +207,25 @@ __global__ void dirty_dilate_kernel(const int32_t *__restrict__ nbr, const uint8
   mask_out[j] = 1;
   tflag[pos[j] >> 5] = 1;
   if (tflag_bo) tflag_bo[bo_pos[j] >> 5] = 1;
+}
+
+// the same from a list of the source set's rows (a short list beats a pass over every site of the
+// scale); entries may repeat, -1 is skipped
+__global__ void dirty_dilate_list_kernel(const int32_t *__restrict__ nbr, const int32_t *__restrict__ rows,
+                                         const int32_t *__restrict__ d_count, int64_t n_fixed,
+                                         uint8_t *__restrict__ mask_out, uint8_t *__restrict__ tflag,
+                                         const int32_t *__restrict__ pos, uint8_t *__restrict__ tflag_bo,
+                                         const int32_t *__restrict__ bo_pos) {
+  const int64_t n = d_count ? (int64_t)*d_count : n_fixed;
+  for (int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; t < n * 27; t += (int64_t)gridDim.x * blockDim.x) {
+    const int r = rows[t / 27];
+    if (r < 0) continue;
+    const int j = nbr[(int64_t)r * 27 + t % 27];
+    if (j < 0) continue;
+    mask_out[j] = 1;
+    tflag[pos[j] >> 5] = 1;
+    if (tflag_bo) tflag_bo[bo_pos[j] >> 5] = 1;
+  }
 }
 
 __global__ void dirty_parents_kernel(const int32_t *__restrict__ parent, const uint8_t *__restrict__ mask_fine,
@@ -605,11 +626,25 @@ static int run_dirty_node(insc_net *net, int id, hipStream_t s) {
   switch (d.kind) {
     case D_INPUT:
       return INSC_OK;  // marked by the input layer
-    case D_DILATE:
+    case D_DILATE: {
       if (L.n_upper == 0) return INSC_OK;
+      const DirtyNode &src = net->dirty[d.src0];
+      if (src.kind == D_INPUT && net->frame_sop && net->frame_P * 8 <= L.n_upper) {
+        // the source is the frame's own points
+        if (net->frame_P == 0) return INSC_OK;
+        hipLaunchKernelGGL(dirty_dilate_list_kernel, dim3(grid_for(net->frame_P * 27, 256)), dim3(256), 0, s, L.nbr,
+                           net->frame_sop, (const int32_t *)nullptr, net->frame_P, d.mask, d.tflag, L.pos, tbo, L.bo_pos);
+        break;
+      }
+      if (src.compact) {
+        hipLaunchKernelGGL(dirty_dilate_list_kernel, dim3(grid_for(src.expect_rows * 27 * 2, 256, 1 << 16)), dim3(256), 0, s,
+                           L.nbr, src.crows, src.ccount, 0, d.mask, d.tflag, L.pos, tbo, L.bo_pos);
+        break;
+      }
       hipLaunchKernelGGL(dirty_dilate_kernel, dim3(grid_for(L.n_upper * 27, 256, 1ll << 30)), dim3(256), 0, s, L.nbr,
                          net->dirty[d.src0].mask, d.mask, d.tflag, L.pos, tbo, L.bo_pos, L.grid->d_n, L.n_upper);
       break;
+    }
     case D_PARENTS: {
       const Level &F = net->levels[d.level - 1];
       if (F.n_upper == 0) return INSC_OK;
@@ -1055,6 +1090,8 @@ int insc_net_forward(insc_net *net, const int32_t *d_coords, int coord_cols, con
 
   if (net->profiling) INSC_HIP(hipEventRecord(net->ev[0], s));
   int32_t *sop = net->site_of_point + net->n_points;
+  net->frame_sop = sop;
+  net->frame_P = P;
   // An incremental frame of moderate size inserts at all scales in one launch, which also leaves
   // the new site counts in host memory; the host picks them up further down, while the GPU is busy
   // with the neighbour maps and orders of the new sites.
