@@ -257,22 +257,30 @@ def kernel_table(device, reps=20):
         return total * 1e-3 / reps
 
     rows = []
+    # HBM bytes per call from the counter summary of this very table (FETCH_SIZE + WRITE_SIZE, calibrated)
+    recs = profile_records("path_kernels_cfg2.txt") or []
+    traffic = {r["row"]: float(r["fetch_bytes"]) + float(r["write_bytes"]) for r in recs if "row" in r}
 
-    def add(name, sec, nbytes, note):
+    def add(name, sec, nbytes, note, key=None):
         gbs = nbytes / sec / 1e9
-        rows.append({"kernel": name, "us": round(sec * 1e6, 1), "algorithmic_bytes": int(nbytes),
-                     "GB/s": round(gbs, 1), "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4), "units": note})
+        row = {"kernel": name, "us": round(sec * 1e6, 1), "algorithmic_bytes": int(nbytes),
+               "GB/s": round(gbs, 1), "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4), "units": note}
+        if key in traffic:
+            row["traffic_bytes"] = int(traffic[key])
+            row["traffic_over_algorithmic"] = round(traffic[key] / nbytes, 2)
+            row["hbm_GB/s_on_traffic"] = round(traffic[key] / sec / 1e9, 1)
+        rows.append(row)
 
     # the box's own copy bandwidth at this size, as the reference point for the rows below
     t = timed(lambda: y.copy_(x))
     add("device-to-device copy (torch; reference point, not a kernel of the path)", t, NF * C * 8, "%d x %d" % (NF, C))
     t = timed(lambda: lib.insc_grid_insert(grid, ptr(c4), I64(P), ptr(sop), ctypes.byref(n_sites), st),
               pre=lambda: lib.insc_grid_clear(grid, st))
-    add("hash grid insert (claim, scan, assign, resolve; incl. count read-back)", t, P * 32, "%d points -> %d sites" % (P, n_sites.value))
+    add("hash grid insert (claim, scan, assign, resolve; incl. count read-back)", t, P * 32, "%d points -> %d sites" % (P, n_sites.value), key="insert")
     t = timed(lambda: lib.insc_grid_query(grid, ptr(c4), I64(P), ptr(sop), st))
-    add("hash grid query", t, P * 28, "%d queries" % P)
+    add("hash grid query", t, P * 28, "%d queries" % P, key="query")
     t = timed(lambda: lib.insc_rulebook_ssc3(grid, I64(0), I64(N), ptr(nbr), 0, st))
-    add("SSC 3^3 rulebook (dense neighbour map, 27 probes per site)", t, N * (16 + 27 * 8 + 27 * 4), "%d sites" % N)
+    add("SSC 3^3 rulebook (dense neighbour map, 27 probes per site)", t, N * (16 + 27 * 8 + 27 * 4), "%d sites" % N, key="ssc")
 
     def down():
         lib.insc_rulebook_down2(grid, coarse, I64(0), I64(N), ptr(parent), ptr(offset), ptr(child), I64(N), st)
@@ -282,10 +290,10 @@ def kernel_table(device, reps=20):
         child.fill_(-1)
 
     t = timed(down, pre=down_pre)
-    add("stride-2 rulebook (coarse grid insert + parent/offset/child maps)", t, N * 36, "%d fine sites" % N)
+    add("stride-2 rulebook (coarse grid insert + parent/offset/child maps)", t, N * 36, "%d fine sites" % N, key="down")
     t = timed(lambda: lib.insc_bn_leaky(ptr(x), I64(C), ptr(y), I64(C), ptr(mean), ptr(var), None, None,
                                          ctypes.c_float(1e-4), ctypes.c_float(0.0), None, None, I64(NF), C, st))
-    add("batch norm + ReLU (eval)", t, NF * C * 8, "%d x %d" % (NF, C))
+    add("batch norm + ReLU (eval)", t, NF * C * 8, "%d x %d" % (NF, C), key="bn")
 
     def inp():
         lib.insc_input_accumulate(ptr(fp), I64(P), C, ptr(sop), 4, ptr(acc), ptr(cnt), I64(N), st)
@@ -296,9 +304,9 @@ def kernel_table(device, reps=20):
         cnt.zero_()
 
     t = timed(inp, pre=inp_pre)
-    add("input layer (mode 4: per-voxel mean)", t, P * (4 * C + 4) + N * 4 * C, "%d points x %d -> %d sites" % (P, C, N))
+    add("input layer (mode 4: per-voxel mean)", t, P * (4 * C + 4) + N * 4 * C, "%d points x %d -> %d sites" % (P, C, N), key="input")
     t = timed(lambda: lib.insc_output_gather(ptr(y), I64(C), ptr(sop), I64(P), C, ptr(outp), st))
-    add("output layer (row gather)", t, P * (4 * C + 4) + P * 4 * C, "%d points x %d" % (P, C))
+    add("output layer (row gather)", t, P * (4 * C + 4) + P * 4 * C, "%d points x %d" % (P, C), key="output")
     # label fusion: one frame of 20-class scores folded into the per-voxel (label, confidence) table
     NCLS = 20
     table = ctypes.c_void_p()
@@ -307,7 +315,7 @@ def kernel_table(device, reps=20):
     lib.insc_labels_update(table, ptr(c4), ptr(scores), I64(NCLS), I64(P), NCLS, st)  # the voxels exist from here on
     t = timed(lambda: lib.insc_labels_update(table, ptr(c4), ptr(scores), I64(NCLS), I64(P), NCLS, st))
     add("label fusion update (argmax + per-voxel confidence rule)", t, P * (16 + 4 * NCLS + 12) + N * 16,
-        "%d points x %d classes -> %d voxels" % (P, NCLS, N))
+        "%d points x %d classes -> %d voxels" % (P, NCLS, N), key="labels")
     lib.insc_labels_destroy(table)
     lib.insc_grid_destroy(grid)
     lib.insc_grid_destroy(coarse)
