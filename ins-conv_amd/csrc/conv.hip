@@ -1380,6 +1380,167 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NB * ST > 4
   }
 }
 
+// ---------------------------------------------------------------------------------------
+// Wide 3^3 layers of middling size (a few hundred to a few thousand tiles): one wavefront per unit
+// (tile, output block), nothing shared between wavefronts - no barrier, no partial sums through LDS,
+// no wait for the slowest of four.  To give the bits of conv_mfma_kernel<1, 27, MAP_NBR, ST> the
+// wavefront keeps that kernel's ST partial sums - the items (k, ch) with (k * nch + ch) % ST == p, in
+// ascending order, bias in sum 0 - in ST accumulators and adds them in order at the end.  Units
+// follow the cost-ordered tile schedule, output blocks of a tile side by side, so the four
+// wavefronts of a block mostly work on the same tile and meet its map slice and gathered rows in L1.
+// ---------------------------------------------------------------------------------------
+constexpr int OWN_DEPTH = 2;  // items in flight per wavefront (three change nothing and cost a wavefront per SIMD)
+template <int ST>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) void conv_own_kernel(
+    const float *__restrict__ in, int64_t ld_in, float *__restrict__ out, int64_t ld_out,
+    const float *__restrict__ Wp, const float *__restrict__ bias, const int32_t *__restrict__ rows,
+    const int32_t *__restrict__ d_n_rows, int64_t n_rows, int Cin, int Cout, int nbt, int nbtp,
+    const uint8_t *__restrict__ tile_flags, uint32_t in_bytes, uint32_t wp_bytes, BnEpilogue ep, TilePlan plan) {
+  constexpr int K = 27;
+  constexpr int NSTAGE = (TILE_M * K + 63) / 64;
+  __shared__ int nlb[4][TILE_M * K];
+  const int64_t n = d_n_rows ? min((int64_t)*d_n_rows, n_rows) : n_rows;
+  const int64_t ntiles = (n + TILE_M - 1) / TILE_M, units = ntiles * nbt;
+  const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), lane = threadIdx.x & 63;
+  const int r = lane & 31, h = lane >> 5;
+  const int64_t u = (int64_t)blockIdx.x * 4 + wave;
+  if (u >= units) return;  // (wavefronts are on their own: no workgroup barrier anywhere below)
+  const int tile = __builtin_amdgcn_readfirstlane(plan.sched[u / nbt]);
+  const int ob = (int)(u % nbt);
+  if (tile_flags && !tile_flags[tile]) return;
+  const int nch = conv_nch(Cin);
+  int *nl = nlb[wave];
+  // the tile's slice of the map: 27 coalesced runs of the plan
+  int st[NSTAGE];
+#pragma unroll
+  for (int i = 0; i < NSTAGE; i++) {
+    const int e = i * 64 + lane;  // e = k * 32 + row
+    st[i] = e < TILE_M * K ? plan.map[(int64_t)(e >> 5) * plan.ld + (int64_t)tile * TILE_M + (e & 31)] : -1;
+  }
+  const int64_t pr = (int64_t)tile * TILE_M + r;
+  const int my_row = pr < n ? (rows ? rows[pr] : (int)pr) : -1;
+  const unsigned tmask = (unsigned)__builtin_amdgcn_readfirstlane((int)plan.tmask[tile]);
+  const int c = ob * 32 + r;
+  const float bv = (bias && c < Cout) ? bias[c] : 0.0f;
+  const float ew = (ep.out2 && c < Cout) ? ep.w[c] : 0.0f;
+  const float eb = (ep.out2 && c < Cout) ? ep.b[c] : 0.0f;
+#pragma unroll
+  for (int i = 0; i < NSTAGE; i++) {
+    const int e = i * 64 + lane;
+    if (e < TILE_M * K) nl[e] = st[i];
+  }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+  f16v acc[ST];
+#pragma unroll
+  for (int pp = 0; pp < ST; pp++) {
+#pragma unroll
+    for (int v = 0; v < 16; v++) acc[pp][v] = pp == 0 ? bv : 0.0f;
+  }
+  if (tmask) {
+    struct Cursor {
+      int k, ch;
+      unsigned rest;
+    };
+    auto step = [&](const Cursor &cu) -> Cursor {  // past the end: k = -1
+      const bool wrap = cu.ch + 1 >= nch;
+      const int nk = cu.rest ? __builtin_ctz(cu.rest) : -1;
+      Cursor nx;
+      nx.ch = wrap ? 0 : cu.ch + 1;
+      nx.k = wrap ? nk : cu.k;
+      nx.rest = wrap ? (cu.rest & (cu.rest - 1)) : cu.rest;
+      return nx;
+    };
+    const __amdgpu_buffer_rsrc_t rin = make_rsrc(in, in_bytes), rw = make_rsrc(Wp, wp_bytes);
+    const uint32_t ld4 = (uint32_t)ld_in * 4u, lane16 = (uint32_t)lane * 16u;
+    auto gather = [&](const Cursor &cu) -> Frag {
+      const int kk = cu.k < 0 ? 0 : cu.k;
+      const int src = nl[kk * TILE_M + r];
+      const bool on = cu.k >= 0 && src >= 0 && (h == 0 || Cin - cu.ch * 32 >= 32);
+      const uint32_t voff = on ? (uint32_t)src * ld4 + (uint32_t)(cu.ch * 128 + h * 64) : BUF_OOB;
+      Frag f;
+#pragma unroll
+      for (int q = 0; q < 4; q++) f.q[q] = buf_load16(rin, voff + 16u * q, 0);
+      return f;
+    };
+    auto wload = [&](const Cursor &cu) -> Frag {
+      const int wt = ((cu.k < 0 ? 0 : cu.k) * nch + cu.ch) * nbtp + ob;
+      const uint32_t soff = (uint32_t)__builtin_amdgcn_readfirstlane(wt * 4096);
+      const uint32_t voff = cu.k >= 0 ? lane16 : BUF_OOB;
+      Frag f;
+#pragma unroll
+      for (int q = 0; q < 4; q++) f.q[q] = buf_load16(rw, voff + 1024u * q, soff);
+      return f;
+    };
+    const int nitems = __builtin_popcount(tmask) * nch;
+    Cursor first;
+    first.k = __builtin_ctz(tmask);
+    first.ch = 0;
+    first.rest = tmask & (tmask - 1);
+    constexpr int D = OWN_DEPTH;
+    Frag g[D], bw[D];
+    Cursor ci = first, c0 = first;
+#pragma unroll
+    for (int d = 0; d < D - 1; d++) {
+      g[d] = gather(ci);
+      bw[d] = wload(ci);
+      ci = step(ci);
+    }
+    for (int t0i = 0; t0i < nitems; t0i += D) {
+#pragma unroll
+      for (int uu = 0; uu < D; uu++) {
+        g[(uu + D - 1) % D] = gather(ci);
+        bw[(uu + D - 1) % D] = wload(ci);
+        ci = step(ci);
+        // which partial sum the item on the matrix cores belongs to (-1 past the last item)
+        const int part = t0i + uu < nitems ? ((c0.k * nch + c0.ch) & (ST - 1)) : -1;
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int pp = 0; pp < ST; pp++) {
+          if (part != pp) continue;  // (one copy of the MFMA block per partial sum: the accumulator is a compile-time choice)
+#pragma unroll
+          for (int s2 = 0; s2 < 16; s2++)
+            acc[pp] = __builtin_amdgcn_mfma_f32_32x32x2f32(frag_at(g[uu], s2), frag_at(bw[uu], s2), acc[pp], 0, 0, 0);
+        }
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+        c0 = step(c0);
+      }
+    }
+  }
+  // rows and epilogue (D layout of the 32x32 MFMA: lane holds column (lane & 31), rows 8*(v/4) + 4*(lane>>5) + (v&3))
+  const __amdgpu_buffer_rsrc_t rout = make_rsrc(out, out ? BUF_OOB : 0u), rout2 = make_rsrc(ep.out2, ep.out2 ? BUF_OOB : 0u);
+  const __amdgpu_buffer_rsrc_t rres = make_rsrc(ep.res, ep.res ? BUF_OOB : 0u);
+  const uint32_t ldo4 = (uint32_t)ld_out * 4u, ldo24 = (uint32_t)ep.ld2 * 4u, ldr4 = (uint32_t)ep.ldr * 4u;
+  int rid[16];
+#pragma unroll
+  for (int v = 0; v < 16; v++) rid[v] = __shfl(my_row, 8 * (v >> 2) + 4 * h + (v & 3), 64);
+  float rv[16];
+#pragma unroll
+  for (int v = 0; v < 16; v++)
+    rv[v] = __uint_as_float((unsigned)__builtin_amdgcn_raw_buffer_load_b32(
+        rres, (int)((rid[v] >= 0 && c < Cout) ? __umul24((unsigned)rid[v], ldr4) + (uint32_t)c * 4u : BUF_OOB), 0, 0));
+#pragma unroll
+  for (int v = 0; v < 16; v++) {
+    const bool ok = rid[v] >= 0 && c < Cout;
+    float a = acc[0][v];
+#pragma unroll
+    for (int pp = 1; pp < ST; pp++) a += acc[pp][v];
+    if (ep.res) a += rv[v];
+    if (out)
+      __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(a), rout,
+                                            (int)(ok ? __umul24((unsigned)rid[v], ldo4) + (uint32_t)c * 4u : BUF_OOB), 0, 0);
+    if (ep.out2) {
+      const float y = fmaf(a, ew, eb);  // fused batch norm + leaky ReLU
+      __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(y * ((y > 0.0f) ? 1.0f : ep.leak)), rout2,
+                                            (int)(ok ? __umul24((unsigned)rid[v], ldo24) + (uint32_t)c * 4u : BUF_OOB), 0, 0);
+    }
+  }
+}
+
 __global__ void count_rules_kernel(const int32_t *__restrict__ map0, int K, const int32_t *__restrict__ rows,
                                    const int32_t *__restrict__ d_n_rows, int64_t n_rows,
                                    unsigned long long *__restrict__ total) {
@@ -1578,6 +1739,10 @@ static std::atomic<int64_t> g_pers_min_units{512};
 // ... and with at least this many (group of four tiles, output block) units to the kernel whose blocks
 // share the weight tiles through LDS (faster from about 60k sites at 64 channels; same bits again).
 static std::atomic<int64_t> g_shared_min_units{896};
+// ... and, below that, with at least this many (tile, output block) units on the kernel that gives every
+// unit a wavefront of its own (faster than the persistent blocks from about 2000 units: 64 channels at
+// 35-55k sites, the second scale of the 150k-voxel U-Net; same bits again).
+static std::atomic<int64_t> g_own_min_units{2000};
 // Narrow 3^3 layers (Cin, Cout <= 32) with at least this many 32-row tiles run on the persistent
 // kernel that keeps the whole filter in LDS; smaller ones on the one-wavefront-per-tile kernel.
 // Same bits either way.
@@ -1688,6 +1853,13 @@ int launch_conv(const float *in, int64_t ld_in, int64_t in_rows, float *out, int
       const unsigned nblk = (unsigned)std::min<int64_t>((int64_t)device_cus() * per_cu2, wunits);
       hipLaunchKernelGGL((conv_wshare_kernel<1, 4>), dim3(nblk), dim3(256), 0, s, in, ld_in, out, ld_out, Wp, bias, rows,
                          d_n_rows, n_rows, Cin, Cout, nbt, nbtp, tile_flags, in_bytes, wp_bytes, ep, plan);
+      INSC_LAUNCH_CHECK();
+      return INSC_OK;
+    }
+    if (wide_planned && tiles * nbt >= g_own_min_units.load(std::memory_order_relaxed)) {
+      // one wavefront per (tile, output block): enough units that every SIMD gets two or three
+      hipLaunchKernelGGL((conv_own_kernel<4>), dim3((unsigned)cdiv(tiles * nbt, 4)), dim3(256), 0, s, in, ld_in, out, ld_out, Wp,
+                         bias, rows, d_n_rows, n_rows, Cin, Cout, nbt, nbtp, tile_flags, in_bytes, wp_bytes, ep, plan);
       INSC_LAUNCH_CHECK();
       return INSC_OK;
     }
@@ -1816,6 +1988,12 @@ int insc_conv_set_persistent_min_units(int64_t units) {
 int insc_conv_set_shared_weights_min_units(int64_t units) {
   INSC_REQUIRE(units >= 1, INSC_ERR_ARG, "insc_conv_set_shared_weights_min_units: units must be >= 1");
   g_shared_min_units.store(units, std::memory_order_relaxed);
+  return INSC_OK;
+}
+
+int insc_conv_set_wavefront_per_unit_min_units(int64_t units) {
+  INSC_REQUIRE(units >= 1, INSC_ERR_ARG, "insc_conv_set_wavefront_per_unit_min_units: units must be >= 1");
+  g_own_min_units.store(units, std::memory_order_relaxed);
   return INSC_OK;
 }
 

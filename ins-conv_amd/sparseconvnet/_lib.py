@@ -38,6 +38,7 @@ _SIGS = {
     "insc_conv_set_persistent_min_units": [c_i64],
     "insc_conv_set_shared_weights_min_units": [c_i64],
     "insc_conv_set_filter_lds_min_tiles": [c_i64],
+    "insc_conv_set_wavefront_per_unit_min_units": [c_i64],
     "insc_deconv_down2": [vp, c_i64, c_i64, vp, c_i64, vp, vp, vp, vp, vp, vp, vp, c_i64, c_int, c_int, vp],
     "insc_bn_leaky": [vp, c_i64, vp, c_i64, vp, vp, vp, vp, c_f32, c_f32, vp, vp, c_i64, c_int, vp],
     "insc_add": [vp, c_i64, vp, c_i64, vp, c_i64, vp, vp, c_i64, c_int, vp],

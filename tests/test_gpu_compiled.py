@@ -11,12 +11,13 @@ from test_gpu_incremental import _frames, _inp
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture(params=[(512, 896, 4096), (1, 1 << 40, 4096), (512, 1, 4096), (512, 896, 1)],
+@pytest.fixture(params=[(512, 896, 4096, 2000), (1, 1 << 40, 4096, 1 << 40), (512, 1, 4096, 2000), (512, 896, 1, 2000),
+                        (512, 1 << 40, 4096, 1)],
                 ids=["default-launch-policy", "persistent-kernel-forced", "shared-weights-kernel-forced",
-                     "filter-in-lds-kernel-forced"])
+                     "filter-in-lds-kernel-forced", "wavefront-per-unit-kernel-forced"])
 def persistent_min_units(request):
     """The 3^3 layers of these small scenes stay below the thresholds of the three persistent
-    kernels; the second and third run force the wide layers onto one and the other, the fourth the
+    kernels; the second, third and fifth run force the wide layers onto one of them, the fourth the
     narrow layers (at most 32 channels) onto the kernel that keeps its filter in LDS - each with the
     fused batch norm / residual epilogues and the dirty-tile flags of the executor."""
     from sparseconvnet._lib import lib
@@ -24,10 +25,12 @@ def persistent_min_units(request):
     lib.insc_conv_set_persistent_min_units(request.param[0])
     lib.insc_conv_set_shared_weights_min_units(request.param[1])
     lib.insc_conv_set_filter_lds_min_tiles(request.param[2])
+    lib.insc_conv_set_wavefront_per_unit_min_units(request.param[3])
     yield request.param
     lib.insc_conv_set_persistent_min_units(512)
     lib.insc_conv_set_shared_weights_min_units(896)
     lib.insc_conv_set_filter_lds_min_tiles(4096)
+    lib.insc_conv_set_wavefront_per_unit_min_units(2000)
 
 
 @pytest.mark.parametrize("levels,m", [(3, 16), (7, 32)])

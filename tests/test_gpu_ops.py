@@ -98,8 +98,12 @@ def test_persistent_kernels_give_the_bits_of_the_per_tile_kernel(S, orc, Cin, Co
     a = torch.full((sc.n, Cout), 3.0, device="cuda")
     c = torch.full((sc.n, Cout), -3.0, device="cuda")
     d = torch.full((sc.n, Cout), 5.0, device="cuda")
+    e = torch.full((sc.n, Cout), 11.0, device="cuda")
     try:
         lib.insc_conv_set_shared_weights_min_units(1 << 40)
+        lib.insc_conv_set_wavefront_per_unit_min_units(1)  # a wavefront of its own per (tile, output block)
+        S.ssc_rows_planned(feats, e, W, bt, sc, m.ssc_plan(sc))
+        lib.insc_conv_set_wavefront_per_unit_min_units(1 << 40)
         lib.insc_conv_set_persistent_min_units(1)
         S.ssc_rows_planned(feats, a, W, bt, sc, m.ssc_plan(sc))
         lib.insc_conv_set_persistent_min_units(1 << 40)
@@ -116,8 +120,10 @@ def test_persistent_kernels_give_the_bits_of_the_per_tile_kernel(S, orc, Cin, Co
     finally:
         lib.insc_conv_set_persistent_min_units(512)
         lib.insc_conv_set_shared_weights_min_units(896)
+        lib.insc_conv_set_wavefront_per_unit_min_units(2000)
     assert torch.equal(a, c)
     assert torch.equal(d, c)
+    assert torch.equal(e, c)
     nt = (sc.n + 31) // 32
     plan = m.ssc_plan(sc)
     sched = plan[3][:nt].cpu().numpy()
@@ -180,7 +186,7 @@ def test_filter_in_lds_kernel_against_oracle_and_per_tile_kernel(S, orc, Cin, Co
 @pytest.mark.parametrize("n", [1, 20, 33, 130, 1025])
 def test_persistent_kernels_on_tiny_and_ragged_scenes(S, n):
     """One site, one tile, two tiles, a group of four tiles with a partial fifth, a partial last tile:
-    all three kernels of a 64->64 layer give the same bits."""
+    all four kernels of a 64->64 layer give the same bits."""
     from sparseconvnet._lib import lib
 
     rng = np.random.default_rng(n)
@@ -193,17 +199,21 @@ def test_persistent_kernels_on_tiny_and_ragged_scenes(S, n):
     W = cu((rng.normal(size=(27, 64, 64)) * 0.05).astype(np.float32))
     outs = []
     try:
-        for pers, shared in [(1 << 40, 1 << 40), (1, 1 << 40), (1 << 40, 1)]:
+        for pers, shared, own in [(1 << 40, 1 << 40, 1 << 40), (1, 1 << 40, 1 << 40), (1 << 40, 1, 1 << 40),
+                                  (1 << 40, 1 << 40, 1)]:
             lib.insc_conv_set_persistent_min_units(pers)
             lib.insc_conv_set_shared_weights_min_units(shared)
+            lib.insc_conv_set_wavefront_per_unit_min_units(own)
             o = torch.full((sc.n, 64), float(len(outs)), device="cuda")
             S.ssc_rows_planned(feats, o, W, None, sc, m.ssc_plan(sc))
             outs.append(o)
     finally:
         lib.insc_conv_set_persistent_min_units(512)
         lib.insc_conv_set_shared_weights_min_units(896)
+        lib.insc_conv_set_wavefront_per_unit_min_units(2000)
     assert torch.equal(outs[0], outs[1])
     assert torch.equal(outs[0], outs[2])
+    assert torch.equal(outs[0], outs[3])
     assert torch.isfinite(outs[0]).all() and outs[0].abs().max().item() > 0
 
 
