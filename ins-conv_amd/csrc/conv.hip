@@ -1389,8 +1389,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NB * ST > 4
 // follow the cost-ordered tile schedule, output blocks of a tile side by side, so the four
 // wavefronts of a block mostly work on the same tile and meet its map slice and gathered rows in L1.
 // ---------------------------------------------------------------------------------------
-constexpr int OWN_DEPTH = 2;  // items in flight per wavefront (three change nothing and cost a wavefront per SIMD)
-template <int ST>
+// D = items in flight per wavefront (2 with three wavefronts per SIMD; deeper rings at two wavefronts per
+// SIMD measured the same: the layer is bound by the bytes a compute unit pulls through its L1, not by latency).
+template <int ST, int D>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) void conv_own_kernel(
     const float *__restrict__ in, int64_t ld_in, float *__restrict__ out, int64_t ld_out,
     const float *__restrict__ Wp, const float *__restrict__ bias, const int32_t *__restrict__ rows,
@@ -1479,7 +1480,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
     first.k = __builtin_ctz(tmask);
     first.ch = 0;
     first.rest = tmask & (tmask - 1);
-    constexpr int D = OWN_DEPTH;
     Frag g[D], bw[D];
     Cursor ci = first, c0 = first;
 #pragma unroll
@@ -1858,7 +1858,8 @@ int launch_conv(const float *in, int64_t ld_in, int64_t in_rows, float *out, int
     }
     if (wide_planned && tiles * nbt >= g_own_min_units.load(std::memory_order_relaxed)) {
       // one wavefront per (tile, output block): enough units that every SIMD gets two or three
-      hipLaunchKernelGGL((conv_own_kernel<4>), dim3((unsigned)cdiv(tiles * nbt, 4)), dim3(256), 0, s, in, ld_in, out, ld_out, Wp,
+      hipLaunchKernelGGL((conv_own_kernel<4, 2>), dim3((unsigned)cdiv(tiles * nbt, 4)), dim3(256), 0, s, in, ld_in, out, ld_out, Wp,
+
                          bias, rows, d_n_rows, n_rows, Cin, Cout, nbt, nbtp, tile_flags, in_bytes, wp_bytes, ep, plan);
       INSC_LAUNCH_CHECK();
       return INSC_OK;
