@@ -472,7 +472,25 @@ __global__ __launch_bounds__((S == 1 ? CONV_WAVES : S) * 64) void conv_mfma_kern
 #pragma unroll
       for (int v = 0; v < 16; v++)
         acc[0][v] = __hip_atomic_load(all + v * 64 + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      for (int gg = 1; gg < G; gg++) {
+      // (the sums of up to three more blocks are requested together and added in block order: one
+      // trip to memory instead of one per block)
+      float pv[3][16];
+#pragma unroll
+      for (int gg = 1; gg < 4; gg++) {
+        if (gg < G) {
+#pragma unroll
+          for (int v = 0; v < 16; v++)
+            pv[gg - 1][v] = __hip_atomic_load(all + gg * 1024 + v * 64 + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+      }
+#pragma unroll
+      for (int gg = 1; gg < 4; gg++) {
+        if (gg < G) {
+#pragma unroll
+          for (int v = 0; v < 16; v++) acc[0][v] += pv[gg - 1][v];
+        }
+      }
+      for (int gg = 4; gg < G; gg++) {
 #pragma unroll
         for (int v = 0; v < 16; v++)
           acc[0][v] += __hip_atomic_load(all + gg * 1024 + v * 64 + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -1386,31 +1404,45 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NB * ST > 4
 // no wait for the slowest of four.  To give the bits of conv_mfma_kernel<1, 27, MAP_NBR, ST> the
 // wavefront keeps that kernel's ST partial sums - the items (k, ch) with (k * nch + ch) % ST == p, in
 // ascending order, bias in sum 0 - in ST accumulators and adds them in order at the end.  Units
-// follow the cost-ordered tile schedule, output blocks of a tile side by side, so the four
-// wavefronts of a block mostly work on the same tile and meet its map slice and gathered rows in L1.
+// follow the cost-ordered tile schedule, output blocks of a tile side by side on neighbouring SIMDs of
+// one compute unit, so they meet the tile's map slice and gathered rows in L1.
 // ---------------------------------------------------------------------------------------
 // D = items in flight per wavefront (2 with three wavefronts per SIMD; deeper rings at two wavefronts per
-// SIMD measured the same: the layer is bound by the bytes a compute unit pulls through its L1, not by latency).
+// SIMD measured the same, and so did fewer wavefronts that draw their units from a counter: what the
+// launch lasts is the SIMD with the largest sum of items, hence the fixed assignment below).
+constexpr int OWN_WAVES = 12;  // one block per compute unit, three wavefronts per SIMD
 template <int ST, int D>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) void conv_own_kernel(
+__global__ __launch_bounds__(OWN_WAVES * 64) __attribute__((amdgpu_waves_per_eu(3, 3))) void conv_own_kernel(
     const float *__restrict__ in, int64_t ld_in, float *__restrict__ out, int64_t ld_out,
     const float *__restrict__ Wp, const float *__restrict__ bias, const int32_t *__restrict__ rows,
     const int32_t *__restrict__ d_n_rows, int64_t n_rows, int Cin, int Cout, int nbt, int nbtp,
     const uint8_t *__restrict__ tile_flags, uint32_t in_bytes, uint32_t wp_bytes, BnEpilogue ep, TilePlan plan) {
   constexpr int K = 27;
   constexpr int NSTAGE = (TILE_M * K + 63) / 64;
-  __shared__ int nlb[4][TILE_M * K];
+  __shared__ int nlb[OWN_WAVES][TILE_M * K];
   const int64_t n = d_n_rows ? min((int64_t)*d_n_rows, n_rows) : n_rows;
   const int64_t ntiles = (n + TILE_M - 1) / TILE_M, units = ntiles * nbt;
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), lane = threadIdx.x & 63;
   const int r = lane & 31, h = lane >> 5;
-  const int64_t u = (int64_t)blockIdx.x * 4 + wave;
-  if (u >= units) return;  // (wavefronts are on their own: no workgroup barrier anywhere below)
-  const int tile = __builtin_amdgcn_readfirstlane(plan.sched[u / nbt]);
-  const int ob = (int)(u % nbt);
-  if (tile_flags && !tile_flags[tile]) return;
   const int nch = conv_nch(Cin);
   int *nl = nlb[wave];
+  // (wavefronts are on their own: no workgroup barrier anywhere below)
+  // One block per compute unit; wavefront w sits on SIMD w % 4, so bin = (block, w % 4) names a SIMD and
+  // round = w / 4 one of its three wavefronts.  Units come by falling cost: round 0 hands them to the bins
+  // in order, every later round in reverse order, so the SIMDs that drew the expensive units of round 0
+  // get the cheap ones afterwards (largest sum of a SIMD at 39k sites and 64 channels: 72 items against
+  // 90 when every SIMD takes three units in a row; 66 is the best any assignment reaches).
+  const int64_t nbins = (int64_t)gridDim.x * 4;
+  const int64_t bin = (int64_t)blockIdx.x * 4 + (wave & 3);
+  for (int64_t rnd = wave >> 2; rnd * nbins < units; rnd += OWN_WAVES / 4) {
+  const int64_t u = rnd * nbins + (rnd == 0 ? bin : nbins - 1 - bin);
+  if (u >= units) continue;
+  const int tile = __builtin_amdgcn_readfirstlane(plan.sched[u / nbt]);
+  const int ob = (int)(u % nbt);
+  if (tile_flags && !tile_flags[tile]) continue;
+  // (the slice of the last unit has been read to the end before this one overwrites it)
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
   // the tile's slice of the map: 27 coalesced runs of the plan
   int st[NSTAGE];
 #pragma unroll
@@ -1539,6 +1571,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
                                             (int)(ok ? __umul24((unsigned)rid[v], ldo24) + (uint32_t)c * 4u : BUF_OOB), 0, 0);
     }
   }
+  }  // units of this wavefront
 }
 
 __global__ void count_rules_kernel(const int32_t *__restrict__ map0, int K, const int32_t *__restrict__ rows,
@@ -1735,14 +1768,16 @@ int pack_weights(const float *W, int K, int Cin, int Cout, float *Wp, hipStream_
 // Launches of a wide 3^3 layer with at least this many (tile, output block) units and a tile
 // schedule go to the persistent kernel (below, one block per unit has all of them resident at once
 // anyway).  Both kernels give the same bits; the bound only moves time.
-static std::atomic<int64_t> g_pers_min_units{512};
+static std::atomic<int64_t> g_pers_min_units{650};
 // ... and with at least this many (group of four tiles, output block) units to the kernel whose blocks
 // share the weight tiles through LDS (faster from about 60k sites at 64 channels; same bits again).
 static std::atomic<int64_t> g_shared_min_units{896};
-// ... and, below that, with at least this many (tile, output block) units on the kernel that gives every
-// unit a wavefront of its own (faster than the persistent blocks from about 2000 units: 64 channels at
-// 35-55k sites, the second scale of the 150k-voxel U-Net; same bits again).
-static std::atomic<int64_t> g_own_min_units{2000};
+// ... and, below that, with at least this many (tile, output block) units - half as many again for layers
+// of more than 64 input channels, whose units are longer - on the kernel that gives every unit a wavefront
+// of its own.  (Below, too few SIMDs get a unit: at 64 channels 44 us against 40 us at 1318 units, 45
+// against 51 at 1730, 54 against 68 at 2452 = 39k sites; at 128 -> 64 channels 83 against 81 at 1730, 99
+// against 95 at 2044, 102 against 110 at 2452.  Same bits again.)
+static std::atomic<int64_t> g_own_min_units{1500};
 // Narrow 3^3 layers (Cin, Cout <= 32) with at least this many 32-row tiles run on the persistent
 // kernel that keeps the whole filter in LDS; smaller ones on the one-wavefront-per-tile kernel.
 // Same bits either way.
@@ -1856,11 +1891,12 @@ int launch_conv(const float *in, int64_t ld_in, int64_t in_rows, float *out, int
       INSC_LAUNCH_CHECK();
       return INSC_OK;
     }
-    if (wide_planned && tiles * nbt >= g_own_min_units.load(std::memory_order_relaxed)) {
-      // one wavefront per (tile, output block): enough units that every SIMD gets two or three
-      hipLaunchKernelGGL((conv_own_kernel<4, 2>), dim3((unsigned)cdiv(tiles * nbt, 4)), dim3(256), 0, s, in, ld_in, out, ld_out, Wp,
-
-                         bias, rows, d_n_rows, n_rows, Cin, Cout, nbt, nbtp, tile_flags, in_bytes, wp_bytes, ep, plan);
+    const int64_t own_min = g_own_min_units.load(std::memory_order_relaxed);
+    if (wide_planned && tiles * nbt >= (Cin > 64 ? own_min + own_min / 2 : own_min)) {
+      // one wavefront per (tile, output block): enough units that every SIMD gets one to three
+      hipLaunchKernelGGL((conv_own_kernel<4, 2>), dim3((unsigned)device_cus()), dim3(OWN_WAVES * 64), 0, s, in, ld_in, out,
+                         ld_out, Wp, bias, rows, d_n_rows, n_rows, Cin, Cout, nbt, nbtp, tile_flags, in_bytes, wp_bytes, ep,
+                         plan);
       INSC_LAUNCH_CHECK();
       return INSC_OK;
     }

@@ -1,4 +1,4 @@
-"""Pins the whole-network oracle (tests/oracle_net.py walking the module tree, and with it the
+"""Pins the whole-network oracle (oracle/oracle_net.py walking the module tree, and with it the
 wiring of the UNet builder) against a dense-grid PyTorch model written by hand from the
 reference's architecture text (sparseconvnet/networkArchitectures.py:202-300 with residual
 blocks, model.py:8-26): conv3d / conv_transpose3d / per-channel affine on [1, C, G, G, G] float64
