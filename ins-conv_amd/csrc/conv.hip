@@ -179,12 +179,14 @@ __device__ __forceinline__ float frag_at(const Frag &f, int s) {
 // handful of non-MFMA instructions per 16 MFMAs (ordinary VALU work does not overlap with MFMAs
 // on this part, so it is paid in matrix-core time).
 // Items in flight per wavefront (ring depth): whole-tile wavefronts, and wavefronts that share a
-// tile (few of them per SIMD, so each must cover more latency itself).
+// tile.  (For the latter a ring of four measured 4-10 % slower than one of two at every scale of the
+// U-Net: with 91 instead of 140 registers more wavefronts fit a SIMD, and a turn of the unrolled loop
+// wastes fewer steps past a wavefront's last item.)
 #ifndef INSC_CONV_DEPTH
 #define INSC_CONV_DEPTH 3
 #endif
 #ifndef INSC_CONV_DEPTH_SPLIT
-#define INSC_CONV_DEPTH_SPLIT 4
+#define INSC_CONV_DEPTH_SPLIT 2
 #endif
 
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
@@ -553,7 +555,10 @@ __global__ __launch_bounds__((S == 1 ? CONV_WAVES : S) * 64) void conv_mfma_kern
 // same MFMA sequence), so both kernels give the same bits.
 // ---------------------------------------------------------------------------------------
 constexpr int WL_WAVES = 12;
-constexpr int WL_DEPTH = 4;
+#ifndef INSC_WL_DEPTH
+#define INSC_WL_DEPTH 4
+#endif
+constexpr int WL_DEPTH = INSC_WL_DEPTH;
 constexpr int WL_MIN_TILES = 4096;  // smaller launches go to conv_mfma_kernel (default of the knob below)
 constexpr int WL_SCHED = 256;  // a block orders up to this many tiles of its own by cost
 
@@ -754,18 +759,20 @@ __global__ __launch_bounds__(WL_WAVES * 64) void conv_wlds_kernel(
       // The loads of the item D - 1 ahead and the weight tile of the next item are issued in the
       // shadow of this item's MFMAs (a dependent MFMA issues every 64 cycles; whatever sits between
       // two of them is free), in four slices pinned by scheduling barriers.
+      // (one turn of the loop covers both rings: D register slots for the gathered rows, two for the weights)
+      constexpr int TURN = D % 2 == 0 ? D : 2 * D;
       Frag bw[2];
       bw[0] = wread(kq[0]);
-      for (int i0 = 0; i0 < nitems; i0 += D) {
+      for (int i0 = 0; i0 < nitems; i0 += TURN) {
 #pragma unroll
-        for (int u = 0; u < D; u++) {
+        for (int u = 0; u < TURN; u++) {
           const bool real = i0 + u < nitems;
           const Frag &bf = bw[u % 2];
           __builtin_amdgcn_sched_barrier(0);
           if (real) {
 #pragma unroll
             for (int s = 0; s < 4; s++)
-              acc = __builtin_amdgcn_mfma_f32_32x32x2f32(frag_at(g[u], s), frag_at(bf, s), acc, 0, 0, 0);
+              acc = __builtin_amdgcn_mfma_f32_32x32x2f32(frag_at(g[u % D], s), frag_at(bf, s), acc, 0, 0, 0);
           }
           __builtin_amdgcn_sched_barrier(0);
           const int kn = next_k();
@@ -775,7 +782,7 @@ __global__ __launch_bounds__(WL_WAVES * 64) void conv_wlds_kernel(
           if (real) {
 #pragma unroll
             for (int s = 4; s < 8; s++)
-              acc = __builtin_amdgcn_mfma_f32_32x32x2f32(frag_at(g[u], s), frag_at(bf, s), acc, 0, 0, 0);
+              acc = __builtin_amdgcn_mfma_f32_32x32x2f32(frag_at(g[u % D], s), frag_at(bf, s), acc, 0, 0, 0);
           }
           __builtin_amdgcn_sched_barrier(0);
           {
@@ -788,7 +795,7 @@ __global__ __launch_bounds__(WL_WAVES * 64) void conv_wlds_kernel(
           if (real) {
 #pragma unroll
             for (int s = 8; s < 12; s++)
-              acc = __builtin_amdgcn_mfma_f32_32x32x2f32(frag_at(g[u], s), frag_at(bf, s), acc, 0, 0, 0);
+              acc = __builtin_amdgcn_mfma_f32_32x32x2f32(frag_at(g[u % D], s), frag_at(bf, s), acc, 0, 0, 0);
           }
           __builtin_amdgcn_sched_barrier(0);
           bw[(u + 1) % 2] = wread(kq[(u + 1) % D]);
@@ -796,7 +803,7 @@ __global__ __launch_bounds__(WL_WAVES * 64) void conv_wlds_kernel(
           if (real) {
 #pragma unroll
             for (int s = 12; s < 16; s++)
-              acc = __builtin_amdgcn_mfma_f32_32x32x2f32(frag_at(g[u], s), frag_at(bf, s), acc, 0, 0, 0);
+              acc = __builtin_amdgcn_mfma_f32_32x32x2f32(frag_at(g[u % D], s), frag_at(bf, s), acc, 0, 0, 0);
           }
           __builtin_amdgcn_sched_barrier(0);
         }
