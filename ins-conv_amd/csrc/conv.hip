@@ -310,15 +310,14 @@ __global__ __launch_bounds__((S == 1 ? CONV_WAVES : S) * 64) void conv_mfma_kern
 #pragma unroll
     for (int w = 0; w < S; w++) act |= wmask[w];
     act = (unsigned)__builtin_amdgcn_readfirstlane((int)act);
-    rest = 0;
-    for (unsigned m = act; m; m &= m - 1) {
-      const int k = __builtin_ctz(m);
-      const int c0 = (ws - k * nch) & (ST - 1);
-      if (c0 < nch) {
-        rest |= 1u << k;
-        nitems += (nch - c0 + ST - 1) / ST;
-      }
-    }
+    // (lane k looks at offset k: one ballot and a sum over the lanes instead of a scalar loop over the offsets)
+    const int c0 = (ws - lane * nch) & (ST - 1);
+    const bool has = lane < K && ((act >> (lane & 31)) & 1u) && c0 < nch;
+    rest = (unsigned)__ballot(has);
+    int cnt = has ? (nch - c0 + ST - 1) >> __builtin_ctz(ST) : 0;
+#pragma unroll
+    for (int d = 16; d > 0; d >>= 1) cnt += __shfl_xor(cnt, d, 64);
+    nitems = __builtin_amdgcn_readfirstlane(cnt);
   }
 
   f16v acc[NB];
