@@ -174,14 +174,14 @@ int insc_conv_ssc_plan(const float *d_in, int64_t ld_in, int64_t n_in_rows, floa
                        const int32_t *d_plan, int64_t plan_ld, const uint32_t *d_tmask, const int32_t *d_sched,
                        const int32_t *d_order, const int32_t *d_n_rows, int64_t n_rows, int Cin, int Cout,
                        void *stream);
-/* A 3^3 layer of 64..127 input channels with a tile schedule runs on persistent blocks once it has
- * at least `units` (tile, 32-column output block) pairs (default 650); below, one block per pair.
- * With at least `units` (four consecutive tiles, output block) pairs (default 896) it runs on the
- * kernel whose blocks share the weight tiles through LDS.  Same bits in all cases: tuning and
- * test knobs with no counterpart in the reference. */
+/* Launch policy of a 3^3 layer of 64..159 input channels with a tile schedule: by default one block per
+ * (tile, 32-column output block) pair; persistent blocks once it has at least `units` pairs (off by
+ * default: the one-block-per-pair kernel measures faster at every size); with at least `units` (four
+ * consecutive tiles, output block) pairs (default 896) the kernel whose blocks share the weight tiles
+ * through LDS.  Same bits in all cases: tuning and test knobs with no counterpart in the reference. */
 int insc_conv_set_persistent_min_units(int64_t units);
 int insc_conv_set_shared_weights_min_units(int64_t units);
-/* ... and between the two, from `units` (tile, output block) pairs up (default 1500; half as many again
+/* ... and between the two, from `units` (tile, output block) pairs up (default 2400; half as many again
  * for more than 64 input channels), on the kernel that gives every pair a wavefront of its own.  Same
  * bits again. */
 int insc_conv_set_wavefront_per_unit_min_units(int64_t units);

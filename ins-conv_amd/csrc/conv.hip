@@ -229,16 +229,36 @@ __global__ __launch_bounds__((S == 1 ? CONV_WAVES : S) * 64) void conv_mfma_kern
   const int r = lane & 31, h = lane >> 5;
   // (with a tile schedule the blocks of a split launch take the tiles by falling cost: blocks go to the
   // compute units round robin, so every unit then holds a mix of expensive and cheap tiles)
-  const int64_t slot = S == 1 ? (int64_t)blockIdx.x * WAVES + wave : (int64_t)blockIdx.x;
+  // Which (tile slot, output block, share of the split) this block works on.  Split launches with a
+  // tile schedule renumber their blocks: the hardware hands out blocks in the order x, y, z, round robin
+  // over the compute units, so block L goes - all blocks being resident at once - to unit L mod CUS.
+  // Ranked by cost (tile slot major: the output blocks and shares of a tile cost the same), round 0 of
+  // CUS blocks takes ranks in order and every other round in reverse order, so that the compute unit that
+  // drew the most expensive block of one round gets the cheapest of the next.
+  unsigned bx = blockIdx.x, by = blockIdx.y, bz = blockIdx.z;
+  if (S > 1 && MODE == MAP_NBR && K == 27 && plan.map != nullptr && plan.sched != nullptr) {
+    constexpr unsigned CUS = 256;
+    const unsigned gyz = gridDim.y * gridDim.z;
+    const unsigned total = (unsigned)((n + TILE_M - 1) / TILE_M) * gyz;
+    const unsigned L = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+    if (L >= total) return;  // (launches are sized by an upper bound of the row count)
+    const unsigned rnd = L / CUS, pos = L % CUS, m = min(CUS, total - rnd * CUS);
+    const unsigned R = rnd * CUS + ((rnd & 1u) ? m - 1 - pos : pos);
+    bx = R / gyz;
+    const unsigned rem = R - bx * gyz;
+    by = rem / gridDim.z;
+    bz = rem - by * gridDim.z;
+  }
+  const int64_t slot = S == 1 ? (int64_t)bx * WAVES + wave : (int64_t)bx;
   const bool by_cost = MODE == MAP_NBR && K == 27 && plan.map != nullptr && plan.sched != nullptr && slot * TILE_M < n;
   const int64_t t0 = (by_cost ? (int64_t)plan.sched[slot] : slot) * TILE_M;
-  const int cb0 = blockIdx.y * NB;  // first output-channel block of this column group
+  const int cb0 = by * NB;  // first output-channel block of this column group
   const int nch = conv_nch(Cin);
   // the items of a tile are dealt to S wavefronts in each of G = gridDim.z blocks
-  const int G = S == 1 ? 1 : (int)gridDim.z, ST = S * G, ws = wave * G + (S == 1 ? 0 : (int)blockIdx.z);
+  const int G = S == 1 ? 1 : (int)gridDim.z, ST = S * G, ws = wave * G + (S == 1 ? 0 : (int)bz);
 
   // blocks beyond the row count leave at once (launches are sized by an upper bound of it)
-  if ((S == 1 ? (int64_t)blockIdx.x * WAVES : (int64_t)blockIdx.x) * TILE_M >= n) return;
+  if ((S == 1 ? (int64_t)bx * WAVES : (int64_t)bx) * TILE_M >= n) return;
   // a tile is skipped when it lies beyond the row count or, with tile flags, is not marked
   const bool live = t0 < n && (!tile_flags || tile_flags[t0 >> 5]);
   int my_row = -1;
@@ -457,8 +477,8 @@ __global__ __launch_bounds__((S == 1 ? CONV_WAVES : S) * 64) void conv_mfma_kern
       // The G blocks of a (tile, output block) leave their sums in memory; the one that arrives
       // last adds them in block order (so the result does not depend on the arrival order),
       // writes the rows and puts the arrival counter back to zero.  Nobody waits for anybody.
-      const int unit = (int)(blockIdx.x * gridDim.y + blockIdx.y);
-      float *mine = part + ((int64_t)unit * G + blockIdx.z) * 1024;
+      const int unit = (int)(bx * gridDim.y + by);
+      float *mine = part + ((int64_t)unit * G + bz) * 1024;
 #pragma unroll
       // (stores and loads of the sums go past the XCD-local L2 - device-scope atomics - so that no
       // cache write-back or invalidation is needed: a full fence flushes the whole L2 and costs
@@ -1771,19 +1791,19 @@ int pack_weights(const float *W, int K, int Cin, int Cout, float *Wp, hipStream_
   return INSC_OK;
 }
 
-// Launches of a wide 3^3 layer with at least this many (tile, output block) units and a tile
-// schedule go to the persistent kernel (below, one block per unit has all of them resident at once
-// anyway).  Both kernels give the same bits; the bound only moves time.
-static std::atomic<int64_t> g_pers_min_units{650};
-// ... and with at least this many (group of four tiles, output block) units to the kernel whose blocks
-// share the weight tiles through LDS (faster from about 60k sites at 64 channels; same bits again).
+// Launch policy of wide 3^3 layers (64..159 input channels, a tile schedule).  All kernels give the same
+// bits; the bounds only move time.
+// The persistent kernel is off by default: since the one-block-per-unit kernel keeps two items in flight
+// and numbers its blocks for balance across the compute units it is the faster one at every size measured
+// (96 -> 96 at 10k sites: 37 us against 43 us; 64 -> 64 at 21k sites: 36 against 46).
+static std::atomic<int64_t> g_pers_min_units{INT64_MAX};
+// With at least this many (group of four tiles, output block) units: the kernel whose blocks share the
+// weight tiles through LDS (faster from about 60k sites at 64 channels).
 static std::atomic<int64_t> g_shared_min_units{896};
-// ... and, below that, with at least this many (tile, output block) units - half as many again for layers
-// of more than 64 input channels, whose units are longer - on the kernel that gives every unit a wavefront
-// of its own.  (Below, too few SIMDs get a unit: at 64 channels 44 us against 40 us at 1318 units, 45
-// against 51 at 1730, 54 against 68 at 2452 = 39k sites; at 128 -> 64 channels 83 against 81 at 1730, 99
-// against 95 at 2044, 102 against 110 at 2452.  Same bits again.)
-static std::atomic<int64_t> g_own_min_units{1500};
+// Below that, with at least this many (tile, output block) units - half as many again for layers of more
+// than 64 input channels, whose units are longer - the kernel that gives every unit a wavefront of its own
+// (64 -> 64: 55 us against 57 us at 2452 units = 39k sites, 54 against 48 at 2044).
+static std::atomic<int64_t> g_own_min_units{2400};
 // Narrow 3^3 layers (Cin, Cout <= 32) with at least this many 32-row tiles run on the persistent
 // kernel that keeps the whole filter in LDS; smaller ones on the one-wavefront-per-tile kernel.
 // Same bits either way.

@@ -27,10 +27,10 @@ def persistent_min_units(request):
     lib.insc_conv_set_filter_lds_min_tiles(request.param[2])
     lib.insc_conv_set_wavefront_per_unit_min_units(request.param[3])
     yield request.param
-    lib.insc_conv_set_persistent_min_units(650)
+    lib.insc_conv_set_persistent_min_units((1 << 63) - 1)
     lib.insc_conv_set_shared_weights_min_units(896)
     lib.insc_conv_set_filter_lds_min_tiles(4096)
-    lib.insc_conv_set_wavefront_per_unit_min_units(1500)
+    lib.insc_conv_set_wavefront_per_unit_min_units(2400)
 
 
 @pytest.mark.parametrize("levels,m", [(3, 16), (7, 32)])

@@ -118,9 +118,9 @@ def test_persistent_kernels_give_the_bits_of_the_per_tile_kernel(S, orc, Cin, Co
         d.fill_(9.0)
         S.ssc_rows_planned(feats, d, W, bt, sc, m.ssc_plan(sc))
     finally:
-        lib.insc_conv_set_persistent_min_units(650)
+        lib.insc_conv_set_persistent_min_units((1 << 63) - 1)
         lib.insc_conv_set_shared_weights_min_units(896)
-        lib.insc_conv_set_wavefront_per_unit_min_units(1500)
+        lib.insc_conv_set_wavefront_per_unit_min_units(2400)
     assert torch.equal(a, c)
     assert torch.equal(d, c)
     assert torch.equal(e, c)
@@ -208,9 +208,9 @@ def test_persistent_kernels_on_tiny_and_ragged_scenes(S, n):
             S.ssc_rows_planned(feats, o, W, None, sc, m.ssc_plan(sc))
             outs.append(o)
     finally:
-        lib.insc_conv_set_persistent_min_units(650)
+        lib.insc_conv_set_persistent_min_units((1 << 63) - 1)
         lib.insc_conv_set_shared_weights_min_units(896)
-        lib.insc_conv_set_wavefront_per_unit_min_units(1500)
+        lib.insc_conv_set_wavefront_per_unit_min_units(2400)
     assert torch.equal(outs[0], outs[1])
     assert torch.equal(outs[0], outs[2])
     assert torch.equal(outs[0], outs[3])
