@@ -183,7 +183,7 @@ __device__ __forceinline__ float frag_at(const Frag &f, int s) {
 // U-Net: with 91 instead of 140 registers more wavefronts fit a SIMD, and a turn of the unrolled loop
 // wastes fewer steps past a wavefront's last item.)
 #ifndef INSC_CONV_DEPTH
-#define INSC_CONV_DEPTH 3
+#define INSC_CONV_DEPTH 2
 #endif
 #ifndef INSC_CONV_DEPTH_SPLIT
 #define INSC_CONV_DEPTH_SPLIT 2
@@ -649,11 +649,22 @@ __global__ __launch_bounds__(WL_WAVES * 64) void conv_wlds_kernel(
   // The wavefronts of a block draw its tiles from a counter in LDS
   // (tile costs differ by 3x: a fixed deal per wavefront leaves the slowest one far behind).
   // draw(): the next tile of this block that has work, or ntiles.
+  // With fewer than three tiles per wavefront the draws ahead of the tile pipeline (up to three tiles
+  // in hand per wavefront) would leave late wavefronts with nothing: then the turns are dealt instead,
+  // wavefront w takes w, w + WL_WAVES, ...
+  const bool dealt = my_tiles < 3 * WL_WAVES;
+  int my_turn = wave;
   auto draw = [&]() -> int64_t {
     for (;;) {
-      int v = 0;
-      if (lane == 0) v = atomicAdd(&next_turn, 1);
-      const int turn = __builtin_amdgcn_readfirstlane(v);
+      int turn;
+      if (dealt) {
+        turn = my_turn;
+        my_turn += WL_WAVES;
+      } else {
+        int v = 0;
+        if (lane == 0) v = atomicAdd(&next_turn, 1);
+        turn = __builtin_amdgcn_readfirstlane(v);
+      }
       if (turn >= my_tiles) return ntiles;
       const int64_t t = (int64_t)(lpt ? sched_l[turn] : turn) * gridDim.x + brank;
       if (!tile_flags || tile_flags[t]) return t;
