@@ -1899,7 +1899,9 @@ int launch_conv(const float *in, int64_t ld_in, int64_t in_rows, float *out, int
     if (G > 1) S = 4;
     const bool wide_planned = mode == MAP_NBR && K == 27 && S == 4 && G == 1 && !lat && plan.map && plan.sched &&
                               small_ids && ep.ldr * 4 < (1 << 24) && out_rows * ep.ldr * 4 < (int64_t)BUF_OOB;
-    if (wide_planned && cdiv(tiles, 4) * nbt >= g_shared_min_units.load(std::memory_order_relaxed)) {
+    // (a layer with one output block has half the weight bytes per gathered row to share: 64 -> 32 at 150k
+    // sites takes 95 us there against 88 us with a wavefront per unit, so its bound is twice as high)
+    if (wide_planned && cdiv(tiles, 4) * nbt >= g_shared_min_units.load(std::memory_order_relaxed) * (nbt == 1 ? 2 : 1)) {
       // blocks of four tiles that share the weight tiles through LDS
       // with enough units left, two output blocks per gathered chunk (eight accumulators: two
       // wavefronts per SIMD instead of three, but a third fewer bytes per MFMA)
