@@ -221,7 +221,7 @@ __global__ __launch_bounds__((S == 1 ? CONV_WAVES : S) * 64) void conv_mfma_kern
   static_assert(S == 1 || NB == 1, "split tiles use one output block per wavefront");
   constexpr int WAVES = S == 1 ? CONV_WAVES : S;
   __shared__ int nbl[S == 1 ? WAVES : 1][TILE_M * K];
-  __shared__ float red[S > 1 ? S - 1 : 1][S > 1 ? 16 * 64 : 1];
+  __shared__ float red[S > 1 ? S : 1][S > 1 ? 16 * 64 : 1];  // (slot S - 1: only when all wavefronts share the tail)
   __shared__ unsigned wmask[S];
   const int64_t n = d_n_rows ? min((int64_t)*d_n_rows, n_rows) : n_rows;
   // (the wavefront's number as a scalar: the item cursor below then runs on the scalar unit)
@@ -355,7 +355,7 @@ __global__ __launch_bounds__((S == 1 ? CONV_WAVES : S) * 64) void conv_mfma_kern
 #pragma unroll
   for (int b = 0; b < NB; b++) {
     const int c = (cb0 + b) * 32 + r;
-    const bool on = ep.out2 && c < Cout && (S == 1 || wave == 0);
+    const bool on = ep.out2 && c < Cout;
     ew[b] = on ? ep.w[c] : 0.0f;
     eb[b] = on ? ep.b[c] : 0.0f;
   }
@@ -461,63 +461,88 @@ __global__ __launch_bounds__((S == 1 ? CONV_WAVES : S) * 64) void conv_mfma_kern
   }
 
   if (S > 1) {
-    // partial sums of wavefronts 1..S-1 go through LDS and are added in wavefront order
-    if (wave > 0) {
+    // Every wavefront leaves its partial sum in LDS; each then adds up - in wavefront order - and
+    // finishes 16 / S of the rows of the tile, so that the tail of the block (partial sums through
+    // memory, residual loads, two stores per row with a fused batch norm) is shared by all of them.
+    // D layout of the 32x32 MFMA: lane holds column (lane & 31), rows 8*(v/4) + 4*(lane>>5) + (v&3).
+    constexpr int NV = 16 / (S > 1 ? S : 16);
 #pragma unroll
-      for (int v = 0; v < 16; v++) red[wave - 1][v * 64 + lane] = acc[0][v];
-    }
+    for (int v = 0; v < 16; v++) red[wave][v * 64 + lane] = acc[0][v];
     __syncthreads();
-    if (wave > 0) return;
+    float a[NV];
+    int rid[NV];
 #pragma unroll
-    for (int w = 0; w < S - 1; w++) {
+    for (int j = 0; j < NV; j++) {
+      const int v = wave * NV + j;
+      a[j] = red[0][v * 64 + lane];
 #pragma unroll
-      for (int v = 0; v < 16; v++) acc[0][v] += red[w][v * 64 + lane];
+      for (int w = 1; w < S; w++) a[j] += red[w][v * 64 + lane];
+      rid[j] = __shfl(my_row, 8 * (v >> 2) + 4 * h + (v & 3), 64);
     }
     if (G > 1) {
-      // The G blocks of a (tile, output block) leave their sums in memory; the one that arrives
-      // last adds them in block order (so the result does not depend on the arrival order),
-      // writes the rows and puts the arrival counter back to zero.  Nobody waits for anybody.
-      const int unit = (int)(bx * gridDim.y + by);
-      float *mine = part + ((int64_t)unit * G + bz) * 1024;
-#pragma unroll
+      // The G blocks of a (tile, output block) leave their sums in memory; of the G wavefronts that
+      // hold the same rows, the one that arrives last adds the sums in block order (so the result
+      // does not depend on the arrival order), writes the rows and puts the arrival counter back to
+      // zero.  Nobody waits for anybody.
       // (stores and loads of the sums go past the XCD-local L2 - device-scope atomics - so that no
       // cache write-back or invalidation is needed: a full fence flushes the whole L2 and costs
       // more than the layer)
-      for (int v = 0; v < 16; v++)
-        __hip_atomic_store(mine + v * 64 + lane, acc[0][v], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const int unit = (int)(bx * gridDim.y + by);
+      float *mine = part + ((int64_t)unit * G + bz) * 1024 + (wave * NV) * 64 + lane;
+#pragma unroll
+      for (int j = 0; j < NV; j++) __hip_atomic_store(mine + j * 64, a[j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the stores have been acknowledged
       int old = 0;
-      if (lane == 0) old = atomicAdd(pcount + unit, 1);
+      if (lane == 0) old = atomicAdd(pcount + unit * S + wave, 1);
       if (__builtin_amdgcn_readfirstlane(old) != G - 1) return;
-      const float *all = part + (int64_t)unit * G * 1024;
+      const float *all = part + (int64_t)unit * G * 1024 + (wave * NV) * 64 + lane;
+      // (the sums of up to four blocks are requested together and added in block order: one trip to
+      // memory instead of one per block)
+      float pv[4][NV];
 #pragma unroll
-      for (int v = 0; v < 16; v++)
-        acc[0][v] = __hip_atomic_load(all + v * 64 + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      // (the sums of up to three more blocks are requested together and added in block order: one
-      // trip to memory instead of one per block)
-      float pv[3][16];
-#pragma unroll
-      for (int gg = 1; gg < 4; gg++) {
+      for (int gg = 0; gg < 4; gg++) {
         if (gg < G) {
 #pragma unroll
-          for (int v = 0; v < 16; v++)
-            pv[gg - 1][v] = __hip_atomic_load(all + gg * 1024 + v * 64 + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          for (int j = 0; j < NV; j++)
+            pv[gg][j] = __hip_atomic_load(all + gg * 1024 + j * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
       }
 #pragma unroll
+      for (int j = 0; j < NV; j++) a[j] = pv[0][j];
+#pragma unroll
       for (int gg = 1; gg < 4; gg++) {
         if (gg < G) {
 #pragma unroll
-          for (int v = 0; v < 16; v++) acc[0][v] += pv[gg - 1][v];
+          for (int j = 0; j < NV; j++) a[j] += pv[gg][j];
         }
       }
       for (int gg = 4; gg < G; gg++) {
 #pragma unroll
-        for (int v = 0; v < 16; v++)
-          acc[0][v] += __hip_atomic_load(all + gg * 1024 + v * 64 + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        for (int j = 0; j < NV; j++)
+          a[j] += __hip_atomic_load(all + gg * 1024 + j * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
-      if (lane == 0) pcount[unit] = 0;
+      if (lane == 0) pcount[unit * S + wave] = 0;
     }
+    const int c = cb0 * 32 + r;
+    if (c >= Cout) return;
+    if (ep.res) {
+      float rv[NV];
+#pragma unroll
+      for (int j = 0; j < NV; j++) rv[j] = rid[j] >= 0 ? ep.res[(int64_t)rid[j] * ep.ldr + c] : 0.0f;
+#pragma unroll
+      for (int j = 0; j < NV; j++) a[j] += rv[j];
+      __builtin_amdgcn_sched_barrier(0);  // (the sums stay above the stores)
+    }
+#pragma unroll
+    for (int j = 0; j < NV; j++) {
+      if (rid[j] < 0) continue;
+      if (out) out[(int64_t)rid[j] * ld_out + c] = a[j];
+      if (ep.out2) {
+        const float y = fmaf(a[j], ew[0], eb[0]);  // fused batch norm + leaky ReLU
+        ep.out2[(int64_t)rid[j] * ep.ld2 + c] = y * ((y > 0.0f) ? 1.0f : ep.leak);
+      }
+    }
+    return;
   }
 
   // D layout of the 32x32 MFMA: lane holds column (lane & 31), rows 8*(v/4) + 4*(lane>>5) + (v&3).
@@ -1962,7 +1987,7 @@ int launch_conv(const float *in, int64_t ld_in, int64_t in_rows, float *out, int
       int rc = workspace(WS_CONV, s, units * G * 1024 * sizeof(float), &ws);
       if (rc) return rc;
       part = (float *)ws;
-      if ((rc = zero_counters(s, units, &pcount))) return rc;
+      if ((rc = zero_counters(s, units * (size_t)S, &pcount))) return rc;  // one counter per wavefront of a unit
     }
     bool shape_ok = true;
 #define INSC_CONV_LAUNCH(NBV, KV, MV, SV)                                                                       \
