@@ -496,11 +496,12 @@ __global__ __launch_bounds__((S == 1 ? CONV_WAVES : S) * 64) void conv_mfma_kern
       if (lane == 0) old = atomicAdd(pcount + unit * S + wave, 1);
       if (__builtin_amdgcn_readfirstlane(old) != G - 1) return;
       const float *all = part + (int64_t)unit * G * 1024 + (wave * NV) * 64 + lane;
-      // (the sums of up to four blocks are requested together and added in block order: one trip to
+      // (the sums of up to eight blocks are requested together and added in block order: one trip to
       // memory instead of one per block)
-      float pv[4][NV];
+      constexpr int GP = 8;
+      float pv[GP][NV];
 #pragma unroll
-      for (int gg = 0; gg < 4; gg++) {
+      for (int gg = 0; gg < GP; gg++) {
         if (gg < G) {
 #pragma unroll
           for (int j = 0; j < NV; j++)
@@ -510,13 +511,13 @@ __global__ __launch_bounds__((S == 1 ? CONV_WAVES : S) * 64) void conv_mfma_kern
 #pragma unroll
       for (int j = 0; j < NV; j++) a[j] = pv[0][j];
 #pragma unroll
-      for (int gg = 1; gg < 4; gg++) {
+      for (int gg = 1; gg < GP; gg++) {
         if (gg < G) {
 #pragma unroll
           for (int j = 0; j < NV; j++) a[j] += pv[gg][j];
         }
       }
-      for (int gg = 4; gg < G; gg++) {
+      for (int gg = GP; gg < G; gg++) {
 #pragma unroll
         for (int j = 0; j < NV; j++)
           a[j] += __hip_atomic_load(all + gg * 1024 + j * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -1916,7 +1917,9 @@ int launch_conv(const float *in, int64_t ld_in, int64_t in_rows, float *out, int
     const int NB = (S == 1 && Cin >= 96) ? 1 : NB0;
     // (the split across blocks is for scales with few tiles; in a U-Net the width grows with the depth,
     // and a layer that narrows to at most 96 channels sits at a fine scale with many tiles)
-    int G = (split && K == 27 && Cout > 96) ? (Cin >= 160 ? 4 : Cin >= 128 ? 2 : 1) : 1;
+    // (eight blocks from 224 channels: the coarsest scale of a seven-scale U-Net, three tiles, where a
+    // wavefront's item loop is most of the launch - 15 -> 12 us; at 192 channels it gains nothing)
+    int G = (split && K == 27 && Cout > 96) ? (Cin >= 224 ? 8 : Cin >= 160 ? 4 : Cin >= 128 ? 2 : 1) : 1;
     if (lat) {
       G = Cin >= 128 ? 4 : Cin >= 64 ? 2 : 1;
       S = 4;
