@@ -608,9 +608,90 @@ __global__ __launch_bounds__(1024) void order_append_sorted_batch_kernel(OrderBa
   const OrderJob &j = b.job[blockIdx.x];
   order_append_sorted_body<MODE>(j.d_n, j.coords, j.nbr, j.offset, j.aux, j.order, j.pos, key);
 }
+// The new sites in the order grouped by the position inside the parent cell (eight groups, each in the
+// sequence of the processing order just written): a stable counting sort of that order, which gives
+// what sorting by (group, position) gives.  One workgroup of 1024 threads, thread t owns the positions
+// 8t .. 8t+7 of the new sites; counts per group travel as eight 16-bit fields in two 64-bit words
+// (at most SORT_NEW_MAX = 8192 sites, so no field overflows).
+__device__ __forceinline__ void order_append_grouped_body(const int32_t *__restrict__ d_n,
+                                                          const int32_t *__restrict__ offset,
+                                                          const int32_t *__restrict__ order,
+                                                          int32_t *__restrict__ bo_order, int32_t *__restrict__ bo_pos,
+                                                          uint64_t *lds) {
+  const int first = d_n[1], n = d_n[0] - first;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  if (n <= 0) return;
+  if (n > SORT_NEW_MAX) {
+    for (int i = tid; i < n; i += 1024) {
+      bo_order[first + i] = first + i;
+      bo_pos[first + i] = first + i;
+    }
+    return;
+  }
+  int v[8], o[8];
+  uint64_t c0 = 0, c1 = 0;  // groups 0..3 and 4..7
+#pragma unroll
+  for (int e = 0; e < 8; e++) {
+    const int q = tid * 8 + e;
+    v[e] = q < n ? order[first + q] : -1;
+    o[e] = v[e] >= 0 ? (offset[v[e]] & 7) : 0;
+    if (v[e] >= 0) {
+      if (o[e] < 4) c0 += 1ull << (16 * o[e]);
+      else c1 += 1ull << (16 * (o[e] - 4));
+    }
+  }
+  // inclusive scan over the threads: inside a wavefront, then over the 16 wavefronts through LDS
+  uint64_t s0 = c0, s1 = c1;
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const uint64_t a0 = __shfl_up(s0, d, 64), a1 = __shfl_up(s1, d, 64);
+    if (lane >= d) {
+      s0 += a0;
+      s1 += a1;
+    }
+  }
+  if (lane == 63) {
+    lds[wave * 2] = s0;
+    lds[wave * 2 + 1] = s1;
+  }
+  __syncthreads();
+  uint64_t w0 = 0, w1 = 0, t0 = 0, t1 = 0;  // sums of the wavefronts before this one; of all
+  for (int w = 0; w < 16; w++) {
+    const uint64_t a0 = lds[w * 2], a1 = lds[w * 2 + 1];
+    if (w < wave) {
+      w0 += a0;
+      w1 += a1;
+    }
+    t0 += a0;
+    t1 += a1;
+  }
+  const uint64_t e0 = w0 + s0 - c0, e1 = w1 + s1 - c1;  // exclusive: sites of each group before this thread
+  int base[8], run[8];
+  int acc = 0;
+#pragma unroll
+  for (int g = 0; g < 8; g++) {
+    base[g] = acc;
+    acc += (int)(((g < 4 ? t0 : t1) >> (16 * (g & 3))) & 0xFFFF);
+    run[g] = (int)(((g < 4 ? e0 : e1) >> (16 * (g & 3))) & 0xFFFF);
+  }
+#pragma unroll
+  for (int e = 0; e < 8; e++) {
+    if (v[e] < 0) continue;
+    int dest = 0;
+#pragma unroll
+    for (int g = 0; g < 8; g++) {
+      if (o[e] == g) {
+        dest = first + base[g] + run[g];
+        run[g]++;
+      }
+    }
+    bo_order[dest] = v[e];
+    bo_pos[v[e]] = dest;
+  }
+}
+
 // both orders of a scale by one workgroup: the processing order of the 3^3 layers, then - where the
-// scale has a coarser one above it - the order grouped by the position inside the parent cell, which
-// sorts by the position in the first
+// scale has a coarser one above it - the order grouped by the position inside the parent cell
 struct OrderBothJob {
   const int32_t *d_n, *coords, *nbr, *offset;  // offset null: no second order
   int32_t *order, *pos, *bo_order, *bo_pos;
@@ -623,8 +704,8 @@ __global__ __launch_bounds__(1024) void order_append_both_batch_kernel(OrderBoth
   const OrderBothJob &j = b.job[blockIdx.x];
   order_append_sorted_body<0>(j.d_n, j.coords, j.nbr, nullptr, nullptr, j.order, j.pos, key);
   if (!j.offset) return;
-  __syncthreads();  // the positions written above are read below, and the keys are reused
-  order_append_sorted_body<1>(j.d_n, nullptr, nullptr, j.offset, j.pos, j.bo_order, j.bo_pos, key);
+  __syncthreads();  // the order written above is read below (by other threads than wrote it), and the LDS is reused
+  order_append_grouped_body(j.d_n, j.offset, j.order, j.bo_order, j.bo_pos, key);
 }
 
 int order_append_new_sites(const insc_grid *g, int32_t *d_order, int32_t *d_pos, int64_t n_new_upper, hipStream_t s) {
