@@ -121,7 +121,7 @@ def ssc_workload(device, channels=(32, 64)):
     return step, info, (xs[0], stacks[0])
 
 
-def conv_roofline(device, reps=30, warm=200):
+def conv_roofline(device, reps=200, warm=30):
     """Average duration of the 32-channel submanifold convolution kernel at 500k voxels and the
     roofline figures derived from it."""
     import torch
