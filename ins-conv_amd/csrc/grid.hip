@@ -777,10 +777,14 @@ __global__ __launch_bounds__(256) void frame_claim_kernel(FrameInsertArgs a, con
       r = REC_SITE | (uint32_t)raw.z;
       break;
     }
+    const bool seen = k == key;  // the slot already held this key when it was read
     if (k == INSC_EMPTY_KEY) k = atomicCAS(&L.table[s].key, INSC_EMPTY_KEY, (unsigned long long)key);
     if (k == INSC_EMPTY_KEY || k == key) {
       r = (uint32_t)s;
-      atomicMin(&L.table[s].val, VAL_PENDING + p);
+      // (the claim of a smaller row that this row has seen stands: the value only ever goes down, so a
+      // stale read errs on the side of one more atomic.  At a coarse scale thousands of rows of a full
+      // frame fall into one cell, and same-address atomics are served one at a time.)
+      if (!(seen && raw.z >= VAL_PENDING && raw.z <= VAL_PENDING + p)) atomicMin(&L.table[s].val, VAL_PENDING + p);
       break;
     }
     s = (s + 1) & L.mask;
@@ -906,12 +910,102 @@ __global__ void frame_link_kernel(FrameInsertArgs a, int P, const int32_t *__res
   if (par >= 0 && F.child) F.child[(int64_t)par * 8 + F.offset[i]] = i;
 }
 
+// Frames of more points than one workgroup per scale can rank: the same three steps with the ranking
+// done by a prefix sum over all (scale, row) pairs at once - flag (is this row the winner of its
+// cell; if not, which row is), scan, assign (a winner publishes its id and the site's coordinates;
+// every row works out its site from the prefix sums alone, a loser through its winner's row, so no
+// row has to wait for another one's write).
+__global__ __launch_bounds__(256) void frame_flag_kernel(FrameInsertArgs a, int P, const uint32_t *__restrict__ rec,
+                                                         int32_t *__restrict__ flag, int32_t *__restrict__ rep,
+                                                         int32_t *__restrict__ n_before) {
+  const int l = blockIdx.y;
+  const FrameLevelDev &L = a.lv[l];
+  const int p = blockIdx.x * 256 + threadIdx.x;
+  if (p == 0) {
+    n_before[l] = L.d_n[0];
+    if (l == 0) flag[(int64_t)a.n_levels * P] = 0;  // (one entry past the end: the scan then leaves the grand total there)
+  }
+  if (p >= P) return;
+  const int64_t idx = (int64_t)l * P + p;
+  const uint32_t r = rec[idx];
+  int f = 0, w = -1;
+  if (r != REC_NONE && !(r & REC_SITE)) {
+    const int v = table_val(L.table, (int64_t)r);
+    if (v == VAL_PENDING + p)
+      f = 1;
+    else if (v >= VAL_PENDING && v != VAL_UNSET)
+      w = v - VAL_PENDING;
+  }
+  flag[idx] = f;
+  rep[idx] = w;
+}
+
+__global__ __launch_bounds__(256) void frame_assign_kernel(FrameInsertArgs a, const int32_t *__restrict__ coords_in,
+                                                           int cols, int P, const int32_t *__restrict__ bad,
+                                                           int32_t frame, int32_t *__restrict__ sop,
+                                                           int32_t *__restrict__ site, const uint32_t *__restrict__ rec,
+                                                           const int32_t *__restrict__ excl,
+                                                           const int32_t *__restrict__ rep,
+                                                           const int32_t *__restrict__ n_before_all, int32_t *h_counts) {
+  const int l = blockIdx.y;
+  const FrameLevelDev &L = a.lv[l];
+  const int p = blockIdx.x * 256 + threadIdx.x;
+  const int n_before = n_before_all[l];
+  const int64_t lp = (int64_t)l * P;
+  const bool dropped = bad[0] == frame;
+  if (p == 0) {
+    int total = dropped ? 0 : excl[lp + P] - excl[lp];
+    if (total > L.capacity - n_before) total = (int)(L.capacity - n_before);  // (the error flag is up)
+    L.d_n[1] = n_before;
+    L.d_n[0] = n_before + total;
+    if (h_counts) {
+      h_counts[2 * l] = n_before + total;
+      h_counts[2 * l + 1] = dropped ? 0 : __hip_atomic_load(L.d_err, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (l == 0) h_counts[2 * a.n_levels] = dropped ? frame : 0;
+    }
+  }
+  if (p >= P) return;
+  const uint32_t r = rec[lp + p];
+  int st = -1;
+  if (dropped) {
+    // the frame is dropped: its claims leave the table, no row gets a site
+    if (r != REC_NONE && !(r & REC_SITE)) {
+      __hip_atomic_store(&L.table[r].val, VAL_UNSET, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(&L.table[r].key, INSC_EMPTY_KEY, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  } else if (r != REC_NONE) {
+    if (r & REC_SITE) {
+      st = (int)(r & ~REC_SITE);
+    } else {
+      const int e = excl[lp + p];
+      const bool win = excl[lp + p + 1] - e == 1;
+      const int wrow = win ? p : rep[lp + p];
+      if (wrow >= 0) {
+        const int id = n_before + (win ? e : excl[lp + wrow]) - excl[lp];
+        if (id < L.capacity) {
+          st = id;
+          if (win) {
+            const int4 c = frame_point(coords_in, cols, p, l);
+            __hip_atomic_store(&L.table[r].val, id, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            reinterpret_cast<int4 *>(L.coords)[id] = c;
+            if (L.offset) L.offset[id] = (c.x & 1) * 4 + (c.y & 1) * 2 + (c.z & 1);
+          }
+        } else if (win) {
+          atomicOr(L.d_err, 2);
+        }
+      }
+    }
+  }
+  site[lp + p] = st;
+  if (l == 0) sop[p] = st;
+}
+
 int frame_insert_levels(const FrameInsertLevel *lv, int n_levels, const int32_t *d_coords, int cols, int64_t P,
                         int32_t *d_bad, int32_t frame, int32_t *d_sop, int32_t *h_counts, hipStream_t s) {
   if (P <= 0) return INSC_OK;
-  if (n_levels < 1 || n_levels > 16 || P > FINISH_SMALL_MAX) {
-    set_error("frame_insert_levels: %d scales, %lld points (at most 16 scales, %d points)", n_levels, (long long)P,
-              FINISH_SMALL_MAX);
+  if (n_levels < 1 || n_levels > 16 || P * n_levels >= (1ll << 30)) {
+    set_error("frame_insert_levels: %d scales, %lld points (at most 16 scales, 2^30 (scale, point) pairs)", n_levels,
+              (long long)P);
     return INSC_ERR_ARG;
   }
   FrameInsertArgs a;
@@ -926,15 +1020,28 @@ int frame_insert_levels(const FrameInsertLevel *lv, int n_levels, const int32_t 
     a.lv[l] = FrameLevelDev{g->table, g->n_slots - 1, g->capacity_sites, g->coords, g->d_n, g->d_err,
                             lv[l].parent, lv[l].offset, lv[l].child};
   }
+  const bool large = P > FINISH_SMALL_MAX;
+  const size_t PL = (size_t)P * n_levels;
   void *ws;
-  int rc = workspace(WS_API, s, (size_t)P * n_levels * 2 * sizeof(int32_t) + 256, &ws);
+  int rc = workspace(WS_API, s, PL * (large ? 4 : 2) * sizeof(int32_t) + 512, &ws);
   if (rc) return rc;
   int32_t *site = (int32_t *)ws;
-  uint32_t *rec = (uint32_t *)(site + P * n_levels);
+  uint32_t *rec = (uint32_t *)(site + PL);
   hipLaunchKernelGGL(frame_claim_kernel, dim3(grid_for(P, 256), (unsigned)n_levels), dim3(256), 0, s, a, d_coords, cols,
                      (int)P, d_bad, frame, rec);
-  hipLaunchKernelGGL(frame_finish_kernel, dim3((unsigned)n_levels), dim3(1024), 0, s, a, d_coords, cols, (int)P,
-                     (const int32_t *)d_bad, frame, d_sop, site, (const uint32_t *)rec, h_counts);
+  if (large) {
+    int32_t *rep = (int32_t *)(rec + PL), *flag = rep + PL, *n_before = flag + PL + 1;
+    hipLaunchKernelGGL(frame_flag_kernel, dim3(grid_for(P, 256), (unsigned)n_levels), dim3(256), 0, s, a, (int)P,
+                       (const uint32_t *)rec, flag, rep, n_before);
+    INSC_LAUNCH_CHECK();
+    if ((rc = scan_exclusive_i32(flag, flag, (int64_t)PL + 1, nullptr, s))) return rc;
+    hipLaunchKernelGGL(frame_assign_kernel, dim3(grid_for(P, 256), (unsigned)n_levels), dim3(256), 0, s, a, d_coords, cols,
+                       (int)P, (const int32_t *)d_bad, frame, d_sop, site, (const uint32_t *)rec, (const int32_t *)flag,
+                       (const int32_t *)rep, (const int32_t *)n_before, h_counts);
+  } else {
+    hipLaunchKernelGGL(frame_finish_kernel, dim3((unsigned)n_levels), dim3(1024), 0, s, a, d_coords, cols, (int)P,
+                       (const int32_t *)d_bad, frame, d_sop, site, (const uint32_t *)rec, h_counts);
+  }
   if (n_levels > 1)
     hipLaunchKernelGGL(frame_link_kernel, dim3(grid_for(P, 256), (unsigned)(n_levels - 1)), dim3(256), 0, s, a, (int)P,
                        (const int32_t *)site);
@@ -946,7 +1053,7 @@ int frame_insert_levels(const FrameInsertLevel *lv, int n_levels, const int32_t 
   return INSC_OK;
 }
 
-int64_t frame_insert_max_points() { return FINISH_SMALL_MAX; }
+int64_t frame_insert_max_points() { return (1ll << 30) / 16 - 1; }
 
 // ---- insert without allocation -------------------------------------------------------------
 // Scratch of insc_grid_insert_noalloc: the slot every row of the call claimed (what the grid's own,

@@ -1092,10 +1092,11 @@ int insc_net_forward(insc_net *net, const int32_t *d_coords, int coord_cols, con
   int32_t *sop = net->site_of_point + net->n_points;
   net->frame_sop = sop;
   net->frame_P = P;
-  // An incremental frame of moderate size inserts at all scales in one launch, which also leaves
-  // the new site counts in host memory; the host picks them up further down, while the GPU is busy
-  // with the neighbour maps and orders of the new sites.
-  const bool fused_insert = inc && P > 0 && P <= frame_insert_max_points();
+  // A frame inserts at all scales at once (three launches up to 16k points, seven beyond), which also
+  // leaves the new site counts in host memory; the host picks them up further down, while the GPU is
+  // busy with the neighbour maps and orders of the new sites.  (The scale-by-scale chain below is left
+  // for frames beyond 2^26 points.)
+  const bool fused_insert = P > 0 && P <= frame_insert_max_points();
   if (P > 0) {
     Level &L0 = net->levels[0];
     if (fused_insert) {
@@ -1158,13 +1159,7 @@ int insc_net_forward(insc_net *net, const int32_t *d_coords, int coord_cols, con
       if ((rc = order_append_new_sites_both_batch(grids, cnbrs, offsets, orders, poss, bo_orders, bo_poss, L, P, s)))
         return rc;
       if ((rc = tile_plan_append_batch(app, P, s))) return rc;
-    } else {
-      for (int l = 0; l < L; l++) {
-        Level &Lv = net->levels[l];
-        if ((rc = order_append_new_sites(Lv.grid, Lv.order, Lv.pos, P, s))) return rc;
-        if (l + 1 < L && (rc = order_append_new_sites(Lv.grid, Lv.bo_order, Lv.bo_pos, P, s))) return rc;
-      }
-    }
+    }  // (a full frame builds its orders from scratch further down, once the counts are known)
     // ---- input scale: accumulate the points' features per site ----------------------------
     DirtyNode &din = net->dirty[net->tensors[0].dirty];
     const unsigned nb = grid_for(P, 256);
@@ -1177,7 +1172,12 @@ int insc_net_forward(insc_net *net, const int32_t *d_coords, int coord_cols, con
   if (!inc) {
     // A full frame may synchronise: learn the exact counts, then build the processing orders
     // (pattern-sorted for the 3^3 convolutions, offset-grouped for the deconvolutions).
-    if ((rc = sync_counts(net, s, "insc_net_forward"))) return rc;
+    if (fused_insert) {
+      INSC_HIP(hipEventSynchronize(net->ev_counts));
+      if ((rc = apply_counts(net, "insc_net_forward"))) return rc;
+    } else if ((rc = sync_counts(net, s, "insc_net_forward"))) {
+      return rc;
+    }
     for (int l = 0; l < L; l++) {
       Level &Lv = net->levels[l];
       if (Lv.n == 0) continue;

@@ -87,12 +87,55 @@ __global__ __launch_bounds__(SCAN_THREADS) void scan_final(const int32_t *__rest
 
 __global__ void scan_zero_total(int32_t *total) { *total = 0; }
 
+// Short inputs (the digit counts of a radix pass, the rows of a coarse scale): one workgroup of 1024
+// threads, up to 32 consecutive values per thread, one launch instead of three.
+constexpr int SCAN_ONE_THREADS = 1024;
+constexpr int SCAN_ONE_ITEMS = 32;
+constexpr int SCAN_ONE_MAX = SCAN_ONE_THREADS * SCAN_ONE_ITEMS;
+__global__ __launch_bounds__(SCAN_ONE_THREADS) void scan_one_block(const int32_t *__restrict__ in,
+                                                                   int32_t *__restrict__ out, int n,
+                                                                   int32_t *__restrict__ total) {
+  __shared__ int wsum[SCAN_ONE_THREADS / 64];
+  const int per = (n + SCAN_ONE_THREADS - 1) / SCAN_ONE_THREADS;  // <= SCAN_ONE_ITEMS
+  const int base = threadIdx.x * per;
+  int v[SCAN_ONE_ITEMS];
+  int sum = 0;
+#pragma unroll
+  for (int i = 0; i < SCAN_ONE_ITEMS; i++) {
+    v[i] = (i < per && base + i < n) ? in[base + i] : 0;
+    sum += v[i];
+  }
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int inc = wave_incl_scan(sum);
+  if (lane == 63) wsum[w] = inc;
+  __syncthreads();  // (also: every value has been read before the first one is written - in may be out)
+  int off = 0, tot = 0;
+#pragma unroll
+  for (int i = 0; i < SCAN_ONE_THREADS / 64; i++) {
+    const int t = wsum[i];
+    if (i < w) off += t;
+    tot += t;
+  }
+  int ex = off + inc - sum;
+#pragma unroll
+  for (int i = 0; i < SCAN_ONE_ITEMS; i++) {
+    if (i < per && base + i < n) out[base + i] = ex;
+    ex += v[i];
+  }
+  if (threadIdx.x == 0 && total) *total = tot;
+}
+
 int scan_exclusive_i32(const int32_t *in, int32_t *out, int64_t n, int32_t *total, hipStream_t s) {
   if (n <= 0) {
     if (total) {
       hipLaunchKernelGGL(scan_zero_total, dim3(1), dim3(1), 0, s, total);
       INSC_LAUNCH_CHECK();
     }
+    return INSC_OK;
+  }
+  if (n <= SCAN_ONE_MAX) {
+    hipLaunchKernelGGL(scan_one_block, dim3(1), dim3(SCAN_ONE_THREADS), 0, s, in, out, (int)n, total);
+    INSC_LAUNCH_CHECK();
     return INSC_OK;
   }
   int64_t nb = cdiv(n, SCAN_TILE);
