@@ -191,6 +191,50 @@ def test_a_frame_with_a_bad_coordinate_is_dropped_whole():
         assert torch.equal(net(_inp(vox, rgb), increment=False), ref)
 
 
+def test_frames_of_more_than_16k_points_full_incremental_and_dropped():
+    """Frames beyond 16 384 points rank their new cells with a device-wide prefix sum instead of one
+    workgroup per scale: a full frame and an incremental frame of that size (the latter with points
+    that fall on old cells, on new cells, and twice on the same new cell) must equal the module tree
+    bit for bit, and such a frame with one bad coordinate must leave nothing behind."""
+    import sparseconvnet as scn
+    from sparseconvnet._lib import InscError
+    from workloads.netdefs import NaiveUNet
+
+    vox = scenes.indoor_scene(seed=51, n=60000, dims=(200, 160, 60), n_boxes=12, side_rng=(10, 40))
+    rng = np.random.default_rng(51)
+    rgb = rng.uniform(0, 1, (len(vox), 3)).astype(np.float32)
+    n0 = 30000
+    # second frame: 30k new voxels, 3k of the old ones again, 2k of the new ones twice
+    idx = np.concatenate([np.arange(n0, len(vox)), rng.integers(0, n0, 3000), rng.integers(n0, len(vox), 2000)])
+    idx = idx[rng.permutation(len(idx))]
+    p1, f1 = vox[idx], rng.uniform(0, 1, (len(idx), 3)).astype(np.float32)
+    assert n0 > 16384 and len(p1) > 16384
+    model = NaiveUNet(m=16, levels=5, seed=17).cuda()
+    mod_model = copy.deepcopy(model)
+    for mod in mod_model.modules():
+        if isinstance(mod, scn.OutputLayer):
+            mod.all_points = True
+    net = scn.compile(model.sparseModel, capacity_sites=1 << 16)
+    with torch.no_grad():
+        a = net(_inp(vox[:n0], rgb[:n0]), increment=False)
+        b = mod_model.sparseModel(_inp(vox[:n0], rgb[:n0]), False)
+        assert torch.equal(a, b)
+        bad = p1.copy()
+        bad[12345, 0] = 1 << 20
+        with pytest.raises(InscError) as e:
+            net(_inp(bad, f1), increment=True)
+        assert e.value.code == -5
+        assert net.sites_per_level()[0] == n0
+        a = net(_inp(p1, f1), increment=True, all_points=True)
+        b = mod_model.sparseModel(_inp(p1, f1), True)
+        assert torch.equal(a, b)
+        assert net.sites_per_level()[0] == len(vox)
+        # and against a full forward over all points (the mean of a voxel's points is formed in row order)
+        pts_all, f_all = np.concatenate([vox[:n0], p1]), np.concatenate([rgb[:n0], f1])
+        full = copy.deepcopy(model).sparseModel(_inp(pts_all, f_all))
+        assert torch.equal(a, full)
+
+
 def test_grid_reports_a_bad_coordinate_once_and_stays_usable():
     import ctypes
 
