@@ -955,12 +955,19 @@ __global__ __launch_bounds__(256) void frame_assign_kernel(FrameInsertArgs a, co
   const bool dropped = bad[0] == frame;
   if (p == 0) {
     int total = dropped ? 0 : excl[lp + P] - excl[lp];
-    if (total > L.capacity - n_before) total = (int)(L.capacity - n_before);  // (the error flag is up)
+    // (more new sites than the scale has room for: the rows beyond get no site below; the flag is worked
+    // out here as well, since those rows may raise it only after this thread has read it)
+    const bool over = total > L.capacity - n_before;
+    if (over) {
+      total = (int)(L.capacity - n_before);
+      atomicOr(L.d_err, 2);
+    }
     L.d_n[1] = n_before;
     L.d_n[0] = n_before + total;
     if (h_counts) {
       h_counts[2 * l] = n_before + total;
-      h_counts[2 * l + 1] = dropped ? 0 : __hip_atomic_load(L.d_err, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      h_counts[2 * l + 1] =
+          dropped ? 0 : (__hip_atomic_load(L.d_err, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) | (over ? 2 : 0));
       if (l == 0) h_counts[2 * a.n_levels] = dropped ? frame : 0;
     }
   }

@@ -233,6 +233,14 @@ def test_frames_of_more_than_16k_points_full_incremental_and_dropped():
         pts_all, f_all = np.concatenate([vox[:n0], p1]), np.concatenate([rgb[:n0], f1])
         full = copy.deepcopy(model).sparseModel(_inp(pts_all, f_all))
         assert torch.equal(a, full)
+        # a full frame of that size that fails leaves no state behind; the next full frame is sound
+        with pytest.raises(InscError) as e:
+            net(_inp(bad, f1), increment=False)
+        assert e.value.code == -5
+        with pytest.raises(InscError) as e:
+            net(_inp(vox[:10], rgb[:10]), increment=True)
+        assert e.value.code == -4
+        assert torch.equal(net(_inp(pts_all, f_all), increment=False), full)
 
 
 def test_grid_reports_a_bad_coordinate_once_and_stays_usable():
