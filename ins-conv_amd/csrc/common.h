@@ -63,6 +63,14 @@ struct BnEpilogue {
   // element-wise sum of a residual block, folded into the convolution that ends the block)
   const float *res = nullptr;
   int64_t ldr = 0;
+  // optional second batch norm, over another matrix with the producer's rows and columns (the other
+  // half of a channel concatenation whose batch norm this producer computes as well):
+  //   side_out[row][c] = leaky(side_in[row][c] * side_w[c] + side_b[c]), row stride of side_out = ld2,
+  // same leak.  Deconvolutions only (conv_mfma_kernel with the parent map).
+  const float *side_in = nullptr;
+  int64_t ld_side = 0;
+  float *side_out = nullptr;
+  const float *side_w = nullptr, *side_b = nullptr;
 };
 // w = gamma / sqrt(var + eps), b = beta - mean * w   (gamma / beta nullable)
 int bn_scale_shift(const float *mean, const float *var, const float *gamma, const float *beta, float eps, int C,

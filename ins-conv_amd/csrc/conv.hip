@@ -351,13 +351,16 @@ __global__ __launch_bounds__((S == 1 ? CONV_WAVES : S) * 64) void conv_mfma_kern
 
   // per-channel scale / shift of the fused batch norm for this lane's columns (loaded here so
   // that the latency is hidden behind the main loop)
-  float ew[NB], eb[NB];
+  float ew[NB], eb[NB], sw[NB], sb[NB];
 #pragma unroll
   for (int b = 0; b < NB; b++) {
     const int c = (cb0 + b) * 32 + r;
     const bool on = ep.out2 && c < Cout;
     ew[b] = on ? ep.w[c] : 0.0f;
     eb[b] = on ? ep.b[c] : 0.0f;
+    const bool son = MODE == MAP_PARENT && ep.side_in && c < Cout;
+    sw[b] = son ? ep.side_w[c] : 0.0f;
+    sb[b] = son ? ep.side_b[c] : 0.0f;
   }
 
   if (rest) {
@@ -534,6 +537,12 @@ __global__ __launch_bounds__((S == 1 ? CONV_WAVES : S) * 64) void conv_mfma_kern
       for (int j = 0; j < NV; j++) a[j] += rv[j];
       __builtin_amdgcn_sched_barrier(0);  // (the sums stay above the stores)
     }
+    float sv[NV];
+    if (MODE == MAP_PARENT && ep.side_in) {
+#pragma unroll
+      for (int j = 0; j < NV; j++) sv[j] = rid[j] >= 0 ? ep.side_in[(int64_t)rid[j] * ep.ld_side + c] : 0.0f;
+      __builtin_amdgcn_sched_barrier(0);  // (all loads above the stores)
+    }
 #pragma unroll
     for (int j = 0; j < NV; j++) {
       if (rid[j] < 0) continue;
@@ -541,6 +550,10 @@ __global__ __launch_bounds__((S == 1 ? CONV_WAVES : S) * 64) void conv_mfma_kern
       if (ep.out2) {
         const float y = fmaf(a[j], ew[0], eb[0]);  // fused batch norm + leaky ReLU
         ep.out2[(int64_t)rid[j] * ep.ld2 + c] = y * ((y > 0.0f) ? 1.0f : ep.leak);
+      }
+      if (MODE == MAP_PARENT && ep.side_in) {
+        const float y = fmaf(sv[j], sw[0], sb[0]);  // batch norm of the other half of a joined matrix
+        ep.side_out[(int64_t)rid[j] * ep.ld2 + c] = y * ((y > 0.0f) ? 1.0f : ep.leak);
       }
     }
     return;
@@ -585,6 +598,23 @@ __global__ __launch_bounds__((S == 1 ? CONV_WAVES : S) * 64) void conv_mfma_kern
         if ((cb0 + b) * 32 + r < Cout) {
           const float y = fmaf(acc[b][v], ew[b], eb[b]);
           op2[b * 32] = y * ((y > 0.0f) ? 1.0f : ep.leak);
+        }
+    }
+  }
+  if (MODE == MAP_PARENT && ep.side_in) {
+    // batch norm of the other half of a joined matrix, same rows and columns
+#pragma unroll
+    for (int v = 0; v < 16; v++) {
+      float x[NB];
+#pragma unroll
+      for (int b = 0; b < NB; b++)
+        x[b] = (rid[v] >= 0 && (cb0 + b) * 32 + r < Cout) ? ep.side_in[(int64_t)rid[v] * ep.ld_side + (cb0 + b) * 32 + r] : 0.0f;
+      if (rid[v] < 0) continue;
+#pragma unroll
+      for (int b = 0; b < NB; b++)
+        if ((cb0 + b) * 32 + r < Cout) {
+          const float y = fmaf(x[b], sw[b], sb[b]);
+          ep.side_out[(int64_t)rid[v] * ep.ld2 + (cb0 + b) * 32 + r] = y * ((y > 0.0f) ? 1.0f : ep.leak);
         }
     }
   }
@@ -1854,6 +1884,10 @@ int launch_conv(const float *in, int64_t ld_in, int64_t in_rows, float *out, int
                 const uint8_t *tile_flags, const uint8_t *row_mask, hipStream_t s, BnEpilogue ep, TilePlan plan,
                 int latency, int64_t expect_rows) {
   if (n_rows == 0) return INSC_OK;
+  if (ep.side_in && !(mode == MAP_PARENT && K == 8 && conv_uses_mfma(in, ld_in, Cin, K) && ep.side_out && ep.side_w && ep.side_b)) {
+    set_error("conv: a second batch norm in the epilogue is for deconvolutions on the matrix-core kernel only");
+    return INSC_ERR_ARG;
+  }
   if (expect_rows <= 0 || expect_rows > n_rows) expect_rows = n_rows;
   if (plan.map && (mode != MAP_NBR || K != 27 || plan.ld * 27 * 4 >= (int64_t)BUF_OOB || plan.ld < cdiv(n_rows, TILE_M) * TILE_M))
     plan = TilePlan();  // only the 3^3 map has a plan; an unusable one is ignored

@@ -69,6 +69,8 @@ struct Op {
   float *bn_w = nullptr, *bn_b = nullptr;  // per-channel scale / shift of an OP_BN, owned
   int fused_add = -1;                      // convolution side: index of the OP_ADD it also computes
   int fused_bn = -1;                       // producer side: index of the OP_BN it also computes
+  int fused_join_bn = -1;                  // deconvolution side: OP_BN over a join of its output with another tensor
+  int join_other = -1;                     //   ... that other tensor
   bool write_raw = true;                   // producer side: its own output has other readers
   bool fused = false;                      // OP_BN / OP_ADD side: computed by its producer, no kernel of its own
 };
@@ -576,6 +578,23 @@ static int run_op(insc_net *net, const Op &op, bool incremental, hipStream_t s) 
     ep.out2 = tensor_ptr(net, bn.out);
     ep.ld2 = tensor_ld(net, bn.out);
   }
+  if (op.fused_join_bn >= 0) {
+    // batch norm of [other | own output]: columns of the normalised matrix by the place each half has
+    // in the joined one
+    const Op &bn = net->ops[op.fused_join_bn];
+    const Tensor &Tj = net->tensors[bn.in0], &Tx = net->tensors[op.out], &Ty = net->tensors[op.join_other];
+    const int cx = Tx.col0 - Tj.col0, cy = Ty.col0 - Tj.col0;
+    ep.w = bn.bn_w + cx;
+    ep.b = bn.bn_b + cx;
+    ep.leak = bn.leak;
+    ep.out2 = tensor_ptr(net, bn.out) + cx;
+    ep.ld2 = tensor_ld(net, bn.out);
+    ep.side_in = tensor_ptr(net, op.join_other);
+    ep.ld_side = tensor_ld(net, op.join_other);
+    ep.side_out = tensor_ptr(net, bn.out) + cy;
+    ep.side_w = bn.bn_w + cy;
+    ep.side_b = bn.bn_b + cy;
+  }
   const float *in0 = tensor_ptr(net, op.in0);
   const int64_t ld0 = tensor_ld(net, op.in0);
   const int64_t rows0 = net->buffers[net->tensors[op.in0].buf].rows;
@@ -948,6 +967,33 @@ int insc_net_finalize(insc_net *net, int out_tensor, int64_t capacity_sites, voi
         T.kept = false;
       }
     }
+    // A batch norm over a channel concatenation [other | deconvolution output] (the decoder of a
+    // U-Net): the deconvolution normalises its own columns in its epilogue and, row by row, the other
+    // tensor's columns as well - same rows (the sets of rows due must be the same one), same column
+    // blocks (equal widths), and the other tensor is complete by then.
+    for (int i = 0; i < (int)net->ops.size(); i++) {
+      Op &bn = net->ops[i];
+      if (bn.kind != OP_BN || bn.fused || bn.in0 == bn.out || producer[bn.out] != i) continue;
+      int jn = -1;
+      for (int k = 0; k < i; k++)
+        if (net->ops[k].kind == OP_JOIN && net->ops[k].out == bn.in0) jn = k;
+      if (jn < 0) continue;
+      const Op &J = net->ops[jn];
+      for (int side = 0; side < 2; side++) {
+        const int x = side ? J.in0 : J.in1, y = side ? J.in1 : J.in0;  // x: the deconvolution's output
+        const int a = producer[x], py = producer[y];
+        if (a < 0 || a > i || py < 0 || py > a) continue;
+        Op &A = net->ops[a];
+        if (A.kind != OP_DECONV || A.fused_bn >= 0 || A.fused_join_bn >= 0 || A.Cin % 16 != 0) continue;
+        const Tensor &Tx = net->tensors[x], &Ty = net->tensors[y];
+        if (Tx.C != Ty.C || Tx.C != A.Cout || !Ty.kept) continue;
+        if (Tx.dirty != net->tensors[bn.out].dirty) continue;
+        A.fused_join_bn = i;
+        A.join_other = y;
+        bn.fused = true;
+        break;
+      }
+    }
   }
   // Fold the element-wise sum that ends a residual block into the convolution that feeds it
   // (the other operand must exist by then and both must be due on the same rows).
@@ -970,7 +1016,7 @@ int insc_net_finalize(insc_net *net, int out_tensor, int64_t capacity_sites, voi
         if (a < 0 || a > i || readers[x] != 1) continue;
         Op &A = net->ops[a];
         const bool conv = A.kind == OP_SSC || A.kind == OP_CONV || A.kind == OP_DECONV || A.kind == OP_NIN;
-        if (!conv || A.fused_bn >= 0 || A.fused_add >= 0) continue;
+        if (!conv || A.fused_bn >= 0 || A.fused_join_bn >= 0 || A.fused_add >= 0) continue;
         if (other != 0 && (producer[other] < 0 || producer[other] > a)) continue;  // not computed yet when A runs
         if (!net->tensors[other].kept) continue;
         if (net->tensors[x].dirty != net->tensors[add.out].dirty) continue;
