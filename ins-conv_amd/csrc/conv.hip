@@ -232,9 +232,9 @@ __global__ __launch_bounds__((S == 1 ? CONV_WAVES : S) * 64) void conv_mfma_kern
   // Which (tile slot, output block, share of the split) this block works on.  Split launches with a
   // tile schedule renumber their blocks: the hardware hands out blocks in the order x, y, z, round robin
   // over the compute units, so block L goes - all blocks being resident at once - to unit L mod CUS.
-  // Ranked by cost (tile slot major: the output blocks and shares of a tile cost the same), round 0 of
-  // CUS blocks takes ranks in order and every other round in reverse order, so that the compute unit that
-  // drew the most expensive block of one round gets the cheapest of the next.
+  // Ranked by cost (tile slot major: the output blocks and shares of a tile cost the same), the first CUS
+  // blocks take ranks in order, the next CUS in reverse order and so on in turns, so that the compute unit
+  // that drew the most expensive block of one turn gets the cheapest of the next.
   unsigned bx = blockIdx.x, by = blockIdx.y, bz = blockIdx.z;
   if (S > 1 && MODE == MAP_NBR && K == 27 && plan.map != nullptr && plan.sched != nullptr) {
     constexpr unsigned CUS = 256;
@@ -1521,9 +1521,9 @@ __global__ __launch_bounds__(OWN_WAVES * 64) __attribute__((amdgpu_waves_per_eu(
   int *nl = nlb[wave];
   // (wavefronts are on their own: no workgroup barrier anywhere below)
   // One block per compute unit; wavefront w sits on SIMD w % 4, so bin = (block, w % 4) names a SIMD and
-  // round = w / 4 one of its three wavefronts.  Units come by falling cost: round 0 hands them to the bins
-  // in order, every later round in reverse order, so the SIMDs that drew the expensive units of round 0
-  // get the cheap ones afterwards (largest sum of a SIMD at 39k sites and 64 channels: 72 items against
+  // turn = w / 4 one of its three wavefronts.  Units come by falling cost: the first turn hands them to the
+  // bins in order, every later turn in reverse order, so the SIMDs that drew the expensive units of the
+  // first turn get the cheap ones afterwards (largest sum of a SIMD at 39k sites and 64 channels: 72 items against
   // 90 when every SIMD takes three units in a row; 66 is the best any assignment reaches).
   const int64_t nbins = (int64_t)gridDim.x * 4;
   const int64_t bin = (int64_t)blockIdx.x * 4 + (wave & 3);
