@@ -19,10 +19,14 @@ namespace insc {
 
 enum OpKind { OP_SSC, OP_BN, OP_CONV, OP_DECONV, OP_NIN, OP_ADD, OP_COPY, OP_JOIN };
 enum DirtyKind { D_INPUT, D_DILATE, D_PARENTS, D_CHILDREN, D_UNION };
-// Scales this small are recomputed whole by incremental frames.  (128 tiles: every launch has all its
-// tiles resident at once, and with the eight 3^3 layers of such a scale and of each coarser one a
-// change anywhere reaches nearly every site of it anyway.)
+// Scales this small are recomputed whole by incremental frames: the input scale up to 128 tiles, the
+// coarser ones up to 512.  (Every launch then has all its tiles resident at once - what it lasts is its
+// longest block, not the number of blocks - and with the eight 3^3 layers of such a scale and of each
+// coarser one a change anywhere reaches nearly every site of it anyway: in the 150k-voxel sweep the sets
+// of the 10k-site scale hold 10 405 to 10 414 of its 10 414 sites.  No set is computed for such a scale:
+// 1 % of the frame.  The input scale keeps the lower bound: its sets start at the frame's own voxels.)
 constexpr int64_t DIRTY_FULL_SITES = 4096;
+constexpr int64_t DIRTY_FULL_SITES_COARSE = 16384;
 // Scales from this size on may run a layer over a list of dirty rows instead of over flagged tiles.
 constexpr int64_t COMPACT_MIN_SITES = 32768;
 
@@ -1284,13 +1288,13 @@ int insc_net_forward(insc_net *net, const int32_t *d_coords, int coord_cols, con
   // ---- dirty sets, then the layers ---------------------------------------------------------
   if (net->profiling) INSC_HIP(hipEventRecord(net->ev[1], s));
   if (inc) {
-    // A scale of at most DIRTY_FULL_SITES sites is recomputed whole: every set of it and of the
+    // A scale of at most DIRTY_FULL_SITES (_COARSE above the input scale) sites is recomputed whole: every set of it and of the
     // coarser scales is "all rows" (recomputing a clean row reproduces its bits).  Being all rows
     // is inherited along the program - the children of all coarse sites are all fine sites, a
     // union with everything is everything, ... - so the decoder's sets at the finer scales are
     // known to be full as well.  Such sets cost no launch and keep no mask.
     int l_full = L;
-    for (int l = L - 1; l >= 0 && net->levels[l].n <= DIRTY_FULL_SITES; l--) l_full = l;
+    for (int l = L - 1; l >= 0 && net->levels[l].n <= (l == 0 ? DIRTY_FULL_SITES : DIRTY_FULL_SITES_COARSE); l--) l_full = l;
     net->dirty_full.assign(net->dirty.size(), 0);
     for (size_t i = 0; i < net->dirty.size(); i++) {  // (a set's sources come before it)
       const DirtyNode &dn = net->dirty[i];
