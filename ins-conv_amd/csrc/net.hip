@@ -1228,18 +1228,33 @@ int insc_net_forward(insc_net *net, const int32_t *d_coords, int coord_cols, con
     } else if ((rc = sync_counts(net, s, "insc_net_forward"))) {
       return rc;
     }
+    {
+      // the small scales: all their sites came with this frame's one insert, and the single-workgroup
+      // sorts of the incremental path order them - all of them in one launch - instead of some fifty
+      // launches per scale
+      const insc_grid *sg[16];
+      const int32_t *snbr[16], *soff[16];
+      int32_t *sord[16], *spos[16], *sbo[16], *sbp[16];
+      int ns = 0;
+      int64_t nmax = 0;
+      for (int l = 0; l < L; l++) {
+        Level &Lv = net->levels[l];
+        if (Lv.n == 0 || Lv.n > order_sorted_max()) continue;
+        sg[ns] = Lv.grid;
+        snbr[ns] = Lv.nbr;
+        soff[ns] = l + 1 < L ? Lv.offset : nullptr;
+        sord[ns] = Lv.order;
+        spos[ns] = Lv.pos;
+        sbo[ns] = Lv.bo_order;
+        sbp[ns] = Lv.bo_pos;
+        nmax = std::max(nmax, Lv.n);
+        ns++;
+      }
+      if (ns > 0 && (rc = order_append_new_sites_both_batch(sg, snbr, soff, sord, spos, sbo, sbp, ns, nmax, s))) return rc;
+    }
     for (int l = 0; l < L; l++) {
       Level &Lv = net->levels[l];
-      if (Lv.n == 0) continue;
-      if (Lv.n <= order_sorted_max()) {
-        // a small scale: all its sites came with this frame's one insert, and the single-workgroup
-        // sorts of the incremental path order them in two launches instead of some fifty
-        if ((rc = order_append_new_sites_sorted(Lv.grid, Lv.nbr, Lv.order, Lv.pos, Lv.n, s))) return rc;
-        if (l + 1 < L)
-          if ((rc = order_append_new_sites_by_offset(Lv.grid, Lv.offset, Lv.pos, Lv.bo_order, Lv.bo_pos, Lv.n, s)))
-            return rc;
-        continue;
-      }
+      if (Lv.n == 0 || Lv.n <= order_sorted_max()) continue;
       if ((rc = insc_order_build(Lv.grid, Lv.nbr, 0, Lv.n, Lv.order, stream))) return rc;
       hipLaunchKernelGGL(invert_perm_kernel, dim3(grid_for(Lv.n, 256)), dim3(256), 0, s, Lv.order, Lv.n, Lv.pos);
       if (l + 1 < L) {
