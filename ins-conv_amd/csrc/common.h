@@ -43,6 +43,7 @@ int device_cus();
 int zero_counters(hipStream_t stream, size_t count, int32_t **out);
 
 // ---- device primitives (scan_sort.hip) -------------------------------------------------
+int sort_pairs_u64_into(uint64_t *keys, int32_t *vals_in, int32_t *vals_out, int64_t n, int key_bits, hipStream_t s);
 int scan_exclusive_i32(const int32_t *in, int32_t *out, int64_t n, int32_t *total, hipStream_t s);
 int sort_pairs_u64(uint64_t *keys, int32_t *vals, int64_t n, int key_bits, hipStream_t s);
 

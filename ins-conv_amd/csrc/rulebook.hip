@@ -183,13 +183,14 @@ int insc_order_build(const insc_grid *g, const int32_t *d_nbr, int64_t first, in
   if (n == 0) return INSC_OK;
   hipStream_t s = (hipStream_t)stream;
   void *ws;
-  int rc = workspace(WS_API, s, sizeof(uint64_t) * (size_t)n, &ws);
+  int rc = workspace(WS_API, s, (sizeof(uint64_t) + sizeof(int32_t)) * (size_t)n, &ws);
   if (rc) return rc;
   uint64_t *keys = (uint64_t *)ws;
+  int32_t *ids = (int32_t *)(keys + n);  // (the unsorted site ids: the sort delivers into d_order, no copy back)
   hipLaunchKernelGGL(order_key_kernel, dim3(grid_for(n, 256)), dim3(256), 0, s, insc_grid_coords(g), d_nbr, first, n,
-                     keys, d_order + first);
+                     keys, ids);
   INSC_LAUNCH_CHECK();
-  return sort_pairs_u64(keys, d_order + first, n, ORDER_KEY_BITS, s);
+  return sort_pairs_u64_into(keys, ids, d_order + first, n, ORDER_KEY_BITS, s);
 }
 
 int insc_order_by_offset(const int32_t *d_order, const int32_t *d_offset, int64_t n, int32_t *d_out, void *stream) {
@@ -197,12 +198,13 @@ int insc_order_by_offset(const int32_t *d_order, const int32_t *d_offset, int64_
   if (n == 0) return INSC_OK;
   hipStream_t s = (hipStream_t)stream;
   void *ws;
-  int rc = workspace(WS_API, s, sizeof(uint64_t) * (size_t)n, &ws);
+  int rc = workspace(WS_API, s, (sizeof(uint64_t) + sizeof(int32_t)) * (size_t)n, &ws);
   if (rc) return rc;
   uint64_t *keys = (uint64_t *)ws;
-  hipLaunchKernelGGL(offset_key_kernel, dim3(grid_for(n, 256)), dim3(256), 0, s, d_order, d_offset, n, keys, d_out);
+  int32_t *ids = (int32_t *)(keys + n);
+  hipLaunchKernelGGL(offset_key_kernel, dim3(grid_for(n, 256)), dim3(256), 0, s, d_order, d_offset, n, keys, ids);
   INSC_LAUNCH_CHECK();
-  return sort_pairs_u64(keys, d_out, n, 3, s);
+  return sort_pairs_u64_into(keys, ids, d_out, n, 3, s);
 }
 
 int insc_dirty_mark(const int32_t *d_site_of_point, int64_t P, uint8_t *d_mask, void *stream) {

@@ -255,6 +255,50 @@ int sort_pairs_u64(uint64_t *keys, int32_t *vals, int64_t n, int key_bits, hipSt
   return INSC_OK;
 }
 
+// The same sort with the values delivered into another array: vals_out gets the values in key order,
+// keys and vals_in are scratch afterwards.  No copy at the end, whatever the number of passes.
+int sort_pairs_u64_into(uint64_t *keys, int32_t *vals_in, int32_t *vals_out, int64_t n, int key_bits, hipStream_t s) {
+  if (n <= 0) return INSC_OK;
+  if (key_bits > 64) key_bits = 64;
+  const int passes = key_bits <= 0 ? 0 : (key_bits + 7) / 8;
+  if (n == 1 || passes == 0) {
+    INSC_HIP(hipMemcpyAsync(vals_out, vals_in, sizeof(int32_t) * (size_t)n, hipMemcpyDeviceToDevice, s));
+    return INSC_OK;
+  }
+  const int64_t nb64 = cdiv(n, SORT_TILE);
+  if (nb64 > (1 << 22)) {
+    set_error("sort_pairs_u64_into: n=%lld too large", (long long)n);
+    return INSC_ERR_ARG;
+  }
+  const int nb = (int)nb64;
+  size_t off_keys = 0;
+  size_t off_vals = off_keys + sizeof(uint64_t) * (size_t)n;
+  size_t off_cnt = (off_vals + sizeof(int32_t) * (size_t)n + 255) & ~(size_t)255;
+  size_t bytes = off_cnt + sizeof(int32_t) * 256 * (size_t)nb;
+  void *ws;
+  int rc = workspace(WS_SORT, s, bytes, &ws);
+  if (rc) return rc;
+  uint64_t *k2 = (uint64_t *)((char *)ws + off_keys);
+  int32_t *v2 = (int32_t *)((char *)ws + off_vals);
+  int32_t *counts = (int32_t *)((char *)ws + off_cnt);
+  uint64_t *kin = keys, *kout = k2;
+  int32_t *vin = vals_in, *vout = v2;
+  for (int p = 0; p < passes; p++) {
+    const int shift = 8 * p;
+    const bool last = p + 1 == passes;
+    hipLaunchKernelGGL(sort_hist, dim3(nb), dim3(SORT_THREADS), 0, s, kin, n, shift, counts, nb);
+    rc = scan_exclusive_i32(counts, counts, 256 * (int64_t)nb, nullptr, s);
+    if (rc) return rc;
+    // (the keys of the last pass go where they would have gone; nobody reads them)
+    hipLaunchKernelGGL(sort_scatter, dim3(nb), dim3(SORT_THREADS), 0, s, kin, vin, kout, last ? vals_out : vout, n,
+                       shift, counts, nb);
+    INSC_LAUNCH_CHECK();
+    uint64_t *tk = kin; kin = kout; kout = tk;
+    int32_t *tv = vin; vin = vout; vout = tv;
+  }
+  return INSC_OK;
+}
+
 }  // namespace insc
 
 extern "C" {
