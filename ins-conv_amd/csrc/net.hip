@@ -1542,22 +1542,24 @@ int insc_net_forward_residual(insc_net *net, const int32_t *d_coords, int coord_
   }
   INSC_HIP(hipMemsetAsync(R.in_sum, 0, sizeof(float) * (size_t)P * C0, s));
   INSC_HIP(hipMemsetAsync(R.in_cnt, 0, sizeof(int32_t) * (size_t)P, s));
-  void *ws;
-  if ((rc = workspace(WS_API, s, sizeof(int32_t) * 4 * (size_t)P, &ws))) return rc;
-  int32_t *c4 = (int32_t *)ws;
   const unsigned nb = grid_for(P, 256);
-  hipLaunchKernelGGL(coords_to_int4_kernel, dim3(nb), dim3(256), 0, s, d_coords, coord_cols, P, c4,
-                     (const int32_t *)nullptr, 0);
-  INSC_LAUNCH_CHECK();
-  if ((rc = grid_insert_nosync(R.levels[0].grid, c4, P, R.sop, s))) return rc;
+  // the inserts of all scales at once, as in an exact frame; the counts arrive in host memory
+  net->frame_id = net->frame_id == INT32_MAX ? 1 : net->frame_id + 1;
+  {
+    FrameInsertLevel fl[16];
+    for (int l = 0; l < L; l++) {
+      Level &Lv = R.levels[l];
+      Lv.grid->n_upper = 0;
+      fl[l] = FrameInsertLevel{Lv.grid, Lv.parent, Lv.offset, Lv.child};
+    }
+    if ((rc = frame_insert_levels(fl, L, d_coords, coord_cols, P, net->d_bad, net->frame_id, R.sop, net->h_counts, s)))
+      return rc;
+    INSC_HIP(hipEventRecord(net->ev_counts, s));
+  }
   hipLaunchKernelGGL(chain_push_kernel, dim3(nb), dim3(256), 0, s, R.sop, P, R.chain_head, R.chain_next);
   hipLaunchKernelGGL(chain_sum_kernel, dim3(nb), dim3(256), 0, s, d_feats, C0, R.sop, P, R.chain_head, R.chain_next,
                      R.in_sum, R.in_cnt, (uint8_t *)nullptr, (uint8_t *)nullptr, (const int32_t *)nullptr);
   INSC_LAUNCH_CHECK();
-  for (int l = 0; l + 1 < L; l++) {
-    Level &F = R.levels[l], &Cs = R.levels[l + 1];
-    if ((rc = down2_new_sites(F.grid, Cs.grid, P, F.parent, F.offset, F.child, s))) return rc;
-  }
   {
     // the neighbour maps of all scales in one launch
     const insc_grid *grids[16];
@@ -1568,13 +1570,10 @@ int insc_net_forward_residual(insc_net *net, const int32_t *d_coords, int coord_
     }
     if ((rc = ssc3_new_sites_batch(grids, nbrs, L, P, s))) return rc;
   }
-  // the exact site counts size every later launch (one short host round trip, as in an exact frame)
-  for (int l = 0; l < L; l++) {
-    INSC_HIP(hipMemcpyAsync(net->h_counts + 2 * l, R.levels[l].grid->d_n, sizeof(int32_t), hipMemcpyDeviceToHost, s));
-    INSC_HIP(hipMemcpyAsync(net->h_counts + 2 * l + 1, R.levels[l].grid->d_err, sizeof(int32_t), hipMemcpyDeviceToHost,
-                            s));
-  }
-  INSC_HIP(hipStreamSynchronize(s));
+  // the exact site counts size every later launch (one short wait, as in an exact frame)
+  INSC_HIP(hipEventSynchronize(net->ev_counts));
+  INSC_REQUIRE(net->h_counts[2 * L] != net->frame_id, INSC_ERR_COORD,
+               "insc_net_forward_residual: a coordinate is outside 0..65535 (batch 0..32767)");
   for (int l = 0; l < L; l++) {
     Level &Lv = R.levels[l];
     Lv.n = Lv.n_upper = net->h_counts[2 * l];
