@@ -1951,9 +1951,10 @@ int launch_conv(const float *in, int64_t ld_in, int64_t in_rows, float *out, int
     const int NB = (S == 1 && Cin >= 96) ? 1 : NB0;
     // (the split across blocks is for scales with few tiles; in a U-Net the width grows with the depth,
     // and a layer that narrows to at most 96 channels sits at a fine scale with many tiles)
-    // (eight blocks from 224 channels: the coarsest scale of a seven-scale U-Net, three tiles, where a
-    // wavefront's item loop is most of the launch - 15 -> 12 us; at 192 channels it gains nothing)
-    int G = (split && K == 27 && Cout > 96) ? (Cin >= 224 ? 8 : Cin >= 160 ? 4 : Cin >= 128 ? 2 : 1) : 1;
+    // (eight blocks from 224 -> 192 channels: the two coarsest scales of a seven-scale U-Net, a few tiles,
+    // where a wavefront's item loop is most of the launch - 224 -> 224 at 70 sites 15 -> 12 us; at 192 input
+    // channels, and for 256 -> 128 and 320 -> 160 with their more numerous tiles, it gains nothing)
+    int G = (split && K == 27 && Cout > 96) ? ((Cin >= 224 && Cout >= 192) ? 8 : Cin >= 160 ? 4 : Cin >= 128 ? 2 : 1) : 1;
     if (lat) {
       G = Cin >= 128 ? 4 : Cin >= 64 ? 2 : 1;
       S = 4;
