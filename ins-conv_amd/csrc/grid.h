@@ -42,19 +42,8 @@ constexpr int32_t COORD_SKIP = INT32_MIN;
 // Device-side variants used inside a frame: nothing here synchronises with the host.
 // All of them act on the sites added by the grid's most recent insert, [*d_n_prev, *d_n).
 int grid_insert_nosync(insc_grid *g, const int32_t *d_coords4, int64_t P, int32_t *d_site_of_point, hipStream_t s);
-int ssc3_new_sites(const insc_grid *g, int32_t *d_nbr, int64_t n_new_upper, hipStream_t s);
-int down2_new_sites(const insc_grid *fine, insc_grid *coarse, int64_t n_new_upper, int32_t *d_parent,
-                    int32_t *d_offset, int32_t *d_child, hipStream_t s);
-// order[i] = pos[i] = i for the new sites (appended in id order)
-int order_append_new_sites(const insc_grid *g, int32_t *d_order, int32_t *d_pos, int64_t n_new_upper, hipStream_t s);
-// the same, with the new sites sorted among themselves by the key of insc_order_build (needs their
-// rows of the neighbour map) / grouped by their position inside the parent cell
-int order_append_new_sites_sorted(const insc_grid *g, const int32_t *d_nbr, int32_t *d_order, int32_t *d_pos,
-                                  int64_t n_new_upper, hipStream_t s);
-int order_append_new_sites_by_offset(const insc_grid *g, const int32_t *d_offset, const int32_t *d_pos_in_order,
-                                     int32_t *d_order, int32_t *d_pos, int64_t n_new_upper, hipStream_t s);
-// the three per-grid steps above for several grids (the scales of a network, at most 16) in one
-// launch each; every grid acts on the sites of its own most recent insert
+// the neighbour maps of the new sites of several grids (the scales of a network, at most 16) in one
+// launch; every grid acts on the sites of its own most recent insert
 // plans (nullable; per grid, plan null = none): tile plans to keep up to date with the map - the
 // entries of older sites that gain a neighbour are patched and the offset masks of the tiles the new
 // sites open are cleared; the new sites' own columns follow with tile_plan_append_batch
@@ -66,14 +55,8 @@ struct PlanRef {
 };
 int ssc3_new_sites_batch(const insc_grid *const *grids, int32_t *const *d_nbr, int n, int64_t n_new_upper,
                          hipStream_t s, const PlanRef *plans = nullptr);
-int order_append_new_sites_sorted_batch(const insc_grid *const *grids, const int32_t *const *d_nbr,
-                                        int32_t *const *d_order, int32_t *const *d_pos, int n, int64_t n_new_upper,
-                                        hipStream_t s);
-int order_append_new_sites_by_offset_batch(const insc_grid *const *grids, const int32_t *const *d_offset,
-                                           const int32_t *const *d_pos_in_order, int32_t *const *d_order,
-                                           int32_t *const *d_pos, int n, int64_t n_new_upper, hipStream_t s);
-// The inserts of a whole frame in one launch (at most frame_insert_max_points() points): the points
-// go into lv[0].grid, the sites that adds (halved) into lv[1].grid and so on, with the parent /
+// The inserts of a whole frame at all scales at once: the points go into lv[0].grid, the sites that adds
+// (halved) into lv[1].grid and so on, with the parent /
 // offset / child link of every scale to the next coarser one filled in for the new sites.  Every
 // grid then reports the sites of this insert as its newest ([d_n[1], d_n[0])).  d_coords: int32
 // [P, cols] (cols 3 or 4).  If any coordinate is out of range nothing is inserted anywhere, *d_bad
@@ -85,12 +68,13 @@ struct FrameInsertLevel {
 };
 int frame_insert_levels(const FrameInsertLevel *lv, int n_levels, const int32_t *d_coords, int cols, int64_t P,
                         int32_t *d_bad, int32_t frame, int32_t *d_sop, int32_t *h_counts, hipStream_t s);
-int64_t frame_insert_max_points();
 // looks up, for the current device, the address of the scratch array of insc_grid_insert_noalloc
 // (called by insc_init; the entry point does it itself on a device that was never initialised)
 int grid_noalloc_setup();
-// both appends for several grids in ONE launch (d_offset[i] null: the grid has no coarser scale above
-// it and only gets the first order)
+// The new sites of several grids appended to their processing orders in ONE launch, sorted among
+// themselves by the key of insc_order_build (needs their rows of the neighbour map), and to the orders
+// grouped by their position inside the parent cell (d_offset[i] null: the grid has no coarser scale
+// above it and only gets the first order)
 int order_append_new_sites_both_batch(const insc_grid *const *grids, const int32_t *const *d_nbr,
                                       const int32_t *const *d_offset, int32_t *const *d_order, int32_t *const *d_pos,
                                       int32_t *const *d_bo_order, int32_t *const *d_bo_pos, int n, int64_t n_new_upper,

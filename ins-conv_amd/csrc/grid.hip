@@ -319,12 +319,7 @@ __device__ __forceinline__ void ssc3_nbr_new_body(const Slot *__restrict__ table
     }
   }
 }
-__global__ void ssc3_nbr_new_kernel(const Slot *__restrict__ table, int64_t mask,
-                                    const int32_t *__restrict__ site_coords, const int32_t *__restrict__ d_n,
-                                    int32_t *__restrict__ nbr) {
-  ssc3_nbr_new_body(table, mask, site_coords, d_n, nbr);
-}
-// the same for several grids (the scales of a network) in one launch: blockIdx.y picks the grid
+// for several grids (the scales of a network) in one launch: blockIdx.y picks the grid
 struct NewSitesJob {
   const Slot *table;
   int64_t mask;
@@ -341,42 +336,6 @@ struct NewSitesBatch {
 __global__ void ssc3_nbr_new_batch_kernel(NewSitesBatch b) {
   const NewSitesJob &j = b.job[blockIdx.y];
   ssc3_nbr_new_body(j.table, j.mask, j.coords, j.d_n, j.nbr, j.plan, j.tmask, j.pos, j.ld);
-}
-
-__global__ void down2_coords_new_kernel(const int32_t *__restrict__ fine_coords, const int32_t *__restrict__ d_n,
-                                        int64_t n_upper, int32_t *__restrict__ half, int32_t *__restrict__ offset) {
-  const int64_t first = d_n[1], n = (int64_t)d_n[0] - first;
-  int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (t >= n_upper) return;
-  if (t >= n) {
-    reinterpret_cast<int4 *>(half)[t] = make_int4(COORD_SKIP, 0, 0, 0);
-    return;
-  }
-  int4 c = reinterpret_cast<const int4 *>(fine_coords)[first + t];
-  offset[first + t] = (c.x & 1) * 4 + (c.y & 1) * 2 + (c.z & 1);
-  reinterpret_cast<int4 *>(half)[t] = make_int4(c.x >> 1, c.y >> 1, c.z >> 1, c.w);
-}
-
-// parent_tmp[t] = coarse site of new fine site first+t
-__global__ void down2_link_new_kernel(const int32_t *__restrict__ parent_tmp, const int32_t *__restrict__ d_n,
-                                      int32_t *__restrict__ parent, const int32_t *__restrict__ offset,
-                                      int32_t *__restrict__ child) {
-  const int64_t first = d_n[1], n = (int64_t)d_n[0] - first;
-  int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (t >= n) return;
-  const int64_t i = first + t;
-  const int p = parent_tmp[t];
-  parent[i] = p;
-  if (p >= 0 && child) child[(int64_t)p * 8 + offset[i]] = (int)i;
-}
-
-__global__ void order_append_kernel(const int32_t *__restrict__ d_n, int32_t *__restrict__ order,
-                                    int32_t *__restrict__ pos) {
-  const int64_t first = d_n[1], n = (int64_t)d_n[0] - first;
-  int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (t >= n) return;
-  order[first + t] = (int)(first + t);
-  if (pos) pos[first + t] = (int)(first + t);
 }
 
 static int grid_alloc_table(insc_grid *g, int64_t capacity_sites) {
@@ -468,39 +427,10 @@ int grid_insert_nosync(insc_grid *g, const int32_t *d_coords4, int64_t P, int32_
   return grid_insert_launch(g, d_coords4, P, d_site_of_point, s);
 }
 
-int ssc3_new_sites(const insc_grid *g, int32_t *d_nbr, int64_t n_new_upper, hipStream_t s) {
-  if (n_new_upper <= 0) return INSC_OK;
-  hipLaunchKernelGGL(ssc3_nbr_new_kernel, dim3(grid_for(n_new_upper * 27, 256, 1ll << 30)), dim3(256), 0, s, g->table,
-                     g->n_slots - 1, g->coords, g->d_n, d_nbr);
-  INSC_LAUNCH_CHECK();
-  return INSC_OK;
-}
-
-int down2_new_sites(const insc_grid *fine, insc_grid *coarse, int64_t n_new_upper, int32_t *d_parent,
-                    int32_t *d_offset, int32_t *d_child, hipStream_t s) {
-  if (n_new_upper <= 0) return INSC_OK;
-  void *ws;
-  int rc = workspace(WS_API, s, sizeof(int32_t) * 5 * (size_t)n_new_upper, &ws);
-  if (rc) return rc;
-  int32_t *half = (int32_t *)ws;
-  int32_t *parent_tmp = half + 4 * n_new_upper;
-  const unsigned nb = grid_for(n_new_upper, 256);
-  hipLaunchKernelGGL(down2_coords_new_kernel, dim3(nb), dim3(256), 0, s, fine->coords, fine->d_n, n_new_upper, half,
-                     d_offset);
-  INSC_LAUNCH_CHECK();
-  rc = grid_insert_nosync(coarse, half, n_new_upper, parent_tmp, s);
-  if (rc) return rc;
-  hipLaunchKernelGGL(down2_link_new_kernel, dim3(nb), dim3(256), 0, s, parent_tmp, fine->d_n, d_parent, d_offset,
-                     d_child);
-  INSC_LAUNCH_CHECK();
-  return INSC_OK;
-}
-
 // The sites of the last insert, appended to a processing order sorted among themselves (one
 // workgroup, bitonic sort in LDS): tiles made of sites in arrival order use every filter offset
 // and gather from all over the scene, which costs a convolution a quarter of its speed.
-//   MODE 0: key = Morton code of the 64^3 block | neighbour pattern (the key of insc_order_build)
-//   MODE 1: key = position inside the parent cell | position in the MODE 0 order (`aux`)
+// Key = Morton code of the 64^3 block | neighbour pattern (the key of insc_order_build).
 // More new sites than SORT_NEW_MAX keep their arrival order (any order gives the same results).
 constexpr int SORT_NEW_MAX = 8192;
 __device__ __forceinline__ uint64_t spread3_10(uint64_t v) {  // 10 bits -> every third bit
@@ -511,12 +441,9 @@ __device__ __forceinline__ uint64_t spread3_10(uint64_t v) {  // 10 bits -> ever
   v = (v | (v << 2)) & 0x9249249ull;
   return v;
 }
-template <int MODE>
 __device__ __forceinline__ void order_append_sorted_body(const int32_t *__restrict__ d_n,
                                                          const int32_t *__restrict__ coords,
-                                                         const int32_t *__restrict__ nbr,
-                                                         const int32_t *__restrict__ offset,
-                                                         const int32_t *__restrict__ aux, int32_t *__restrict__ order,
+                                                         const int32_t *__restrict__ nbr, int32_t *__restrict__ order,
                                                          int32_t *__restrict__ pos, uint64_t *key) {
   // key: SORT_NEW_MAX 64-bit words of LDS, one per new site: sort key in the upper 51 bits, index of
   // the site among the new ones in the lower 13
@@ -536,18 +463,13 @@ __device__ __forceinline__ void order_append_sorted_body(const int32_t *__restri
     uint64_t k = ~0ull;
     if (i < n) {
       const int v = first + i;
-      if (MODE == 0) {
-        const int4 c = reinterpret_cast<const int4 *>(coords)[v];
-        uint32_t m = 0;
-        for (int j = 0; j < 27; j++) m |= (nbr[(int64_t)v * 27 + j] >= 0 ? 1u : 0u) << j;
-        // (8 bits of block coordinate per axis: blocks 16384 voxels apart share a group, harmless)
-        const uint64_t mort = spread3_10((uint64_t)((c.x >> 6) & 255)) | (spread3_10((uint64_t)((c.y >> 6) & 255)) << 1) |
-                              (spread3_10((uint64_t)((c.z >> 6) & 255)) << 2);
-        k = (mort << 27) | (uint64_t)m;
-      } else {
-        k = ((uint64_t)(offset[v] & 7) << 32) | (uint32_t)aux[v];
-      }
-      k = (k << 13) | (uint64_t)i;
+      const int4 c = reinterpret_cast<const int4 *>(coords)[v];
+      uint32_t m = 0;
+      for (int j = 0; j < 27; j++) m |= (nbr[(int64_t)v * 27 + j] >= 0 ? 1u : 0u) << j;
+      // (8 bits of block coordinate per axis: blocks 16384 voxels apart share a group, harmless)
+      const uint64_t mort = spread3_10((uint64_t)((c.x >> 6) & 255)) | (spread3_10((uint64_t)((c.y >> 6) & 255)) << 1) |
+                            (spread3_10((uint64_t)((c.z >> 6) & 255)) << 2);
+      k = (((mort << 27) | (uint64_t)m) << 13) | (uint64_t)i;
     }
     key[i] = k;
   }
@@ -582,31 +504,6 @@ __device__ __forceinline__ void order_append_sorted_body(const int32_t *__restri
     order[first + i] = v;
     if (pos) pos[v] = first + i;
   }
-}
-template <int MODE>
-__global__ __launch_bounds__(1024) void order_append_sorted_kernel(const int32_t *__restrict__ d_n,
-                                                                   const int32_t *__restrict__ coords,
-                                                                   const int32_t *__restrict__ nbr,
-                                                                   const int32_t *__restrict__ offset,
-                                                                   const int32_t *__restrict__ aux,
-                                                                   int32_t *__restrict__ order,
-                                                                   int32_t *__restrict__ pos) {
-  __shared__ uint64_t key[SORT_NEW_MAX];
-  order_append_sorted_body<MODE>(d_n, coords, nbr, offset, aux, order, pos, key);
-}
-// one workgroup per grid
-struct OrderJob {
-  const int32_t *d_n, *coords, *nbr, *offset, *aux;
-  int32_t *order, *pos;
-};
-struct OrderBatch {
-  OrderJob job[16];
-};
-template <int MODE>
-__global__ __launch_bounds__(1024) void order_append_sorted_batch_kernel(OrderBatch b) {
-  __shared__ uint64_t key[SORT_NEW_MAX];
-  const OrderJob &j = b.job[blockIdx.x];
-  order_append_sorted_body<MODE>(j.d_n, j.coords, j.nbr, j.offset, j.aux, j.order, j.pos, key);
 }
 // The new sites in the order grouped by the position inside the parent cell (eight groups, each in the
 // sequence of the processing order just written): a stable counting sort of that order, which gives
@@ -702,17 +599,10 @@ struct OrderBothBatch {
 __global__ __launch_bounds__(1024) void order_append_both_batch_kernel(OrderBothBatch b) {
   __shared__ uint64_t key[SORT_NEW_MAX];
   const OrderBothJob &j = b.job[blockIdx.x];
-  order_append_sorted_body<0>(j.d_n, j.coords, j.nbr, nullptr, nullptr, j.order, j.pos, key);
+  order_append_sorted_body(j.d_n, j.coords, j.nbr, j.order, j.pos, key);
   if (!j.offset) return;
   __syncthreads();  // the order written above is read below (by other threads than wrote it), and the LDS is reused
   order_append_grouped_body(j.d_n, j.offset, j.order, j.bo_order, j.bo_pos, key);
-}
-
-int order_append_new_sites(const insc_grid *g, int32_t *d_order, int32_t *d_pos, int64_t n_new_upper, hipStream_t s) {
-  if (n_new_upper <= 0) return INSC_OK;
-  hipLaunchKernelGGL(order_append_kernel, dim3(grid_for(n_new_upper, 256)), dim3(256), 0, s, g->d_n, d_order, d_pos);
-  INSC_LAUNCH_CHECK();
-  return INSC_OK;
 }
 
 int64_t order_sorted_max() { return SORT_NEW_MAX; }
@@ -1060,7 +950,6 @@ int frame_insert_levels(const FrameInsertLevel *lv, int n_levels, const int32_t 
   return INSC_OK;
 }
 
-int64_t frame_insert_max_points() { return (1ll << 30) / 16 - 1; }
 
 // ---- insert without allocation -------------------------------------------------------------
 // Scratch of insc_grid_insert_noalloc: the slot every row of the call claimed (what the grid's own,
@@ -1119,36 +1008,6 @@ int ssc3_new_sites_batch(const insc_grid *const *grids, int32_t *const *d_nbr, i
   return INSC_OK;
 }
 
-int order_append_new_sites_sorted_batch(const insc_grid *const *grids, const int32_t *const *d_nbr,
-                                        int32_t *const *d_order, int32_t *const *d_pos, int n, int64_t n_new_upper,
-                                        hipStream_t s) {
-  if (n <= 0 || n_new_upper <= 0) return INSC_OK;
-  if (n > 16) {
-    set_error("order_append_new_sites_sorted_batch: at most 16 grids");
-    return INSC_ERR_ARG;
-  }
-  OrderBatch b;
-  for (int i = 0; i < n; i++) b.job[i] = OrderJob{grids[i]->d_n, grids[i]->coords, d_nbr[i], nullptr, nullptr, d_order[i], d_pos[i]};
-  hipLaunchKernelGGL(order_append_sorted_batch_kernel<0>, dim3((unsigned)n), dim3(1024), 0, s, b);
-  INSC_LAUNCH_CHECK();
-  return INSC_OK;
-}
-
-int order_append_new_sites_by_offset_batch(const insc_grid *const *grids, const int32_t *const *d_offset,
-                                           const int32_t *const *d_pos_in_order, int32_t *const *d_order,
-                                           int32_t *const *d_pos, int n, int64_t n_new_upper, hipStream_t s) {
-  if (n <= 0 || n_new_upper <= 0) return INSC_OK;
-  if (n > 16) {
-    set_error("order_append_new_sites_by_offset_batch: at most 16 grids");
-    return INSC_ERR_ARG;
-  }
-  OrderBatch b;
-  for (int i = 0; i < n; i++) b.job[i] = OrderJob{grids[i]->d_n, nullptr, nullptr, d_offset[i], d_pos_in_order[i], d_order[i], d_pos[i]};
-  hipLaunchKernelGGL(order_append_sorted_batch_kernel<1>, dim3((unsigned)n), dim3(1024), 0, s, b);
-  INSC_LAUNCH_CHECK();
-  return INSC_OK;
-}
-
 int order_append_new_sites_both_batch(const insc_grid *const *grids, const int32_t *const *d_nbr,
                                       const int32_t *const *d_offset, int32_t *const *d_order, int32_t *const *d_pos,
                                       int32_t *const *d_bo_order, int32_t *const *d_bo_pos, int n, int64_t n_new_upper,
@@ -1162,24 +1021,6 @@ int order_append_new_sites_both_batch(const insc_grid *const *grids, const int32
   for (int i = 0; i < n; i++)
     b.job[i] = OrderBothJob{grids[i]->d_n, grids[i]->coords, d_nbr[i], d_offset[i], d_order[i], d_pos[i], d_bo_order[i], d_bo_pos[i]};
   hipLaunchKernelGGL(order_append_both_batch_kernel, dim3((unsigned)n), dim3(1024), 0, s, b);
-  INSC_LAUNCH_CHECK();
-  return INSC_OK;
-}
-
-int order_append_new_sites_sorted(const insc_grid *g, const int32_t *d_nbr, int32_t *d_order, int32_t *d_pos,
-                                  int64_t n_new_upper, hipStream_t s) {
-  if (n_new_upper <= 0) return INSC_OK;
-  hipLaunchKernelGGL(order_append_sorted_kernel<0>, dim3(1), dim3(1024), 0, s, g->d_n, g->coords, d_nbr, nullptr,
-                     nullptr, d_order, d_pos);
-  INSC_LAUNCH_CHECK();
-  return INSC_OK;
-}
-
-int order_append_new_sites_by_offset(const insc_grid *g, const int32_t *d_offset, const int32_t *d_pos_in_order,
-                                     int32_t *d_order, int32_t *d_pos, int64_t n_new_upper, hipStream_t s) {
-  if (n_new_upper <= 0) return INSC_OK;
-  hipLaunchKernelGGL(order_append_sorted_kernel<1>, dim3(1), dim3(1024), 0, s, g->d_n, nullptr, nullptr, d_offset,
-                     d_pos_in_order, d_order, d_pos);
   INSC_LAUNCH_CHECK();
   return INSC_OK;
 }

@@ -345,27 +345,6 @@ __global__ void gather_out_kernel(const float *__restrict__ in, int64_t ld_in, c
   }
 }
 
-// A frame is all or nothing: the first pass raises *bad if any coordinate of the frame cannot be
-// represented, the second pass then turns EVERY point of the frame into one the insert skips, so
-// that no grid, map or running sum changes and the host can report the error after the frame's one
-// round trip.  The flag holds the number of the last frame that raised it (frames are numbered from 1),
-// so it never needs clearing.
-__global__ void coords_check_kernel(const int32_t *__restrict__ in, int cols, int64_t P, int32_t *__restrict__ bad,
-                                    int32_t frame) {
-  int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (p >= P) return;
-  const int32_t *c = in + p * cols;
-  if (!coord_ok(c[0], c[1], c[2], cols > 3 ? c[3] : 0)) bad[0] = frame;
-}
-__global__ void coords_to_int4_kernel(const int32_t *__restrict__ in, int cols, int64_t P, int32_t *__restrict__ out,
-                                      const int32_t *__restrict__ bad, int32_t frame) {
-  int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (p >= P) return;
-  const int32_t *c = in + p * cols;
-  reinterpret_cast<int4 *>(out)[p] =
-      (bad && bad[0] == frame) ? make_int4(COORD_SKIP, 0, 0, 0) : make_int4(c[0], c[1], c[2], cols > 3 ? c[3] : 0);
-}
-
 // -----------------------------------------------------------------------------------------
 // host side
 // -----------------------------------------------------------------------------------------
@@ -512,22 +491,7 @@ static int points_reserve(insc_net *net, int64_t need, hipStream_t s) {
   return INSC_OK;
 }
 
-// the site counts and error flags of all scales, as they lie in net->h_counts
-static int apply_counts(insc_net *net, const char *who);
-
-static int sync_counts(insc_net *net, hipStream_t s, const char *who) {
-  const int L = net->n_levels;
-  INSC_HIP(hipMemcpyAsync(net->h_counts + 2 * L, net->d_bad, sizeof(int32_t), hipMemcpyDeviceToHost, s));
-  for (int l = 0; l < L; l++) {
-    INSC_HIP(hipMemcpyAsync(net->h_counts + 2 * l, net->levels[l].grid->d_n, sizeof(int32_t),
-                            hipMemcpyDeviceToHost, s));
-    INSC_HIP(hipMemcpyAsync(net->h_counts + 2 * l + 1, net->levels[l].grid->d_err, sizeof(int32_t),
-                            hipMemcpyDeviceToHost, s));
-  }
-  INSC_HIP(hipStreamSynchronize(s));
-  return apply_counts(net, who);
-}
-
+// the site counts and error flags of all scales, as the insert kernels left them in net->h_counts
 static int apply_counts(insc_net *net, const char *who) {
   const int L = net->n_levels;
   for (int l = 0; l < L; l++) {
@@ -1144,12 +1108,10 @@ int insc_net_forward(insc_net *net, const int32_t *d_coords, int coord_cols, con
   net->frame_P = P;
   // A frame inserts at all scales at once (three launches up to 16k points, seven beyond), which also
   // leaves the new site counts in host memory; the host picks them up further down, while the GPU is
-  // busy with the neighbour maps and orders of the new sites.  (The scale-by-scale chain below is left
-  // for frames beyond 2^26 points.)
-  const bool fused_insert = P > 0 && P <= frame_insert_max_points();
+  // busy with the neighbour maps and orders of the new sites.
   if (P > 0) {
     Level &L0 = net->levels[0];
-    if (fused_insert) {
+    {
       FrameInsertLevel fl[16];
       for (int l = 0; l < L; l++) {
         Level &Lv = net->levels[l];
@@ -1158,22 +1120,6 @@ int insc_net_forward(insc_net *net, const int32_t *d_coords, int coord_cols, con
       if ((rc = frame_insert_levels(fl, L, d_coords, coord_cols, P, net->d_bad, net->frame_id, sop, net->h_counts, s)))
         return rc;
       INSC_HIP(hipEventRecord(net->ev_counts, s));
-    } else {
-      // ---- input scale: insert ----------------------------------------------------------------
-      void *ws;
-      if ((rc = workspace(WS_API, s, sizeof(int32_t) * 4 * (size_t)P, &ws))) return rc;
-      int32_t *c4 = (int32_t *)ws;
-      hipLaunchKernelGGL(coords_check_kernel, dim3(grid_for(P, 256)), dim3(256), 0, s, d_coords, coord_cols, P, net->d_bad,
-                         net->frame_id);
-      hipLaunchKernelGGL(coords_to_int4_kernel, dim3(grid_for(P, 256)), dim3(256), 0, s, d_coords, coord_cols, P, c4,
-                         net->d_bad, net->frame_id);
-      INSC_LAUNCH_CHECK();
-      if ((rc = grid_insert_nosync(L0.grid, c4, P, sop, s))) return rc;
-      // ---- coarser scales: the new sites of a scale are the parents of the new sites below ---
-      for (int l = 0; l + 1 < L; l++) {
-        Level &F = net->levels[l], &Cs = net->levels[l + 1];
-        if ((rc = down2_new_sites(F.grid, Cs.grid, P, F.parent, F.offset, F.child, s))) return rc;
-      }
     }
     // ---- neighbour maps and processing orders of the new sites, all scales per launch ------
     const insc_grid *grids[16];
@@ -1222,11 +1168,9 @@ int insc_net_forward(insc_net *net, const int32_t *d_coords, int coord_cols, con
   if (!inc) {
     // A full frame may synchronise: learn the exact counts, then build the processing orders
     // (pattern-sorted for the 3^3 convolutions, offset-grouped for the deconvolutions).
-    if (fused_insert) {
+    if (P > 0) {
       INSC_HIP(hipEventSynchronize(net->ev_counts));
       if ((rc = apply_counts(net, "insc_net_forward"))) return rc;
-    } else if ((rc = sync_counts(net, s, "insc_net_forward"))) {
-      return rc;
     }
     {
       // the small scales: all their sites came with this frame's one insert, and the single-workgroup
@@ -1269,11 +1213,9 @@ int insc_net_forward(insc_net *net, const int32_t *d_coords, int coord_cols, con
     // (tens of microseconds) buys launches sized to the real number of tiles.  With the bound
     // "every new point is a new site at every scale" a coarse scale of 70 sites would be
     // launched for thousands, and idle blocks cost more than the convolution itself.
-    if (fused_insert) {
+    if (P > 0) {
       INSC_HIP(hipEventSynchronize(net->ev_counts));
       if ((rc = apply_counts(net, "insc_net_forward"))) return rc;
-    } else if ((rc = sync_counts(net, s, "insc_net_forward"))) {
-      return rc;
     }
   }
 
