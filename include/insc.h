@@ -70,6 +70,23 @@ int insc_grid_reserve(insc_grid *g, int64_t capacity_sites, void *stream);
  * 766-796; kernels CUDPPWrapper.cu:72-100,212-231). */
 int insc_grid_insert(insc_grid *g, const int32_t *d_coords4, int64_t P, int32_t *d_site_of_point, int64_t *h_n_sites,
                      void *stream);
+/* The points of a frame inserted at ALL scales of a network at once: grids[0] takes the points
+ * (d_coords: int32 [P, coord_cols], coord_cols 3 or 4), grids[l] the cells coordinate >> l, and for
+ * every scale l < n_scales - 1 the link to the next coarser one is filled in for the sites this call
+ * adds: d_parent[l][i] = coarse site, d_offset[l][i] = (x&1)*4 + (y&1)*2 + (z&1), d_child[l][parent*8 +
+ * offset] = i (rows of new coarse sites must have been filled with -1 by the caller).  Same grids, ids
+ * and links as insc_grid_insert on grids[0] followed by insc_rulebook_down2 scale by scale - the
+ * reference's order of construction (Metadata.cpp inputLayer, then getRuleBook / ConvolutionRules.h:
+ * 344-380 per scale) - in 3 to 7 kernel launches for any number of scales: a site that is new at scale l
+ * has only new sites below it, so the ids that chain hands out follow the smallest row of the point
+ * list that falls into each new cell, which every scale can work out from the points themselves.
+ * d_site_of_point: [P] site at grids[0].  h_n_sites (nullable): [n_scales] site counts after the call.
+ * Differences to the chain: a frame is all or nothing (one bad coordinate: INSC_ERR_COORD and nothing
+ * is inserted anywhere), and no grid grows (every grid must have room for P more sites:
+ * INSC_ERR_CAPACITY otherwise; insc_grid_reserve beforehand).  The call synchronises the stream. */
+int insc_grid_insert_scales(insc_grid *const *grids, int32_t *const *d_parent, int32_t *const *d_offset,
+                            int32_t *const *d_child, int n_scales, const int32_t *d_coords, int coord_cols, int64_t P,
+                            int32_t *d_site_of_point, int64_t *h_n_sites, void *stream);
 /* insc_grid_insert for callers that cannot allocate device memory (code under HIP graph capture,
  * tight serving loops, harnesses that forbid it).  No counterpart in the reference.  Same result
  * as insc_grid_insert, with two limits: at most 16384 points per call (INSC_ERR_CAPACITY beyond),

@@ -1255,4 +1255,53 @@ int insc_rulebook_down2(const insc_grid *fine, insc_grid *coarse, int64_t first,
   return INSC_OK;
 }
 
+int insc_grid_insert_scales(insc_grid *const *grids, int32_t *const *d_parent, int32_t *const *d_offset,
+                            int32_t *const *d_child, int n_scales, const int32_t *d_coords, int coord_cols, int64_t P,
+                            int32_t *d_site_of_point, int64_t *h_n_sites, void *stream) {
+  INSC_REQUIRE(grids && n_scales >= 1 && n_scales <= 16, INSC_ERR_ARG, "insc_grid_insert_scales: 1..16 scales");
+  INSC_REQUIRE(P >= 0 && (coord_cols == 3 || coord_cols == 4), INSC_ERR_ARG, "insc_grid_insert_scales: bad arguments");
+  INSC_REQUIRE(P == 0 || (d_coords && d_site_of_point), INSC_ERR_ARG, "insc_grid_insert_scales: null pointer");
+  INSC_REQUIRE(n_scales == 1 || (d_parent && d_offset && d_child), INSC_ERR_ARG,
+               "insc_grid_insert_scales: the link arrays are missing");
+  hipStream_t s = (hipStream_t)stream;
+  FrameInsertLevel lv[16];
+  for (int l = 0; l < n_scales; l++) {
+    INSC_REQUIRE(grids[l], INSC_ERR_ARG, "insc_grid_insert_scales: grid %d is null", l);
+    for (int k = 0; k < l; k++) INSC_REQUIRE(grids[k] != grids[l], INSC_ERR_ARG, "insc_grid_insert_scales: grid %d given twice", l);
+    const bool link = l + 1 < n_scales;
+    INSC_REQUIRE(!link || (d_parent[l] && d_offset[l] && d_child[l]), INSC_ERR_ARG,
+                 "insc_grid_insert_scales: link arrays of scale %d are null", l);
+    lv[l] = FrameInsertLevel{grids[l], link ? d_parent[l] : nullptr, link ? d_offset[l] : nullptr, link ? d_child[l] : nullptr};
+  }
+  if (P > 0) {
+    // the flag "some coordinate is bad" and the counts the kernels leave: 2 * scales + 2 words
+    void *ws;
+    int rc = workspace(WS_SORT, s, 64 * sizeof(int32_t), &ws);
+    if (rc) return rc;
+    int32_t *d_bad = (int32_t *)ws, *d_counts = d_bad + 1;
+    INSC_HIP(hipMemsetAsync(d_bad, 0, sizeof(int32_t), s));
+    if ((rc = frame_insert_levels(lv, n_scales, d_coords, coord_cols, P, d_bad, 1, d_site_of_point, d_counts, s))) return rc;
+    int32_t dropped = 0;
+    INSC_HIP(hipMemcpyAsync(&dropped, d_counts + 2 * n_scales, sizeof(int32_t), hipMemcpyDeviceToHost, s));
+    INSC_HIP(hipStreamSynchronize(s));
+    // the exact counts, and the capacity flag of every scale (reported once, then cleared)
+    int first_err = INSC_OK;
+    for (int l = 0; l < n_scales; l++) {
+      rc = grid_sync_errors(grids[l], s, "insc_grid_insert_scales");
+      if (rc && !first_err) first_err = rc;
+    }
+    INSC_REQUIRE(dropped != 1, INSC_ERR_COORD,
+                 "insc_grid_insert_scales: a coordinate is outside 0..65535 (batch 0..32767); nothing was inserted");
+    if (first_err) return first_err;
+  }
+  if (h_n_sites)
+    for (int l = 0; l < n_scales; l++) {
+      int64_t n = 0;
+      int rc = insc_grid_size(grids[l], &n, stream);
+      if (rc) return rc;
+      h_n_sites[l] = n;
+    }
+  return INSC_OK;
+}
+
 }  // extern "C"

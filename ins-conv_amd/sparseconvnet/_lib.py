@@ -22,6 +22,8 @@ _SIGS = {
     "insc_grid_reserve": [vp, c_i64, vp],
     "insc_grid_insert": [vp, vp, c_i64, vp, ctypes.POINTER(c_i64), vp],
     "insc_grid_insert_noalloc": [vp, vp, c_i64, vp, ctypes.POINTER(c_i64), vp],
+    "insc_grid_insert_scales": [ctypes.POINTER(vp), ctypes.POINTER(vp), ctypes.POINTER(vp), ctypes.POINTER(vp), c_int,
+                                vp, c_int, c_i64, vp, ctypes.POINTER(c_i64), vp],
     "insc_grid_query": [vp, vp, c_i64, vp, vp],
     "insc_grid_size": [vp, ctypes.POINTER(c_i64), vp],
     "insc_rulebook_ssc3": [vp, c_i64, c_i64, vp, c_int, vp],

@@ -192,3 +192,97 @@ def test_down2_rulebook_matches_oracle(S, orc):
     bo = m.deconv_order(fine, d)[:fine.n].cpu().numpy()
     assert (np.sort(bo) == np.arange(fine.n)).all()
     assert (np.diff(off[bo]) >= 0).all()
+
+
+@pytest.mark.parametrize("P", [3000, 40000])
+def test_insert_at_all_scales_equals_the_scale_by_scale_chain(S, P):
+    """insc_grid_insert_scales (claim / rank / link at every scale straight from the points) must leave
+    the same grids - site ids, coordinates - and the same parent / offset / child links as the chain it
+    replaces, insc_grid_insert followed by insc_rulebook_down2 scale by scale; two frames, the second
+    with points on old cells, on new cells and repeated, below and above the 16k points one workgroup
+    per scale ranks."""
+    import ctypes
+
+    from sparseconvnet._lib import InscError, lib, ptr, stream_ptr
+
+    L = 5
+    vox = scenes.indoor_scene(seed=61, n=2 * P, dims=(200, 160, 60), n_boxes=12, side_rng=(10, 40)).astype(np.int32)
+    rng = np.random.default_rng(61)
+    idx2 = np.concatenate([np.arange(P, 2 * P), rng.integers(0, P, P // 8), rng.integers(P, 2 * P, P // 8)])
+    frames = [vox[:P], vox[idx2[rng.permutation(len(idx2))]]]
+    cap = 4 * P
+    vp = ctypes.c_void_p
+
+    def new_grids():
+        gs = []
+        for _ in range(L):
+            g = vp()
+            lib.insc_grid_create(I64(cap), ctypes.byref(g))
+            gs.append(g)
+        par = [torch.full((cap,), -7, dtype=torch.int32, device="cuda") for _ in range(L - 1)]
+        off = [torch.full((cap,), -7, dtype=torch.int32, device="cuda") for _ in range(L - 1)]
+        chi = [torch.full((cap, 8), -1, dtype=torch.int32, device="cuda") for _ in range(L - 1)]
+        return gs, par, off, chi
+
+    def sizes(gs):
+        out = []
+        for g in gs:
+            n = I64(0)
+            lib.insc_grid_size(g, ctypes.byref(n), stream_ptr())
+            out.append(n.value)
+        return out
+
+    # the chain
+    ga, pa, oa, ca = new_grids()
+    sop_a = []
+    for f in frames:
+        c = dev(f)
+        sop = torch.empty(len(f), dtype=torch.int32, device="cuda")
+        before = sizes(ga)
+        lib.insc_grid_insert(ga[0], ptr(c), I64(len(f)), ptr(sop), None, stream_ptr())
+        after0 = sizes(ga)[0]
+        first, n = before[0], after0 - before[0]
+        for l in range(L - 1):
+            nb = sizes(ga)[l + 1]
+            lib.insc_rulebook_down2(ga[l], ga[l + 1], I64(first), I64(n), ptr(pa[l]), ptr(oa[l]), ptr(ca[l]), I64(cap),
+                                    stream_ptr())
+            first, n = nb, sizes(ga)[l + 1] - nb
+        sop_a.append(sop)
+    # all scales at once
+    gb, pb, ob, cb = new_grids()
+    arr = lambda xs: (vp * len(xs))(*[x if isinstance(x, vp) else vp(x.data_ptr()) for x in xs])
+    sop_b = []
+    counts = (I64 * L)()
+    for f in frames:
+        c = dev(f)
+        sop = torch.empty(len(f), dtype=torch.int32, device="cuda")
+        lib.insc_grid_insert_scales(arr(gb), arr(pb + [pb[0]]), arr(ob + [ob[0]]), arr(cb + [cb[0]]), L, ptr(c), 4,
+                                    I64(len(f)), ptr(sop), counts, stream_ptr())
+        sop_b.append(sop)
+    na, nb_ = sizes(ga), sizes(gb)
+    assert na == nb_ == list(counts)
+    for a, b in zip(sop_a, sop_b):
+        assert torch.equal(a, b)
+    for l in range(L):
+        from sparseconvnet.SCN import _from_ptr
+
+        dv = torch.device("cuda", torch.cuda.current_device())
+        ca_ = _from_ptr(lib.insc_grid_coords(ga[l]), (na[l], 4), torch.int32, dv)
+        cb_ = _from_ptr(lib.insc_grid_coords(gb[l]), (na[l], 4), torch.int32, dv)
+        assert torch.equal(ca_, cb_), "site coordinates of scale %d" % l
+        if l + 1 < L:
+            assert torch.equal(pa[l][:na[l]], pb[l][:na[l]]), "parents of scale %d" % l
+            assert torch.equal(oa[l][:na[l]], ob[l][:na[l]]), "offsets of scale %d" % l
+            assert torch.equal(ca[l][:na[l + 1]], cb[l][:na[l + 1]]), "children of scale %d" % (l + 1)
+    # a bad coordinate: nothing is inserted anywhere, the grids stay usable
+    bad = frames[1].copy()
+    bad[7, 2] = 1 << 17
+    c = dev(bad)
+    sop = torch.empty(len(bad), dtype=torch.int32, device="cuda")
+    with pytest.raises(InscError) as e:
+        lib.insc_grid_insert_scales(arr(gb), arr(pb + [pb[0]]), arr(ob + [ob[0]]), arr(cb + [cb[0]]), L, ptr(c), 4,
+                                    I64(len(bad)), ptr(sop), counts, stream_ptr())
+    assert e.value.code == -5
+    assert sizes(gb) == na
+    for g in ga + gb:
+        lib.insc_grid_destroy(g)
