@@ -79,6 +79,10 @@ int order_append_new_sites_both_batch(const insc_grid *const *grids, const int32
                                       const int32_t *const *d_offset, int32_t *const *d_order, int32_t *const *d_pos,
                                       int32_t *const *d_bo_order, int32_t *const *d_bo_pos, int n, int64_t n_new_upper,
                                       hipStream_t s);
+// insc_grid_clear for several grids in one launch; with grid i the int32 array minus1[i] (n_minus1[i]
+// words, nullable) is set to -1, and `zero` (nullable, zero_bytes a multiple of 4) is zeroed
+int grid_clear_batch(insc_grid *const *grids, int32_t *const *minus1, const int64_t *n_minus1, int n, void *zero,
+                     int64_t zero_bytes, hipStream_t s);
 // most sites the two sorted appends put in order (more keep their arrival order)
 int64_t order_sorted_max();
 // device pointer to the site count before the most recent insert

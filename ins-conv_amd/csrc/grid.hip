@@ -607,6 +607,67 @@ __global__ __launch_bounds__(1024) void order_append_both_batch_kernel(OrderBoth
 
 int64_t order_sorted_max() { return SORT_NEW_MAX; }
 
+// Several grids emptied in one launch, and with each (optionally) an int32 array set to -1 - the child
+// map that hangs off it - and one more array zeroed (running sums of an input layer).
+struct ClearJob {
+  Slot *table;
+  int64_t n_slots;
+  int32_t *d_n, *d_err;
+  int32_t *minus1;
+  int64_t n_minus1;
+};
+struct ClearBatch {
+  ClearJob job[16];
+  uint32_t *zero;  // 4-byte words
+  int64_t n_zero;
+};
+__global__ __launch_bounds__(256) void grid_clear_batch_kernel(ClearBatch b, int n) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if ((int)blockIdx.y == n) {
+    for (int64_t i = t; i < b.n_zero; i += stride) b.zero[i] = 0u;
+    return;
+  }
+  const ClearJob &j = b.job[blockIdx.y];
+  for (int64_t i = t; i < j.n_slots; i += stride) {
+    Slot e;
+    e.key = INSC_EMPTY_KEY;
+    e.val = VAL_UNSET;
+    e.pad = 0;
+    j.table[i] = e;
+  }
+  for (int64_t i = t; i < j.n_minus1; i += stride) j.minus1[i] = -1;
+  if (t == 0) {
+    j.d_n[0] = 0;
+    j.d_n[1] = 0;
+    *j.d_err = 0;
+  }
+}
+
+int grid_clear_batch(insc_grid *const *grids, int32_t *const *minus1, const int64_t *n_minus1, int n, void *zero,
+                     int64_t zero_bytes, hipStream_t s) {
+  if (n <= 0 || n > 16 || (zero_bytes & 3)) {
+    set_error("grid_clear_batch: 1..16 grids, a multiple of four bytes to zero");
+    return INSC_ERR_ARG;
+  }
+  ClearBatch b;
+  int64_t most = zero_bytes / 4;
+  for (int i = 0; i < n; i++) {
+    insc_grid *g = grids[i];
+    b.job[i] = ClearJob{g->table, g->n_slots, g->d_n, g->d_err, minus1 ? minus1[i] : nullptr,
+                        (minus1 && minus1[i]) ? n_minus1[i] : 0};
+    most = std::max(most, std::max(g->n_slots, b.job[i].n_minus1));
+    g->n_upper = 0;
+    g->n_exact = 0;
+  }
+  b.zero = (uint32_t *)zero;
+  b.n_zero = zero ? zero_bytes / 4 : 0;
+  hipLaunchKernelGGL(grid_clear_batch_kernel, dim3(grid_for(most, 256, 2048), (unsigned)(n + (b.n_zero ? 1 : 0))), dim3(256),
+                     0, s, b, n);
+  INSC_LAUNCH_CHECK();
+  return INSC_OK;
+}
+
 // ---- the inserts of a whole frame, all scales at once ----------------------------------------
 // The reference inserts scale by scale: the sites a frame adds at one scale are halved and inserted
 // at the next coarser one, a chain in which every step waits for the ids of the step before.  The

@@ -1074,14 +1074,19 @@ int insc_net_forward(insc_net *net, const int32_t *d_coords, int coord_cols, con
   net->frame_id = net->frame_id == INT32_MAX ? 1 : net->frame_id + 1;
 
   if (!inc) {
+    // all grids emptied, the child maps back to -1 and the input layer's running sums to zero: one launch
+    insc_grid *gs[16];
+    int32_t *chi[16];
+    int64_t nchi[16];
     for (int l = 0; l < L; l++) {
       Level &Lv = net->levels[l];
-      if ((rc = insc_grid_clear(Lv.grid, stream))) return rc;
+      gs[l] = Lv.grid;
+      chi[l] = (l + 1 < L && Lv.child_rows) ? Lv.child : nullptr;
+      nchi[l] = Lv.child_rows * 8;
       Lv.n = Lv.n_upper = 0;
-      if (l + 1 < L && Lv.child_rows)
-        if ((rc = fill_i32(Lv.child, Lv.child_rows * 8, -1, s))) return rc;
     }
-    INSC_HIP(hipMemsetAsync(net->in_sum, 0, sizeof(float) * (size_t)net->levels[0].cap * C0, s));
+    if ((rc = grid_clear_batch(gs, chi, nchi, L, net->in_sum, (int64_t)sizeof(float) * net->levels[0].cap * C0, s)))
+      return rc;
     INSC_HIP(hipMemsetAsync(net->in_cnt, 0, sizeof(int32_t) * (size_t)net->levels[0].cap, s));
     net->n_points = 0;
     net->have_state = false;
@@ -1476,13 +1481,17 @@ int insc_net_forward_residual(insc_net *net, const int32_t *d_coords, int coord_
   if ((rc = rframe_reserve(net, P, s))) return rc;
 
   // ---- the frame's own site set --------------------------------------------------------------
-  for (int l = 0; l < L; l++) {
-    Level &Lv = R.levels[l];
-    if ((rc = insc_grid_clear(Lv.grid, stream))) return rc;
-    if (l + 1 < L)
-      if ((rc = fill_i32(Lv.child, P * 8, -1, s))) return rc;  // a scale has at most P sites
+  {
+    insc_grid *gs[16];
+    int32_t *chi[16];
+    int64_t nchi[16];
+    for (int l = 0; l < L; l++) {
+      gs[l] = R.levels[l].grid;
+      chi[l] = l + 1 < L ? R.levels[l].child : nullptr;
+      nchi[l] = P * 8;  // a scale has at most P sites
+    }
+    if ((rc = grid_clear_batch(gs, chi, nchi, L, R.in_sum, (int64_t)sizeof(float) * P * C0, s))) return rc;
   }
-  INSC_HIP(hipMemsetAsync(R.in_sum, 0, sizeof(float) * (size_t)P * C0, s));
   INSC_HIP(hipMemsetAsync(R.in_cnt, 0, sizeof(int32_t) * (size_t)P, s));
   const unsigned nb = grid_for(P, 256);
   // the inserts of all scales at once, as in an exact frame; the counts arrive in host memory
