@@ -95,45 +95,52 @@ __global__ void grid_claim_kernel(Slot *table, int64_t mask, const int32_t *__re
   atomicMin(&table[found].val, VAL_PENDING + (int)p);
 }
 
+// pass 2 of a large insert: flag the winning rows for the scan and leave for every row what pass 3
+// needs in site_of_point: the winner's row (>= 0), -1 for a skipped row, or -2 - id for a cell that
+// held a site before this insert.  Row 0 also saves the site count from before the insert beside
+// the scan's total, so that pass 3 can replace the counters while its other threads still read it.
 __global__ void grid_flag_kernel(const Slot *__restrict__ table, const int32_t *__restrict__ slot_of_point, int64_t P,
-                                 int32_t *__restrict__ flags) {
+                                 int32_t *__restrict__ flags, int32_t *__restrict__ site_of_point,
+                                 const int32_t *__restrict__ d_n, int32_t *__restrict__ n_before) {
   int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (p >= P) return;
+  if (p == 0) *n_before = d_n[0];
   int s = slot_of_point[p];
-  flags[p] = (s >= 0 && table[s].val == VAL_PENDING + (int)p) ? 1 : 0;
+  int v = s >= 0 ? table[s].val : -1;
+  flags[p] = (s >= 0 && v == VAL_PENDING + (int)p) ? 1 : 0;
+  site_of_point[p] = s < 0 ? -1 : v >= VAL_PENDING ? v - VAL_PENDING : -2 - v;
 }
 
-// pass 3: winners take id = n_before + rank, publish it in the slot and record the coordinates
+// pass 3: winners take id = n_before + rank, publish it in the slot and record the coordinates; every
+// row learns its site from its winner's rank; row 0 moves the counters on
 __global__ void grid_assign_kernel(Slot *table, const int32_t *__restrict__ coords4,
                                    const int32_t *__restrict__ slot_of_point, const int32_t *__restrict__ excl,
-                                   int64_t P, const int32_t *__restrict__ d_n, int32_t *__restrict__ site_coords,
-                                   int64_t capacity_sites, int32_t *d_err) {
+                                   int64_t P, int32_t *__restrict__ d_n, const int32_t *__restrict__ total,
+                                   int32_t *__restrict__ site_coords, int64_t capacity_sites, int32_t *d_err,
+                                   int32_t *__restrict__ site_of_point) {
   int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (p >= P) return;
-  int s = slot_of_point[p];
-  if (s < 0 || table[s].val != VAL_PENDING + (int)p) return;
-  int id = *d_n + excl[p];
-  if (id >= capacity_sites) {
-    atomicOr(d_err, 2);
+  const int n_before = total[1];
+  if (p == 0) {
+    d_n[1] = n_before;
+    d_n[0] = n_before + total[0];
+  }
+  int r = site_of_point[p];
+  if (r < 0) {
+    if (r < -1) site_of_point[p] = -2 - r;
     return;
   }
-  table[s].val = id;
-  reinterpret_cast<int4 *>(site_coords)[id] = reinterpret_cast<const int4 *>(coords4)[p];
-}
-
-__global__ void grid_resolve_kernel(const Slot *__restrict__ table, const int32_t *__restrict__ slot_of_point,
-                                    int64_t P, int32_t *__restrict__ site_of_point, int32_t *d_n,
-                                    const int32_t *__restrict__ total) {
-  int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (p < P) {
-    int s = slot_of_point[p];
-    int v = (s >= 0) ? table[s].val : -1;
-    site_of_point[p] = (v >= 0 && v < VAL_PENDING) ? v : -1;
+  int id = n_before + excl[r];
+  if (id >= capacity_sites) {
+    site_of_point[p] = -1;
+    if (r == p) atomicOr(d_err, 2);
+    return;
   }
-}
-__global__ void grid_bump_kernel(int32_t *d_n, const int32_t *total) {
-  d_n[1] = d_n[0];
-  d_n[0] += *total;
+  site_of_point[p] = id;
+  if (r == p) {
+    table[slot_of_point[p]].val = id;
+    reinterpret_cast<int4 *>(site_coords)[id] = reinterpret_cast<const int4 *>(coords4)[p];
+  }
 }
 
 // Passes 2-4 and the counter update in one workgroup, for inserts of up to FINISH_SMALL_MAX rows
@@ -402,15 +409,13 @@ static int grid_insert_launch(insc_grid *g, const int32_t *d_coords4, int64_t P,
     g->n_exact = -1;
     return INSC_OK;
   }
-  hipLaunchKernelGGL(grid_flag_kernel, dim3(nb), dim3(256), 0, s, g->table, g->slot_of_point, P, g->flags);
+  hipLaunchKernelGGL(grid_flag_kernel, dim3(nb), dim3(256), 0, s, g->table, g->slot_of_point, P, g->flags,
+                     d_site_of_point, g->d_n, total + 1);
   INSC_LAUNCH_CHECK();
   rc = scan_exclusive_i32(g->flags, g->flags, P, total, s);
   if (rc) return rc;
   hipLaunchKernelGGL(grid_assign_kernel, dim3(nb), dim3(256), 0, s, g->table, d_coords4, g->slot_of_point, g->flags,
-                     P, g->d_n, g->coords, g->capacity_sites, g->d_err);
-  hipLaunchKernelGGL(grid_resolve_kernel, dim3(nb), dim3(256), 0, s, g->table, g->slot_of_point, P, d_site_of_point,
-                     g->d_n, total);
-  hipLaunchKernelGGL(grid_bump_kernel, dim3(1), dim3(1), 0, s, g->d_n, total);
+                     P, g->d_n, total, g->coords, g->capacity_sites, g->d_err, d_site_of_point);
   INSC_LAUNCH_CHECK();
   g->n_upper += P;
   g->n_exact = -1;
