@@ -72,6 +72,20 @@ struct BnEpilogue {
   int64_t ld_side = 0;
   float *side_out = nullptr;
   const float *side_w = nullptr, *side_b = nullptr;
+  // optional second source of a split launch (residual frames: the saved features join the frame's
+  // own): a second set of blocks per (tile, output block) gathers from src2_in through src2_map
+  // (in the place of map0; a parent map shares map1) with the same weights, and the sums of both
+  // sets are added up in block order.  src2_rows: rows of src2_in.
+  const float *src2_in = nullptr;
+  int64_t src2_ld = 0, src2_rows = 0;
+  const int32_t *src2_map = nullptr;
+  // optional: the batch norm behind out2 is that of a residual frame (incre_bn_kernel, same
+  // arithmetic): for a row whose site existed (pre_exist[row] = its saved row, or -1)
+  //   out2 = leaky(w * pre_in[saved row] + (w * x + b)) - pre_out[saved row].
+  // Split launches of 3^3 layers with latency != 0 only.
+  const int32_t *pre_exist = nullptr;
+  const float *pre_in = nullptr, *pre_out = nullptr;
+  int64_t ld_pin = 0, ld_pout = 0;
 };
 // w = gamma / sqrt(var + eps), b = beta - mean * w   (gamma / beta nullable)
 int bn_scale_shift(const float *mean, const float *var, const float *gamma, const float *beta, float eps, int C,
@@ -116,6 +130,9 @@ int launch_conv(const float *in, int64_t ld_in, int64_t in_rows, float *out, int
                 const int32_t *rows, const int32_t *d_n_rows, int64_t n_rows, int Cin, int Cout,
                 const uint8_t *tile_flags, const uint8_t *row_mask, hipStream_t s, BnEpilogue ep = BnEpilogue(),
                 TilePlan plan = TilePlan(), int latency = 0, int64_t expect_rows = 0);
+// whether launch_conv takes a second source (BnEpilogue::src2_*) for this shape
+bool conv_two_sources_ok(int mode, int K, const float *in, int64_t ld_in, const float *in2, int64_t ld_in2,
+                         int64_t in2_rows, int Cin, int latency);
 int64_t packed_floats(int K, int Cin, int Cout);
 int pack_weights(const float *W, int K, int Cin, int Cout, float *Wp, hipStream_t s);
 int launch_bn(const float *in, int64_t ld_in, float *out, int64_t ld_out, const float *mean, const float *var,
@@ -130,6 +147,17 @@ int launch_incre_bn(const float *in, int64_t ld_in, float *out, int64_t ld_out, 
                     const float *gamma, const float *beta, float eps, float leak, const float *w, const float *b,
                     const int32_t *pre_exist, const float *pre_in, int64_t ld_pin, const float *pre_out,
                     int64_t ld_pout, int64_t n, int C, hipStream_t s);
+// the two convolutions of a residual frame (incre.hip; insc_incre_conv_ssc / insc_incre_deconv_down2
+// with an optional element-wise sum: out = result + res; the 3^3 one also takes the batch norm of
+// a residual frame in ep where conv_two_sources_ok says that it runs as one launch)
+int incre_conv_ssc(const float *in, int64_t ld_in, const float *pre_in, int64_t ld_pre, int64_t n_pre_rows, float *out,
+                   int64_t ld_out, const float *W, const float *Wp, const float *bias, const int32_t *nbr,
+                   const int32_t *nbr_pre, int64_t n, int Cin, int Cout, BnEpilogue ep, hipStream_t s);
+int incre_deconv_down2(const float *in, int64_t ld_in, int64_t n_in_rows, const float *pre_in, int64_t ld_pre,
+                       int64_t n_pre_rows, float *out, int64_t ld_out, const float *W, const float *Wp,
+                       const float *bias, const int32_t *parent, const int32_t *offset, const int32_t *pre_exist_in,
+                       const int32_t *pre_exist_out, int64_t n_rows, int Cin, int Cout, const float *res, int64_t ldr,
+                       hipStream_t s);
 int launch_input_finish(const float *sum, const int32_t *cnt, int mode, float *out, int64_t ld_out,
                         const int32_t *rows, const int32_t *d_n_rows, int64_t n_rows, int C,
                         const uint8_t *row_mask, hipStream_t s);
@@ -144,6 +172,12 @@ static inline unsigned grid_for(int64_t n, int block, int64_t cap = 1 << 20) {
 
 // ---- device helpers shared by the streaming kernels ------------------------------------
 __device__ __forceinline__ float leaky(float o, float leak) { return o * ((o > 0.0f) ? 1.0f : leak); }
+// a - b as a subtraction of its own, never contracted with the product that formed a (two code
+// sites that must give the same bits use it)
+__device__ __forceinline__ float sub_exact(float a, float b) {
+#pragma clang fp contract(off)
+  return a - b;
+}
 
 // per-channel scale / shift of inference batch norm; every kernel that normalises goes through
 // this one function so that fused and unfused paths give the same bits

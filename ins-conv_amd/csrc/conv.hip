@@ -254,8 +254,19 @@ __global__ __launch_bounds__((S == 1 ? CONV_WAVES : S) * 64) void conv_mfma_kern
   const int64_t t0 = (by_cost ? (int64_t)plan.sched[slot] : slot) * TILE_M;
   const int cb0 = by * NB;  // first output-channel block of this column group
   const int nch = conv_nch(Cin);
-  // the items of a tile are dealt to S wavefronts in each of G = gridDim.z blocks
-  const int G = S == 1 ? 1 : (int)gridDim.z, ST = S * G, ws = wave * G + (S == 1 ? 0 : (int)bz);
+  // the items of a tile are dealt to S wavefronts in each of G blocks; gridDim.z = GZ holds G blocks
+  // per source (two sources: the blocks from G on gather from the second one, through its own map)
+  const int GZ = S == 1 ? 1 : (int)gridDim.z;
+  const bool second = S > 1 && ep.src2_in != nullptr && (int)bz >= GZ / 2;
+  const int G = (S > 1 && ep.src2_in != nullptr) ? GZ / 2 : GZ, ST = S * G;
+  const int ws = wave * G + (S == 1 ? 0 : (int)bz - (second ? G : 0));
+  if (second) {
+    in = ep.src2_in;
+    ld_in = ep.src2_ld;
+    in_bytes = (uint32_t)(ep.src2_rows * ep.src2_ld * 4);
+    map0 = ep.src2_map;
+    bias = nullptr;
+  }
 
   // blocks beyond the row count leave at once (launches are sized by an upper bound of it)
   if ((S == 1 ? (int64_t)bx * WAVES : (int64_t)bx) * TILE_M >= n) return;
@@ -263,6 +274,10 @@ __global__ __launch_bounds__((S == 1 ? CONV_WAVES : S) * 64) void conv_mfma_kern
   const bool live = t0 < n && (!tile_flags || tile_flags[t0 >> 5]);
   int my_row = -1;
   if (live && t0 + r < n) my_row = rows ? rows[t0 + r] : (int)(t0 + r);
+  // (residual-frame batch norm in the epilogue: the saved row of this lane's row, asked for here so
+  // that the main loop hides the load)
+  int my_pe = -1;
+  if (S > 1 && ep.pre_exist && my_row >= 0) my_pe = ep.pre_exist[my_row];
 
   // stage the tile's slice of the neighbour map in LDS and find the offsets it uses; all the
   // loads are issued before the first one is consumed.  With a tile plan (the map transposed into
@@ -316,6 +331,25 @@ __global__ __launch_bounds__((S == 1 ? CONV_WAVES : S) * 64) void conv_mfma_kern
   if (S > 1 && lane == 0) wmask[wave] = mymask;
   __syncthreads();
   if (!live) return;  // the whole block (S > 1) or wavefront (S == 1) is idle; no barrier follows
+  // Split launches: what the tail of this wavefront will read besides the sums - the other operand of a
+  // folded element-wise sum, the saved rows of a residual frame's batch norm - is asked for here, for
+  // the rows the wavefront finishes, so that the main loop hides these loads.
+  constexpr int NVP = S > 1 ? 16 / S : 1;
+  float pre_res[NVP], pre_pin[NVP], pre_pout[NVP];
+  int pre_pe[NVP];
+  if (S > 1) {
+    const int c = cb0 * 32 + r;
+#pragma unroll
+    for (int j = 0; j < NVP; j++) {
+      const int v = wave * NVP + j, src_lane = 8 * (v >> 2) + 4 * h + (v & 3);
+      const int row = __shfl(my_row, src_lane, 64);
+      pre_pe[j] = __shfl(my_pe, src_lane, 64);
+      pre_res[j] = (ep.res && row >= 0 && c < Cout) ? ep.res[(int64_t)row * ep.ldr + c] : 0.0f;
+      const bool sv = pre_pe[j] >= 0 && c < Cout;
+      pre_pin[j] = sv ? ep.pre_in[(int64_t)pre_pe[j] * ep.ld_pin + c] : 0.0f;
+      pre_pout[j] = sv ? ep.pre_out[(int64_t)pre_pe[j] * ep.ld_pout + c] : 0.0f;
+    }
+  }
   // Offsets some row of the tile uses.  With S wavefronts per tile, the (offset k, chunk ch)
   // items are dealt out by (k * nch + ch) % S: wavefront w takes, of offset k, the chunks
   // ch0(k), ch0(k) + S, ... with ch0(k) = (w - k * nch) mod S.  The deal depends on k, ch and
@@ -482,8 +516,8 @@ __global__ __launch_bounds__((S == 1 ? CONV_WAVES : S) * 64) void conv_mfma_kern
       for (int w = 1; w < S; w++) a[j] += red[w][v * 64 + lane];
       rid[j] = __shfl(my_row, 8 * (v >> 2) + 4 * h + (v & 3), 64);
     }
-    if (G > 1) {
-      // The G blocks of a (tile, output block) leave their sums in memory; of the G wavefronts that
+    if (GZ > 1) {
+      // The blocks of a (tile, output block) leave their sums in memory; of the wavefronts that
       // hold the same rows, the one that arrives last adds the sums in block order (so the result
       // does not depend on the arrival order), writes the rows and puts the arrival counter back to
       // zero.  Nobody waits for anybody.
@@ -491,57 +525,61 @@ __global__ __launch_bounds__((S == 1 ? CONV_WAVES : S) * 64) void conv_mfma_kern
       // cache write-back or invalidation is needed: a full fence flushes the whole L2 and costs
       // more than the layer)
       const int unit = (int)(bx * gridDim.y + by);
-      float *mine = part + ((int64_t)unit * G + bz) * 1024 + (wave * NV) * 64 + lane;
+      float *mine = part + ((int64_t)unit * GZ + bz) * 1024 + (wave * NV) * 64 + lane;
 #pragma unroll
       for (int j = 0; j < NV; j++) __hip_atomic_store(mine + j * 64, a[j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the stores have been acknowledged
       int old = 0;
       if (lane == 0) old = atomicAdd(pcount + unit * S + wave, 1);
-      if (__builtin_amdgcn_readfirstlane(old) != G - 1) return;
-      const float *all = part + (int64_t)unit * G * 1024 + (wave * NV) * 64 + lane;
-      // (the sums of up to eight blocks are requested together and added in block order: one trip to
-      // memory instead of one per block)
+      if (__builtin_amdgcn_readfirstlane(old) != GZ - 1) return;
+      const float *all = part + (int64_t)unit * GZ * 1024 + (wave * NV) * 64 + lane;
+      // (the sums of eight blocks at a time are requested together and added in block order: one trip
+      // to memory per eight blocks instead of one per block)
       constexpr int GP = 8;
-      float pv[GP][NV];
+      for (int g0 = 0; g0 < GZ; g0 += GP) {
+        float pv[GP][NV];
 #pragma unroll
-      for (int gg = 0; gg < GP; gg++) {
-        if (gg < G) {
+        for (int gg = 0; gg < GP; gg++) {
+          if (g0 + gg < GZ) {
 #pragma unroll
-          for (int j = 0; j < NV; j++)
-            pv[gg][j] = __hip_atomic_load(all + gg * 1024 + j * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            for (int j = 0; j < NV; j++)
+              pv[gg][j] = __hip_atomic_load(all + (g0 + gg) * 1024 + j * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          }
         }
-      }
 #pragma unroll
-      for (int j = 0; j < NV; j++) a[j] = pv[0][j];
+        for (int gg = 0; gg < GP; gg++) {
+          if (g0 + gg < GZ) {
 #pragma unroll
-      for (int gg = 1; gg < GP; gg++) {
-        if (gg < G) {
-#pragma unroll
-          for (int j = 0; j < NV; j++) a[j] += pv[gg][j];
+            for (int j = 0; j < NV; j++) a[j] = (g0 + gg == 0) ? pv[0][j] : a[j] + pv[gg][j];
+          }
         }
-      }
-      for (int gg = GP; gg < G; gg++) {
-#pragma unroll
-        for (int j = 0; j < NV; j++)
-          a[j] += __hip_atomic_load(all + gg * 1024 + j * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
       if (lane == 0) pcount[unit * S + wave] = 0;
     }
     const int c = cb0 * 32 + r;
     if (c >= Cout) return;
     if (ep.res) {
-      float rv[NV];
 #pragma unroll
-      for (int j = 0; j < NV; j++) rv[j] = rid[j] >= 0 ? ep.res[(int64_t)rid[j] * ep.ldr + c] : 0.0f;
-#pragma unroll
-      for (int j = 0; j < NV; j++) a[j] += rv[j];
-      __builtin_amdgcn_sched_barrier(0);  // (the sums stay above the stores)
+      for (int j = 0; j < NV; j++) a[j] += pre_res[j];
     }
     float sv[NV];
     if (MODE == MAP_PARENT && ep.side_in) {
 #pragma unroll
       for (int j = 0; j < NV; j++) sv[j] = rid[j] >= 0 ? ep.side_in[(int64_t)rid[j] * ep.ld_side + c] : 0.0f;
       __builtin_amdgcn_sched_barrier(0);  // (all loads above the stores)
+    }
+    if (MODE == MAP_NBR && K == 27 && ep.pre_exist && ep.out2) {
+      // batch norm of a residual frame, with the saved input and output of the rows that existed
+#pragma unroll
+      for (int j = 0; j < NV; j++) {
+        if (rid[j] < 0) continue;
+        if (out) out[(int64_t)rid[j] * ld_out + c] = a[j];
+        const float o = fmaf(a[j], ew[0], eb[0]);
+        const float y =
+            pre_pe[j] >= 0 ? sub_exact(leaky(fmaf(pre_pin[j], ew[0], o), ep.leak), pre_pout[j]) : leaky(o, ep.leak);
+        ep.out2[(int64_t)rid[j] * ep.ld2 + c] = y;
+      }
+      return;
     }
 #pragma unroll
     for (int j = 0; j < NV; j++) {
@@ -1878,6 +1916,16 @@ static std::atomic<int64_t> g_wl_min_tiles{WL_MIN_TILES};
 
 // W: raw [K,Cin,Cout] weights (always needed by the generic kernel); Wp: packed weights or
 // null, in which case they are packed into scratch memory first.
+// Whether one launch can gather from two sources (BnEpilogue::src2_*): the shapes that the split
+// kernel serves - 3^3 layers of a residual frame (latency != 0) and stride-2 deconvolutions, from 32
+// input channels on.
+bool conv_two_sources_ok(int mode, int K, const float *in, int64_t ld_in, const float *in2, int64_t ld_in2,
+                         int64_t in2_rows, int Cin, int latency) {
+  if (!in2 || Cin < 32 || !conv_uses_mfma(in, ld_in, Cin, K) || !conv_uses_mfma(in2, ld_in2, Cin, K)) return false;
+  if (in2_rows < 0 || in2_rows * ld_in2 * 4 >= (int64_t)BUF_OOB) return false;
+  return (mode == MAP_NBR && K == 27 && latency) || (mode == MAP_PARENT && K == 8);
+}
+
 int launch_conv(const float *in, int64_t ld_in, int64_t in_rows, float *out, int64_t ld_out, const float *W,
                 const float *Wp, const float *bias, const int32_t *map0, const int32_t *map1, int mode, int K,
                 const int32_t *rows, const int32_t *d_n_rows, int64_t n_rows, int Cin, int Cout,
@@ -1886,6 +1934,16 @@ int launch_conv(const float *in, int64_t ld_in, int64_t in_rows, float *out, int
   if (n_rows == 0) return INSC_OK;
   if (ep.side_in && !(mode == MAP_PARENT && K == 8 && conv_uses_mfma(in, ld_in, Cin, K) && ep.side_out && ep.side_w && ep.side_b)) {
     set_error("conv: a second batch norm in the epilogue is for deconvolutions on the matrix-core kernel only");
+    return INSC_ERR_ARG;
+  }
+  if (ep.src2_in && !conv_two_sources_ok(mode, K, in, ld_in, ep.src2_in, ep.src2_ld, ep.src2_rows, Cin, latency)) {
+    set_error("conv: no kernel with two sources for this shape (K=%d, map mode %d, Cin=%d)", K, mode, Cin);
+    return INSC_ERR_ARG;
+  }
+  if (ep.src2_in) plan = TilePlan();  // (a plan describes the first source's map only)
+  if (ep.pre_exist && !(ep.out2 && ep.pre_in && ep.pre_out && latency && mode == MAP_NBR && K == 27 && Cin >= 32 &&
+                        conv_uses_mfma(in, ld_in, Cin, K))) {
+    set_error("conv: the batch norm of a residual frame is fused into 3^3 layers on the split kernel only (Cin=%d)", Cin);
     return INSC_ERR_ARG;
   }
   if (expect_rows <= 0 || expect_rows > n_rows) expect_rows = n_rows;
@@ -1943,11 +2001,12 @@ int launch_conv(const float *in, int64_t ld_in, int64_t in_rows, float *out, int
     // its most expensive tile): the items of every 3^3 tile are dealt to four wavefronts whatever
     // the width, and to more blocks for the wide layers.  Also a function of the layer shape only.
     const bool lat = latency && mode == MAP_NBR && K == 27 && Cin >= 32;
-    const bool split = lat || (Cin >= 64 && K > 1 && (mode == MAP_NBR || (mode == MAP_PARENT && Cin >= 96)));
+    const bool two = ep.src2_in != nullptr;  // (checked above: a shape that the split kernel serves)
+    const bool split = lat || two || (Cin >= 64 && K > 1 && (mode == MAP_NBR || (mode == MAP_PARENT && Cin >= 96)));
     const int NB0 = split ? 1 : conv_nb_per_group(Cout);
     const int nbtp = conv_nbt_padded(Cout);
     int S = 1;
-    if (split) S = K == 27 ? (Cin >= 160 ? 8 : 4) : (Cin >= 96 ? 4 : 1);  // K == 8: conv and deconv
+    if (split) S = K == 27 ? (Cin >= 160 ? 8 : 4) : ((Cin >= 96 || two) ? 4 : 1);  // K == 8: conv and deconv
     const int NB = (S == 1 && Cin >= 96) ? 1 : NB0;
     // (the split across blocks is for scales with few tiles; in a U-Net the width grows with the depth,
     // and a layer that narrows to at most 96 channels sits at a fine scale with many tiles)
@@ -2016,13 +2075,14 @@ int launch_conv(const float *in, int64_t ld_in, int64_t in_rows, float *out, int
       return INSC_OK;
     }
     const unsigned gx = (unsigned)(S == 1 ? cdiv(tiles, CONV_WAVES) : tiles);
-    dim3 grid(gx, (unsigned)(NB == 1 ? nbt : nbtp / NB), (unsigned)G), block((S == 1 ? CONV_WAVES : S) * 64);
+    const int GZ = two ? 2 * G : G;  // blocks per (tile, output block): G per source
+    dim3 grid(gx, (unsigned)(NB == 1 ? nbt : nbtp / NB), (unsigned)GZ), block((S == 1 ? CONV_WAVES : S) * 64);
     float *part = nullptr;
     int32_t *pcount = nullptr;
-    if (G > 1) {
+    if (GZ > 1) {
       const size_t units = (size_t)gx * grid.y;
       void *ws;
-      int rc = workspace(WS_CONV, s, units * G * 1024 * sizeof(float), &ws);
+      int rc = workspace(WS_CONV, s, units * GZ * 1024 * sizeof(float), &ws);
       if (rc) return rc;
       part = (float *)ws;
       if ((rc = zero_counters(s, units * (size_t)S, &pcount))) return rc;  // one counter per wavefront of a unit

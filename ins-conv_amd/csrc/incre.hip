@@ -8,7 +8,8 @@
 // convolution leaves the rows around the frame's sites untouched.
 //
 // All kernels are streaming (one thread per channel group of a row); the two convolutions are
-// the ordinary kernels run twice, the second pass gathering the saved features.
+// the ordinary kernels with the saved features as a second source (a second set of blocks in
+// the same launch, or a second pass for the shapes without such a kernel).
 #include "common.h"
 #include "grid.h"
 
@@ -61,9 +62,9 @@ __global__ __launch_bounds__(256) void incre_bn_kernel(const float *__restrict__
     }
     const float o = fmaf(in[row * ld_in + c], w, b);
     const int pe = pre_exist[row];
-    float y;
+    float y;  // (the same operations, one by one, as the fused form in the convolution's epilogue)
     if (pe >= 0)
-      y = leaky(fmaf(pre_in[(int64_t)pe * ld_pin + c], w, o), leak) - pre_out[(int64_t)pe * ld_pout + c];
+      y = sub_exact(leaky(fmaf(pre_in[(int64_t)pe * ld_pin + c], w, o), leak), pre_out[(int64_t)pe * ld_pout + c]);
     else
       y = leaky(o, leak);
     out[row * ld_out + c] = y;
@@ -115,6 +116,81 @@ int launch_incre_bn(const float *in, int64_t ld_in, float *out, int64_t ld_out, 
   return INSC_OK;
 }
 
+int incre_conv_ssc(const float *in, int64_t ld_in, const float *pre_in, int64_t ld_pre, int64_t n_pre_rows, float *out,
+                   int64_t ld_out, const float *W, const float *Wp, const float *bias, const int32_t *nbr,
+                   const int32_t *nbr_pre, int64_t n, int Cin, int Cout, BnEpilogue ep, hipStream_t s) {
+  // rules inside the frame's site set, on the residual features (CUDA/Convolution.cpp:264-268,283);
+  // new sites also gather the saved features of their neighbours in the saved set (:274,287)
+  const float *res = ep.res;
+  const int64_t ldr = ep.ldr;
+  if (n_pre_rows == 0)
+    return launch_conv(in, ld_in, n, out, ld_out, W, Wp, bias, nbr, nullptr, MAP_NBR, 27, nullptr, nullptr, n, Cin, Cout,
+                       nullptr, nullptr, s, ep, TilePlan(), 1);
+  if (conv_two_sources_ok(MAP_NBR, 27, in, ld_in, pre_in, ld_pre, n_pre_rows, Cin, 1)) {
+    // one launch: a second set of blocks per tile walks the saved features
+    ep.src2_in = pre_in;
+    ep.src2_ld = ld_pre;
+    ep.src2_rows = n_pre_rows;
+    ep.src2_map = nbr_pre;
+    return launch_conv(in, ld_in, n, out, ld_out, W, Wp, bias, nbr, nullptr, MAP_NBR, 27, nullptr, nullptr, n, Cin, Cout,
+                       nullptr, nullptr, s, ep, TilePlan(), 1);
+  }
+  // two passes, the second adding to the first (and the element-wise sum, if any, behind them)
+  if (ep.out2 || ep.pre_exist) {
+    set_error("incre_conv_ssc: no fused batch norm for a layer that runs in two passes (Cin=%d)", Cin);
+    return INSC_ERR_ARG;
+  }
+  int rc = launch_conv(in, ld_in, n, out, ld_out, W, Wp, bias, nbr, nullptr, MAP_NBR, 27, nullptr, nullptr, n, Cin, Cout,
+                       nullptr, nullptr, s, BnEpilogue(), TilePlan(), 1);
+  if (rc) return rc;
+  BnEpilogue e2;
+  e2.res = out;
+  e2.ldr = ld_out;
+  rc = launch_conv(pre_in, ld_pre, n_pre_rows, out, ld_out, W, Wp, nullptr, nbr_pre, nullptr, MAP_NBR, 27, nullptr,
+                   nullptr, n, Cin, Cout, nullptr, nullptr, s, e2, TilePlan(), 1);
+  if (rc || !res) return rc;
+  return launch_add(out, ld_out, res, ldr, out, ld_out, nullptr, nullptr, n, Cout, nullptr, s);
+}
+
+int incre_deconv_down2(const float *in, int64_t ld_in, int64_t n_in_rows, const float *pre_in, int64_t ld_pre,
+                       int64_t n_pre_rows, float *out, int64_t ld_out, const float *W, const float *Wp,
+                       const float *bias, const int32_t *parent, const int32_t *offset, const int32_t *pre_exist_in,
+                       const int32_t *pre_exist_out, int64_t n_rows, int Cin, int Cout, const float *res, int64_t ldr,
+                       hipStream_t s) {
+  BnEpilogue ep;
+  ep.res = res;
+  ep.ldr = ldr;
+  if (n_pre_rows == 0)
+    return launch_conv(in, ld_in, n_in_rows, out, ld_out, W, Wp, bias, parent, offset, MAP_PARENT, 8, nullptr, nullptr,
+                       n_rows, Cin, Cout, nullptr, nullptr, s, ep);
+  // the saved coarse row a fine site also reads
+  void *ws;
+  int rc = workspace(WS_INCRE, s, sizeof(int32_t) * (size_t)n_rows, &ws);
+  if (rc) return rc;
+  int32_t *parent2 = (int32_t *)ws;
+  hipLaunchKernelGGL(incre_parent_kernel, dim3(grid_for(n_rows, 256)), dim3(256), 0, s, parent, pre_exist_in,
+                     pre_exist_out, n_rows, n_in_rows, parent2);
+  INSC_LAUNCH_CHECK();
+  if (conv_two_sources_ok(MAP_PARENT, 8, in, ld_in, pre_in, ld_pre, n_pre_rows, Cin, 0)) {
+    ep.src2_in = pre_in;
+    ep.src2_ld = ld_pre;
+    ep.src2_rows = n_pre_rows;
+    ep.src2_map = parent2;
+    return launch_conv(in, ld_in, n_in_rows, out, ld_out, W, Wp, bias, parent, offset, MAP_PARENT, 8, nullptr, nullptr,
+                       n_rows, Cin, Cout, nullptr, nullptr, s, ep);
+  }
+  rc = launch_conv(in, ld_in, n_in_rows, out, ld_out, W, Wp, bias, parent, offset, MAP_PARENT, 8, nullptr, nullptr,
+                   n_rows, Cin, Cout, nullptr, nullptr, s);
+  if (rc) return rc;
+  BnEpilogue e2;
+  e2.res = out;
+  e2.ldr = ld_out;
+  rc = launch_conv(pre_in, ld_pre, n_pre_rows, out, ld_out, W, Wp, nullptr, parent2, offset, MAP_PARENT, 8, nullptr,
+                   nullptr, n_rows, Cin, Cout, nullptr, nullptr, s, e2);
+  if (rc || !res) return rc;
+  return launch_add(out, ld_out, res, ldr, out, ld_out, nullptr, nullptr, n_rows, Cout, nullptr, s);
+}
+
 }  // namespace insc
 
 using namespace insc;
@@ -143,17 +219,8 @@ int insc_incre_conv_ssc(const float *d_in, int64_t ld_in, const float *d_pre_in,
   if (n == 0) return INSC_OK;
   INSC_REQUIRE(d_in && d_out && (d_W || d_Wp) && d_nbr && d_nbr_pre && (d_pre_in || n_pre_rows == 0), INSC_ERR_ARG,
                "insc_incre_conv_ssc: null pointer");
-  hipStream_t s = (hipStream_t)stream;
-  // rules inside the frame's site set, on the residual features (CUDA/Convolution.cpp:264-268,283)
-  int rc = launch_conv(d_in, ld_in, n, d_out, ld_out, d_W, d_Wp, d_bias, d_nbr, nullptr, MAP_NBR, 27, nullptr, nullptr,
-                       n, Cin, Cout, nullptr, nullptr, s, BnEpilogue(), TilePlan(), 1);
-  if (rc || n_pre_rows == 0) return rc;
-  // new sites gather the saved features of their neighbours in the saved set (:274,287)
-  BnEpilogue ep;
-  ep.res = d_out;
-  ep.ldr = ld_out;
-  return launch_conv(d_pre_in, ld_pre, n_pre_rows, d_out, ld_out, d_W, d_Wp, nullptr, d_nbr_pre, nullptr, MAP_NBR, 27,
-                     nullptr, nullptr, n, Cin, Cout, nullptr, nullptr, s, ep, TilePlan(), 1);
+  return incre_conv_ssc(d_in, ld_in, d_pre_in, ld_pre, n_pre_rows, d_out, ld_out, d_W, d_Wp, d_bias, d_nbr, d_nbr_pre, n,
+                        Cin, Cout, BnEpilogue(), (hipStream_t)stream);
 }
 
 int insc_incre_bn_leaky(const float *d_in, int64_t ld_in, float *d_out, int64_t ld_out, const float *d_mean,
@@ -181,22 +248,9 @@ int insc_incre_deconv_down2(const float *d_in, int64_t ld_in, int64_t n_in_rows,
   INSC_REQUIRE(d_in && d_out && (d_W || d_Wp) && d_parent && d_offset && d_pre_exist_in && d_pre_exist_out &&
                    (d_pre_in || n_pre_rows == 0),
                INSC_ERR_ARG, "insc_incre_deconv_down2: null pointer");
-  hipStream_t s = (hipStream_t)stream;
-  int rc = launch_conv(d_in, ld_in, n_in_rows, d_out, ld_out, d_W, d_Wp, d_bias, d_parent, d_offset, MAP_PARENT, 8,
-                       nullptr, nullptr, n_rows, Cin, Cout, nullptr, nullptr, s);
-  if (rc || n_pre_rows == 0) return rc;
-  void *ws;
-  rc = workspace(WS_INCRE, s, sizeof(int32_t) * (size_t)n_rows, &ws);
-  if (rc) return rc;
-  int32_t *parent2 = (int32_t *)ws;
-  hipLaunchKernelGGL(incre_parent_kernel, dim3(grid_for(n_rows, 256)), dim3(256), 0, s, d_parent, d_pre_exist_in,
-                     d_pre_exist_out, n_rows, n_in_rows, parent2);
-  INSC_LAUNCH_CHECK();
-  BnEpilogue ep;
-  ep.res = d_out;
-  ep.ldr = ld_out;
-  return launch_conv(d_pre_in, ld_pre, n_pre_rows, d_out, ld_out, d_W, d_Wp, nullptr, parent2, d_offset, MAP_PARENT, 8,
-                     nullptr, nullptr, n_rows, Cin, Cout, nullptr, nullptr, s, ep);
+  return incre_deconv_down2(d_in, ld_in, n_in_rows, d_pre_in, ld_pre, n_pre_rows, d_out, ld_out, d_W, d_Wp, d_bias,
+                            d_parent, d_offset, d_pre_exist_in, d_pre_exist_out, n_rows, Cin, Cout, nullptr, 0,
+                            (hipStream_t)stream);
 }
 
 int insc_incre_output(const float *d_in, int64_t ld_in, const float *d_pre_in, int64_t ld_pre,

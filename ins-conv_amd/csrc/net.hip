@@ -114,6 +114,7 @@ struct ResidualFrame {
   int64_t cap = 0;                      // sites every scale can hold
   float *in_sum = nullptr;
   int32_t *in_cnt = nullptr, *chain_head = nullptr, *chain_next = nullptr, *sop = nullptr;
+  std::vector<uint8_t> bn_done;         // per op, this frame: a batch norm that its producer has computed
 };
 }  // namespace insc
 
@@ -1403,39 +1404,70 @@ static float *rtensor_ptr(insc_net *net, int t) {
 }
 static int64_t rtensor_ld(insc_net *net, int t) { return net->rf.buffers[net->tensors[t].buf].ld; }
 
-// one layer of a residual frame: every op runs on its own (no fusions), on all rows of the frame
-static int run_op_residual(insc_net *net, const Op &op, hipStream_t s) {
+// one layer of a residual frame, on all rows of the frame: every op runs on its own, except that the
+// element-wise sum of a residual block is formed by the convolution before it
+static int run_op_residual(insc_net *net, int index, hipStream_t s) {
   ResidualFrame &R = net->rf;
+  const Op &op = net->ops[(size_t)index];
+  if (op.kind == OP_BN && R.bn_done[(size_t)index]) return INSC_OK;
   const Tensor &To = net->tensors[op.out];
   const Level &Lo = R.levels[To.level];
   const int64_t n = Lo.n;
   if (n == 0 || op.kind == OP_JOIN) return INSC_OK;
+  if (op.kind == OP_ADD && op.fused) return INSC_OK;  // formed by the convolution that feeds it
   const float *in0 = rtensor_ptr(net, op.in0);
   const int64_t ld0 = rtensor_ld(net, op.in0);
-  float *out = rtensor_ptr(net, op.out);
-  const int64_t ld_out = rtensor_ld(net, op.out);
+  // a convolution that also forms the sum of its residual block writes what the OP_ADD would
+  const Op *add = op.fused_add >= 0 ? &net->ops[op.fused_add] : nullptr;
+  float *out = rtensor_ptr(net, add ? add->out : op.out);
+  const int64_t ld_out = rtensor_ld(net, add ? add->out : op.out);
+  BnEpilogue ep;
+  if (add) {
+    const int other = add->in0 == op.out ? add->in1 : add->in0;
+    ep.res = rtensor_ptr(net, other);
+    ep.ldr = rtensor_ld(net, other);
+  }
   const int li = net->tensors[op.in0].level;
   const int64_t n_in = R.levels[li].n;
   // the saved input of the layer and the saved site count of its scale
   const float *pre0 = net->tensors[op.in0].kept ? tensor_ptr(net, op.in0) : nullptr;
   const int64_t ldp0 = net->tensors[op.in0].kept ? tensor_ld(net, op.in0) : 0;
   const int64_t n_pre_in = net->levels[li].n;
-  void *st = (void *)s;
   switch (op.kind) {
     case OP_SSC:
       INSC_REQUIRE(pre0, INSC_ERR_STATE, "residual frame: the input of a convolution was not kept");
-      return insc_incre_conv_ssc(in0, ld0, pre0, ldp0, n_pre_in, out, ld_out, op.W, op.Wp, op.bias, Lo.nbr,
-                                 R.nbr_pre[To.level], n, op.Cin, op.Cout, st);
+      {
+        // the batch norm that reads the result (the layer's own or, with the sum folded in, the sum's) rides
+        // in the epilogue when the layer runs as one launch
+        const Op &tail = add ? *add : op;
+        const Op *bn = tail.fused_bn >= 0 ? &net->ops[(size_t)tail.fused_bn] : nullptr;
+        if (bn && bn->bn_w && n_pre_in > 0 && net->tensors[bn->in0].kept && net->tensors[bn->out].kept &&
+            conv_two_sources_ok(MAP_NBR, 27, in0, ld0, pre0, ldp0, n_pre_in, op.Cin, 1)) {
+          ep.w = bn->bn_w;
+          ep.b = bn->bn_b;
+          ep.leak = bn->leak;
+          ep.out2 = rtensor_ptr(net, bn->out);
+          ep.ld2 = rtensor_ld(net, bn->out);
+          ep.pre_exist = R.pre_exist[To.level];
+          ep.pre_in = tensor_ptr(net, bn->in0);
+          ep.ld_pin = tensor_ld(net, bn->in0);
+          ep.pre_out = tensor_ptr(net, bn->out);
+          ep.ld_pout = tensor_ld(net, bn->out);
+          R.bn_done[(size_t)tail.fused_bn] = 1;
+        }
+      }
+      return incre_conv_ssc(in0, ld0, pre0, ldp0, n_pre_in, out, ld_out, op.W, op.Wp, op.bias, Lo.nbr,
+                            R.nbr_pre[To.level], n, op.Cin, op.Cout, ep, s);
     case OP_NIN:
       return launch_conv(in0, ld0, n_in, out, ld_out, op.W, op.Wp, op.bias, nullptr, nullptr, MAP_IDENTITY, 1, nullptr,
-                         nullptr, n, op.Cin, op.Cout, nullptr, nullptr, s);
+                         nullptr, n, op.Cin, op.Cout, nullptr, nullptr, s, ep);
     case OP_CONV:
       return launch_conv(in0, ld0, n_in, out, ld_out, op.W, op.Wp, op.bias, R.levels[li].child, nullptr, MAP_NBR, 8,
-                         nullptr, nullptr, n, op.Cin, op.Cout, nullptr, nullptr, s);
+                         nullptr, nullptr, n, op.Cin, op.Cout, nullptr, nullptr, s, ep);
     case OP_DECONV:
       INSC_REQUIRE(pre0, INSC_ERR_STATE, "residual frame: the input of a deconvolution was not kept");
-      return insc_incre_deconv_down2(in0, ld0, n_in, pre0, ldp0, n_pre_in, out, ld_out, op.W, op.Wp, op.bias, Lo.parent,
-                                     Lo.offset, R.pre_exist[li], R.pre_exist[To.level], n, op.Cin, op.Cout, st);
+      return incre_deconv_down2(in0, ld0, n_in, pre0, ldp0, n_pre_in, out, ld_out, op.W, op.Wp, op.bias, Lo.parent,
+                                Lo.offset, R.pre_exist[li], R.pre_exist[To.level], n, op.Cin, op.Cout, ep.res, ep.ldr, s);
     case OP_BN:
       INSC_REQUIRE(pre0 && net->tensors[op.out].kept, INSC_ERR_STATE,
                    "residual frame: the input of a batch norm was not kept (insc_net_enable_residual before finalize)");
@@ -1554,8 +1586,9 @@ int insc_net_forward_residual(insc_net *net, const int32_t *d_coords, int coord_
                                     stream))) {
     return rc;
   }
-  for (const Op &op : net->ops)
-    if ((rc = run_op_residual(net, op, s))) return rc;
+  R.bn_done.assign(net->ops.size(), 0);
+  for (int i = 0; i < (int)net->ops.size(); i++)
+    if ((rc = run_op_residual(net, i, s))) return rc;
   if (d_out) {
     const Tensor &To = net->tensors[net->out_tensor];
     if ((rc = insc_incre_output(rtensor_ptr(net, net->out_tensor), rtensor_ld(net, net->out_tensor),
