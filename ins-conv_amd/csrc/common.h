@@ -157,7 +157,7 @@ int incre_deconv_down2(const float *in, int64_t ld_in, int64_t n_in_rows, const 
                        int64_t n_pre_rows, float *out, int64_t ld_out, const float *W, const float *Wp,
                        const float *bias, const int32_t *parent, const int32_t *offset, const int32_t *pre_exist_in,
                        const int32_t *pre_exist_out, int64_t n_rows, int Cin, int Cout, const float *res, int64_t ldr,
-                       hipStream_t s);
+                       hipStream_t s, const int32_t *parent2 = nullptr);  // parent2: incre_parent_kernel's answer, if at hand
 int launch_input_finish(const float *sum, const int32_t *cnt, int mode, float *out, int64_t ld_out,
                         const int32_t *rows, const int32_t *d_n_rows, int64_t n_rows, int C,
                         const uint8_t *row_mask, hipStream_t s);

@@ -55,6 +55,14 @@ struct PlanRef {
 };
 int ssc3_new_sites_batch(const insc_grid *const *grids, int32_t *const *d_nbr, int n, int64_t n_new_upper,
                          hipStream_t s, const PlanRef *plans = nullptr);
+// Residual frames, all scales in two launches: d_pre_exist[l][i] = the saved site (grid pre[l]) at the
+// coordinates of site i of grids[l], or -1; d_nbr_pre[l] = the 27 saved neighbours of the sites that
+// have none (insc_grid_query + insc_incre_rulebook_ssc3); d_parent2[l][i], for l + 1 < n, = the saved
+// site of the coarse parent (d_parent[l]) of a site that has none.  Sized by n_upper, an upper bound
+// of every scale's site count; the counts themselves are read on the device.
+int incre_links_batch(const insc_grid *const *grids, const insc_grid *const *pre, const int32_t *const *d_parent,
+                      int32_t *const *d_pre_exist, int32_t *const *d_nbr_pre, int32_t *const *d_parent2, int n,
+                      int64_t n_upper, hipStream_t s);
 // The inserts of a whole frame at all scales at once: the points go into lv[0].grid, the sites that adds
 // (halved) into lv[1].grid and so on, with the parent /
 // offset / child link of every scale to the next coarser one filled in for the new sites.  Every

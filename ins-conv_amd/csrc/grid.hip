@@ -1074,6 +1074,66 @@ int ssc3_new_sites_batch(const insc_grid *const *grids, int32_t *const *d_nbr, i
   return INSC_OK;
 }
 
+// ---- residual frames: the links of a frame's site sets to the saved ones, all scales at once ------
+struct IncreLinkJob {
+  const Slot *pre_table;
+  int64_t pre_mask;
+  const int32_t *coords, *d_n, *parent;
+  int32_t *pre_exist, *nbr_pre, *parent2;
+};
+struct IncreLinkBatch {
+  IncreLinkJob job[16];
+};
+// pre_exist (insc_grid_query of the saved grid with the scale's own coordinates) and, for the sites the
+// saved grid does not hold, their neighbours there (incre_ssc3_nbr_kernel).  Thread = (site, offset);
+// every thread looks its own site up, the one of the centre offset records the answer.
+__global__ void incre_links_batch_kernel(IncreLinkBatch b) {
+  const IncreLinkJob &j = b.job[blockIdx.y];
+  const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= (int64_t)j.d_n[0] * 27) return;
+  const int64_t o = t / 27;
+  const int k = (int)(t % 27);
+  const int4 c = reinterpret_cast<const int4 *>(j.coords)[o];
+  const int pe = grid_find(j.pre_table, j.pre_mask, pack_key(c.x, c.y, c.z, c.w));
+  if (k == 13) j.pre_exist[o] = pe;
+  int r = -1;
+  if (pe < 0 && k != 13) {
+    const int x = c.x + k / 9 - 1, y = c.y + (k / 3) % 3 - 1, z = c.z + k % 3 - 1;
+    if (coord_ok(x, y, z, c.w)) r = grid_find(j.pre_table, j.pre_mask, pack_key(x, y, z, c.w));
+  }
+  j.nbr_pre[t] = r;
+}
+// the saved coarse row that a fine site new to the saved set also reads (incre_parent_kernel); job l
+// holds the fine scale's parent map and answer, job l + 1 the coarse scale
+__global__ void incre_parents_batch_kernel(IncreLinkBatch b) {
+  const IncreLinkJob &f = b.job[blockIdx.y], &cs = b.job[blockIdx.y + 1];
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= f.d_n[0]) return;
+  const int p = f.parent[i];
+  f.parent2[i] = (p >= 0 && p < cs.d_n[0] && f.pre_exist[i] < 0) ? cs.pre_exist[p] : -1;
+}
+
+int incre_links_batch(const insc_grid *const *grids, const insc_grid *const *pre, const int32_t *const *d_parent,
+                      int32_t *const *d_pre_exist, int32_t *const *d_nbr_pre, int32_t *const *d_parent2, int n,
+                      int64_t n_upper, hipStream_t s) {
+  if (n <= 0 || n_upper <= 0) return INSC_OK;
+  if (n > 16) {
+    set_error("incre_links_batch: at most 16 grids");
+    return INSC_ERR_ARG;
+  }
+  IncreLinkBatch b;
+  for (int i = 0; i < n; i++)
+    b.job[i] = IncreLinkJob{pre[i]->table, pre[i]->n_slots - 1, grids[i]->coords, grids[i]->d_n,
+                            i + 1 < n ? d_parent[i] : nullptr, d_pre_exist[i], d_nbr_pre[i],
+                            i + 1 < n ? d_parent2[i] : nullptr};
+  hipLaunchKernelGGL(incre_links_batch_kernel, dim3(grid_for(n_upper * 27, 256, 1ll << 30), (unsigned)n), dim3(256), 0,
+                     s, b);
+  if (n > 1)
+    hipLaunchKernelGGL(incre_parents_batch_kernel, dim3(grid_for(n_upper, 256), (unsigned)(n - 1)), dim3(256), 0, s, b);
+  INSC_LAUNCH_CHECK();
+  return INSC_OK;
+}
+
 int order_append_new_sites_both_batch(const insc_grid *const *grids, const int32_t *const *d_nbr,
                                       const int32_t *const *d_offset, int32_t *const *d_order, int32_t *const *d_pos,
                                       int32_t *const *d_bo_order, int32_t *const *d_bo_pos, int n, int64_t n_new_upper,

@@ -156,7 +156,7 @@ int incre_deconv_down2(const float *in, int64_t ld_in, int64_t n_in_rows, const 
                        int64_t n_pre_rows, float *out, int64_t ld_out, const float *W, const float *Wp,
                        const float *bias, const int32_t *parent, const int32_t *offset, const int32_t *pre_exist_in,
                        const int32_t *pre_exist_out, int64_t n_rows, int Cin, int Cout, const float *res, int64_t ldr,
-                       hipStream_t s) {
+                       hipStream_t s, const int32_t *parent2_ready) {
   BnEpilogue ep;
   ep.res = res;
   ep.ldr = ldr;
@@ -164,13 +164,17 @@ int incre_deconv_down2(const float *in, int64_t ld_in, int64_t n_in_rows, const 
     return launch_conv(in, ld_in, n_in_rows, out, ld_out, W, Wp, bias, parent, offset, MAP_PARENT, 8, nullptr, nullptr,
                        n_rows, Cin, Cout, nullptr, nullptr, s, ep);
   // the saved coarse row a fine site also reads
-  void *ws;
-  int rc = workspace(WS_INCRE, s, sizeof(int32_t) * (size_t)n_rows, &ws);
-  if (rc) return rc;
-  int32_t *parent2 = (int32_t *)ws;
-  hipLaunchKernelGGL(incre_parent_kernel, dim3(grid_for(n_rows, 256)), dim3(256), 0, s, parent, pre_exist_in,
-                     pre_exist_out, n_rows, n_in_rows, parent2);
-  INSC_LAUNCH_CHECK();
+  int rc;
+  const int32_t *parent2 = parent2_ready;
+  if (!parent2) {
+    void *ws;
+    rc = workspace(WS_INCRE, s, sizeof(int32_t) * (size_t)n_rows, &ws);
+    if (rc) return rc;
+    hipLaunchKernelGGL(incre_parent_kernel, dim3(grid_for(n_rows, 256)), dim3(256), 0, s, parent, pre_exist_in,
+                       pre_exist_out, n_rows, n_in_rows, (int32_t *)ws);
+    INSC_LAUNCH_CHECK();
+    parent2 = (const int32_t *)ws;
+  }
   if (conv_two_sources_ok(MAP_PARENT, 8, in, ld_in, pre_in, ld_pre, n_pre_rows, Cin, 0)) {
     ep.src2_in = pre_in;
     ep.src2_ld = ld_pre;

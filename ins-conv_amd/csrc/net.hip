@@ -109,6 +109,7 @@ struct ResidualFrame {
   std::vector<Level> levels;            // grid, nbr, parent, offset, child of the frame's sites
   std::vector<int32_t *> pre_exist;     // [cap] id in the saved site set of the scale, or -1
   std::vector<int32_t *> nbr_pre;       // [cap,27] saved neighbours of the sites new to the saved set
+  std::vector<int32_t *> parent2;       // [cap] saved row of the coarse parent of such a site (scales with a coarser one)
   std::vector<Buffer> buffers;          // same layout as the program's buffers, rows = sites of the frame
   std::vector<int> ld;                  // row stride of every buffer (0: unused)
   int64_t cap = 0;                      // sites every scale can hold
@@ -717,6 +718,8 @@ int insc_net_destroy(insc_net *net) {
   for (int32_t *p : net->rf.pre_exist)
     if (p) (void)hipFree(p);
   for (int32_t *p : net->rf.nbr_pre)
+    if (p) (void)hipFree(p);
+  for (int32_t *p : net->rf.parent2)
     if (p) (void)hipFree(p);
   for (Buffer &B : net->rf.buffers)
     if (B.p) (void)hipFree(B.p);
@@ -1331,6 +1334,7 @@ static int rframe_reserve(insc_net *net, int64_t need, hipStream_t s) {
     R.levels.resize(L);
     R.pre_exist.assign(L, nullptr);
     R.nbr_pre.assign(L, nullptr);
+    R.parent2.assign(L, nullptr);
     R.buffers.resize(net->buffers.size());
     R.ld.assign(net->buffers.size(), 0);
     for (size_t b = 0; b < net->buffers.size(); b++) R.buffers[b].level = net->buffers[b].level;
@@ -1354,6 +1358,8 @@ static int rframe_reserve(insc_net *net, int64_t need, hipStream_t s) {
     free_dev(Lv.child);
     free_dev(R.pre_exist[l]);
     free_dev(R.nbr_pre[l]);
+    free_dev(R.parent2[l]);
+    R.parent2[l] = nullptr;
     Lv.parent = Lv.offset = Lv.child = nullptr;
     if ((rc = dev_alloc(&Lv.nbr, (size_t)cap * 27))) return rc;
     if ((rc = dev_alloc(&R.pre_exist[l], (size_t)cap))) return rc;
@@ -1362,6 +1368,7 @@ static int rframe_reserve(insc_net *net, int64_t need, hipStream_t s) {
       if ((rc = dev_alloc(&Lv.parent, (size_t)cap))) return rc;
       if ((rc = dev_alloc(&Lv.offset, (size_t)cap))) return rc;
       if ((rc = dev_alloc(&Lv.child, (size_t)cap * 8))) return rc;
+      if ((rc = dev_alloc(&R.parent2[l], (size_t)cap))) return rc;
       Lv.child_rows = cap;
     }
     Lv.cap = cap;
@@ -1467,7 +1474,8 @@ static int run_op_residual(insc_net *net, int index, hipStream_t s) {
     case OP_DECONV:
       INSC_REQUIRE(pre0, INSC_ERR_STATE, "residual frame: the input of a deconvolution was not kept");
       return incre_deconv_down2(in0, ld0, n_in, pre0, ldp0, n_pre_in, out, ld_out, op.W, op.Wp, op.bias, Lo.parent,
-                                Lo.offset, R.pre_exist[li], R.pre_exist[To.level], n, op.Cin, op.Cout, ep.res, ep.ldr, s);
+                                Lo.offset, R.pre_exist[li], R.pre_exist[To.level], n, op.Cin, op.Cout, ep.res, ep.ldr, s,
+                                R.parent2[To.level]);
     case OP_BN:
       INSC_REQUIRE(pre0 && net->tensors[op.out].kept, INSC_ERR_STATE,
                    "residual frame: the input of a batch norm was not kept (insc_net_enable_residual before finalize)");
@@ -1552,6 +1560,15 @@ int insc_net_forward_residual(insc_net *net, const int32_t *d_coords, int coord_
       nbrs[l] = R.levels[l].nbr;
     }
     if ((rc = ssc3_new_sites_batch(grids, nbrs, L, P, s))) return rc;
+    // the links to the saved site set, all scales at once
+    const insc_grid *pre[16];
+    const int32_t *par[16];
+    for (int l = 0; l < L; l++) {
+      pre[l] = net->levels[l].grid;
+      par[l] = R.levels[l].parent;
+    }
+    if ((rc = incre_links_batch(grids, pre, par, R.pre_exist.data(), R.nbr_pre.data(), R.parent2.data(), L, P, s)))
+      return rc;
   }
   // the exact site counts size every later launch (one short wait, as in an exact frame)
   INSC_HIP(hipEventSynchronize(net->ev_counts));
@@ -1567,14 +1584,6 @@ int insc_net_forward_residual(insc_net *net, const int32_t *d_coords, int coord_
     INSC_REQUIRE(!(err & 2), INSC_ERR_CAPACITY, "insc_net_forward_residual: capacity of scale %d exceeded", l);
   }
   if ((rc = rframe_buffers(net, s))) return rc;
-  // ---- links to the saved site set -------------------------------------------------------------
-  for (int l = 0; l < L; l++) {
-    Level &Lv = R.levels[l];
-    if (Lv.n == 0) continue;
-    if ((rc = insc_grid_query(net->levels[l].grid, Lv.grid->coords, Lv.n, R.pre_exist[l], stream))) return rc;
-    if ((rc = insc_incre_rulebook_ssc3(Lv.grid, net->levels[l].grid, R.pre_exist[l], Lv.n, R.nbr_pre[l], stream)))
-      return rc;
-  }
   // ---- input layer, layers, output layer -----------------------------------------------------------
   const int64_t n0 = R.levels[0].n;
   if (net->mode == 0) {
