@@ -86,7 +86,7 @@ int grid_noalloc_setup();
 int order_append_new_sites_both_batch(const insc_grid *const *grids, const int32_t *const *d_nbr,
                                       const int32_t *const *d_offset, int32_t *const *d_order, int32_t *const *d_pos,
                                       int32_t *const *d_bo_order, int32_t *const *d_bo_pos, int n, int64_t n_new_upper,
-                                      hipStream_t s);
+                                      hipStream_t s, bool all = false);  // all: every site of each grid, from position 0
 // insc_grid_clear for several grids in one launch; with grid i the int32 array minus1[i] (n_minus1[i]
 // words, nullable) is set to -1, and `zero` (nullable, zero_bytes a multiple of 4) is zeroed
 int grid_clear_batch(insc_grid *const *grids, int32_t *const *minus1, const int64_t *n_minus1, int n, void *zero,

@@ -446,13 +446,12 @@ __device__ __forceinline__ uint64_t spread3_10(uint64_t v) {  // 10 bits -> ever
   v = (v | (v << 2)) & 0x9249249ull;
   return v;
 }
-__device__ __forceinline__ void order_append_sorted_body(const int32_t *__restrict__ d_n,
+__device__ __forceinline__ void order_append_sorted_body(const int first, const int n,
                                                          const int32_t *__restrict__ coords,
                                                          const int32_t *__restrict__ nbr, int32_t *__restrict__ order,
                                                          int32_t *__restrict__ pos, uint64_t *key) {
   // key: SORT_NEW_MAX 64-bit words of LDS, one per new site: sort key in the upper 51 bits, index of
   // the site among the new ones in the lower 13
-  const int first = d_n[1], n = d_n[0] - first;
   const int tid = threadIdx.x;
   if (n <= 0) return;
   if (n > SORT_NEW_MAX) {
@@ -515,12 +514,11 @@ __device__ __forceinline__ void order_append_sorted_body(const int32_t *__restri
 // what sorting by (group, position) gives.  One workgroup of 1024 threads, thread t owns the positions
 // 8t .. 8t+7 of the new sites; counts per group travel as eight 16-bit fields in two 64-bit words
 // (at most SORT_NEW_MAX = 8192 sites, so no field overflows).
-__device__ __forceinline__ void order_append_grouped_body(const int32_t *__restrict__ d_n,
+__device__ __forceinline__ void order_append_grouped_body(const int first, const int n,
                                                           const int32_t *__restrict__ offset,
                                                           const int32_t *__restrict__ order,
                                                           int32_t *__restrict__ bo_order, int32_t *__restrict__ bo_pos,
                                                           uint64_t *lds) {
-  const int first = d_n[1], n = d_n[0] - first;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   if (n <= 0) return;
   if (n > SORT_NEW_MAX) {
@@ -597,6 +595,7 @@ __device__ __forceinline__ void order_append_grouped_body(const int32_t *__restr
 struct OrderBothJob {
   const int32_t *d_n, *coords, *nbr, *offset;  // offset null: no second order
   int32_t *order, *pos, *bo_order, *bo_pos;
+  int all;  // order every site of the grid, not only those of the last insert
 };
 struct OrderBothBatch {
   OrderBothJob job[16];
@@ -604,10 +603,11 @@ struct OrderBothBatch {
 __global__ __launch_bounds__(1024) void order_append_both_batch_kernel(OrderBothBatch b) {
   __shared__ uint64_t key[SORT_NEW_MAX];
   const OrderBothJob &j = b.job[blockIdx.x];
-  order_append_sorted_body(j.d_n, j.coords, j.nbr, j.order, j.pos, key);
+  const int first = j.all ? 0 : j.d_n[1], n = j.d_n[0] - first;
+  order_append_sorted_body(first, n, j.coords, j.nbr, j.order, j.pos, key);
   if (!j.offset) return;
   __syncthreads();  // the order written above is read below (by other threads than wrote it), and the LDS is reused
-  order_append_grouped_body(j.d_n, j.offset, j.order, j.bo_order, j.bo_pos, key);
+  order_append_grouped_body(first, n, j.offset, j.order, j.bo_order, j.bo_pos, key);
 }
 
 int64_t order_sorted_max() { return SORT_NEW_MAX; }
@@ -1137,7 +1137,7 @@ int incre_links_batch(const insc_grid *const *grids, const insc_grid *const *pre
 int order_append_new_sites_both_batch(const insc_grid *const *grids, const int32_t *const *d_nbr,
                                       const int32_t *const *d_offset, int32_t *const *d_order, int32_t *const *d_pos,
                                       int32_t *const *d_bo_order, int32_t *const *d_bo_pos, int n, int64_t n_new_upper,
-                                      hipStream_t s) {
+                                      hipStream_t s, bool all) {
   if (n <= 0 || n_new_upper <= 0) return INSC_OK;
   if (n > 16) {
     set_error("order_append_new_sites_both_batch: at most 16 grids");
@@ -1145,7 +1145,7 @@ int order_append_new_sites_both_batch(const insc_grid *const *grids, const int32
   }
   OrderBothBatch b;
   for (int i = 0; i < n; i++)
-    b.job[i] = OrderBothJob{grids[i]->d_n, grids[i]->coords, d_nbr[i], d_offset[i], d_order[i], d_pos[i], d_bo_order[i], d_bo_pos[i]};
+    b.job[i] = OrderBothJob{grids[i]->d_n, grids[i]->coords, d_nbr[i], d_offset[i], d_order[i], d_pos[i], d_bo_order[i], d_bo_pos[i], all ? 1 : 0};
   hipLaunchKernelGGL(order_append_both_batch_kernel, dim3((unsigned)n), dim3(1024), 0, s, b);
   INSC_LAUNCH_CHECK();
   return INSC_OK;

@@ -49,6 +49,7 @@ struct Level {
   int64_t n_upper = 0;          // bound valid during the frame being enqueued
   int64_t new_upper = 0;        // bound on sites added in this frame
   bool plan_valid = false;      // the tile plan holds every site of the last completed frame
+  int64_t n_sorted = 0;         // sites that the last order built from scratch covers (later ones are appended)
 };
 
 struct Buffer {
@@ -123,6 +124,7 @@ struct insc_net {
   int n_levels = 0, in_channels = 0, mode = 4;
   bool finalized = false, have_state = false;
   bool keep_raw = false;  // keep the input of every batch norm (residual frames read it)
+  int order_refresh_pct = 25;  // an incremental frame re-sorts the orders once this share of a large scale is appended (0: never)
   insc::ResidualFrame rf;
   std::vector<insc::Level> levels;
   std::vector<insc::Buffer> buffers;
@@ -1076,6 +1078,18 @@ int insc_net_forward(insc_net *net, const int32_t *d_coords, int coord_cols, con
   int rc;
   const bool inc = increment != 0;
   net->frame_id = net->frame_id == INT32_MAX ? 1 : net->frame_id + 1;
+  // Sites that arrive with incremental frames are appended to the processing orders, frame by frame, each
+  // batch sorted among itself; tiles made of such batches use more filter offsets and gather from farther
+  // apart than tiles of an order sorted as a whole (a sweep that grew a scene from 37k to 150k voxels in 49
+  // frames: layers 2.42 ms against 2.11 ms per frame).  Once the appended part of a large scale passes a
+  // share of the sorted part, the frame sorts the orders of all scales from scratch, as a full frame does
+  // (results do not depend on the order).
+  bool refresh = false;
+  if (inc && P > 0 && net->order_refresh_pct > 0)
+    for (int l = 0; l < L; l++) {
+      const Level &Lv = net->levels[l];
+      if (Lv.n > order_sorted_max() && (Lv.n - Lv.n_sorted) * 100 > Lv.n_sorted * net->order_refresh_pct) refresh = true;
+    }
 
   if (!inc) {
     // all grids emptied, the child maps back to -1 and the input layer's running sums to zero: one launch
@@ -1119,7 +1133,6 @@ int insc_net_forward(insc_net *net, const int32_t *d_coords, int coord_cols, con
   // leaves the new site counts in host memory; the host picks them up further down, while the GPU is
   // busy with the neighbour maps and orders of the new sites.
   if (P > 0) {
-    Level &L0 = net->levels[0];
     {
       FrameInsertLevel fl[16];
       for (int l = 0; l < L; l++) {
@@ -1154,27 +1167,34 @@ int insc_net_forward(insc_net *net, const int32_t *d_coords, int coord_cols, con
     app.n = L;
     for (int l = 0; l < L; l++) {
       Level &Lv = net->levels[l];
-      const bool keep = inc && Lv.plan_valid;
+      const bool keep = inc && !refresh && Lv.plan_valid;
       prefs[l] = keep ? PlanRef{Lv.plan, Lv.tmask, Lv.pos, Lv.cap} : PlanRef{nullptr, nullptr, nullptr, 0};
       app.job[l] = TilePlanJob{Lv.nbr, Lv.order, Lv.grid->d_n, 0, Lv.cap, keep ? Lv.plan : nullptr, Lv.tmask, nullptr};
     }
     if ((rc = ssc3_new_sites_batch(grids, nbrs, L, P, s, prefs))) return rc;
-    if (inc) {
+    if (inc && !refresh) {
       offsets[L - 1] = nullptr;  // the coarsest scale has no order by position inside a parent cell
       if ((rc = order_append_new_sites_both_batch(grids, cnbrs, offsets, orders, poss, bo_orders, bo_poss, L, P, s)))
         return rc;
       if ((rc = tile_plan_append_batch(app, P, s))) return rc;
-    }  // (a full frame builds its orders from scratch further down, once the counts are known)
-    // ---- input scale: accumulate the points' features per site ----------------------------
+    }  // (a full frame builds its orders from scratch further down, once the counts are known; so does a
+       // frame that refreshes them)
+  }
+  // ---- input scale: accumulate the points' features per site (an incremental frame marks the tiles of
+  // the touched sites, so the sites must have their positions by then) ---------------------------------
+  auto accumulate_input = [&]() -> int {
+    if (P <= 0) return INSC_OK;
     DirtyNode &din = net->dirty[net->tensors[0].dirty];
     const unsigned nb = grid_for(P, 256);
     hipLaunchKernelGGL(chain_push_kernel, dim3(nb), dim3(256), 0, s, sop, P, net->chain_head, net->chain_next);
     hipLaunchKernelGGL(chain_sum_kernel, dim3(nb), dim3(256), 0, s, d_feats, C0, sop, P, net->chain_head,
                        net->chain_next, net->in_sum, net->in_cnt, inc ? din.mask : nullptr,
-                       inc ? din.tflag : nullptr, L0.pos);
+                       inc ? din.tflag : nullptr, net->levels[0].pos);
     INSC_LAUNCH_CHECK();
-  }
-  if (!inc) {
+    return INSC_OK;
+  };
+  if (!refresh && (rc = accumulate_input())) return rc;
+  if (!inc || refresh) {
     // A full frame may synchronise: learn the exact counts, then build the processing orders
     // (pattern-sorted for the 3^3 convolutions, offset-grouped for the deconvolutions).
     if (P > 0) {
@@ -1203,7 +1223,8 @@ int insc_net_forward(insc_net *net, const int32_t *d_coords, int coord_cols, con
         nmax = std::max(nmax, Lv.n);
         ns++;
       }
-      if (ns > 0 && (rc = order_append_new_sites_both_batch(sg, snbr, soff, sord, spos, sbo, sbp, ns, nmax, s))) return rc;
+      if (ns > 0 && (rc = order_append_new_sites_both_batch(sg, snbr, soff, sord, spos, sbo, sbp, ns, nmax, s, true)))
+        return rc;
     }
     for (int l = 0; l < L; l++) {
       Level &Lv = net->levels[l];
@@ -1217,6 +1238,11 @@ int insc_net_forward(insc_net *net, const int32_t *d_coords, int coord_cols, con
       }
       INSC_LAUNCH_CHECK();
     }
+    for (int l = 0; l < L; l++) {
+      net->levels[l].n_sorted = net->levels[l].n;
+      if (refresh) net->levels[l].plan_valid = false;  // rebuilt below for the new order
+    }
+    if (refresh && (rc = accumulate_input())) return rc;
   } else {
     // An incremental frame learns the exact counts here as well: one short host round trip
     // (tens of microseconds) buys launches sized to the real number of tiles.  With the bound
@@ -1307,6 +1333,12 @@ int insc_net_forward(insc_net *net, const int32_t *d_coords, int coord_cols, con
   INSC_HIP(hipStreamSynchronize(s));  // the counts are known already; the call returns when the frame is done
   net->ev_valid = net->profiling;
   if (h_n_sites) *h_n_sites = net->levels[0].n;
+  return INSC_OK;
+}
+
+int insc_net_set_order_refresh(insc_net *net, int percent) {
+  INSC_REQUIRE(net && percent >= 0, INSC_ERR_ARG, "insc_net_set_order_refresh: net is null or percent < 0");
+  net->order_refresh_pct = percent;
   return INSC_OK;
 }
 

@@ -70,6 +70,7 @@ _SIGS = {
     "insc_net_rebind_op": [vp, c_int, vp, vp, vp, vp, vp, vp],
     "insc_net_forward": [vp, vp, c_int, vp, c_i64, c_int, vp, c_int, ctypes.POINTER(c_i64), vp],
     "insc_net_enable_residual": [vp],
+    "insc_net_set_order_refresh": [vp, ctypes.c_int],
     "insc_net_forward_residual": [vp, vp, c_int, vp, c_i64, vp, ctypes.POINTER(c_i64), vp],
     "insc_net_tensor_view": [vp, c_int, ctypes.POINTER(vp), ctypes.POINTER(c_i64), ctypes.POINTER(c_i64),
                              ctypes.POINTER(c_int)],

@@ -204,6 +204,11 @@ class CompiledNet(object):
         self.n_sites_frame = int(n.value)
         return out
 
+    def set_order_refresh(self, percent):
+        """Share (in percent) of appended sites at which an incremental frame re-sorts the processing
+        orders of all scales (insc_net_set_order_refresh); 0 switches the re-sorting off."""
+        lib.insc_net_set_order_refresh(self.h, int(percent))
+
     def profile(self, enable=True):
         """Switch phase timing on/off; returns the last timed frame's phases in ms as a dict
         (structure, dirty, layers, output), or None if no frame was timed yet."""

@@ -110,3 +110,33 @@ def test_dirty_set_rows_of_a_frame():
     assert min(rows0) == touched and max(rows0) >= touched
     # dilation by 3^3 layers grows a set; a frame here touches one end of the scene
     assert [r for k, r in sets[0] if k == "dilate"][0] > touched
+
+
+def test_order_refresh_leaves_every_bit_alone():
+    """An incremental frame that re-sorts the processing orders of its scales (the input scale of this
+    sweep holds 37k..50k sites, so the appended share passes 1 % with every frame) gives the bits of one
+    that keeps appending, and of a full forward over all points so far."""
+    import sparseconvnet as scn
+    from workloads import scenes
+    from workloads.netdefs import NaiveUNet
+
+    seq = scenes.sweep_sequence()[:6]
+    model = NaiveUNet(m=32, levels=7, seed=5).cuda()
+    nets = [scn.compile(copy.deepcopy(model).sparseModel, capacity_sites=60000) for _ in range(3)]
+    nets[0].set_order_refresh(0)   # never
+    nets[1].set_order_refresh(1)   # every frame
+    nets[2].set_order_refresh(12)  # once or twice in this sequence
+    all_p, all_c = seq[0]
+    with torch.no_grad():
+        outs = [n(_inp(*seq[0]), increment=False) for n in nets]
+        assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2])
+        for f in range(1, len(seq)):
+            p, c = seq[f]
+            outs = [n(_inp(p, c), increment=True, all_points=True) for n in nets]
+            assert torch.equal(outs[0], outs[1]), "frame %d" % f
+            assert torch.equal(outs[0], outs[2]), "frame %d" % f
+            all_p = np.concatenate([all_p, p], 0)
+            all_c = np.concatenate([all_c, c], 0)
+        full = scn.compile(copy.deepcopy(model).sparseModel, capacity_sites=60000)(_inp(all_p, all_c), increment=False)
+        assert torch.equal(outs[1], full)
+        assert [int(v) for v in nets[1].sites_per_level()] == [int(v) for v in nets[0].sites_per_level()]
