@@ -150,6 +150,17 @@ int insc_order_build(const insc_grid *g, const int32_t *d_nbr, int64_t first, in
  * the reference (its rulebook is already split by offset, Metadata/Metadata.h:86). */
 int insc_order_by_offset(const int32_t *d_order, const int32_t *d_offset, int64_t n, int32_t *d_out, void *stream);
 
+/* Both orders and their inverses for n_scales (1..8) scales at once, the radix passes of all scales
+ * in the same launches: for scale i over its sites 0..n[i]-1 (1 <= n[i] <= 262144),
+ *   d_order[i]   = what insc_order_build(grids[i], d_nbr[i], 0, n[i]) gives,  d_pos[i][d_order[i][t]] = t,
+ * and, where d_offset[i] is not NULL,
+ *   d_bo_order[i] = what insc_order_by_offset(d_order[i], d_offset[i], n[i]) gives, d_bo_pos[i] its inverse.
+ * Same results as the two calls scale by scale (both are stable sorts of the same keys), in about a
+ * third of the launches.  No counterpart in the reference. */
+int insc_order_build_scales(const insc_grid *const *grids, const int32_t *const *d_nbr, const int32_t *const *d_offset,
+                            const int64_t *n, int n_scales, int32_t *const *d_order, int32_t *const *d_pos,
+                            int32_t *const *d_bo_order, int32_t *const *d_bo_pos, void *stream);
+
 /* ---------------------------------------------------------------------------------------
  * Feature kernels.
  * ------------------------------------------------------------------------------------- */

@@ -55,6 +55,17 @@ struct PlanRef {
 };
 int ssc3_new_sites_batch(const insc_grid *const *grids, int32_t *const *d_nbr, int n, int64_t n_new_upper,
                          hipStream_t s, const PlanRef *plans = nullptr);
+// Processing orders of several scales built from scratch in shared launches (insc_order_build +
+// insc_order_by_offset + their inverses, scale by scale, take three times as many): order / pos = the
+// order of the 3^3 layers and its inverse over sites 0..n-1; with offset != null also bo_order / bo_pos,
+// the same sites grouped by their position inside the parent cell.  n <= SORT_BATCH_MAX_N per scale.
+struct OrderBuildJob {
+  const insc_grid *g;
+  const int32_t *nbr, *offset;
+  int64_t n;
+  int32_t *order, *pos, *bo_order, *bo_pos;
+};
+int order_build_batch(const OrderBuildJob *jobs, int n_jobs, hipStream_t s);
 // Residual frames, all scales in two launches: d_pre_exist[l][i] = the saved site (grid pre[l]) at the
 // coordinates of site i of grids[l], or -1; d_nbr_pre[l] = the 27 saved neighbours of the sites that
 // have none (insc_grid_query + insc_incre_rulebook_ssc3); d_parent2[l][i], for l + 1 < n, = the saved

@@ -1226,7 +1226,19 @@ int insc_net_forward(insc_net *net, const int32_t *d_coords, int coord_cols, con
       if (ns > 0 && (rc = order_append_new_sites_both_batch(sg, snbr, soff, sord, spos, sbo, sbp, ns, nmax, s, true)))
         return rc;
     }
+    // the large scales: radix sorts, all scales pass by pass in the same launches where they fit
+    OrderBuildJob big[16];
+    int n_big = 0;
+    bool batch_ok = true;
     for (int l = 0; l < L; l++) {
+      Level &Lv = net->levels[l];
+      if (Lv.n == 0 || Lv.n <= order_sorted_max()) continue;
+      if (Lv.n > SORT_BATCH_MAX_N || n_big == SORT_BATCH_MAX_JOBS) batch_ok = false;
+      if (batch_ok)
+        big[n_big++] = OrderBuildJob{Lv.grid, Lv.nbr, l + 1 < L ? Lv.offset : nullptr, Lv.n, Lv.order, Lv.pos, Lv.bo_order, Lv.bo_pos};
+    }
+    if (batch_ok && n_big > 0 && (rc = order_build_batch(big, n_big, s))) return rc;
+    for (int l = 0; l < L && !batch_ok; l++) {
       Level &Lv = net->levels[l];
       if (Lv.n == 0 || Lv.n <= order_sorted_max()) continue;
       if ((rc = insc_order_build(Lv.grid, Lv.nbr, 0, Lv.n, Lv.order, stream))) return rc;

@@ -1,5 +1,8 @@
 // Rulebook list form, processing order, dirty-site propagation.
+#include <algorithm>
+
 #include "common.h"
+#include "grid.h"
 
 namespace insc {
 
@@ -65,6 +68,37 @@ __global__ void offset_key_kernel(const int32_t *__restrict__ order, const int32
   const int s = order ? order[t] : (int)t;
   keys[t] = (uint64_t)(offset[s] & 7);
   vals[t] = s;
+}
+
+// the two key kernels for several scales in one launch each (blockIdx.y = scale)
+struct OrderBuildJobDev {
+  const int32_t *coords, *nbr, *offset, *order;
+  uint64_t *keys;
+  int32_t *vals;
+  int64_t n;
+};
+struct OrderBuildBatchDev {
+  OrderBuildJobDev job[SORT_BATCH_MAX_JOBS];
+};
+__global__ void order_key_batch_kernel(OrderBuildBatchDev b) {
+  const OrderBuildJobDev &j = b.job[blockIdx.y];
+  const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= j.n) return;
+  const int4 c = reinterpret_cast<const int4 *>(j.coords)[t];
+  uint32_t m = 0;
+  for (int k = 0; k < 27; k++) m |= (j.nbr[t * 27 + k] >= 0 ? 1u : 0u) << k;
+  const uint64_t mort = spread3((uint64_t)((c.x >> 6) & 15)) | (spread3((uint64_t)((c.y >> 6) & 15)) << 1) |
+                        (spread3((uint64_t)((c.z >> 6) & 15)) << 2);
+  j.keys[t] = ((uint64_t)(c.w & 1) << 39) | (mort << 27) | (uint64_t)m;
+  j.vals[t] = (int)t;
+}
+__global__ void offset_key_batch_kernel(OrderBuildBatchDev b) {
+  const OrderBuildJobDev &j = b.job[blockIdx.y];
+  const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= j.n) return;
+  const int s = j.order[t];
+  j.keys[t] = (uint64_t)(j.offset[s] & 7);
+  j.vals[t] = s;
 }
 
 __global__ void mark_kernel(const int32_t *__restrict__ site_of_point, int64_t P, uint8_t *__restrict__ mask) {
@@ -134,6 +168,60 @@ __global__ void compact_write_kernel(const uint8_t *__restrict__ mask, const int
 
 }  // namespace insc
 
+namespace insc {
+
+int order_build_batch(const OrderBuildJob *jobs, int n_jobs, hipStream_t s) {
+  if (n_jobs <= 0) return INSC_OK;
+  if (n_jobs > SORT_BATCH_MAX_JOBS) {
+    set_error("order_build_batch: at most %d scales", SORT_BATCH_MAX_JOBS);
+    return INSC_ERR_ARG;
+  }
+  size_t bytes = 0;
+  int64_t n_max = 0;
+  for (int i = 0; i < n_jobs; i++) {
+    if (jobs[i].n < 1 || jobs[i].n > SORT_BATCH_MAX_N || !jobs[i].g || !jobs[i].nbr || !jobs[i].order || !jobs[i].pos ||
+        (jobs[i].offset && (!jobs[i].bo_order || !jobs[i].bo_pos))) {
+      set_error("order_build_batch: bad job %d", i);
+      return INSC_ERR_ARG;
+    }
+    bytes += ((sizeof(uint64_t) + sizeof(int32_t)) * (size_t)jobs[i].n + 511) & ~(size_t)255;
+    n_max = std::max(n_max, jobs[i].n);
+  }
+  void *ws;
+  int rc = workspace(WS_API, s, bytes, &ws);
+  if (rc) return rc;
+  char *p = (char *)ws;
+  OrderBuildBatchDev b;
+  SortJob sj[SORT_BATCH_MAX_JOBS];
+  for (int i = 0; i < n_jobs; i++) {
+    uint64_t *keys = (uint64_t *)p;
+    int32_t *vals = (int32_t *)(keys + jobs[i].n);
+    p += ((sizeof(uint64_t) + sizeof(int32_t)) * (size_t)jobs[i].n + 511) & ~(size_t)255;
+    b.job[i] = OrderBuildJobDev{insc_grid_coords(jobs[i].g), jobs[i].nbr, jobs[i].offset, jobs[i].order, keys, vals, jobs[i].n};
+    sj[i] = SortJob{keys, vals, jobs[i].order, jobs[i].pos, jobs[i].n};
+  }
+  hipLaunchKernelGGL(order_key_batch_kernel, dim3(grid_for(n_max, 256), (unsigned)n_jobs), dim3(256), 0, s, b);
+  INSC_LAUNCH_CHECK();
+  if ((rc = sort_pairs_u64_into_batch(sj, n_jobs, ORDER_KEY_BITS, s))) return rc;
+  // the orders grouped by the position inside the parent cell, for the scales that have a coarser one
+  OrderBuildBatchDev b2;
+  int n2 = 0;
+  n_max = 0;
+  for (int i = 0; i < n_jobs; i++) {
+    if (!jobs[i].offset) continue;
+    b2.job[n2] = b.job[i];
+    sj[n2] = SortJob{b.job[i].keys, b.job[i].vals, jobs[i].bo_order, jobs[i].bo_pos, jobs[i].n};
+    n_max = std::max(n_max, jobs[i].n);
+    n2++;
+  }
+  if (n2 == 0) return INSC_OK;
+  hipLaunchKernelGGL(offset_key_batch_kernel, dim3(grid_for(n_max, 256), (unsigned)n2), dim3(256), 0, s, b2);
+  INSC_LAUNCH_CHECK();
+  return sort_pairs_u64_into_batch(sj, n2, 3, s);
+}
+
+}  // namespace insc
+
 using namespace insc;
 
 extern "C" {
@@ -191,6 +279,25 @@ int insc_order_build(const insc_grid *g, const int32_t *d_nbr, int64_t first, in
                      keys, ids);
   INSC_LAUNCH_CHECK();
   return sort_pairs_u64_into(keys, ids, d_order + first, n, ORDER_KEY_BITS, s);
+}
+
+int insc_order_build_scales(const insc_grid *const *grids, const int32_t *const *d_nbr, const int32_t *const *d_offset,
+                            const int64_t *n, int n_scales, int32_t *const *d_order, int32_t *const *d_pos,
+                            int32_t *const *d_bo_order, int32_t *const *d_bo_pos, void *stream) {
+  INSC_REQUIRE(grids && d_nbr && n && d_order && d_pos && n_scales >= 1 && n_scales <= SORT_BATCH_MAX_JOBS, INSC_ERR_ARG,
+               "insc_order_build_scales: 1..%d scales, no null array", SORT_BATCH_MAX_JOBS);
+  OrderBuildJob jobs[SORT_BATCH_MAX_JOBS];
+  for (int i = 0; i < n_scales; i++) {
+    INSC_REQUIRE(grids[i] && n[i] >= 1 && n[i] <= SORT_BATCH_MAX_N && n[i] <= insc_grid_capacity(grids[i]), INSC_ERR_ARG,
+                 "insc_order_build_scales: scale %d has %lld sites (1..%lld, within the grid's capacity)", i,
+                 (long long)n[i], (long long)SORT_BATCH_MAX_N);
+    const int32_t *off = d_offset ? d_offset[i] : nullptr;
+    INSC_REQUIRE(d_nbr[i] && d_order[i] && d_pos[i] && (!off || (d_bo_order && d_bo_pos && d_bo_order[i] && d_bo_pos[i])),
+                 INSC_ERR_ARG, "insc_order_build_scales: null pointer at scale %d", i);
+    jobs[i] = OrderBuildJob{grids[i], d_nbr[i], off, n[i], d_order[i], d_pos[i], off ? d_bo_order[i] : nullptr,
+                            off ? d_bo_pos[i] : nullptr};
+  }
+  return order_build_batch(jobs, n_scales, (hipStream_t)stream);
 }
 
 int insc_order_by_offset(const int32_t *d_order, const int32_t *d_offset, int64_t n, int32_t *d_out, void *stream) {

@@ -1,5 +1,7 @@
 // Device-wide exclusive scan and stable LSD radix sort.  These replace the CUDPP scan /
 // compact / radix-sort calls the reference leans on (CUDA/CUDPPWrapper.hpp:30-217).
+#include <algorithm>
+
 #include "common.h"
 
 namespace insc {
@@ -92,10 +94,8 @@ __global__ void scan_zero_total(int32_t *total) { *total = 0; }
 constexpr int SCAN_ONE_THREADS = 1024;
 constexpr int SCAN_ONE_ITEMS = 32;
 constexpr int SCAN_ONE_MAX = SCAN_ONE_THREADS * SCAN_ONE_ITEMS;
-__global__ __launch_bounds__(SCAN_ONE_THREADS) void scan_one_block(const int32_t *__restrict__ in,
-                                                                   int32_t *__restrict__ out, int n,
-                                                                   int32_t *__restrict__ total) {
-  __shared__ int wsum[SCAN_ONE_THREADS / 64];
+__device__ __forceinline__ void scan_one_block_body(const int32_t *__restrict__ in, int32_t *__restrict__ out, int n,
+                                                    int32_t *__restrict__ total, int *wsum /*[SCAN_ONE_THREADS / 64]*/) {
   const int per = (n + SCAN_ONE_THREADS - 1) / SCAN_ONE_THREADS;  // <= SCAN_ONE_ITEMS
   const int base = threadIdx.x * per;
   int v[SCAN_ONE_ITEMS];
@@ -123,6 +123,12 @@ __global__ __launch_bounds__(SCAN_ONE_THREADS) void scan_one_block(const int32_t
     ex += v[i];
   }
   if (threadIdx.x == 0 && total) *total = tot;
+}
+__global__ __launch_bounds__(SCAN_ONE_THREADS) void scan_one_block(const int32_t *__restrict__ in,
+                                                                   int32_t *__restrict__ out, int n,
+                                                                   int32_t *__restrict__ total) {
+  __shared__ int wsum[SCAN_ONE_THREADS / 64];
+  scan_one_block_body(in, out, n, total, wsum);
 }
 
 int scan_exclusive_i32(const int32_t *in, int32_t *out, int64_t n, int32_t *total, hipStream_t s) {
@@ -157,9 +163,8 @@ constexpr int SORT_THREADS = 256;
 constexpr int SORT_ROUNDS = 8;
 constexpr int SORT_TILE = SORT_THREADS * SORT_ROUNDS;
 
-__global__ __launch_bounds__(SORT_THREADS) void sort_hist(const uint64_t *__restrict__ keys, int64_t n, int shift,
-                                                          int32_t *__restrict__ counts, int nb) {
-  __shared__ int h[256];
+__device__ __forceinline__ void sort_hist_body(const uint64_t *__restrict__ keys, int64_t n, int shift,
+                                               int32_t *__restrict__ counts, int nb, int *h /*[256]*/) {
   h[threadIdx.x] = 0;
   __syncthreads();
   int64_t base = (int64_t)blockIdx.x * SORT_TILE;
@@ -171,14 +176,18 @@ __global__ __launch_bounds__(SORT_THREADS) void sort_hist(const uint64_t *__rest
   __syncthreads();
   counts[(int64_t)threadIdx.x * nb + blockIdx.x] = h[threadIdx.x];
 }
+__global__ __launch_bounds__(SORT_THREADS) void sort_hist(const uint64_t *__restrict__ keys, int64_t n, int shift,
+                                                          int32_t *__restrict__ counts, int nb) {
+  __shared__ int h[256];
+  sort_hist_body(keys, n, shift, counts, nb, h);
+}
 
-__global__ __launch_bounds__(SORT_THREADS) void sort_scatter(const uint64_t *__restrict__ keys_in,
-                                                             const int32_t *__restrict__ vals_in,
-                                                             uint64_t *__restrict__ keys_out,
-                                                             int32_t *__restrict__ vals_out, int64_t n, int shift,
-                                                             const int32_t *__restrict__ offsets, int nb) {
-  __shared__ int base[256];
-  __shared__ int wcount[SORT_THREADS / 64][256];
+// inv (nullable): the inverse of the permutation that vals_out receives, inv[vals_out[i]] = i
+__device__ __forceinline__ void sort_scatter_body(const uint64_t *__restrict__ keys_in,
+                                                  const int32_t *__restrict__ vals_in, uint64_t *__restrict__ keys_out,
+                                                  int32_t *__restrict__ vals_out, int32_t *__restrict__ inv, int64_t n,
+                                                  int shift, const int32_t *__restrict__ offsets, int nb, int *base,
+                                                  int (*wcount)[256]) {
   const int t = threadIdx.x, lane = t & 63, w = t >> 6;
   base[t] = offsets[(int64_t)t * nb + blockIdx.x];
   const int64_t tile = (int64_t)blockIdx.x * SORT_TILE;
@@ -206,6 +215,7 @@ __global__ __launch_bounds__(SORT_THREADS) void sort_scatter(const uint64_t *__r
       for (int i2 = 0; i2 < w; i2++) rank += wcount[i2][digit];
       keys_out[rank] = key;
       vals_out[rank] = val;
+      if (inv) inv[val] = rank;
     }
     __syncthreads();
     int add = 0;
@@ -214,6 +224,48 @@ __global__ __launch_bounds__(SORT_THREADS) void sort_scatter(const uint64_t *__r
     base[t] += add;
     __syncthreads();
   }
+}
+__global__ __launch_bounds__(SORT_THREADS) void sort_scatter(const uint64_t *__restrict__ keys_in,
+                                                             const int32_t *__restrict__ vals_in,
+                                                             uint64_t *__restrict__ keys_out,
+                                                             int32_t *__restrict__ vals_out, int64_t n, int shift,
+                                                             const int32_t *__restrict__ offsets, int nb) {
+  __shared__ int base[256];
+  __shared__ int wcount[SORT_THREADS / 64][256];
+  sort_scatter_body(keys_in, vals_in, keys_out, vals_out, nullptr, n, shift, offsets, nb, base, wcount);
+}
+
+// Several sorts of the same key width, pass by pass in the same launches (blockIdx.y = job): three
+// launches per pass whatever the number of jobs.  Jobs of at most SORT_BATCH_MAX_N pairs (the digit
+// counts of a pass then fit the one-workgroup scan).
+struct SortJobDev {
+  uint64_t *k[2];
+  int32_t *v[2];
+  int32_t *vals_out, *inv, *counts;
+  int64_t n;
+  int nb;
+};
+struct SortBatchDev {
+  SortJobDev job[SORT_BATCH_MAX_JOBS];
+};
+__global__ __launch_bounds__(SORT_THREADS) void sort_hist_batch(SortBatchDev b, int shift, int src) {
+  __shared__ int h[256];
+  const SortJobDev &j = b.job[blockIdx.y];
+  if ((int)blockIdx.x >= j.nb) return;
+  sort_hist_body(j.k[src], j.n, shift, j.counts, j.nb, h);
+}
+__global__ __launch_bounds__(SCAN_ONE_THREADS) void sort_scan_batch(SortBatchDev b) {
+  __shared__ int wsum[SCAN_ONE_THREADS / 64];
+  const SortJobDev &j = b.job[blockIdx.x];
+  scan_one_block_body(j.counts, j.counts, 256 * j.nb, nullptr, wsum);
+}
+__global__ __launch_bounds__(SORT_THREADS) void sort_scatter_batch(SortBatchDev b, int shift, int src, int last) {
+  __shared__ int base[256];
+  __shared__ int wcount[SORT_THREADS / 64][256];
+  const SortJobDev &j = b.job[blockIdx.y];
+  if ((int)blockIdx.x >= j.nb) return;
+  sort_scatter_body(j.k[src], j.v[src], j.k[src ^ 1], last ? j.vals_out : j.v[src ^ 1], last ? j.inv : nullptr, j.n, shift,
+                    j.counts, j.nb, base, wcount);
 }
 
 int sort_pairs_u64(uint64_t *keys, int32_t *vals, int64_t n, int key_bits, hipStream_t s) {
@@ -295,6 +347,57 @@ int sort_pairs_u64_into(uint64_t *keys, int32_t *vals_in, int32_t *vals_out, int
     INSC_LAUNCH_CHECK();
     uint64_t *tk = kin; kin = kout; kout = tk;
     int32_t *tv = vin; vin = vout; vout = tv;
+  }
+  return INSC_OK;
+}
+
+int sort_pairs_u64_into_batch(const SortJob *jobs, int n_jobs, int key_bits, hipStream_t s) {
+  if (n_jobs <= 0) return INSC_OK;
+  if (n_jobs > SORT_BATCH_MAX_JOBS || key_bits <= 0 || key_bits > 64) {
+    set_error("sort_pairs_u64_into_batch: %d jobs, %d key bits", n_jobs, key_bits);
+    return INSC_ERR_ARG;
+  }
+  const int passes = (key_bits + 7) / 8;
+  SortBatchDev b;
+  size_t bytes = 0;
+  int nb_max = 0;
+  for (int i = 0; i < n_jobs; i++) {
+    if (jobs[i].n < 1 || jobs[i].n > SORT_BATCH_MAX_N) {
+      set_error("sort_pairs_u64_into_batch: job %d has %lld pairs (1..%lld)", i, (long long)jobs[i].n,
+                (long long)SORT_BATCH_MAX_N);
+      return INSC_ERR_ARG;
+    }
+    bytes += (sizeof(uint64_t) + sizeof(int32_t)) * (size_t)jobs[i].n + 256 * sizeof(int32_t) * (size_t)cdiv(jobs[i].n, SORT_TILE) + 768;
+  }
+  void *ws;
+  int rc = workspace(WS_SORT, s, bytes, &ws);
+  if (rc) return rc;
+  char *p = (char *)ws;
+  auto take = [&](size_t nbytes) -> void * {
+    void *r = p;
+    p += (nbytes + 255) & ~(size_t)255;
+    return r;
+  };
+  for (int i = 0; i < n_jobs; i++) {
+    SortJobDev &j = b.job[i];
+    j.n = jobs[i].n;
+    j.nb = (int)cdiv(j.n, SORT_TILE);
+    nb_max = std::max(nb_max, j.nb);
+    j.k[0] = jobs[i].keys;
+    j.v[0] = jobs[i].vals_in;
+    j.k[1] = (uint64_t *)take(sizeof(uint64_t) * (size_t)j.n);
+    j.v[1] = (int32_t *)take(sizeof(int32_t) * (size_t)j.n);
+    j.counts = (int32_t *)take(sizeof(int32_t) * 256 * (size_t)j.nb);
+    j.vals_out = jobs[i].vals_out;
+    j.inv = jobs[i].inv_out;
+  }
+  for (int pass = 0; pass < passes; pass++) {
+    const int src = pass & 1, last = pass + 1 == passes;
+    hipLaunchKernelGGL(sort_hist_batch, dim3((unsigned)nb_max, (unsigned)n_jobs), dim3(SORT_THREADS), 0, s, b, 8 * pass, src);
+    hipLaunchKernelGGL(sort_scan_batch, dim3((unsigned)n_jobs), dim3(SCAN_ONE_THREADS), 0, s, b);
+    hipLaunchKernelGGL(sort_scatter_batch, dim3((unsigned)nb_max, (unsigned)n_jobs), dim3(SORT_THREADS), 0, s, b, 8 * pass, src,
+                       last);
+    INSC_LAUNCH_CHECK();
   }
   return INSC_OK;
 }

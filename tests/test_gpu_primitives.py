@@ -286,3 +286,60 @@ def test_insert_at_all_scales_equals_the_scale_by_scale_chain(S, P):
     assert sizes(gb) == na
     for g in ga + gb:
         lib.insc_grid_destroy(g)
+
+
+def test_orders_of_all_scales_at_once_equal_the_scale_by_scale_calls(S):
+    """insc_order_build_scales (the radix passes of all scales in shared launches, inverses written by the
+    last pass) against insc_order_build + insc_order_by_offset per scale: the same permutations, word
+    for word; three scales of very different size, the last one without a coarser scale above it."""
+    import ctypes
+
+    from sparseconvnet._lib import lib, ptr, stream_ptr
+
+    L, P = 3, 60000
+    vox = scenes.indoor_scene(seed=77, n=P, dims=(260, 200, 70), n_boxes=15, side_rng=(10, 50)).astype(np.int32)
+    cap = 2 * P
+    vp = ctypes.c_void_p
+    gs = []
+    for _ in range(L):
+        g = vp()
+        lib.insc_grid_create(I64(cap), ctypes.byref(g))
+        gs.append(g)
+    par = [torch.empty(cap, dtype=torch.int32, device="cuda") for _ in range(L)]
+    off = [torch.empty(cap, dtype=torch.int32, device="cuda") for _ in range(L)]
+    chi = [torch.full((cap, 8), -1, dtype=torch.int32, device="cuda") for _ in range(L)]
+    arr = lambda xs: (vp * len(xs))(*[x if isinstance(x, vp) else vp(x.data_ptr() if x is not None else 0) for x in xs])
+    counts = (I64 * L)()
+    c = dev(vox)
+    sop = torch.empty(P, dtype=torch.int32, device="cuda")
+    lib.insc_grid_insert_scales(arr(gs), arr(par), arr(off), arr(chi), L, ptr(c), 4, I64(P), ptr(sop), counts, stream_ptr())
+    n = list(counts)
+    assert n[0] == P and n[0] > n[1] > n[2] > 8192 // 4
+    nbr = [torch.empty((n[l], 27), dtype=torch.int32, device="cuda") for l in range(L)]
+    for l in range(L):
+        lib.insc_rulebook_ssc3(gs[l], I64(0), I64(n[l]), ptr(nbr[l]), 0, stream_ptr())
+    new = lambda l: torch.full((n[l],), -1, dtype=torch.int32, device="cuda")
+    # scale by scale
+    order_a = [new(l) for l in range(L)]
+    bo_a = [new(l) for l in range(L - 1)]
+    for l in range(L):
+        lib.insc_order_build(gs[l], ptr(nbr[l]), I64(0), I64(n[l]), ptr(order_a[l]), stream_ptr())
+        if l + 1 < L:
+            lib.insc_order_by_offset(ptr(order_a[l]), ptr(off[l]), I64(n[l]), ptr(bo_a[l]), stream_ptr())
+    # all at once
+    order_b, pos_b = [new(l) for l in range(L)], [new(l) for l in range(L)]
+    bo_b, bop_b = [new(l) for l in range(L)], [new(l) for l in range(L)]
+    offs = [off[l] for l in range(L - 1)] + [None]
+    lib.insc_order_build_scales(arr(gs), arr(nbr), arr(offs), (I64 * L)(*n), L, arr(order_b), arr(pos_b), arr(bo_b),
+                                arr(bop_b), stream_ptr())
+    for l in range(L):
+        assert torch.equal(order_a[l], order_b[l]), "order of scale %d" % l
+        ident = torch.arange(n[l], dtype=torch.int32, device="cuda")
+        assert torch.equal(pos_b[l][order_b[l].long()], ident), "inverse of scale %d" % l
+        assert torch.equal(torch.sort(order_b[l]).values, ident)
+        if l + 1 < L:
+            assert torch.equal(bo_a[l], bo_b[l]), "grouped order of scale %d" % l
+            assert torch.equal(bop_b[l][bo_b[l].long()], ident), "inverse of the grouped order of scale %d" % l
+    assert bool((bo_b[L - 1] == -1).all())  # the scale without a coarser one is left alone
+    for g in gs:
+        lib.insc_grid_destroy(g)
