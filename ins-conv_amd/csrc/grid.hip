@@ -711,7 +711,7 @@ __device__ __forceinline__ int4 frame_point(const int32_t *__restrict__ coords_i
 // rec[l * P + p]: what row p found at scale l - REC_SITE | id, the slot it claimed, or REC_NONE
 __global__ __launch_bounds__(256) void frame_claim_kernel(FrameInsertArgs a, const int32_t *__restrict__ coords_in,
                                                           int cols, int P, int32_t *__restrict__ bad, int32_t frame,
-                                                          uint32_t *__restrict__ rec) {
+                                                          uint32_t *__restrict__ rec, int shared_from) {
   const int l = blockIdx.y;
   const FrameLevelDev &L = a.lv[l];
   const int p = blockIdx.x * 256 + threadIdx.x;
@@ -724,26 +724,47 @@ __global__ __launch_bounds__(256) void frame_claim_kernel(FrameInsertArgs a, con
   }
   const int4 c = frame_point(coords_in, cols, p, l);
   const uint64_t key = pack_key(c.x, c.y, c.z, c.w);
-  int64_t s = home_slot(key, L.mask);
+  auto claim = [&]() -> uint32_t {
+    int64_t s = home_slot(key, L.mask);
+    for (int64_t probe = 0; probe <= L.mask && probe < MAX_PROBES; probe++) {
+      const int4 raw = *reinterpret_cast<const int4 *>(&L.table[s]);  // key (two words), val, pad
+      unsigned long long k = ((unsigned long long)(unsigned)raw.y << 32) | (unsigned)raw.x;
+      if (k == key && raw.z >= 0 && raw.z < VAL_PENDING) return REC_SITE | (uint32_t)raw.z;  // numbered before this frame
+      const bool seen = k == key;  // the slot already held this key when it was read
+      if (k == INSC_EMPTY_KEY) k = atomicCAS(&L.table[s].key, INSC_EMPTY_KEY, (unsigned long long)key);
+      if (k == INSC_EMPTY_KEY || k == key) {
+        // (the claim of a smaller row that this row has seen stands: the value only ever goes down, so a
+        // stale read errs on the side of one more atomic)
+        if (!(seen && raw.z >= VAL_PENDING && raw.z <= VAL_PENDING + p)) atomicMin(&L.table[s].val, VAL_PENDING + p);
+        return (uint32_t)s;
+      }
+      s = (s + 1) & L.mask;
+    }
+    return REC_NONE;
+  };
   uint32_t r = REC_NONE;
-  for (int64_t probe = 0; probe <= L.mask && probe < MAX_PROBES; probe++) {
-    const int4 raw = *reinterpret_cast<const int4 *>(&L.table[s]);  // key (two words), val, pad
-    unsigned long long k = ((unsigned long long)(unsigned)raw.y << 32) | (unsigned)raw.x;
-    if (k == key && raw.z >= 0 && raw.z < VAL_PENDING) {  // numbered before this frame
-      r = REC_SITE | (uint32_t)raw.z;
-      break;
+  if (l < shared_from) {
+    r = claim();
+  } else {
+    // From the third scale on, neighbouring rows mostly fall into the same cell (at the coarsest scale of
+    // a full frame thousands of rows per cell), and atomics on one address are served one at a time: the
+    // rows of a wavefront that share a cell send one claim, that of their first lane - the smallest row,
+    // rows ascending with the lanes - and all take its answer.
+    bool todo = true;
+    while (todo) {  // (lanes leave as their cell is served; every turn serves the first waiting lane's cell)
+      const uint64_t waiting = __ballot(true);
+      const int leader = (int)__builtin_ctzll(waiting);
+      const uint32_t klo = (uint32_t)__shfl((int)(uint32_t)key, leader, 64);
+      const uint32_t khi = (uint32_t)__shfl((int)(uint32_t)(key >> 32), leader, 64);
+      const bool same = key == (((uint64_t)khi << 32) | klo);
+      uint32_t mine = REC_NONE;
+      if ((int)(threadIdx.x & 63) == leader) mine = claim();
+      const uint32_t got = (uint32_t)__shfl((int)mine, leader, 64);
+      if (same) {
+        r = got;
+        todo = false;
+      }
     }
-    const bool seen = k == key;  // the slot already held this key when it was read
-    if (k == INSC_EMPTY_KEY) k = atomicCAS(&L.table[s].key, INSC_EMPTY_KEY, (unsigned long long)key);
-    if (k == INSC_EMPTY_KEY || k == key) {
-      r = (uint32_t)s;
-      // (the claim of a smaller row that this row has seen stands: the value only ever goes down, so a
-      // stale read errs on the side of one more atomic.  At a coarse scale thousands of rows of a full
-      // frame fall into one cell, and same-address atomics are served one at a time.)
-      if (!(seen && raw.z >= VAL_PENDING && raw.z <= VAL_PENDING + p)) atomicMin(&L.table[s].val, VAL_PENDING + p);
-      break;
-    }
-    s = (s + 1) & L.mask;
   }
   if (r == REC_NONE) atomicOr(L.d_err, 2);
   rec[(int64_t)l * P + p] = r;
@@ -990,8 +1011,11 @@ int frame_insert_levels(const FrameInsertLevel *lv, int n_levels, const int32_t 
   if (rc) return rc;
   int32_t *site = (int32_t *)ws;
   uint32_t *rec = (uint32_t *)(site + PL);
+  // (frames of many points: from the third scale on the rows of a wavefront share their claims; for a few
+  // thousand points the turns this takes cost more than the atomics they save)
+  const int shared_from = large ? 2 : 16;
   hipLaunchKernelGGL(frame_claim_kernel, dim3(grid_for(P, 256), (unsigned)n_levels), dim3(256), 0, s, a, d_coords, cols,
-                     (int)P, d_bad, frame, rec);
+                     (int)P, d_bad, frame, rec, shared_from);
   if (large) {
     int32_t *rep = (int32_t *)(rec + PL), *flag = rep + PL, *n_before = flag + PL + 1;
     hipLaunchKernelGGL(frame_flag_kernel, dim3(grid_for(P, 256), (unsigned)n_levels), dim3(256), 0, s, a, (int)P,
