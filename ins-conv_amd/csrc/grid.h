@@ -54,7 +54,9 @@ struct PlanRef {
   int64_t ld;
 };
 int ssc3_new_sites_batch(const insc_grid *const *grids, int32_t *const *d_nbr, int n, int64_t n_new_upper,
-                         hipStream_t s, const PlanRef *plans = nullptr);
+                         hipStream_t s, const PlanRef *plans = nullptr, bool all_new = false);
+// (all_new: the caller knows that grids without older sites - d_n[1] == 0 - are to get whole maps, as in a
+// full frame: their rows are set to -1 first and every neighbour pair is looked up once)
 // Processing orders of several scales built from scratch in shared launches (insc_order_build +
 // insc_order_by_offset + their inverses, scale by scale, take three times as many): order / pos = the
 // order of the 3^3 layers and its inverse over sites 0..n-1; with offset != null also bo_order / bo_pos,

@@ -253,6 +253,32 @@ __global__ void ssc3_nbr_kernel(const Slot *__restrict__ table, int64_t mask, co
   if (patch_reverse && r >= 0 && r < first) nbr[(int64_t)r * 27 + (26 - k)] = (int)o;
 }
 
+// The same map when every site of the grid gets its row in this call (n = all sites, rows pre-filled
+// with -1): a site being neighbour k of another makes that one neighbour 26 - k of the first, so a
+// thread per (site, offset < 13) looks the neighbour up and writes both entries - half the probes.
+__device__ __forceinline__ void ssc3_nbr_sym_body(const Slot *__restrict__ table, int64_t mask,
+                                                  const int32_t *__restrict__ site_coords, int64_t n,
+                                                  int32_t *__restrict__ nbr, int64_t t) {
+  if (t >= n * 14) return;
+  const int64_t o = t / 14;
+  const int k = (int)(t % 14);
+  if (k == 13) {
+    nbr[o * 27 + 13] = (int)o;
+    return;
+  }
+  const int4 c = reinterpret_cast<const int4 *>(site_coords)[o];
+  const int x = c.x + k / 9 - 1, y = c.y + (k / 3) % 3 - 1, z = c.z + k % 3 - 1;
+  if (!coord_ok(x, y, z, c.w)) return;
+  const int r = grid_find(table, mask, pack_key(x, y, z, c.w));
+  if (r < 0 || r >= n) return;
+  nbr[o * 27 + k] = r;
+  nbr[(int64_t)r * 27 + (26 - k)] = (int)o;
+}
+__global__ void ssc3_nbr_sym_kernel(const Slot *__restrict__ table, int64_t mask, const int32_t *__restrict__ site_coords,
+                                    int64_t n, int32_t *__restrict__ nbr) {
+  ssc3_nbr_sym_body(table, mask, site_coords, n, nbr, (int64_t)blockIdx.x * blockDim.x + threadIdx.x);
+}
+
 // Neighbours, in another (saved) grid, of the sites that the saved grid does not hold; see
 // insc_incre_rulebook_ssc3
 __global__ void incre_ssc3_nbr_kernel(const Slot *__restrict__ pre_table, int64_t pre_mask,
@@ -299,9 +325,14 @@ __device__ __forceinline__ void ssc3_nbr_new_body(const Slot *__restrict__ table
                                                   const int32_t *__restrict__ d_n, int32_t *__restrict__ nbr,
                                                   int32_t *__restrict__ plan = nullptr,
                                                   uint32_t *__restrict__ tmask = nullptr,
-                                                  const int32_t *__restrict__ pos = nullptr, int64_t ld = 0) {
+                                                  const int32_t *__restrict__ pos = nullptr, int64_t ld = 0,
+                                                  int symmetric = 0) {
   const int64_t first = d_n[1], n = (int64_t)d_n[0] - first;
   int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (symmetric && first == 0 && !plan) {  // every site is new and the rows hold -1: half the probes
+    ssc3_nbr_sym_body(table, mask, site_coords, n, nbr, t);
+    return;
+  }
   if (plan) {
     const int64_t tile = (first + 31) / 32 + t;
     if (tile < (first + n + 31) / 32) tmask[tile] = 0;
@@ -339,10 +370,18 @@ struct NewSitesJob {
 };
 struct NewSitesBatch {
   NewSitesJob job[16];
+  int symmetric;  // grids whose sites are all new have their rows at -1 (ssc3_nbr_fill_batch_kernel)
 };
 __global__ void ssc3_nbr_new_batch_kernel(NewSitesBatch b) {
   const NewSitesJob &j = b.job[blockIdx.y];
-  ssc3_nbr_new_body(j.table, j.mask, j.coords, j.d_n, j.nbr, j.plan, j.tmask, j.pos, j.ld);
+  ssc3_nbr_new_body(j.table, j.mask, j.coords, j.d_n, j.nbr, j.plan, j.tmask, j.pos, j.ld, b.symmetric);
+}
+// rows of the grids whose sites are all new set to -1, ahead of the symmetric form of the kernel above
+__global__ void ssc3_nbr_fill_batch_kernel(NewSitesBatch b) {
+  const NewSitesJob &j = b.job[blockIdx.y];
+  if (j.d_n[1] != 0 || j.plan) return;
+  const int64_t words = (int64_t)j.d_n[0] * 27, stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < words; i += stride) j.nbr[i] = -1;
 }
 
 static int grid_alloc_table(insc_grid *g, int64_t capacity_sites) {
@@ -1076,7 +1115,7 @@ int grid_noalloc_setup() {
 }
 
 int ssc3_new_sites_batch(const insc_grid *const *grids, int32_t *const *d_nbr, int n, int64_t n_new_upper,
-                         hipStream_t s, const PlanRef *plans) {
+                         hipStream_t s, const PlanRef *plans, bool all_new) {
   if (n <= 0 || n_new_upper <= 0) return INSC_OK;
   if (n > 16) {
     set_error("ssc3_new_sites_batch: at most 16 grids");
@@ -1092,6 +1131,10 @@ int ssc3_new_sites_batch(const insc_grid *const *grids, int32_t *const *d_nbr, i
       b.job[i].ld = plans[i].ld;
     }
   }
+  b.symmetric = all_new ? 1 : 0;
+  if (all_new)
+    hipLaunchKernelGGL(ssc3_nbr_fill_batch_kernel, dim3(grid_for(n_new_upper * 27, 1024, 4096), (unsigned)n), dim3(256), 0,
+                       s, b);
   hipLaunchKernelGGL(ssc3_nbr_new_batch_kernel, dim3(grid_for(n_new_upper * 27, 256, 1ll << 30), (unsigned)n), dim3(256),
                      0, s, b);
   INSC_LAUNCH_CHECK();
@@ -1359,6 +1402,15 @@ int insc_rulebook_ssc3(const insc_grid *g, int64_t first, int64_t n, int32_t *d_
                (long long)(first + n), (long long)g->capacity_sites);
   INSC_REQUIRE(n == 0 || d_nbr, INSC_ERR_ARG, "insc_rulebook_ssc3: d_nbr is null");
   if (n == 0) return INSC_OK;
+  if (first == 0 && n == g->n_exact) {
+    // every site of the grid: rows to -1, then half the probes (each found pair fills two entries)
+    int rc = insc_fill_i32(d_nbr, n * 27, -1, stream);
+    if (rc) return rc;
+    hipLaunchKernelGGL(ssc3_nbr_sym_kernel, dim3(grid_for(n * 14, 256, 1ll << 30)), dim3(256), 0, (hipStream_t)stream,
+                       g->table, g->n_slots - 1, g->coords, n, d_nbr);
+    INSC_LAUNCH_CHECK();
+    return INSC_OK;
+  }
   hipLaunchKernelGGL(ssc3_nbr_kernel, dim3(grid_for(n * 27, 256, 1ll << 30)), dim3(256), 0, (hipStream_t)stream,
                      g->table, g->n_slots - 1, g->coords, first, n, d_nbr, patch_reverse);
   INSC_LAUNCH_CHECK();

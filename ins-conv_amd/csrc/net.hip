@@ -1171,7 +1171,7 @@ int insc_net_forward(insc_net *net, const int32_t *d_coords, int coord_cols, con
       prefs[l] = keep ? PlanRef{Lv.plan, Lv.tmask, Lv.pos, Lv.cap} : PlanRef{nullptr, nullptr, nullptr, 0};
       app.job[l] = TilePlanJob{Lv.nbr, Lv.order, Lv.grid->d_n, 0, Lv.cap, keep ? Lv.plan : nullptr, Lv.tmask, nullptr};
     }
-    if ((rc = ssc3_new_sites_batch(grids, nbrs, L, P, s, prefs))) return rc;
+    if ((rc = ssc3_new_sites_batch(grids, nbrs, L, P, s, prefs, !inc))) return rc;
     if (inc && !refresh) {
       offsets[L - 1] = nullptr;  // the coarsest scale has no order by position inside a parent cell
       if ((rc = order_append_new_sites_both_batch(grids, cnbrs, offsets, orders, poss, bo_orders, bo_poss, L, P, s)))
