@@ -45,7 +45,7 @@ int zero_counters(hipStream_t stream, size_t count, int32_t **out);
 // ---- device primitives (scan_sort.hip) -------------------------------------------------
 int sort_pairs_u64_into(uint64_t *keys, int32_t *vals_in, int32_t *vals_out, int64_t n, int key_bits, hipStream_t s);
 int scan_exclusive_i32(const int32_t *in, int32_t *out, int64_t n, int32_t *total, hipStream_t s);
-// Several sorts of the same key width in shared launches (three per 8-bit pass, whatever the number of
+// Several sorts of the same key width in shared launches (two per 8-bit pass, whatever the number of
 // jobs).  Per job: vals_out receives vals_in in key order and inv_out (nullable) the inverse,
 // inv_out[vals_out[i]] = i (the values must then be a permutation of 0..n-1); keys and vals_in are scratch
 // afterwards.  1 <= n <= SORT_BATCH_MAX_N per job.

@@ -162,7 +162,11 @@ int scan_exclusive_i32(const int32_t *in, int32_t *out, int64_t n, int32_t *tota
 constexpr int SORT_THREADS = 256;
 constexpr int SORT_ROUNDS = 8;
 constexpr int SORT_TILE = SORT_THREADS * SORT_ROUNDS;
+constexpr int SORT_FUSED_MAX_BLOCKS = 256;  // up to this many blocks (524 288 pairs) every scatter block sums the counts itself
 
+// counts[digit * nb + block] for the scan over all counts, or - BY_BLOCK - counts[block * 256 + digit] for
+// a scatter that adds them up itself
+template <bool BY_BLOCK>
 __device__ __forceinline__ void sort_hist_body(const uint64_t *__restrict__ keys, int64_t n, int shift,
                                                int32_t *__restrict__ counts, int nb, int *h /*[256]*/) {
   h[threadIdx.x] = 0;
@@ -174,22 +178,51 @@ __device__ __forceinline__ void sort_hist_body(const uint64_t *__restrict__ keys
     if (i < n) atomicAdd(&h[(int)((keys[i] >> shift) & 255)], 1);
   }
   __syncthreads();
-  counts[(int64_t)threadIdx.x * nb + blockIdx.x] = h[threadIdx.x];
+  if (BY_BLOCK)
+    counts[(int64_t)blockIdx.x * 256 + threadIdx.x] = h[threadIdx.x];
+  else
+    counts[(int64_t)threadIdx.x * nb + blockIdx.x] = h[threadIdx.x];
 }
+template <bool FUSED>
 __global__ __launch_bounds__(SORT_THREADS) void sort_hist(const uint64_t *__restrict__ keys, int64_t n, int shift,
                                                           int32_t *__restrict__ counts, int nb) {
   __shared__ int h[256];
-  sort_hist_body(keys, n, shift, counts, nb, h);
+  sort_hist_body<FUSED>(keys, n, shift, counts, nb, h);
 }
 
 // inv (nullable): the inverse of the permutation that vals_out receives, inv[vals_out[i]] = i
+// offsets: the scanned counts, [digit * nb + block]; or - RAW - the counts themselves, [block * 256 + digit]:
+// thread t then adds up the counts of digit t over the blocks (before this one, and all) and the block
+// scans the digit totals, in place of a scan launch between the histogram and the scatter.
+template <bool RAW>
 __device__ __forceinline__ void sort_scatter_body(const uint64_t *__restrict__ keys_in,
                                                   const int32_t *__restrict__ vals_in, uint64_t *__restrict__ keys_out,
                                                   int32_t *__restrict__ vals_out, int32_t *__restrict__ inv, int64_t n,
                                                   int shift, const int32_t *__restrict__ offsets, int nb, int *base,
                                                   int (*wcount)[256]) {
   const int t = threadIdx.x, lane = t & 63, w = t >> 6;
-  base[t] = offsets[(int64_t)t * nb + blockIdx.x];
+  if (RAW) {
+    int before = 0, total = 0;
+    for (int b0 = 0; b0 < nb; b0 += 16) {  // (sixteen loads in flight at a time)
+      int c[16];
+#pragma unroll
+      for (int u = 0; u < 16; u++) c[u] = b0 + u < nb ? offsets[(int64_t)(b0 + u) * 256 + t] : 0;
+#pragma unroll
+      for (int u = 0; u < 16; u++) {
+        if (b0 + u < (int)blockIdx.x) before += c[u];
+        total += c[u];
+      }
+    }
+    const int inc = wave_incl_scan(total);
+    if (lane == 63) wcount[0][w] = inc;
+    __syncthreads();
+    int off = 0;
+    for (int i = 0; i < w; i++) off += wcount[0][i];
+    base[t] = off + inc - total + before;
+    __syncthreads();  // (wcount is cleared below)
+  } else {
+    base[t] = offsets[(int64_t)t * nb + blockIdx.x];
+  }
   const int64_t tile = (int64_t)blockIdx.x * SORT_TILE;
   for (int r = 0; r < SORT_ROUNDS; r++) {
 #pragma unroll
@@ -225,6 +258,7 @@ __device__ __forceinline__ void sort_scatter_body(const uint64_t *__restrict__ k
     __syncthreads();
   }
 }
+template <bool FUSED>
 __global__ __launch_bounds__(SORT_THREADS) void sort_scatter(const uint64_t *__restrict__ keys_in,
                                                              const int32_t *__restrict__ vals_in,
                                                              uint64_t *__restrict__ keys_out,
@@ -232,12 +266,12 @@ __global__ __launch_bounds__(SORT_THREADS) void sort_scatter(const uint64_t *__r
                                                              const int32_t *__restrict__ offsets, int nb) {
   __shared__ int base[256];
   __shared__ int wcount[SORT_THREADS / 64][256];
-  sort_scatter_body(keys_in, vals_in, keys_out, vals_out, nullptr, n, shift, offsets, nb, base, wcount);
+  sort_scatter_body<FUSED>(keys_in, vals_in, keys_out, vals_out, nullptr, n, shift, offsets, nb, base, wcount);
 }
 
-// Several sorts of the same key width, pass by pass in the same launches (blockIdx.y = job): three
-// launches per pass whatever the number of jobs.  Jobs of at most SORT_BATCH_MAX_N pairs (the digit
-// counts of a pass then fit the one-workgroup scan).
+// Several sorts of the same key width, pass by pass in the same launches (blockIdx.y = job): two
+// launches per pass whatever the number of jobs (the scatter adds up the digit counts itself).  Jobs of at
+// most SORT_BATCH_MAX_N pairs, i.e. 128 blocks whose counts every scatter block reads.
 struct SortJobDev {
   uint64_t *k[2];
   int32_t *v[2];
@@ -252,20 +286,15 @@ __global__ __launch_bounds__(SORT_THREADS) void sort_hist_batch(SortBatchDev b, 
   __shared__ int h[256];
   const SortJobDev &j = b.job[blockIdx.y];
   if ((int)blockIdx.x >= j.nb) return;
-  sort_hist_body(j.k[src], j.n, shift, j.counts, j.nb, h);
-}
-__global__ __launch_bounds__(SCAN_ONE_THREADS) void sort_scan_batch(SortBatchDev b) {
-  __shared__ int wsum[SCAN_ONE_THREADS / 64];
-  const SortJobDev &j = b.job[blockIdx.x];
-  scan_one_block_body(j.counts, j.counts, 256 * j.nb, nullptr, wsum);
+  sort_hist_body<true>(j.k[src], j.n, shift, j.counts, j.nb, h);
 }
 __global__ __launch_bounds__(SORT_THREADS) void sort_scatter_batch(SortBatchDev b, int shift, int src, int last) {
   __shared__ int base[256];
   __shared__ int wcount[SORT_THREADS / 64][256];
   const SortJobDev &j = b.job[blockIdx.y];
   if ((int)blockIdx.x >= j.nb) return;
-  sort_scatter_body(j.k[src], j.v[src], j.k[src ^ 1], last ? j.vals_out : j.v[src ^ 1], last ? j.inv : nullptr, j.n, shift,
-                    j.counts, j.nb, base, wcount);
+  sort_scatter_body<true>(j.k[src], j.v[src], j.k[src ^ 1], last ? j.vals_out : j.v[src ^ 1], last ? j.inv : nullptr, j.n,
+                          shift, j.counts, j.nb, base, wcount);
 }
 
 int sort_pairs_u64(uint64_t *keys, int32_t *vals, int64_t n, int key_bits, hipStream_t s) {
@@ -292,10 +321,15 @@ int sort_pairs_u64(uint64_t *keys, int32_t *vals, int64_t n, int key_bits, hipSt
   int32_t *vin = vals, *vout = v2;
   for (int p = 0; p < passes; p++) {
     int shift = 8 * p;
-    hipLaunchKernelGGL(sort_hist, dim3(nb), dim3(SORT_THREADS), 0, s, kin, n, shift, counts, nb);
-    rc = scan_exclusive_i32(counts, counts, 256 * (int64_t)nb, nullptr, s);
-    if (rc) return rc;
-    hipLaunchKernelGGL(sort_scatter, dim3(nb), dim3(SORT_THREADS), 0, s, kin, vin, kout, vout, n, shift, counts, nb);
+    if (nb <= SORT_FUSED_MAX_BLOCKS) {  // (the scatter adds up the digit counts itself: two launches per pass)
+      hipLaunchKernelGGL(sort_hist<true>, dim3(nb), dim3(SORT_THREADS), 0, s, kin, n, shift, counts, nb);
+      hipLaunchKernelGGL(sort_scatter<true>, dim3(nb), dim3(SORT_THREADS), 0, s, kin, vin, kout, vout, n, shift, counts, nb);
+    } else {
+      hipLaunchKernelGGL(sort_hist<false>, dim3(nb), dim3(SORT_THREADS), 0, s, kin, n, shift, counts, nb);
+      rc = scan_exclusive_i32(counts, counts, 256 * (int64_t)nb, nullptr, s);
+      if (rc) return rc;
+      hipLaunchKernelGGL(sort_scatter<false>, dim3(nb), dim3(SORT_THREADS), 0, s, kin, vin, kout, vout, n, shift, counts, nb);
+    }
     INSC_LAUNCH_CHECK();
     uint64_t *tk = kin; kin = kout; kout = tk;
     int32_t *tv = vin; vin = vout; vout = tv;
@@ -338,12 +372,18 @@ int sort_pairs_u64_into(uint64_t *keys, int32_t *vals_in, int32_t *vals_out, int
   for (int p = 0; p < passes; p++) {
     const int shift = 8 * p;
     const bool last = p + 1 == passes;
-    hipLaunchKernelGGL(sort_hist, dim3(nb), dim3(SORT_THREADS), 0, s, kin, n, shift, counts, nb);
-    rc = scan_exclusive_i32(counts, counts, 256 * (int64_t)nb, nullptr, s);
-    if (rc) return rc;
     // (the keys of the last pass go where they would have gone; nobody reads them)
-    hipLaunchKernelGGL(sort_scatter, dim3(nb), dim3(SORT_THREADS), 0, s, kin, vin, kout, last ? vals_out : vout, n,
-                       shift, counts, nb);
+    if (nb <= SORT_FUSED_MAX_BLOCKS) {
+      hipLaunchKernelGGL(sort_hist<true>, dim3(nb), dim3(SORT_THREADS), 0, s, kin, n, shift, counts, nb);
+      hipLaunchKernelGGL(sort_scatter<true>, dim3(nb), dim3(SORT_THREADS), 0, s, kin, vin, kout, last ? vals_out : vout, n,
+                         shift, counts, nb);
+    } else {
+      hipLaunchKernelGGL(sort_hist<false>, dim3(nb), dim3(SORT_THREADS), 0, s, kin, n, shift, counts, nb);
+      rc = scan_exclusive_i32(counts, counts, 256 * (int64_t)nb, nullptr, s);
+      if (rc) return rc;
+      hipLaunchKernelGGL(sort_scatter<false>, dim3(nb), dim3(SORT_THREADS), 0, s, kin, vin, kout, last ? vals_out : vout, n,
+                         shift, counts, nb);
+    }
     INSC_LAUNCH_CHECK();
     uint64_t *tk = kin; kin = kout; kout = tk;
     int32_t *tv = vin; vin = vout; vout = tv;
@@ -394,7 +434,6 @@ int sort_pairs_u64_into_batch(const SortJob *jobs, int n_jobs, int key_bits, hip
   for (int pass = 0; pass < passes; pass++) {
     const int src = pass & 1, last = pass + 1 == passes;
     hipLaunchKernelGGL(sort_hist_batch, dim3((unsigned)nb_max, (unsigned)n_jobs), dim3(SORT_THREADS), 0, s, b, 8 * pass, src);
-    hipLaunchKernelGGL(sort_scan_batch, dim3((unsigned)n_jobs), dim3(SCAN_ONE_THREADS), 0, s, b);
     hipLaunchKernelGGL(sort_scatter_batch, dim3((unsigned)nb_max, (unsigned)n_jobs), dim3(SORT_THREADS), 0, s, b, 8 * pass, src,
                        last);
     INSC_LAUNCH_CHECK();
