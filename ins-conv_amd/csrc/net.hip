@@ -1201,10 +1201,21 @@ int insc_net_forward(insc_net *net, const int32_t *d_coords, int coord_cols, con
       INSC_HIP(hipEventSynchronize(net->ev_counts));
       if ((rc = apply_counts(net, "insc_net_forward"))) return rc;
     }
-    {
-      // the small scales: all their sites came with this frame's one insert, and the single-workgroup
-      // sorts of the incremental path order them - all of them in one launch - instead of some fifty
-      // launches per scale
+    // With a large scale around, the radix passes that it needs carry the other scales along in the same
+    // launches (their duration is the largest scale's); otherwise - or where a scale exceeds what those
+    // shared launches take - the small scales are sorted by one workgroup each, all in one launch.
+    OrderBuildJob big[16];
+    int n_big = 0, n_nonempty = 0;
+    bool any_large = false, batch_ok = true;
+    for (int l = 0; l < L; l++) {
+      const Level &Lv = net->levels[l];
+      if (Lv.n == 0) continue;
+      n_nonempty++;
+      if (Lv.n > order_sorted_max()) any_large = true;
+      if (Lv.n > SORT_BATCH_MAX_N) batch_ok = false;
+    }
+    batch_ok = batch_ok && any_large && n_nonempty <= SORT_BATCH_MAX_JOBS;
+    if (!batch_ok) {
       const insc_grid *sg[16];
       const int32_t *snbr[16], *soff[16];
       int32_t *sord[16], *spos[16], *sbo[16], *sbp[16];
@@ -1225,19 +1236,14 @@ int insc_net_forward(insc_net *net, const int32_t *d_coords, int coord_cols, con
       }
       if (ns > 0 && (rc = order_append_new_sites_both_batch(sg, snbr, soff, sord, spos, sbo, sbp, ns, nmax, s, true)))
         return rc;
-    }
-    // the large scales: radix sorts, all scales pass by pass in the same launches where they fit
-    OrderBuildJob big[16];
-    int n_big = 0;
-    bool batch_ok = true;
-    for (int l = 0; l < L; l++) {
-      Level &Lv = net->levels[l];
-      if (Lv.n == 0 || Lv.n <= order_sorted_max()) continue;
-      if (Lv.n > SORT_BATCH_MAX_N || n_big == SORT_BATCH_MAX_JOBS) batch_ok = false;
-      if (batch_ok)
+    } else {
+      for (int l = 0; l < L; l++) {
+        Level &Lv = net->levels[l];
+        if (Lv.n == 0) continue;
         big[n_big++] = OrderBuildJob{Lv.grid, Lv.nbr, l + 1 < L ? Lv.offset : nullptr, Lv.n, Lv.order, Lv.pos, Lv.bo_order, Lv.bo_pos};
+      }
+      if ((rc = order_build_batch(big, n_big, s))) return rc;
     }
-    if (batch_ok && n_big > 0 && (rc = order_build_batch(big, n_big, s))) return rc;
     for (int l = 0; l < L && !batch_ok; l++) {
       Level &Lv = net->levels[l];
       if (Lv.n == 0 || Lv.n <= order_sorted_max()) continue;
