@@ -335,8 +335,8 @@ int insc_net_enable_residual(insc_net *net);
  * which a scale's rows are cut into 32-row tiles), each frame's batch sorted among itself.  Once the
  * appended part of a scale of more than 8192 sites exceeds `percent` % of the part that was sorted
  * as a whole, the next incremental frame sorts the orders of all scales from scratch, as a full
- * frame does (about 0.5 ms once, for layers that then run some 10 % faster).  Results do not
- * depend on the order.  Default 25; 0: never.  No counterpart in the reference, which rebuilds
+ * frame does (0.1-0.2 ms once, for layers that then run some 10 % faster).  Results do not
+ * depend on the order.  Default 10; 0: never.  No counterpart in the reference, which rebuilds
  * its rulebooks on every call. */
 int insc_net_set_order_refresh(insc_net *net, int percent);
 /* Re-pack the weights after the caller changed them in place. */

@@ -124,7 +124,7 @@ struct insc_net {
   int n_levels = 0, in_channels = 0, mode = 4;
   bool finalized = false, have_state = false;
   bool keep_raw = false;  // keep the input of every batch norm (residual frames read it)
-  int order_refresh_pct = 25;  // an incremental frame re-sorts the orders once this share of a large scale is appended (0: never)
+  int order_refresh_pct = 10;  // an incremental frame re-sorts the orders once this share of a large scale is appended (0: never)
   insc::ResidualFrame rf;
   std::vector<insc::Level> levels;
   std::vector<insc::Buffer> buffers;
