@@ -353,7 +353,8 @@ int insc_net_rebind_op(insc_net *net, int op, const float *d_W, const float *d_b
  * increment == 0 forgets all state and runs a full forward; increment != 0 appends the points
  * and recomputes only the rows they affect.  d_out (nullable) receives one row of the output
  * tensor per point of this frame (out_all == 0) or per point since the last full frame.
- * Returns when the frame has completed.  A frame is all or nothing: if any of its coordinates is
+ * Returns once the frame is enqueued on `stream` (the host has waited for the site counts of the
+ * frame's insert by then, nothing else); d_out and the state are ready in stream order.  A frame is all or nothing: if any of its coordinates is
  * outside the representable range the call returns INSC_ERR_COORD and the state is that of the
  * previous frame (after a full frame that failed: no state; the next frame must be a full one). */
 int insc_net_forward(insc_net *net, const int32_t *d_coords, int coord_cols, const float *d_feats, int64_t P,

@@ -1348,7 +1348,8 @@ int insc_net_forward(insc_net *net, const int32_t *d_coords, int coord_cols, con
   net->n_points += P;
   net->have_state = true;
   if (net->profiling) INSC_HIP(hipEventRecord(net->ev[4], s));
-  INSC_HIP(hipStreamSynchronize(s));  // the counts are known already; the call returns when the frame is done
+  // (no wait here: the host has had the site counts since the structure phase, the output rows are ready in
+  // stream order, and what the caller enqueues next - a classifier on d_out - follows without a gap)
   net->ev_valid = net->profiling;
   if (h_n_sites) *h_n_sites = net->levels[0].n;
   return INSC_OK;
