@@ -710,6 +710,9 @@ def main():
                   "points_per_frame_mean": int(np.mean([len(seq[f][0]) for f in range(first, n_inc + 1)])),
                   "points_last_frame": int(len(seq[n_inc][0])),
                   "sites_at_start": sites_at_start, "sites_at_end": net.n_sites,
+                  "order_refresh": "library default: an incremental frame re-sorts the processing orders of its "
+                                   "scales once 10 % of a large scale has been appended (several of the timed "
+                                   "frames do)",
                   "sites_per_level_at_end": net.sites_per_level()[:7]}
         extra = {"frame_at_150k_ms": round(per_frame[-1], 3),
                  "median_ms": round(float(np.median(per_frame)), 3),
