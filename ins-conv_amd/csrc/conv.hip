@@ -68,11 +68,15 @@ __global__ __launch_bounds__(256) void conv_generic_kernel(const float *__restri
 }
 
 // ---------------------------------------------------------------------------------------
-// 3^3 layers with 1..4 input channels (the RGB stem of a U-Net): same thread layout and the same
-// order of operations as the generic kernel (so the same bits), but the 27 x CIN weights of a
-// thread's output channel stay in registers over all its rows, and the 27 neighbour ids and the
-// input values of a row are fetched in batches instead of one dependent load after the other.
+// 3^3 layers with 1..4 input channels (the RGB stem of a U-Net): same thread layout - a thread per (row,
+// output channel) - and the same order of operations as the generic kernel (so the same bits), but the
+// 27 x CIN weights of a thread's output channel stay in registers over all its rows, and the neighbour ids
+// and input values of a batch of rows are fetched once per block, one (row, offset) per thread, and read
+// back from LDS by the threads of the row (one 16-byte broadcast read per offset): with every thread
+// fetching its row's 27 ids and 81 values itself the kernel was bound by the number of load instructions
+// (92 us for 150k rows and 32 output channels).
 // ---------------------------------------------------------------------------------------
+constexpr int STEM_ROWS = 16;  // rows per batch at most (those of 256 / Cout rows that a block handles at a time)
 template <int CIN>
 __global__ __launch_bounds__(256) void conv_stem_kernel(const float *__restrict__ in, int64_t ld_in,
                                                         float *__restrict__ out, int64_t ld_out,
@@ -82,41 +86,52 @@ __global__ __launch_bounds__(256) void conv_stem_kernel(const float *__restrict_
                                                         const int32_t *__restrict__ d_n_rows, int64_t n_rows,
                                                         int Cout, const uint8_t *__restrict__ row_mask,
                                                         BnEpilogue ep) {
-  constexpr int K = 27, GK = 9;  // offsets per batch
+  constexpr int K = 27;
+  __shared__ float4 xs[2][STEM_ROWS][K];  // input values of (row, offset); two batches in turn
+  __shared__ int vs[2][STEM_ROWS][K];     // 1: the row has a neighbour at the offset
+  __shared__ int rid[2][STEM_ROWS];       // row of the batch, -1: none
   const int64_t n = d_n_rows ? min((int64_t)*d_n_rows, n_rows) : n_rows;
-  const int cpb = 256 / Cout;  // rows per block (Cout <= 256)
+  const int cpb = min(256 / Cout, STEM_ROWS);  // rows per batch (Cout <= 256)
   const int lr = threadIdx.x / Cout, co = threadIdx.x % Cout;
-  if (lr >= cpb) return;
+  const bool worker = lr < cpb;
   float w[K][CIN];
 #pragma unroll
   for (int k = 0; k < K; k++)
 #pragma unroll
-    for (int ci = 0; ci < CIN; ci++) w[k][ci] = W[((int64_t)k * CIN + ci) * Cout + co];
-  const float bv = bias ? bias[co] : 0.0f;
-  const float ew = ep.out2 ? ep.w[co] : 0.0f, eb = ep.out2 ? ep.b[co] : 0.0f;
-  for (int64_t t = (int64_t)blockIdx.x * cpb + lr; t < n; t += (int64_t)gridDim.x * cpb) {
-    const int row = rows ? rows[t] : (int)t;
-    if (row < 0 || (row_mask && !row_mask[row])) continue;
-    int src[K];
+    for (int ci = 0; ci < CIN; ci++) w[k][ci] = worker ? W[((int64_t)k * CIN + ci) * Cout + co] : 0.0f;
+  const float bv = (bias && worker) ? bias[co] : 0.0f;
+  const float ew = (ep.out2 && worker) ? ep.w[co] : 0.0f, eb = (ep.out2 && worker) ? ep.b[co] : 0.0f;
+  int buf = 0;
+  for (int64_t t0 = (int64_t)blockIdx.x * cpb; t0 < n; t0 += (int64_t)gridDim.x * cpb, buf ^= 1) {
+    // fetch: one (row, offset) per thread
+    for (int e = threadIdx.x; e < cpb * K; e += 256) {
+      const int er = e / K, k = e - er * K;
+      const int64_t t = t0 + er;
+      int row = t < n ? (rows ? rows[t] : (int)t) : -1;
+      if (row >= 0 && row_mask && !row_mask[row]) row = -1;
+      const int src = row >= 0 ? map0[(int64_t)row * K + k] : -1;
+      float x[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+      if (src >= 0) {
+        const float *p = in + (int64_t)src * ld_in;
 #pragma unroll
-    for (int k = 0; k < K; k++) src[k] = map0[(int64_t)row * K + k];
+        for (int ci = 0; ci < CIN; ci++) x[ci] = p[ci];
+      }
+      xs[buf][er][k] = make_float4(x[0], x[1], x[2], x[3]);
+      vs[buf][er][k] = src >= 0 ? 1 : 0;
+      if (k == 0) rid[buf][er] = row;
+    }
+    __syncthreads();  // (one barrier per batch: the next batch fills the other buffer)
+    const int row = worker ? rid[buf][lr] : -1;
+    if (row < 0) continue;
     float acc = bv;
 #pragma unroll
-    for (int g = 0; g < K / GK; g++) {
-      float x[GK][CIN];
+    for (int k = 0; k < K; k++) {
+      const float4 xv = xs[buf][lr][k];
+      const float x[4] = {xv.x, xv.y, xv.z, xv.w};
+      float a = acc;
 #pragma unroll
-      for (int j = 0; j < GK; j++) {
-        const float *p = in + (int64_t)max(src[g * GK + j], 0) * ld_in;
-#pragma unroll
-        for (int ci = 0; ci < CIN; ci++) x[j][ci] = p[ci];
-      }
-#pragma unroll
-      for (int j = 0; j < GK; j++) {
-        float a = acc;
-#pragma unroll
-        for (int ci = 0; ci < CIN; ci++) a = fmaf(x[j][ci], w[g * GK + j][ci], a);
-        acc = src[g * GK + j] >= 0 ? a : acc;
-      }
+      for (int ci = 0; ci < CIN; ci++) a = fmaf(x[ci], w[k][ci], a);
+      acc = vs[buf][lr][k] ? a : acc;
     }
     if (ep.res) acc += ep.res[(int64_t)row * ep.ldr + co];
     if (out) out[(int64_t)row * ld_out + co] = acc;
@@ -2149,7 +2164,7 @@ int launch_conv(const float *in, int64_t ld_in, int64_t in_rows, float *out, int
     const int cpb = 256 / Cout;
     if (mode == MAP_NBR && K == 27 && Cin <= 4) {
       // enough blocks to fill the machine, few enough that the weights are fetched rarely
-      const dim3 sg(grid_for(n_rows, cpb, (unsigned)device_cus() * 8));
+      const dim3 sg(grid_for(n_rows, std::min(cpb, STEM_ROWS), (unsigned)device_cus() * 8));
 #define INSC_STEM(CI)                                                                                          \
   hipLaunchKernelGGL(conv_stem_kernel<CI>, sg, dim3(256), 0, s, in, ld_in, out, ld_out, W, bias, map0, rows, \
                      d_n_rows, n_rows, Cout, row_mask, ep)
