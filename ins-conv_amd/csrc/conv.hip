@@ -1741,15 +1741,29 @@ __global__ void count_rules_kernel(const int32_t *__restrict__ map0, int K, cons
 __device__ __forceinline__ void tile_plan_body(const int32_t *__restrict__ nbr, const int32_t *__restrict__ order,
                                                const int32_t *__restrict__ d_n, int64_t n_rows, int64_t ld,
                                                int32_t *__restrict__ map, uint32_t *__restrict__ tmask) {
+  // A block transposes the rows of 256 positions through LDS: the rows are read 27 consecutive words at a
+  // time (consecutive threads, consecutive offsets), the plan is written one 1 KB run per offset.  (With a
+  // thread per position reading its own row every load instruction touched 64 different lines.)
+  __shared__ int site_l[256];
+  __shared__ int row_l[256 * 27];  // [position][offset]: stride 27, odd, so the reads below are conflict-free
   const int64_t n = d_n ? min((int64_t)*d_n, n_rows) : n_rows;
   const int64_t padded = (n + TILE_M - 1) / TILE_M * TILE_M;
-  const int64_t p = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t p0 = (int64_t)blockIdx.x * 256, p = p0 + threadIdx.x;
+  if (p0 >= padded) return;  // (the whole block)
+  site_l[threadIdx.x] = p < n ? (order ? order[p] : (int)p) : -1;
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < 27; i++) {
+    const int e = i * 256 + threadIdx.x, lp = e / 27, k = e - lp * 27;
+    const int site = site_l[lp];
+    row_l[e] = site >= 0 ? nbr[(int64_t)site * 27 + k] : -1;
+  }
+  __syncthreads();
   if (p >= padded) return;  // whole 32-lane groups leave together (padded is a multiple of 32)
-  const int site = p < n ? (order ? order[p] : (int)p) : -1;
   unsigned m = 0;
 #pragma unroll
   for (int k = 0; k < 27; k++) {
-    const int v = site >= 0 ? nbr[(int64_t)site * 27 + k] : -1;
+    const int v = row_l[threadIdx.x * 27 + k];
     map[(int64_t)k * ld + p] = v;
     if (v >= 0) m |= 1u << k;
   }
