@@ -25,6 +25,18 @@
 
 typedef int32_t Int;
 
+/* Arithmetic type of the feature operators.  The default build (float) is the restatement of
+ * the reference's fp32 CPU path.  A second build with -DORC_REAL=double (liborc64.so) runs the
+ * same operators, in the same order, in double precision: the yardstick that says how far each
+ * fp32 implementation - the reference's order of operations as restated here, and the HIP
+ * kernels' - is from the exact result, so that a tolerance can be stated per element. */
+#ifndef ORC_REAL
+#define ORC_REAL float
+#endif
+typedef ORC_REAL real;
+#define REAL_POW(x, y) (sizeof(real) == sizeof(float) ? (real)powf((float)(x), (float)(y)) : (real)pow((double)(x), (double)(y)))
+int orc_real_bytes(void) { return (int)sizeof(real); }
+
 /* ------------------------------------------------------------------------------------
  * Point -> site map.  Stands in for google::dense_hash_map<Point<4>, Int, IntArrayHash>
  * (Metadata/Metadata.h:95-106); the hash is the reference's FNV variant
@@ -126,12 +138,12 @@ void orc_grid_query(const Int *site_coords4, int64_t N, const Int *q4, int64_t Q
  * mode 4.  Written without the rule table: rows are visited in input order, which gives
  * each site the same order of additions.
  * ------------------------------------------------------------------------------------ */
-void orc_input_forward(const float *in, int64_t P, int C, const Int *site_of_point, const Int *count, int64_t N,
-                       int average, float *out) {
-  memset(out, 0, sizeof(float) * N * C);
+void orc_input_forward(const real *in, int64_t P, int C, const Int *site_of_point, const Int *count, int64_t N,
+                       int average, real *out) {
+  memset(out, 0, sizeof(real) * N * C);
   for (int64_t p = 0; p < P; p++) {
     Int s = site_of_point[p];
-    float mult = (average && count[s] > 0) ? 1.0f / (float)count[s] : 1.0f;
+    real mult = (average && count[s] > 0) ? 1.0f / (real)count[s] : 1.0f;
     for (int c = 0; c < C; c++) out[(int64_t)s * C + c] += mult * in[p * C + c];
   }
 }
@@ -139,9 +151,9 @@ void orc_input_forward(const float *in, int64_t P, int C, const Int *site_of_poi
 /* Output layer forward.  Follows CPU/IOLayers.cpp:99-115 (cpu_OutputLayer_updateOutput ->
  * InputLayer_BackwardPass with average=false): every original input row receives its
  * site's feature row, multiplier 1. */
-void orc_output_forward(const float *feats, int C, const Int *site_of_point, int64_t P, float *out) {
+void orc_output_forward(const real *feats, int C, const Int *site_of_point, int64_t P, real *out) {
   for (int64_t p = 0; p < P; p++)
-    memcpy(out + p * C, feats + (int64_t)site_of_point[p] * C, sizeof(float) * C);
+    memcpy(out + p * C, feats + (int64_t)site_of_point[p] * C, sizeof(real) * C);
 }
 
 /* ------------------------------------------------------------------------------------
@@ -240,7 +252,7 @@ int64_t orc_down2_rules(const Int *fine_coords4, int64_t Nf, Int *parent, Int *o
  * reference returns).  Within one offset every destination row occurs at most once, so
  * the parallel add is race-free (the reference relies on the same fact).
  * ------------------------------------------------------------------------------------ */
-double orc_conv_forward(const float *in, float *out, int64_t n_out, const float *W, const float *bias, const Int *pairs,
+double orc_conv_forward(const real *in, real *out, int64_t n_out, const real *W, const real *bias, const Int *pairs,
                         const Int *counts, int K, int Cin, int Cout, int swap) {
   for (int64_t r = 0; r < n_out; r++)
     for (int c = 0; c < Cout; c++) out[r * Cout + c] = bias ? bias[c] : 0.0f;
@@ -251,23 +263,23 @@ double orc_conv_forward(const float *in, float *out, int64_t n_out, const float 
     if (nr) {
       flops += (double)nr * Cin * Cout;
       const Int *r = pairs + 2 * base;
-      const float *w = W + (int64_t)k * Cin * Cout;
-      float *rows = (float *)malloc(sizeof(float) * nr * Cout);
+      const real *w = W + (int64_t)k * Cin * Cout;
+      real *rows = (real *)malloc(sizeof(real) * nr * Cout);
 #pragma omp parallel for schedule(static)
       for (int64_t i = 0; i < nr; i++) {
-        const float *x = in + (int64_t)r[2 * i + (swap ? 1 : 0)] * Cin;
-        float *y = rows + i * Cout;
+        const real *x = in + (int64_t)r[2 * i + (swap ? 1 : 0)] * Cin;
+        real *y = rows + i * Cout;
         for (int c = 0; c < Cout; c++) y[c] = 0.0f;
         for (int ci = 0; ci < Cin; ci++) {
-          float xv = x[ci];
-          const float *wr = w + (int64_t)ci * Cout;
+          real xv = x[ci];
+          const real *wr = w + (int64_t)ci * Cout;
           for (int c = 0; c < Cout; c++) y[c] += xv * wr[c];
         }
       }
 #pragma omp parallel for schedule(static)
       for (int64_t i = 0; i < nr; i++) {
-        float *t = out + (int64_t)r[2 * i + (swap ? 0 : 1)] * Cout;
-        const float *s = rows + i * Cout;
+        real *t = out + (int64_t)r[2 * i + (swap ? 0 : 1)] * Cout;
+        const real *s = rows + i * Cout;
         for (int c = 0; c < Cout; c++) t[c] += s[c];
       }
       free(rows);
@@ -283,19 +295,19 @@ double orc_conv_forward(const float *in, float *out, int64_t n_out, const float 
  * invstd = powf(var + eps, -0.5); w = invstd * gamma; b = -mean * w + beta;
  * y = x*w + b; y *= (y > 0) ? 1 : leakiness.
  * ------------------------------------------------------------------------------------ */
-void orc_bn_forward(const float *in, float *out, int64_t N, int C, const float *mean, const float *var,
-                    const float *gamma, const float *beta, float eps, float leakiness) {
-  float *w = (float *)malloc(sizeof(float) * C), *b = (float *)malloc(sizeof(float) * C);
+void orc_bn_forward(const real *in, real *out, int64_t N, int C, const real *mean, const real *var,
+                    const real *gamma, const real *beta, float eps, float leakiness) {
+  real *w = (real *)malloc(sizeof(real) * C), *b = (real *)malloc(sizeof(real) * C);
   for (int c = 0; c < C; c++) {
-    float invstd = powf(var[c] + eps, -0.5f);
+    real invstd = REAL_POW(var[c] + (real)eps, (real)-0.5);
     w[c] = invstd * (gamma ? gamma[c] : 1.0f);
     b[c] = -mean[c] * w[c] + (beta ? beta[c] : 0.0f);
   }
 #pragma omp parallel for schedule(static)
   for (int64_t r = 0; r < N; r++)
     for (int c = 0; c < C; c++) {
-      float o = in[r * C + c] * w[c] + b[c];
-      float s = (o > 0) ? 1.0f : leakiness;
+      real o = in[r * C + c] * w[c] + b[c];
+      real s = (o > 0) ? 1.0f : leakiness;
       out[r * C + c] = o * s;
     }
   free(w);
@@ -304,14 +316,14 @@ void orc_bn_forward(const float *in, float *out, int64_t N, int C, const float *
 
 /* Network-in-network (1x1 linear).  Follows CPU/NetworkInNetwork.cpp:8-23:
  * out = bias (or zero); out.addmm_(in, W).  Returns multiply-adds. */
-double orc_nin_forward(const float *in, float *out, int64_t N, const float *W, const float *bias, int Cin, int Cout) {
+double orc_nin_forward(const real *in, real *out, int64_t N, const real *W, const real *bias, int Cin, int Cout) {
 #pragma omp parallel for schedule(static)
   for (int64_t r = 0; r < N; r++) {
-    float *y = out + r * Cout;
+    real *y = out + r * Cout;
     for (int c = 0; c < Cout; c++) y[c] = bias ? bias[c] : 0.0f;
     for (int ci = 0; ci < Cin; ci++) {
-      float xv = in[r * Cin + ci];
-      const float *wr = W + (int64_t)ci * Cout;
+      real xv = in[r * Cin + ci];
+      const real *wr = W + (int64_t)ci * Cout;
       for (int c = 0; c < Cout; c++) y[c] += xv * wr[c];
     }
   }

@@ -11,31 +11,50 @@ import subprocess
 import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-_LIB = None
+_LIBS = {}
+_REAL = np.float32  # arithmetic type of the feature operators: float32 (the reference's) or float64
 
 _i32p = ctypes.POINTER(ctypes.c_int32)
-_f32p = ctypes.POINTER(ctypes.c_float)
 
 
-def build(force=False):
-    so = os.path.join(_HERE, "liborc.so")
+def build(force=False, real=np.float32):
+    name = "liborc.so" if real == np.float32 else "liborc64.so"
+    so = os.path.join(_HERE, name)
     if force or not os.path.exists(so):
-        subprocess.check_call(["make", "-C", _HERE, "-B", "liborc.so"], stdout=subprocess.DEVNULL)
+        subprocess.check_call(["make", "-C", _HERE, "-B", name], stdout=subprocess.DEVNULL)
     return so
 
 
 def lib():
-    global _LIB
-    if _LIB is None:
-        L = ctypes.CDLL(build())
+    if _REAL not in _LIBS:
+        L = ctypes.CDLL(build(real=_REAL))
         L.orc_grid_build.restype = ctypes.c_int64
         L.orc_ssc_rules.restype = ctypes.c_int64
         L.orc_down2_rules.restype = ctypes.c_int64
         L.orc_conv_forward.restype = ctypes.c_double
         L.orc_nin_forward.restype = ctypes.c_double
         L.orc_num_threads.restype = ctypes.c_int
-        _LIB = L
-    return _LIB
+        L.orc_real_bytes.restype = ctypes.c_int
+        if L.orc_real_bytes() != np.dtype(_REAL).itemsize:
+            raise RuntimeError("oracle library built for another arithmetic type")
+        _LIBS[_REAL] = L
+    return _LIBS[_REAL]
+
+
+class double_precision(object):
+    """`with double_precision():` runs the plain feature operators below (input / output layer,
+    rulebook convolution, batch norm, 1x1) through the double-precision build of the same C text
+    (liborc64.so): same operations in the same order, no fp32 rounding.  It is the yardstick
+    that fp32 results - the oracle's own and the HIP library's - are measured against; the
+    residual (incre_*) and pooling operators stay float32."""
+
+    def __enter__(self):
+        global _REAL
+        self._saved, _REAL = _REAL, np.float64
+
+    def __exit__(self, *exc):
+        global _REAL
+        _REAL = self._saved
 
 
 def _ip(a):
@@ -43,7 +62,10 @@ def _ip(a):
 
 
 def _fp(a):
-    return a.ctypes.data_as(_f32p) if a is not None else None
+    if a is None:
+        return None
+    assert a.dtype == _REAL
+    return a.ctypes.data_as(ctypes.c_void_p)  # data_as keeps the array alive for the call
 
 
 def _c4(coords):
@@ -56,7 +78,7 @@ def _c4(coords):
 
 
 def _f(a):
-    return np.ascontiguousarray(a, dtype=np.float32)
+    return np.ascontiguousarray(a, dtype=_REAL)
 
 
 def num_threads():
@@ -85,7 +107,7 @@ def input_forward(feats, site_of_point, count, mode=4):
     f = _f(feats)
     P, C = f.shape
     N = len(count)
-    out = np.empty((N, C), np.float32)
+    out = np.empty((N, C), _REAL)
     lib().orc_input_forward(_fp(f), ctypes.c_int64(P), C, _ip(np.ascontiguousarray(site_of_point, np.int32)),
                             _ip(np.ascontiguousarray(count, np.int32)), ctypes.c_int64(N), int(mode == 4), _fp(out))
     return out
@@ -94,7 +116,7 @@ def input_forward(feats, site_of_point, count, mode=4):
 def output_forward(feats, site_of_point):
     f = _f(feats)
     sop = np.ascontiguousarray(site_of_point, np.int32)
-    out = np.empty((len(sop), f.shape[1]), np.float32)
+    out = np.empty((len(sop), f.shape[1]), _REAL)
     lib().orc_output_forward(_fp(f), f.shape[1], _ip(sop), ctypes.c_int64(len(sop)), _fp(out))
     return out
 
@@ -133,7 +155,7 @@ def conv_forward(feats, W, bias, pairs, counts, n_out, swap=False):
     f, W = _f(feats), _f(W)
     K, Cin, Cout = W.shape
     assert f.shape[1] == Cin and len(counts) == K
-    out = np.empty((n_out, Cout), np.float32)
+    out = np.empty((n_out, Cout), _REAL)
     b = _f(bias) if bias is not None else None
     p = np.ascontiguousarray(pairs, np.int32)
     c = np.ascontiguousarray(counts, np.int32)
@@ -154,7 +176,7 @@ def bn_forward(feats, mean, var, gamma, beta, eps=1e-4, leakiness=0.0):
 
 def nin_forward(feats, W, bias=None):
     f, W = _f(feats), _f(W)
-    out = np.empty((f.shape[0], W.shape[1]), np.float32)
+    out = np.empty((f.shape[0], W.shape[1]), _REAL)
     b = _f(bias) if bias is not None else None
     lib().orc_nin_forward(_fp(f), _fp(out), ctypes.c_int64(f.shape[0]), _fp(W), _fp(b), W.shape[0], W.shape[1])
     return out

@@ -61,7 +61,7 @@ def _forward(module, x, save):
         ctx.coords[size] = sc
         ctx.site_of_point = sop
         ctx.count = cnt
-        f = orc.input_forward(np.asarray(feats, np.float32), sop, cnt, mode=module.mode)
+        f = orc.input_forward(np.asarray(feats), sop, cnt, mode=module.mode)
         return OTensor(f, size, ctx)
     if isinstance(module, scn.OutputLayer):
         return orc.output_forward(x.features, x.ctx.site_of_point)
@@ -71,7 +71,7 @@ def _forward(module, x, save):
         f = x[0].features
         for t in x[1:]:
             f = f + t.features
-        return OTensor(f.astype(np.float32), x[0].spatial_size, x[0].ctx)
+        return OTensor(f.astype(x[0].features.dtype), x[0].spatial_size, x[0].ctx)
     if isinstance(module, scn.JoinTable):
         return OTensor(np.concatenate([t.features for t in x], 1), x[0].spatial_size, x[0].ctx)
     if isinstance(module, scn.Sequential):

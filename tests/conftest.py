@@ -19,3 +19,13 @@ def orc():
 
     oracle.lib()
     return oracle
+
+
+def pytest_terminal_summary(terminalreporter):
+    """The float errors the parity checks observed (tests/parity.py), one line per check."""
+    import parity
+
+    if parity.REPORT:
+        terminalreporter.section("parity report (tolerance 1e-5 + 1e-4*|ref| per element)")
+        for line in parity.REPORT:
+            terminalreporter.write_line(line)

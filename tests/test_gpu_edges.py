@@ -7,6 +7,8 @@ import numpy as np
 import pytest
 import torch
 
+import parity
+
 from workloads import scenes
 
 pytestmark = pytest.mark.gpu
@@ -45,8 +47,7 @@ def test_batch_of_scenes_equals_scenes_run_alone():
     assert torch.equal(both[inv[:len(va)]], alone_a)
     assert torch.equal(both[inv[len(va):]], alone_b)
     ref = oracle_net.forward(cpu.sparseModel, [pts, rgb, 2])
-    scale = max(1.0, float(np.abs(ref).max()))
-    np.testing.assert_allclose(both.cpu().numpy(), ref, rtol=1e-4, atol=1e-5 * scale)
+    parity.check("two samples in one batch, 4-level U-Net", both.cpu().numpy(), ref)
 
 
 def test_sites_on_the_border_of_the_coordinate_range(orc):
@@ -137,8 +138,7 @@ def test_residual_frames_disjoint_from_and_inside_the_saved_scene():
         alone = ref_model.sparseModel(_inp(far, rgb[:1500]))
         # (not the same bits: a residual frame's convolutions use the launch shape for small row
         # counts, which adds the terms of a row in another order)
-        scale = max(1.0, float(alone.abs().max()))
-        np.testing.assert_allclose(got.cpu().numpy(), alone.cpu().numpy(), rtol=1e-4, atol=1e-5 * scale)
+        parity.check("residual frame away from the saved scene vs plain forward", got.cpu().numpy(), alone.cpu().numpy())
         # saved voxels, same colours, one point per voxel: mean unchanged -> residual 0
         idx = np.random.default_rng(48).permutation(len(vox))[:1200]
         got = net(_inp(vox[idx], rgb[idx]), increment="residual")

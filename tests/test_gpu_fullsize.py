@@ -11,6 +11,7 @@ import numpy as np
 import pytest
 import torch
 
+import parity
 from workloads import scenes
 
 pytestmark = pytest.mark.gpu
@@ -169,14 +170,13 @@ def test_workload3_layer_stack_against_oracle(S, orc, C):
             ref, _ = orc.conv_forward(ref, conv.weight.cpu().numpy(), b, pairs, counts, len(sc))
             ref = orc.bn_forward(ref, bn.running_mean.cpu().numpy(), bn.running_var.cpu().numpy(),
                                  bn.weight.cpu().numpy(), bn.bias.cpu().numpy(), bn.eps, 0.0)
-            scale = max(1.0, float(np.abs(ref).max()))
-            np.testing.assert_allclose(x.features.cpu().numpy(), ref, rtol=1e-4, atol=1e-5 * scale)
+            parity.check("workload 3, C=%d, end to end after layer %d" % (C, layer), x.features.cpu().numpy(), ref)
 
 
-def test_workload4_full_unet_forward_against_oracle():
+def test_workload4_full_unet_forward_against_oracle(orc):
     """The 150k-voxel scene (165k points) through the network executor and through the module tree,
-    against the same module tree evaluated on the CPU oracle (1e-4 relative, 1e-5 absolute relative to
-    the tensor's largest value, as for every whole-network comparison)."""
+    against the same module tree evaluated on the CPU oracle in fp32 and in double precision: every
+    element within 1e-5 + 1e-4 * |reference| of both (nothing scaled by the tensor's maximum)."""
     import sparseconvnet as scn
     from oracle import oracle_net
     from workloads.netdefs import NaiveUNet
@@ -191,11 +191,10 @@ def test_workload4_full_unet_forward_against_oracle():
     assert net.n_sites == len(vox) == 150000
     assert torch.equal(feats, feats_mod)
     ref = oracle_net.forward(model.sparseModel, [pts, rgb, 1])
+    with orc.double_precision():
+        ref64 = oracle_net.forward(model.sparseModel, [pts, rgb, 1])
     assert feats.shape == ref.shape == (len(pts), 32)
-    scale = max(1.0, float(np.abs(ref).max()))
-    err = np.abs(feats.cpu().numpy() - ref)
-    tol = 1e-5 * scale + 1e-4 * np.abs(ref)
-    assert (err <= tol).all(), "max err %.3e, worst excess %.3e" % (err.max(), (err - tol).max())
+    parity.check("workload 4, full U-Net forward, 150k voxels", feats.cpu().numpy(), ref, ref64)
 
 
 @pytest.mark.parametrize("C", [32, 64])
@@ -229,7 +228,7 @@ def test_workload3_convolution_is_independent_of_order_and_staging(S, C):
     torch.testing.assert_close(a, b, rtol=1e-5, atol=1e-6)
 
 
-def test_workload5_sweep_equals_a_full_forward_every_tenth_frame():
+def test_workload5_sweep_equals_a_full_forward_every_tenth_frame(orc):
     """All 50 frames of the sweep through the executor; after every tenth frame and after the last
     one a second executor runs ONE full forward over every point seen so far, in arrival order: the
     features of all points must be equal bit for bit.  The final scene is also compared with the CPU
@@ -260,8 +259,8 @@ def test_workload5_sweep_equals_a_full_forward_every_tenth_frame():
     from oracle import oracle_net
 
     oref = oracle_net.forward(model.sparseModel, [allp, allc, 1])
-    scale = max(1.0, float(np.abs(oref).max()))
-    err = np.abs(out.cpu().numpy() - oref)
-    assert (err <= 1e-5 * scale + 1e-4 * np.abs(oref)).all(), "sweep end vs oracle: max err %.3e" % err.max()
+    with orc.double_precision():
+        oref64 = oracle_net.forward(model.sparseModel, [allp, allc, 1])
+    parity.check("workload 5, last frame of the sweep, 150k voxels", out.cpu().numpy(), oref, oref64)
     assert set(phases) == {"structure", "dirty", "layers", "output"}
     assert 0.5 < sum(phases.values()) < 50.0

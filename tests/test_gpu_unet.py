@@ -4,6 +4,7 @@ import numpy as np
 import pytest
 import torch
 
+import parity
 from workloads import scenes
 
 pytestmark = pytest.mark.gpu
@@ -18,18 +19,10 @@ def _scene(n, seed, dup=0.1):
     return pts, rgb
 
 
-def _check(a, b, what):
-    """1e-4 relative / 1e-5 absolute, the tolerance stated for float32 outputs; for a deep
-    network the absolute term is taken relative to the tensor's scale (max |value|)."""
-    scale = max(1.0, float(np.abs(b).max()))
-    err = np.abs(a - b)
-    tol = 1e-5 * scale + 1e-4 * np.abs(b)
-    assert (err <= tol).all(), "%s: max err %.3e (scale %.3e), worst excess %.3e" % (
-        what, err.max(), scale, (err - tol).max())
 
 
 @pytest.mark.parametrize("levels,m", [(3, 16), (7, 32)])
-def test_unet_full_forward_matches_oracle(levels, m):
+def test_unet_full_forward_matches_oracle(orc, levels, m):
     from oracle import oracle_net
     from workloads.netdefs import NaiveUNet
 
@@ -40,10 +33,13 @@ def test_unet_full_forward_matches_oracle(levels, m):
         feats = model.sparseModel([coords, torch.from_numpy(rgb).cuda(), 1])
         logits = model.linear(feats)
     ref_feats = oracle_net.forward(model.sparseModel, [pts, rgb, 1])
+    with orc.double_precision():
+        ref64 = oracle_net.forward(model.sparseModel, [pts, rgb, 1])
     assert feats.shape == ref_feats.shape == (len(pts), m)
-    _check(feats.cpu().numpy(), ref_feats, "U-Net features")
+    parity.check("U-Net features, %d levels, m=%d, 6000 voxels" % (levels, m), feats.cpu().numpy(), ref_feats, ref64)
     w, b = model.linear.weight.detach().cpu().numpy(), model.linear.bias.detach().cpu().numpy()
-    _check(logits.cpu().numpy(), ref_feats @ w.T + b, "logits")
+    parity.check("logits, %d levels" % levels, logits.cpu().numpy(), ref_feats @ w.T + b,
+                 ref64 @ w.T.astype(np.float64) + b)
 
 
 def test_unet_is_deterministic():
