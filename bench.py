@@ -165,6 +165,11 @@ def conv_roofline(device, reps=200, warm=300):
     return {
         "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
         "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
+        "bound_in_practice": "mfma issue: `achieved` counts ALGORITHMIC bytes (every gathered row once per rule); the L2 "
+                             "serves most of that reuse, so the HBM itself moves `traffic` bytes per launch "
+                             "(hbm_GB/s_on_traffic), and what the kernel waits for is matrix-core issue (mfma_frac)",
+        "hbm_GB/s_on_traffic": round(traffic / t / 1e9, 1) if traffic else None,
+        "hbm_frac_on_traffic": round(traffic / t / 1e9 / HBM_PEAK_GBS, 4) if traffic else None,
         "kernel": "conv_wlds_kernel (SSC 3^3, 32->32, filter in LDS, persistent blocks; 500k sites, %d rules)" % n_rules,
         "avg_us": round(t * 1e6, 1), "algorithmic_bytes": int(bytes_alg),
         "traffic_note": traffic_note,
@@ -173,7 +178,7 @@ def conv_roofline(device, reps=200, warm=300):
     }
 
 
-def wide_conv_row(device, C=64, reps=20, warm=60):
+def wide_conv_row(device, C=64, reps=40, warm=60):
     """The 64-channel submanifold convolution of workload 3 (500k voxels), which is bound by the
     matrix cores rather than by HBM: us per launch and the fraction of the fp32 MFMA peak."""
     import torch
@@ -186,7 +191,14 @@ def wide_conv_row(device, C=64, reps=20, warm=60):
     sc = m.ssc_rulebook(x.spatial_size)
     out = torch.empty((sc.n, conv.nOut), device=device)
     plan = m.ssc_plan(sc)
+    # (warm-up on another kernel that computes the same layer - the weight-sharing kernel switched off - so
+    # that a profiler's table for conv_wshare_kernel holds the timed launches and five before them only)
+    from sparseconvnet._lib import lib
+    lib.insc_conv_set_shared_weights_min_units(1 << 40)
     for _ in range(warm):
+        SCN.ssc_rows_planned(x.features, out, conv.weight, None, sc, plan)
+    lib.insc_conv_set_shared_weights_min_units(896)
+    for _ in range(5):
         SCN.ssc_rows_planned(x.features, out, conv.weight, None, sc, plan)
     torch.cuda.synchronize()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -204,10 +216,64 @@ def wide_conv_row(device, C=64, reps=20, warm=60):
             "GB/s_on_algorithmic_bytes": round(bytes_alg / t / 1e9, 1)}
 
 
+def split_layer_row(device, C=96, shift=2, reps=200, warm=200):
+    """The kernel the incremental frame spends most of its time in - conv_mfma_kernel<1, 27, 0, 4>,
+    the items of a 32-row tile dealt to four wavefronts - on the layer it serves most often: 3^3,
+    96 -> 96 channels, at the third scale of the 150 000-voxel scene (10 414 sites), alone in a loop.
+    Useful and issued flops against the fp32 MFMA peak."""
+    import numpy as np
+    import torch
+
+    import sparseconvnet as scn
+    from sparseconvnet import SCN
+    from workloads import scenes
+
+    _, _, vox = scenes.unet_scene()
+    coarse = vox.copy()
+    coarse[:, :3] >>= shift
+    _, first = np.unique(coarse, axis=0, return_index=True)
+    coarse = coarse[np.sort(first)]
+    size = torch.LongTensor([4096 >> shift] * 3)
+    rng = np.random.default_rng(7)
+    f = torch.from_numpy(rng.normal(size=(len(coarse), C)).astype(np.float32)).to(device)
+    x = scn.InputLayer(3, size, mode=4)([torch.from_numpy(coarse[:, :3].astype(np.int64)), f, 1])
+    m = x.metadata
+    sc = m.ssc_rulebook(size)
+    plan = m.ssc_plan(sc)
+    w = torch.from_numpy((rng.normal(size=(27, C, C)) * (2.0 / C / 27) ** 0.5).astype(np.float32)).to(device)
+    out = torch.empty((sc.n, C), device=device)
+    for _ in range(warm):
+        SCN.ssc_rows_planned(x.features, out, w, None, sc, plan)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        SCN.ssc_rows_planned(x.features, out, w, None, sc, plan)
+    e1.record()
+    torch.cuda.synchronize()
+    t = e0.elapsed_time(e1) * 1e-3 / reps
+    rules = m.n_ssc_rules(sc)
+    tiles = (sc.n + 31) // 32
+    tmask = plan[1][:tiles].cpu().numpy().astype(np.uint32)
+    slots = 32 * int(sum(bin(int(v)).count("1") for v in tmask))
+    useful, issued = 2.0 * rules * C * C, 2.0 * slots * C * C
+    return {"kernel": "conv_mfma_kernel<1, 27, 0, 4> (SSC 3^3, %d->%d, one 32-row tile and output block per block of four "
+                      "wavefronts; %d sites = scale %d of the 150 000-voxel scene, %d rules, %d tiles)"
+                      % (C, C, sc.n, shift, rules, tiles),
+            "bound": "mfma", "avg_us": round(t * 1e6, 1), "unit": "TFLOP/s", "peak": MFMA_FP32_PEAK_TFLOPS,
+            "achieved": round(useful / t / 1e12, 2), "frac": round(useful / t / 1e12 / MFMA_FP32_PEAK_TFLOPS, 4),
+            "issued_tflops": round(issued / t / 1e12, 2),
+            "issued_frac": round(issued / t / 1e12 / MFMA_FP32_PEAK_TFLOPS, 4),
+            "rule_slot_fill": round(useful / issued, 3),
+            "offsets_used_per_tile": round(slots / 32.0 / tiles, 2),
+            "note": "alone in a loop, plain epilogue; inside a frame the same layer also adds the residual, applies the "
+                    "next batch norm and writes two outputs"}
+
+
 # ---------------------------------------------------------------------------------------------
 # the bandwidth-bound kernels of the path, one C call each, against the HBM roofline
 # ---------------------------------------------------------------------------------------------
-def kernel_table(device, reps=20):
+def kernel_table(device, reps=20, strict=True):
     """us per call, achieved GB/s on ALGORITHMIC bytes and fraction of the HBM peak for the hash
     grid, the rulebooks, batch norm and the input/output layers, on the workload-2 scene (200k
     voxels, 1024^3, plus 10 % repeated points) and, for the feature kernels, 500k x 32 floats."""
@@ -267,8 +333,15 @@ def kernel_table(device, reps=20):
 
     rows = []
     # HBM bytes per call from the counter summary of this very table (FETCH_SIZE + WRITE_SIZE, calibrated)
-    recs = profile_records("path_kernels_cfg2.txt") or []
-    traffic = {r["row"]: float(r["fetch_bytes"]) + float(r["write_bytes"]) for r in recs if "row" in r}
+    recs = profile_records("path_kernels_cfg2.txt")
+    traffic = {r["row"]: float(r["fetch_bytes"]) + float(r["write_bytes"]) for r in recs or [] if "row" in r}
+    if recs is not None and strict:  # (--kernels-only, the run a summary is cut from, passes strict=False)
+        # a summary that lacks a row, or holds a zero for it (a kernel renamed since the summary was cut),
+        # must not pass for a measurement
+        for key in ("insert", "query", "ssc", "down", "bn", "input", "output", "labels"):
+            if not traffic.get(key, 0.0) > 0.0:
+                raise SystemExit("bench.py: profiles/path_kernels_cfg2.txt holds no (or a zero) TRAFFIC record for row "
+                                 "'%s': regenerate the summary" % key)
 
     def add(name, sec, nbytes, note, key=None):
         gbs = nbytes / sec / 1e9
@@ -334,11 +407,16 @@ def kernel_table(device, reps=20):
 # ---------------------------------------------------------------------------------------------
 # workloads 4 and 5: the U-Net of the reference's example, through the network executor
 # ---------------------------------------------------------------------------------------------
-def unet_model(device):
-    import sparseconvnet as scn
+def unet_only(device):
     from workloads.netdefs import NaiveUNet
 
-    model = NaiveUNet(m=32, levels=7, seed=4).to(device)
+    return NaiveUNet(m=32, levels=7, seed=4).to(device)
+
+
+def unet_model(device):
+    import sparseconvnet as scn
+
+    model = unet_only(device)
     return model, scn.compile(model.sparseModel, capacity_sites=1 << 18)
 
 
@@ -370,6 +448,104 @@ def residual_row(model, seq, frames, last, device):
                                    % (len(seq[last][0]), rnet.sites_per_level()[0])}
 
 
+def time_sweep(call, frames, first):
+    """Frame 0 as a full forward, frames 1 .. first-1 untimed, the rest timed back to back with one
+    synchronisation per frame.  `call(frame, increment)` runs one frame including the classifier.
+    Returns (per-frame ms of the timed frames, their total in seconds)."""
+    import torch
+
+    with torch.no_grad():
+        call(frames[0], False)
+        for f in range(1, first):
+            call(frames[f], True)
+        torch.cuda.synchronize()
+        per_frame = []
+        t0 = time.perf_counter()
+        for f in range(first, len(frames)):
+            t1 = time.perf_counter()
+            call(frames[f], True)
+            torch.cuda.synchronize()
+            per_frame.append((time.perf_counter() - t1) * 1e3)
+        dt = time.perf_counter() - t0
+    return per_frame, dt
+
+
+def to_host_long(pts, rgb, device):
+    """A frame as the reference's callers hand it over (ioLayers.py:52-69): coordinates as a CPU
+    LongTensor [P,3], features on the GPU, batch size 1."""
+    import numpy as np
+    import torch
+
+    return [torch.from_numpy(pts[:, :3].astype(np.int64)), torch.from_numpy(rgb).to(device), 1]
+
+
+def target_frame_rows(model, net, device, reps=10):
+    """The frame the latency target is stated on: a full forward over the first 145 000 voxels of the
+    room (untimed), then ONE incremental frame of 5 000 new voxels + 1 500 re-observed ones (timed,
+    classifier included); median of `reps` such pairs.  Once with the re-observed voxels drawn from
+    the whole scene (as in the sweep) and once from the part of the scene nearest the new voxels."""
+    import numpy as np
+    import torch
+
+    from workloads import scenes
+
+    out = {}
+    for key, old_from in (("frame_5k_on_150k_ms", "scene"), ("frame_5k_on_150k_frontier_ms", "frontier")):
+        (p0, c0), (p1, c1) = scenes.target_frame(old_from=old_from)
+        base, frame = to_dev(p0, c0, device), to_dev(p1, c1, device)
+        ts = []
+        with torch.no_grad():
+            for _ in range(reps + 2):
+                net(base, increment=False)
+                torch.cuda.synchronize()
+                t1 = time.perf_counter()
+                model.linear(net(frame, increment=True))
+                torch.cuda.synchronize()
+                ts.append((time.perf_counter() - t1) * 1e3)
+        if net.n_sites != 150000:
+            sys.exit("bench.py: the target frame ended on %d voxels, not 150 000" % net.n_sites)
+        out[key] = round(float(np.median(ts[2:])), 3)
+        if old_from == "scene":
+            out["frame_5k_on_150k_dirty_rows"] = [
+                {"scale": l, "sites": int(net.sites_per_level()[l]), "min": min(r for _, r in sets),
+                 "max": max(r for _, r in sets)} for l, sets in enumerate(net.dirty_rows()) if sets]
+            out["frame_5k_on_150k_work"] = frame_work_summary(net, out[key])
+    out["frame_5k_on_150k_note"] = ("full forward over 145 000 voxels (untimed), then one incremental frame of 5 000 new "
+                                    "voxels + 1 500 re-observed voxels (6 500 points), classifier included; median of %d; "
+                                    "'_frontier': the re-observed voxels come from the 10 %% of the scene nearest the new "
+                                    "ones instead of from anywhere in it" % reps)
+    return out
+
+
+def frame_work_summary(net, frame_ms):
+    """Flop accounting of the frame the executor ran last (insc_net_frame_work): useful flops =
+    2 * rules * Cin * Cout summed over its convolutions, issued = 2 * 32 * (offsets used per 32-row
+    tile) * Cin * Cout (what the matrix cores are handed, empty rule slots included; the 3-channel
+    stem runs on the vector units and counts as issued = useful), both over the whole frame's
+    wall time against the fp32 MFMA peak."""
+    useful = issued = 0.0
+    by_scale = {}
+    for w in net.frame_work():
+        u = 2.0 * w["rules"] * w["cin"] * w["cout"]
+        up32 = lambda c: (c + 31) // 32 * 32
+        i = 2.0 * w["slots"] * up32(w["cin"]) * up32(w["cout"]) if w["cin"] >= 16 else u
+        useful += u
+        issued += i
+        b = by_scale.setdefault(w["level"], [0.0, 0.0, 0])
+        b[0] += u
+        b[1] += i
+        b[2] += 1
+    t = frame_ms * 1e-3
+    return {"useful_gflop": round(useful / 1e9, 2), "issued_gflop": round(issued / 1e9, 2),
+            "useful_tflops": round(useful / t / 1e12, 2), "issued_tflops": round(issued / t / 1e12, 2),
+            "useful_frac_of_fp32_mfma_peak": round(useful / t / 1e12 / MFMA_FP32_PEAK_TFLOPS, 4),
+            "issued_frac_of_fp32_mfma_peak": round(issued / t / 1e12 / MFMA_FP32_PEAK_TFLOPS, 4),
+            "rule_slot_fill": round(useful / issued, 3) if issued else None,
+            "by_scale": [{"scale": l, "convolutions": b[2], "useful_gflop": round(b[0] / 1e9, 2),
+                          "issued_gflop": round(b[1] / 1e9, 2)} for l, b in sorted(by_scale.items())],
+            "note": "whole frame: structure, dirty sets, all layers and the classifier are inside the time"}
+
+
 def to_dev(pts, rgb, device):
     import numpy as np
     import torch
@@ -398,7 +574,9 @@ def cpu_baseline_unet():
     return {
         "value": round(dt * 1e3, 1), "unit": "ms/frame", "cores": orc.num_threads(), "kind": "port",
         "sample": "one full U-Net forward (rulebooks + 53 SSC + 6 conv + 6 deconv + 65 BN) over the final "
-                  "150k-voxel scene of the sweep, 165k points; the reference CPU path has no incremental mode",
+                  "150k-voxel scene of the sweep, 165k points; the reference CPU path has no incremental mode.  "
+                  "A port, not the reference's speed: the per-offset contraction is a plain OpenMP loop nest where "
+                  "the reference calls at::mm (CPU/Convolution.cpp:131-147)",
     }
 
 
@@ -628,6 +806,8 @@ def main():
                     help="run only the dominant-kernel measurement (short; used under rocprofv3)")
     ap.add_argument("--wide-only", action="store_true",
                     help="run only the 64-channel layer at 500k voxels (short; used under rocprofv3)")
+    ap.add_argument("--split-only", action="store_true",
+                    help="run only the 96-channel layer at the third scale of the U-Net scene (short; used under rocprofv3)")
     ap.add_argument("--no-extras", action="store_true",
                     help="skip the roofline, wide-layer and kernel-table rows (used under rocprofv3)")
     args = ap.parse_args()
@@ -643,7 +823,7 @@ def main():
     torch.cuda.set_device(device)
 
     if args.kernels_only:
-        print(json.dumps({"kernels": kernel_table(device)}))
+        print(json.dumps({"kernels": kernel_table(device, strict=False)}))
         return
     if args.residual_only:
         from workloads import scenes
@@ -655,6 +835,9 @@ def main():
         return
     if args.wide_only:
         print(json.dumps({"wide_layer": wide_conv_row(device)}))
+        return
+    if args.split_only:
+        print(json.dumps({"split_layer": split_layer_row(device)}))
         return
     if args.roofline_only:
         # plus a plain copy of known size (500k x 32 floats: 64 MB read, 64 MB written), the
@@ -682,32 +865,35 @@ def main():
                      "scene must have grown to 150k voxels): need 1 <= steps <= 40 and warmup + steps <= %d"
                      % (n_inc, n_inc))
         first = n_inc - K + 1  # first timed frame; frames 1 .. first - 1 (at least W of them) are untimed
+        import sparseconvnet as scn
+
         model, net = unet_model(device)
         frames = [to_dev(p, c, device) for p, c in seq]
-        with torch.no_grad():
-            # the logits of a frame's points = Linear(features of those points)
-            net(frames[0], increment=False)
-            for f in range(1, first):
-                model.linear(net(frames[f], increment=True))
-            torch.cuda.synchronize()
-            sites_at_start = net.n_sites
-            per_frame = []
-            t0 = time.perf_counter()
-            for f in range(first, n_inc + 1):
-                t1 = time.perf_counter()
-                model.linear(net(frames[f], increment=True))
-                torch.cuda.synchronize()
-                per_frame.append((time.perf_counter() - t1) * 1e3)
-            dt = time.perf_counter() - t0
+        # the logits of a frame's points = Linear(features of those points)
+        per_frame, dt = time_sweep(lambda x, inc: model.linear(net(x, increment=inc)), frames, first)
         if net.n_sites != 150000:
             sys.exit("bench.py: the sweep ended on %d voxels, not on the 150 000 the metric names" % net.n_sites)
+        seen = np.unique(np.concatenate([p for p, _ in seq[:first]]), axis=0)
+        sites_at_start = int(len(seen))
+        new_per_frame = []
+        have = set(map(tuple, seen[:, :3].tolist()))
+        for f in range(first, n_inc + 1):
+            pts = set(map(tuple, seq[f][0][:, :3].tolist()))
+            new_per_frame.append(len(pts - have))
+            have |= pts
         ms = dt * 1e3 / K
         value, metric, unit, hib = round(ms, 3), "incremental frame latency ms (UNet, 150k vox)", "ms", False
         config = {"workload": "cfg5: the last %d incremental U-Net frames (%d..%d) of the 50-frame sweep (m=32, 7 "
                               "levels, InputLayer mode 4 .. OutputLayer + Linear(32,20)); frames 0..%d untimed; the "
-                              "scene grows from %d to 150 000 voxels over the timed frames"
-                              % (K, first, n_inc, first - 1, sites_at_start),
+                              "scene grows from %d to 150 000 voxels over the timed frames.  The sweep's draws of "
+                              "3k-8k new voxels per frame are scaled so that 50 frames end on 150 000 voxels: a "
+                              "timed frame really adds %d-%d new voxels (mean %d) plus 1k-2k re-observed ones; "
+                              "the frame the latency target names (5 000 new voxels onto a scene that then has "
+                              "150 000) is measured separately: frame_5k_on_150k_ms"
+                              % (K, first, n_inc, first - 1, sites_at_start, min(new_per_frame), max(new_per_frame),
+                                 int(np.mean(new_per_frame))),
                   "points_per_frame_mean": int(np.mean([len(seq[f][0]) for f in range(first, n_inc + 1)])),
+                  "new_voxels_per_frame_mean": int(np.mean(new_per_frame)),
                   "points_last_frame": int(len(seq[n_inc][0])),
                   "sites_at_start": sites_at_start, "sites_at_end": net.n_sites,
                   "order_refresh": "library default: an incremental frame re-sorts the processing orders of its "
@@ -724,6 +910,56 @@ def main():
         extra["dirty_rows_last_frame"] = [
             {"scale": l, "sites": int(sites[l]), "min": min(r for _, r in sets), "max": max(r for _, r in sets)}
             for l, sets in enumerate(net.dirty_rows()) if sets]
+        # flop accounting of the last timed frame against the fp32 MFMA peak (the frame is bound by
+        # matrix-core issue at the coarse scales, not by HBM)
+        extra["frame"] = frame_work_summary(net, per_frame[-1])
+        if not args.no_extras:
+            # (a) the same frames through the reference's own call path: model(x, increment) on the module
+            # tree with CPU int64 coordinates (model.py:23-26, ioLayers.py:52-69); the whole-network
+            # Sequential hands them to the executor by itself.  (b) the explicit executor fed the same
+            # host coordinates.  (c) the module tree layer by layer (one C call per layer from Python).
+            hframes = [to_host_long(p, c, device) for p, c in seq]
+            model_b = unet_only(device)
+            pf, _ = time_sweep(lambda x, inc: model_b(x, increment=inc), hframes, first)
+            extra["module_api_frame_ms"] = round(float(np.mean(pf)), 3)
+            extra["module_api_frame_at_150k_ms"] = round(pf[-1], 3)
+            if model_b.sparseModel.why_not_compiled() is not None or "_exec" not in model_b.sparseModel.__dict__:
+                sys.exit("bench.py: the module path did not reach the executor: %s" % model_b.sparseModel.why_not_compiled())
+            pf, _ = time_sweep(lambda x, inc: model.linear(net(x, increment=inc)), hframes, first)
+            extra["executor_cpu_coords_frame_ms"] = round(float(np.mean(pf)), 3)
+            prev = scn.set_auto_compile(False)
+            try:
+                model_c = unet_only(device)
+                pf, _ = time_sweep(lambda x, inc: model_c(x, increment=inc), hframes, first)
+            finally:
+                scn.set_auto_compile(prev)
+            extra["module_api_layer_by_layer_frame_ms"] = round(float(np.mean(pf)), 3)
+            extra["module_api_note"] = ("the same %d frames, mean ms per frame, classifier included: module_api = "
+                                        "model([coords int64 on the HOST [P,3], features on the GPU, 1], increment) on "
+                                        "the module tree, as a user of the reference calls it (the Sequential traces "
+                                        "itself into the executor at its first frame); executor_cpu_coords = the explicit "
+                                        "scn.compile() object fed the same host coordinates; layer_by_layer = the module "
+                                        "tree with the executor switched off (one C call per layer from Python); "
+                                        "`value` = the executor fed int32 device coordinates" % K)
+            del model_b, model_c
+            # (d) full forward over the whole 150k-voxel scene (workload 4), same executor: what a frame
+            # costs without the incremental path
+            pts4, rgb4, _ = scenes.unet_scene()
+            x4 = to_dev(pts4, rgb4, device)
+            with torch.no_grad():
+                for _ in range(3):
+                    model.linear(net(x4, increment=False))
+                torch.cuda.synchronize()
+                t1 = time.perf_counter()
+                for _ in range(10):
+                    model.linear(net(x4, increment=False))
+                torch.cuda.synchronize()
+                extra["full_forward_ms"] = round((time.perf_counter() - t1) * 100.0, 3)
+            extra["full_forward_note"] = ("full U-Net forward over the 150 000-voxel scene (165 000 points), mean of 10: an "
+                                          "incremental frame of this sweep dirties every row from the second scale on, so "
+                                          "it saves the structure phase and part of the input scale, not the layers")
+            # (e) the frame the latency target is stated on
+            extra.update(target_frame_rows(model, net, device))
         if not args.no_residual:
             extra.update(residual_row(model, seq, frames, n_inc, device))
         cpu_fn = cpu_baseline_unet
@@ -803,6 +1039,8 @@ def main():
     if not args.no_extras:
         out["roofline"] = conv_roofline(device)
         out["wide_layer"] = wide_conv_row(device)
+        if args.workload in ("incr", "unet"):
+            out["split_layer"] = split_layer_row(device)
         out["kernels"] = kernel_table(device)
     # the CPU leg comes last: the GPU idles during it, and a measurement taken right after would
     # start at idle clocks

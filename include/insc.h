@@ -339,14 +339,16 @@ int insc_net_enable_residual(insc_net *net);
  * depend on the order.  Default 10; 0: never.  No counterpart in the reference, which rebuilds
  * its rulebooks on every call. */
 int insc_net_set_order_refresh(insc_net *net, int percent);
-/* Re-pack the weights after the caller changed them in place. */
+/* Re-pack the weights after the caller changed them in place.  The rows cached by earlier frames
+ * were computed with the old parameters and are forgotten: the next frame must be a full one
+ * (an incremental or residual frame before it returns INSC_ERR_STATE). */
 int insc_net_refresh_weights(insc_net *net, void *stream);
 /* Ops added so far (joins included); the op added last has index insc_net_op_count() - 1. */
 int insc_net_op_count(const insc_net *net);
 /* Point op `op` at parameters that moved (e.g. the caller's framework re-allocated them when a
  * checkpoint was restored): d_W / d_bias for a convolution op, d_mean / d_var / d_gamma / d_beta for
  * a batch norm; same shapes as when the op was added.  Follow with insc_net_refresh_weights.
- * No counterpart in the reference, whose modules pass their tensors on every call. */
+ * Like that call it forgets the cached state of earlier frames.  No counterpart in the reference, whose modules pass their tensors on every call. */
 int insc_net_rebind_op(insc_net *net, int op, const float *d_W, const float *d_bias, const float *d_mean,
                        const float *d_var, const float *d_gamma, const float *d_beta);
 /* One frame: d_coords int32 [P,coord_cols] (x,y,z[,batch]), d_feats float32 [P,in_channels].
@@ -354,8 +356,11 @@ int insc_net_rebind_op(insc_net *net, int op, const float *d_W, const float *d_b
  * and recomputes only the rows they affect.  d_out (nullable) receives one row of the output
  * tensor per point of this frame (out_all == 0) or per point since the last full frame.
  * Returns once the frame is enqueued on `stream` (the host has waited for the site counts of the
- * frame's insert by then, nothing else); d_out and the state are ready in stream order.  A frame is all or nothing: if any of its coordinates is
- * outside the representable range the call returns INSC_ERR_COORD and the state is that of the
+ * frame's insert by then, nothing else); d_out and the state are ready in stream order, and
+ * d_coords, d_feats and d_out must stay valid - the two inputs unmodified - until the stream has
+ * reached the end of the frame (kernels that read them may still be running when the call
+ * returns; work enqueued on the same stream afterwards is ordered behind them).
+ * A frame is all or nothing: if any of its coordinates is outside the representable range the call returns INSC_ERR_COORD and the state is that of the
  * previous frame (after a full frame that failed: no state; the next frame must be a full one). */
 int insc_net_forward(insc_net *net, const int32_t *d_coords, int coord_cols, const float *d_feats, int64_t P,
                      int increment, float *d_out, int out_all, int64_t *h_n_sites, void *stream);
@@ -374,6 +379,15 @@ int insc_net_dirty_counts(insc_net *net, int max_sets, int *h_n_sets, int *h_lev
  * Returns once the frame's site counts are known; the layers may still be running on the stream. */
 int insc_net_forward_residual(insc_net *net, const int32_t *d_coords, int coord_cols, const float *d_feats, int64_t P,
                               float *d_out, int64_t *h_n_sites, void *stream);
+/* What every convolution of the last completed frame worked on (diagnostics for flop accounting; the
+ * reference's operators return their multiply-add count instead, e.g. CUDA/Convolution.cpp:152-218).
+ * For convolution i in program order (i < *h_n_ops <= max_ops): h_kind[i] (0 3^3 submanifold,
+ * 2 strided, 3 transposed, 4 1x1), h_level[i] = scale of its output, h_cin[i], h_cout[i], and over
+ * the 32-row tiles it computed in that frame h_rows[i] = output rows, h_rules[i] = rules,
+ * h_slots[i] = 32 x offsets used per tile.  Useful multiply-adds = rules x Cin x Cout; the matrix
+ * cores are issued slots x Cin x Cout.  Synchronises. */
+int insc_net_frame_work(insc_net *net, int max_ops, int *h_n_ops, int *h_kind, int *h_level, int *h_cin, int *h_cout,
+                        int64_t *h_rows, int64_t *h_rules, int64_t *h_slots, void *stream);
 int insc_net_tensor_view(insc_net *net, int tensor, float **d_ptr, int64_t *ld, int64_t *rows, int *channels);
 int insc_net_counts(insc_net *net, int64_t *h_sites_per_level, int64_t *h_points);
 /* Phase timing (the reference brackets the same phases with easy_profiler blocks,

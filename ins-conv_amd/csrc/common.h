@@ -35,8 +35,9 @@ int hip_fail(hipError_t e, const char *what, const char *file, int line);
 // Arena 0 belongs to the scan primitive, arena 1 to the sort primitive, arena 2 to the
 // API-level function that is running (none of which calls another arena-2 user; the convolution
 // launcher packs weights there when the caller brings none), arena 5 to the residual-frame
-// operators, which call that launcher.
-enum { WS_SCAN = 0, WS_SORT = 1, WS_API = 2, WS_CONV = 3, WS_LABELS = 4, WS_INCRE = 5 };
+// operators, which call that launcher, arena 6 to the flag and count words of
+// insc_grid_insert_scales (whose helpers use arenas 0-2).
+enum { WS_SCAN = 0, WS_SORT = 1, WS_API = 2, WS_CONV = 3, WS_LABELS = 4, WS_INCRE = 5, WS_INSERT = 6 };
 int workspace(int which, hipStream_t stream, size_t bytes, void **out);
 int device_cus();
 // `count` int32 counters per (device, stream), zero at kernel start; users leave them at zero
@@ -112,6 +113,7 @@ struct TilePlan {
   int64_t ld = 0;
   const uint32_t *tmask = nullptr;
   const int32_t *sched = nullptr;  // [ld / 32] tiles by falling cost, or null
+  unsigned cus = 256;              // compute units of the device (launch_conv fills it in)
 };
 int build_tile_plan(const int32_t *nbr, const int32_t *order, const int32_t *d_n, int64_t n_rows, int64_t ld,
                     int32_t *map, uint32_t *tmask, int32_t *sched, hipStream_t s);

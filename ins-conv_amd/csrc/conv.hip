@@ -252,7 +252,7 @@ __global__ __launch_bounds__((S == 1 ? CONV_WAVES : S) * 64) void conv_mfma_kern
   // that drew the most expensive block of one turn gets the cheapest of the next.
   unsigned bx = blockIdx.x, by = blockIdx.y, bz = blockIdx.z;
   if (S > 1 && MODE == MAP_NBR && K == 27 && plan.map != nullptr && plan.sched != nullptr) {
-    constexpr unsigned CUS = 256;
+    const unsigned CUS = plan.cus;
     const unsigned gyz = gridDim.y * gridDim.z;
     const unsigned total = (unsigned)((n + TILE_M - 1) / TILE_M) * gyz;
     const unsigned L = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
@@ -539,14 +539,28 @@ __global__ __launch_bounds__((S == 1 ? CONV_WAVES : S) * 64) void conv_mfma_kern
       // (stores and loads of the sums go past the XCD-local L2 - device-scope atomics - so that no
       // cache write-back or invalidation is needed: a full fence flushes the whole L2 and costs
       // more than the layer)
+      // Why the last arrival sees every sum.  (1) The sums are written with agent-scope atomic stores:
+      // on this part such a store is not kept in the writer's XCD-local L2 but written through to the
+      // level all XCDs share, and it is acknowledged from there.  (2) vmcnt(0) makes the wavefront wait
+      // for those acknowledgements before it issues the counter's read-modify-write, which is performed
+      // at that same shared level: a wavefront's increment is ordered after its own sums.  (3) The
+      // wavefront that reads GZ - 1 back has therefore been preceded by all other increments, hence by
+      // all other sums.  (4) Its loads below are issued only after that value has returned (the branch
+      // depends on it; wavefronts issue in order) and are agent-scope atomic loads, which do not hit a
+      // stale line of the reader's own L2.  The compiler fences pin the program order this relies on
+      // (they emit no instructions).  An acquire/release pair at agent scope would say the same in the
+      // language's terms but writes back and invalidates the whole L2.
       const int unit = (int)(bx * gridDim.y + by);
       float *mine = part + ((int64_t)unit * GZ + bz) * 1024 + (wave * NV) * 64 + lane;
 #pragma unroll
       for (int j = 0; j < NV; j++) __hip_atomic_store(mine + j * 64, a[j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __atomic_signal_fence(__ATOMIC_SEQ_CST);
       __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the stores have been acknowledged
+      __atomic_signal_fence(__ATOMIC_SEQ_CST);
       int old = 0;
       if (lane == 0) old = atomicAdd(pcount + unit * S + wave, 1);
       if (__builtin_amdgcn_readfirstlane(old) != GZ - 1) return;
+      __atomic_signal_fence(__ATOMIC_SEQ_CST);
       const float *all = part + (int64_t)unit * GZ * 1024 + (wave * NV) * 64 + lane;
       // (the sums of eight blocks at a time are requested together and added in block order: one trip
       // to memory per eight blocks instead of one per block)
@@ -1978,6 +1992,7 @@ int launch_conv(const float *in, int64_t ld_in, int64_t in_rows, float *out, int
   if (expect_rows <= 0 || expect_rows > n_rows) expect_rows = n_rows;
   if (plan.map && (mode != MAP_NBR || K != 27 || plan.ld * 27 * 4 >= (int64_t)BUF_OOB || plan.ld < cdiv(n_rows, TILE_M) * TILE_M))
     plan = TilePlan();  // only the 3^3 map has a plan; an unusable one is ignored
+  plan.cus = (unsigned)device_cus();
   if (conv_uses_mfma(in, ld_in, Cin, K)) {
     // the gather addresses rows with 32-bit byte offsets (buffer loads)
     const int64_t in_bytes64 = in_rows * ld_in * 4, wp_bytes64 = packed_floats(K, Cin, Cout) * 4;

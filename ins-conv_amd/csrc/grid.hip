@@ -1478,7 +1478,7 @@ int insc_grid_insert_scales(insc_grid *const *grids, int32_t *const *d_parent, i
   if (P > 0) {
     // the flag "some coordinate is bad" and the counts the kernels leave: 2 * scales + 2 words
     void *ws;
-    int rc = workspace(WS_SORT, s, 64 * sizeof(int32_t), &ws);
+    int rc = workspace(WS_INSERT, s, 64 * sizeof(int32_t), &ws);
     if (rc) return rc;
     int32_t *d_bad = (int32_t *)ws, *d_counts = d_bad + 1;
     INSC_HIP(hipMemsetAsync(d_bad, 0, sizeof(int32_t), s));

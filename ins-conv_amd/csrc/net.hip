@@ -123,6 +123,7 @@ struct ResidualFrame {
 struct insc_net {
   int n_levels = 0, in_channels = 0, mode = 4;
   bool finalized = false, have_state = false;
+  bool last_inc = false;  // the last completed frame was an incremental one (its dirty flags are still in place)
   bool keep_raw = false;  // keep the input of every batch norm (residual frames read it)
   int order_refresh_pct = 10;  // an incremental frame re-sorts the orders once this share of a large scale is appended (0: never)
   insc::ResidualFrame rf;
@@ -659,6 +660,53 @@ static int run_dirty_node(insc_net *net, int id, hipStream_t s) {
   return INSC_OK;
 }
 
+
+// What one convolution of the last frame worked on (diagnostics): one wavefront per 32-row tile of the
+// layer's processing order (or of its list of dirty rows).  For the tiles the layer computed:
+// acc[0] += output rows, acc[1] += rules (existing (row, offset) pairs), acc[2] += 32 x offsets the
+// tile uses (the (row, offset) slots the matrix cores are issued work for, empty ones included).
+__global__ __launch_bounds__(256) void conv_work_kernel(const int32_t *__restrict__ map0, const int32_t *__restrict__ map1,
+                                                        int mode, int K, const int32_t *__restrict__ rows,
+                                                        const int32_t *__restrict__ d_n, int64_t n_rows,
+                                                        const uint8_t *__restrict__ tile_flags,
+                                                        unsigned long long *__restrict__ acc) {
+  const int64_t n = d_n ? min((int64_t)*d_n, n_rows) : n_rows;
+  const int64_t t = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (t * 32 >= n) return;
+  if (tile_flags && !tile_flags[t]) return;
+  const int64_t p = t * 32 + (lane & 31);
+  unsigned bits = 0;
+  int rules = 0, valid = 0;
+  if (lane < 32 && p < n) {
+    const int64_t row = rows ? rows[p] : p;
+    valid = 1;
+    if (mode == MAP_NBR) {
+      for (int k = 0; k < K; k++)
+        if (map0[row * K + k] >= 0) {
+          bits |= 1u << k;
+          rules++;
+        }
+    } else if (mode == MAP_PARENT) {
+      bits = 1u << map1[row];
+      rules = 1;
+    } else {
+      bits = 1u;
+      rules = 1;
+    }
+  }
+  for (int o = 32; o >= 1; o >>= 1) {
+    bits |= __shfl_xor(bits, o);
+    rules += __shfl_xor(rules, o);
+    valid += __shfl_xor(valid, o);
+  }
+  if (lane == 0) {
+    atomicAdd(acc + 0, (unsigned long long)valid);
+    atomicAdd(acc + 1, (unsigned long long)rules);
+    atomicAdd(acc + 2, (unsigned long long)(__popc(bits) * 32));
+  }
+}
+
 }  // namespace insc
 
 using namespace insc;
@@ -1016,9 +1064,12 @@ int insc_net_finalize(insc_net *net, int out_tensor, int64_t capacity_sites, voi
   return INSC_OK;
 }
 
-/* Re-pack the weights after the caller changed them in place. */
+/* Re-pack the weights after the caller changed them in place.  The rows cached by earlier frames were
+ * computed with the old parameters, so they are forgotten: the next frame must be a full one (an
+ * incremental or residual frame before it fails with INSC_ERR_STATE instead of mixing old and new rows). */
 int insc_net_refresh_weights(insc_net *net, void *stream) {
   INSC_REQUIRE(net && net->finalized, INSC_ERR_STATE, "insc_net_refresh_weights: net is not finalized");
+  net->have_state = false;
   for (Op &op : net->ops)
     if (op.Wp) {
       const int K = op.kind == OP_SSC ? 27 : op.kind == OP_NIN ? 1 : 8;
@@ -1040,6 +1091,7 @@ int insc_net_rebind_op(insc_net *net, int op, const float *d_W, const float *d_b
                        const float *d_var, const float *d_gamma, const float *d_beta) {
   INSC_REQUIRE(net && op >= 0 && op < (int)net->ops.size(), INSC_ERR_ARG, "insc_net_rebind_op: no op %d", op);
   Op &o = net->ops[op];
+  net->have_state = false;  // cached rows belong to the old parameters
   if (o.kind == OP_SSC || o.kind == OP_CONV || o.kind == OP_DECONV || o.kind == OP_NIN) {
     INSC_REQUIRE(d_W, INSC_ERR_ARG, "insc_net_rebind_op: op %d is a convolution and needs d_W", op);
     o.W = d_W;
@@ -1064,14 +1116,18 @@ int insc_net_rebind_op(insc_net *net, int op, const float *d_W, const float *d_b
  * d_out (nullable): one row of the output tensor per point - of this frame's points
  * (out_all == 0, [P,C]) or of every point since the last full frame (out_all != 0).
  * h_n_sites (nullable): receives the number of active sites at the input scale.
- * The call returns after the frame has completed (it reads the site counts back). */
+ * The call returns once the frame is ENQUEUED on `stream` (it waits only for the site counts of the
+ * structure phase).  d_coords, d_feats and d_out are read / written by kernels that may still be
+ * running when it returns: they must stay valid, and the inputs unmodified, until the stream has
+ * reached the end of the frame (work enqueued on the same stream afterwards is ordered behind it). */
 int insc_net_forward(insc_net *net, const int32_t *d_coords, int coord_cols, const float *d_feats, int64_t P,
                      int increment, float *d_out, int out_all, int64_t *h_n_sites, void *stream) {
   INSC_REQUIRE(net && net->finalized, INSC_ERR_STATE, "insc_net_forward: net is not finalized");
   INSC_REQUIRE(P >= 0 && (P == 0 || (d_coords && d_feats)) && (coord_cols == 3 || coord_cols == 4), INSC_ERR_ARG,
                "insc_net_forward: bad arguments");
   INSC_REQUIRE(!increment || net->have_state, INSC_ERR_STATE,
-               "insc_net_forward: incremental frame before any full frame");
+               "insc_net_forward: incremental frame without a full frame before it (none yet, or the weights "
+               "were rebound / refreshed since)");
   hipStream_t s = (hipStream_t)stream;
   const int L = net->n_levels;
   const int C0 = net->in_channels;
@@ -1347,6 +1403,7 @@ int insc_net_forward(insc_net *net, const int32_t *d_coords, int coord_cols, con
   }
   net->n_points += P;
   net->have_state = true;
+  net->last_inc = inc;
   if (net->profiling) INSC_HIP(hipEventRecord(net->ev[4], s));
   // (no wait here: the host has had the site counts since the structure phase, the output rows are ready in
   // stream order, and what the caller enqueues next - a classifier on d_out - follows without a gap)
@@ -1722,6 +1779,81 @@ int insc_net_dirty_counts(insc_net *net, int max_sets, int *h_n_sets, int *h_lev
   for (int i = 0; i < ns; i++)
     h_rows[i] = (i < (int)net->dirty_full.size() && net->dirty_full[(size_t)i]) ? net->levels[net->dirty[i].level].n
                                                                                 : (int64_t)h[(size_t)i];
+  return INSC_OK;
+}
+
+/* What every convolution of the last completed frame (insc_net_forward) worked on - diagnostics for
+ * the benchmark's flop accounting.  For convolution i in program order (i < *h_n_ops <= max_ops):
+ * h_kind[i] (0 3^3 submanifold, 2 strided, 3 transposed, 4 1x1), h_level[i] = scale of its output,
+ * h_cin / h_cout, and over the tiles it computed in that frame (all of them after a full frame, the
+ * flagged ones or the listed rows after an incremental one) h_rows[i] = output rows, h_rules[i] =
+ * rules, h_slots[i] = 32 x (offsets used per tile): useful multiply-adds = rules x Cin x Cout, the
+ * matrix cores are issued slots x Cin x Cout (Cin rounded up to 32).  Synchronises. */
+int insc_net_frame_work(insc_net *net, int max_ops, int *h_n_ops, int *h_kind, int *h_level, int *h_cin, int *h_cout,
+                        int64_t *h_rows, int64_t *h_rules, int64_t *h_slots, void *stream) {
+  INSC_REQUIRE(net && net->finalized && h_n_ops && h_kind && h_level && h_cin && h_cout && h_rows && h_rules && h_slots &&
+                   max_ops >= 0, INSC_ERR_ARG, "insc_net_frame_work: bad arguments");
+  INSC_REQUIRE(net->have_state, INSC_ERR_STATE, "insc_net_frame_work: no frame has run");
+  hipStream_t s = (hipStream_t)stream;
+  std::vector<const Op *> convs;
+  for (const Op &op : net->ops)
+    if (!op.fused && (op.kind == OP_SSC || op.kind == OP_CONV || op.kind == OP_DECONV || op.kind == OP_NIN))
+      convs.push_back(&op);
+  const int nc = std::min<int>(max_ops, (int)convs.size());
+  *h_n_ops = nc;
+  if (nc == 0) return INSC_OK;
+  void *ws;
+  int rc = workspace(WS_API, s, sizeof(unsigned long long) * 3 * (size_t)nc, &ws);
+  if (rc) return rc;
+  unsigned long long *acc = (unsigned long long *)ws;
+  INSC_HIP(hipMemsetAsync(acc, 0, sizeof(unsigned long long) * 3 * (size_t)nc, s));
+  for (int i = 0; i < nc; i++) {
+    const Op &op = *convs[(size_t)i];
+    const Tensor &To = net->tensors[op.out];
+    const Level &Lo = net->levels[To.level];
+    const DirtyNode *d = net->last_inc && !net->dirty_full[(size_t)To.dirty] ? &net->dirty[To.dirty] : nullptr;
+    h_kind[i] = op.kind;
+    h_level[i] = To.level;
+    h_cin[i] = op.Cin;
+    h_cout[i] = op.Cout;
+    if (Lo.n <= 0) continue;
+    const int32_t *map0 = nullptr, *map1 = nullptr, *rows = Lo.order, *d_n = Lo.grid->d_n;
+    const uint8_t *flags = d ? d->tflag : nullptr;
+    int mode = MAP_NBR, K = 27;
+    int64_t n = Lo.n;
+    if (op.kind == OP_SSC) {
+      map0 = Lo.nbr;
+      if (d && d->compact) {
+        rows = d->crows;
+        d_n = d->ccount;
+        flags = nullptr;
+      }
+    } else if (op.kind == OP_NIN) {
+      mode = MAP_IDENTITY;
+      K = 1;
+    } else if (op.kind == OP_CONV) {
+      map0 = net->levels[To.level - 1].child;
+      K = 8;
+    } else {
+      map0 = Lo.parent;
+      map1 = Lo.offset;
+      mode = MAP_PARENT;
+      K = 8;
+      rows = Lo.bo_order;
+      flags = d ? d->tflag_bo : nullptr;
+    }
+    hipLaunchKernelGGL(conv_work_kernel, dim3(grid_for(cdiv(n, 32), 4)), dim3(256), 0, s, map0, map1, mode, K, rows, d_n, n,
+                       flags, acc + 3 * i);
+    INSC_LAUNCH_CHECK();
+  }
+  std::vector<unsigned long long> h(3 * (size_t)nc);
+  INSC_HIP(hipMemcpyAsync(h.data(), acc, sizeof(unsigned long long) * h.size(), hipMemcpyDeviceToHost, s));
+  INSC_HIP(hipStreamSynchronize(s));
+  for (int i = 0; i < nc; i++) {
+    h_rows[i] = (int64_t)h[3 * (size_t)i];
+    h_rules[i] = (int64_t)h[3 * (size_t)i + 1];
+    h_slots[i] = (int64_t)h[3 * (size_t)i + 2];
+  }
   return INSC_OK;
 }
 

@@ -9,7 +9,7 @@ forward_pass_hidden_states = 0
 
 from .sparseConvNetTensor import SparseConvNetTensor  # noqa: E402
 from .metadata import Metadata  # noqa: E402
-from .sequential import Sequential  # noqa: E402
+from .sequential import Sequential, set_auto_compile, get_auto_compile  # noqa: E402
 from .tables import JoinTable, AddTable, ConcatTable, Identity  # noqa: E402
 from .ioLayers import InputLayer, OutputLayer  # noqa: E402
 from .submanifoldConvolution import SubmanifoldConvolution, ValidConvolution  # noqa: E402

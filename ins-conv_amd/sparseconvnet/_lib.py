@@ -79,6 +79,9 @@ _SIGS = {
     "insc_net_dirty_counts": [vp, c_int, ctypes.POINTER(c_int), ctypes.POINTER(c_int), ctypes.POINTER(c_int),
                               ctypes.POINTER(c_i64), vp],
     "insc_net_profile": [vp, c_int, ctypes.POINTER(ctypes.c_float)],
+    "insc_net_frame_work": [vp, c_int, ctypes.POINTER(c_int), ctypes.POINTER(c_int), ctypes.POINTER(c_int),
+                            ctypes.POINTER(c_int), ctypes.POINTER(c_int), ctypes.POINTER(c_i64), ctypes.POINTER(c_i64),
+                            ctypes.POINTER(c_i64), vp],
     "insc_labels_create": [c_i64, c_int, c_f32, ctypes.POINTER(vp)],
     "insc_labels_destroy": [vp],
     "insc_labels_clear": [vp, vp],

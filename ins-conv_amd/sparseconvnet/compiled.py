@@ -8,11 +8,14 @@
 The module path issues one C call per layer from Python; this path hands the whole frame to
 one C call, so an incremental frame costs a few hundred kernel launches and no Python work.
 Results are bit-identical to the module path.  Parameters are read in place (device
-pointers).  Whatever touches every parameter of the model - `.to()` / `.cpu()` + `.cuda()`
-(new storage), `load_state_dict` / `checkpoint_restore` (new values) - is noticed at the next
-call and the executor is pointed at the current tensors and re-packs its weights; after editing
-single parameters in place call `refresh()`.  JoinTable takes two inputs (the U-Net's skip
-connection); wider joins run on the module path only.
+pointers).  A parameter that moved (`.to()`, `.cpu()` + `.cuda()`) or changed through torch
+(`load_state_dict`, `checkpoint_restore`, `copy_`, an optimizer step: anything that bumps the
+tensor's version counter) is noticed at the next call: the executor is pointed at the current
+tensors, re-packs its weights and forgets the rows cached by earlier frames, so the next frame
+must be a full one (an incremental frame raises instead of mixing rows computed with old and
+new parameters).  Writes torch cannot see (a raw kernel on the parameter's memory) need
+`refresh()`.  JoinTable takes two inputs (the U-Net's skip connection); wider joins run on the
+module path only.
 """
 import ctypes
 
@@ -45,6 +48,7 @@ class CompiledNet(object):
         lib.insc_net_create(levels, int(self.in_channels), int(self.input_layer.mode), ctypes.byref(self.h))
         self._keep = []  # tensors whose storage the executor points into
         self._bound = []  # (op index, module) of every op with parameters
+        self._sig_tensors = None
         self._level = {0: 0}
         self._chan = {0: self.in_channels}
         x = 0
@@ -52,11 +56,12 @@ class CompiledNet(object):
             x = self._trace(m, x)
         self.out_tensor = x
         self.out_channels = self._chan[x]
+        self._n_points = 0  # points since the last full frame (rows of an all_points output)
         self.residual = bool(residual)
         if self.residual:
             lib.insc_net_enable_residual(self.h)
         lib.insc_net_finalize(self.h, int(x), I64(int(capacity_sites)), stream_ptr())
-        self._sig = self._signature(False)
+        self._sig = self._signature()
 
     def __del__(self):
         try:
@@ -97,17 +102,22 @@ class CompiledNet(object):
     def _bind_op(self, m):
         self._bound.append((int(lib.insc_net_op_count(self.h)) - 1, m))
 
-    def _signature(self, full):
-        """(address, version) of the bound tensors: all of them, or the first and last op's only."""
-        ops = self._bound if full or len(self._bound) < 2 else (self._bound[0], self._bound[-1])
-        return tuple((t.data_ptr(), t._version) for _, m in ops for t in self._params(m) if t is not None)
+    def _signature(self):
+        """(addresses, versions) of every tensor the ops read (some 330 for the 7-level U-Net).  The
+        tensor objects are looked up once per binding: torch moves and reloads parameters in place
+        (`.to()`, `load_state_dict`), which the address and the version counter show."""
+        ts = self._sig_tensors
+        if ts is None:
+            ts = self._sig_tensors = [t for _, m in self._bound for t in self._params(m) if t is not None]
+        return [t.data_ptr() for t in ts], [t._version for t in ts]
 
     def _rebind(self):
-        self._keep = []
+        keep, self._keep, self._sig_tensors = self._keep, [], None
         for op, m in self._bound:
             lib.insc_net_rebind_op(self.h, op, *[self._dev(t) for t in self._params(m)])
         lib.insc_net_refresh_weights(self.h, stream_ptr())
-        self._sig = self._signature(False)
+        self._sig = self._signature()
+        del keep  # (the old storages stayed alive until the executor stopped pointing at them)
 
     def _trace(self, m, x):
         import sparseconvnet as scn
@@ -165,26 +175,51 @@ class CompiledNet(object):
         """Point the executor at the model's current parameter tensors and re-pack the weights."""
         self._rebind()
 
+    def _coords(self, coords):
+        """int32 on the device.  The reference's callers pass int64 coordinates, on the host
+        (ioLayers.py:52-69 converts to a CPU LongTensor) or on the GPU (demo.py:20): narrowed on
+        the side where they are, so that the host-to-device copy carries half the bytes."""
+        if coords.dtype != torch.int32:
+            coords = coords.to(torch.int32)
+        return coords.to(self.device).contiguous()
+
+    def _changed(self):
+        """Whether a parameter moved or changed since the weights were packed.  Looked at AFTER a
+        frame has been enqueued - the walk over the tensors costs the host some 60 us, which the
+        GPU then spends on the frame instead of waiting for it; the stale pointers stay valid
+        memory because `_keep` holds the old storages."""
+        return self._signature() != self._sig
+
     def __call__(self, input, increment=False, all_points=None):
         coords, feats = input[0], input[1]
         from . import incremental
-        if self._signature(False) != self._sig:  # the model was moved or reloaded since the last call
-            self._rebind()
         if incremental.kind(increment) == "residual":
-            return self._residual(coords, feats)
+            out = self._residual(coords, feats)
+            if self._changed():
+                self._rebind()
+                raise RuntimeError("the model's parameters changed since the last full frame: run a full frame "
+                                   "(increment=False) before the next residual frame")
+            return out
         increment = bool(increment)
         if all_points is None:
             all_points = (not increment) or self.output_layer.all_points
-        c = coords.to(device=self.device, dtype=torch.int32).contiguous()
+        c = self._coords(coords)
         f = feats.detach().to(device=self.device, dtype=torch.float32).contiguous()
         P = c.size(0)
-        n_pts = I64(0)
-        lib.insc_net_counts(self.h, None, ctypes.byref(n_pts))
-        rows = (n_pts.value if increment else 0) + P if all_points else P
+        rows = (self._n_points if increment else 0) + P if all_points else P
         out = torch.empty((rows, self.out_channels), dtype=torch.float32, device=self.device)
         n = I64(0)
-        lib.insc_net_forward(self.h, ptr(c), int(c.size(1)), ptr(f), I64(P), int(bool(increment)), ptr(out),
-                             int(bool(all_points)), ctypes.byref(n), stream_ptr())
+        for attempt in (0, 1):
+            lib.insc_net_forward(self.h, ptr(c), int(c.size(1)), ptr(f), I64(P), int(increment), ptr(out),
+                                 int(bool(all_points)), ctypes.byref(n), stream_ptr())
+            if attempt or not self._changed():
+                break
+            # the frame just enqueued read parameters that have moved or changed since they were packed
+            self._rebind()
+            if increment:
+                raise RuntimeError("the model's parameters changed since the last full frame: the cached rows "
+                                   "belong to the old parameters; run a full frame (increment=False) first")
+        self._n_points = (self._n_points if increment else 0) + P
         self.n_sites = int(n.value)
         self._timed = getattr(self, "_profiling", False)
         return out
@@ -194,7 +229,7 @@ class CompiledNet(object):
         the frame's points only; the saved state is not touched."""
         if not self.residual:
             raise RuntimeError("compile the model with residual=True to run residual frames")
-        c = coords.to(device=self.device, dtype=torch.int32).contiguous()
+        c = self._coords(coords)
         f = feats.detach().to(device=self.device, dtype=torch.float32).contiguous()
         P = c.size(0)
         out = torch.empty((P, self.out_channels), dtype=torch.float32, device=self.device)
@@ -232,6 +267,19 @@ class CompiledNet(object):
         for i in range(n.value):
             out[lv[i]].append((names[kd[i]], int(rows[i])))
         return out
+
+    def frame_work(self):
+        """What every convolution of the last frame worked on: a list of dicts (kind, level, cin, cout,
+        rows, rules, slots) in program order; useful multiply-adds of a layer = rules * cin * cout, the
+        matrix cores are issued slots * cin * cout (insc_net_frame_work).  Synchronises."""
+        cap = 256
+        n = ctypes.c_int(0)
+        kd, lv, ci, co = ((ctypes.c_int * cap)() for _ in range(4))
+        rows, rules, slots = ((I64 * cap)() for _ in range(3))
+        lib.insc_net_frame_work(self.h, cap, ctypes.byref(n), kd, lv, ci, co, rows, rules, slots, stream_ptr())
+        names = {0: "ssc", 2: "conv", 3: "deconv", 4: "nin"}
+        return [dict(kind=names[kd[i]], level=lv[i], cin=ci[i], cout=co[i], rows=int(rows[i]), rules=int(rules[i]),
+                     slots=int(slots[i])) for i in range(n.value)]
 
     def sites_per_level(self):
         a = (I64 * 16)()

@@ -158,8 +158,12 @@ def sweep_sequence(seed=5, n=150000, frames=50, first_frac=0.2):
     """Workload 5: a sensor sweep over the workload-4 room.
 
     Frame 0 holds the ``first_frac`` of the voxels nearest a start pose; each later frame
-    adds the next 3k-8k voxels in order of distance along the sweep and re-observes
-    1k-2k already seen voxels with RGB perturbed by U[-0.1, 0.1].
+    adds the next voxels in order of distance along the sweep and re-observes 1k-2k already
+    seen voxels with RGB perturbed by U[-0.1, 0.1].  The additions are drawn from 3k-8k and
+    then scaled so that ``frames`` frames end exactly on ``n`` voxels: 49 unscaled draws would
+    add some 270k voxels to a 150k-voxel scene, so with the default arguments a frame really
+    adds 1.3k-3.6k voxels (2.4k on average).  ``target_frame`` below is the frame the latency
+    target is stated on (5k new voxels onto a scene that then has 150k).
     Returns a list of (points[P,4] int32, rgb[P,3] float32) per frame.
     """
     vox = indoor_scene(seed=4, n=n, dims=(270, 220, 80), n_boxes=30, side_rng=(15, 60))
@@ -189,3 +193,36 @@ def sweep_sequence(seed=5, n=150000, frames=50, first_frac=0.2):
         out.append((vox[idx][perm].copy(), rgb[perm].copy()))
         seen += adds[f - 1]
     return out
+
+
+def target_frame(seed=6, n=150000, n_new=5000, n_old=1500, old_from="scene"):
+    """The frame the latency target is stated on: 5k new voxels onto a 150k-voxel scene.
+
+    The workload-4 room in the order of the sweep (distance from the start pose): the first
+    ``n - n_new`` voxels are the scene a full forward has seen (one point per voxel, seeded
+    shuffle), and ONE incremental frame then brings exactly ``n_new`` new voxels - the next
+    ones along the sweep, i.e. a shell at the scene's frontier, as a moving sensor delivers
+    them - plus ``n_old`` re-observed voxels with RGB perturbed by U[-0.1, 0.1], drawn from the
+    whole scene (``old_from="scene"``, as in the sweep: the harder case, it dirties every region)
+    or from the 10 % of the scene nearest the frontier (``"frontier"``: what a sensor that moves
+    on still sees).  This mirrors the reference's usage: one full pass, then a frame with
+    increment=True (demo.py:26-38).
+    Returns ((scene_points[n - n_new, 4], scene_rgb), (frame_points[n_new + n_old, 4], frame_rgb)).
+    """
+    vox = indoor_scene(seed=4, n=n, dims=(270, 220, 80), n_boxes=30, side_rng=(15, 60))
+    rng = np.random.default_rng(seed)
+    base_rgb = rng.uniform(0, 1, (len(vox), 3)).astype(np.float32)
+    pose = np.array([1024 + 20, 1024 + 20, 1024 + 30], np.float64)
+    d = np.linalg.norm(vox[:, :3].astype(np.float64) - pose, axis=1)
+    order = np.argsort(d, kind="stable")
+    n0 = n - n_new
+    idx0 = order[:n0][rng.permutation(n0)]
+    if old_from not in ("scene", "frontier"):
+        raise ValueError("old_from must be 'scene' or 'frontier'")
+    near = order[:n0] if old_from == "scene" else order[n0 - n0 // 10:n0]
+    old = near[rng.permutation(len(near))[:n_old]]
+    idx1 = np.concatenate([order[n0:], old])
+    rgb1 = base_rgb[idx1].copy()
+    rgb1[n_new:] = np.clip(rgb1[n_new:] + rng.uniform(-0.1, 0.1, (n_old, 3)).astype(np.float32), 0, 1)
+    perm = rng.permutation(len(idx1))
+    return (vox[idx0].copy(), base_rgb[idx0].copy()), (vox[idx1][perm].copy(), rgb1[perm].copy())

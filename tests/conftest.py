@@ -13,6 +13,27 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: test needs a real MI355X (run with -m gpu)")
 
 
+@pytest.fixture(autouse=True)
+def layer_by_layer_module_path():
+    """A whole-network Sequential hands its frames to the network executor by itself.  The tests compare
+    that executor with the layer-by-layer module path (one C call per layer through the reference's
+    operator names), so here the switch is off unless a test turns it on (`auto_compile` fixture)."""
+    import sparseconvnet as scn
+
+    prev = scn.set_auto_compile(False)
+    yield
+    scn.set_auto_compile(prev)
+
+
+@pytest.fixture
+def auto_compile(layer_by_layer_module_path):
+    import sparseconvnet as scn
+
+    scn.set_auto_compile(True)
+    yield
+    scn.set_auto_compile(False)
+
+
 @pytest.fixture(scope="session")
 def orc():
     from oracle import oracle

@@ -60,6 +60,45 @@ def test_checkpoint_round_trip_through_the_hip_path(tmp_path):
     assert torch.equal(net_again, again)
 
 
+def test_incremental_frame_after_a_reload_is_refused():
+    """Rows cached by earlier frames were computed with the old parameters.  After the parameters
+    change - all of them (load_state_dict) or a single tensor in the middle of the network (copy_) -
+    an incremental frame must not mix old and new rows: the executor raises until a full frame has
+    run, and that full frame plus an increment equals a full forward with the new parameters."""
+    import sparseconvnet as scn
+    from sparseconvnet._lib import InscError
+    from workloads.netdefs import NaiveUNet
+
+    pts, rgb = _scene(5000, seed=52)
+    a, b = (pts[:4000], rgb[:4000]), (pts[4000:], rgb[4000:])
+    model = NaiveUNet(m=16, levels=3, seed=3).cuda()
+    net = scn.compile(model.sparseModel, capacity_sites=8192)
+
+    def change_all():
+        model.load_state_dict(NaiveUNet(m=16, levels=3, seed=5).state_dict())
+
+    def change_one():
+        convs = [m for m in model.modules() if isinstance(m, scn.SubmanifoldConvolution)]
+        mid = convs[len(convs) // 2]  # neither the first nor the last op with parameters
+        mid.weight.copy_(mid.weight * 1.5)
+
+    for change in (change_all, change_one):
+        with torch.no_grad():
+            net(_inp(*a), increment=False)
+            net(_inp(*b), increment=True)  # fine: state and parameters agree
+            change()
+            with pytest.raises(RuntimeError) as err:  # noticed by the wrapper ...
+                net(_inp(*b), increment=True)
+            assert "full frame" in str(err.value)
+            with pytest.raises(InscError) as err:  # ... and the library has dropped its cached rows
+                net(_inp(*b), increment=True)
+            assert "full frame" in str(err.value)
+            net(_inp(*a), increment=False)
+            got = net(_inp(*b), increment=True, all_points=True)
+            want = model.sparseModel(_inp(pts, rgb))
+        assert torch.equal(got, want)
+
+
 def test_zmajor_weights_through_the_hip_path():
     """Weights trained against the z-major offset numbering: the oracle runs the ORIGINAL weights on
     z-major rules; the HIP path runs the converted state_dict."""

@@ -140,3 +140,91 @@ def test_order_refresh_leaves_every_bit_alone():
         full = scn.compile(copy.deepcopy(model).sparseModel, capacity_sites=60000)(_inp(all_p, all_c), increment=False)
         assert torch.equal(outs[1], full)
         assert [int(v) for v in nets[1].sites_per_level()] == [int(v) for v in nets[0].sites_per_level()]
+
+
+def test_whole_network_sequential_runs_through_the_executor_by_itself(auto_compile):
+    """The reference's own loop, unchanged (model.py:23-26, demo.py:26-38): `model(x, increment=False)`
+    then `model(x, increment=True)` on the module tree, coordinates as int64 on the host or on the
+    GPU.  With the switch on, the whole-network Sequential traces itself at the first frame; the
+    outputs equal the layer-by-layer path bit for bit."""
+    import sparseconvnet as scn
+    from workloads.netdefs import NaiveUNet
+
+    frames = _frames(4, seed=35)
+    model = NaiveUNet(m=16, levels=4, seed=9).cuda()
+    ref_model = copy.deepcopy(model)
+    assert scn.get_auto_compile()
+    with torch.no_grad():
+        out = model(_inp(*frames[0]), increment=False)
+        assert model.sparseModel.__dict__["_exec"][0] is not None and model.sparseModel.why_not_compiled() is None
+        scn.set_auto_compile(False)
+        ref = ref_model(_inp(*frames[0]), increment=False)
+        scn.set_auto_compile(True)
+        assert torch.equal(out, ref)
+        for f in range(1, len(frames)):
+            pts, rgb = frames[f]
+            x = _inp(pts, rgb)
+            if f == 2:
+                x[0] = x[0].cuda()  # int64 coordinates on the GPU, as in the reference's demo
+            out = model(x, increment=True)
+            scn.set_auto_compile(False)
+            ref = ref_model(_inp(pts, rgb), increment=True)
+            scn.set_auto_compile(True)
+            assert out.shape == ref.shape == (len(pts), 20)
+            assert torch.equal(out, ref), "frame %d" % f
+    # a copy of the model traces its own executor
+    twin = copy.deepcopy(model)
+    assert "_exec" not in twin.sparseModel.__dict__
+    with torch.no_grad():
+        assert torch.equal(twin(_inp(*frames[0])), ref_model(_inp(*frames[0])))
+
+
+def test_sequential_falls_back_to_the_layer_path(auto_compile):
+    """Trees the tracer does not take run layer by layer, with the tracer's reason kept: here a
+    ConcatTable of three branches joined by one JoinTable."""
+    import sparseconvnet as scn
+
+    torch.manual_seed(3)
+    net = scn.Sequential().add(scn.InputLayer(3, 4096, mode=4)).add(
+        scn.SubmanifoldConvolution(3, 3, 16, 3, False)).add(
+        scn.ConcatTable().add(scn.Identity()).add(scn.SubmanifoldConvolution(3, 16, 16, 3, False)).add(
+            scn.NetworkInNetwork(16, 16, False))).add(
+        scn.JoinTable()).add(scn.BatchNormReLU(48)).add(scn.OutputLayer(3)).cuda()
+    pts, rgb = _frames(2, seed=36)[0]
+    with torch.no_grad():
+        out = net(_inp(pts, rgb))
+        assert "JoinTable" in net.why_not_compiled()
+        scn.set_auto_compile(False)
+        ref = net(_inp(pts, rgb))
+    assert out.shape == (len(pts), 48) and torch.equal(out, ref)
+
+
+def test_sequential_residual_frames_through_the_executor(auto_compile):
+    """With the reference's kind of incremental forward in force (set_incremental_mode("residual")),
+    `model(x, increment=True)` is a residual frame; traced at the first frame, it equals the module
+    tree's Incre_* operators bit for bit."""
+    import sparseconvnet as scn
+    from workloads.netdefs import NaiveUNet
+
+    frames = _frames(3, seed=37)
+    model = NaiveUNet(m=16, levels=3, seed=9).cuda()
+    ref_model = copy.deepcopy(model)
+    scn.set_incremental_mode("residual")
+    try:
+        with torch.no_grad():
+            model(_inp(*frames[0]), increment=False)
+            got = model(_inp(*frames[1]), increment=True)
+            assert model.sparseModel.__dict__["_exec"][0].residual
+            scn.set_auto_compile(False)
+            ref_model(_inp(*frames[0]), increment=False)
+            ref = ref_model(_inp(*frames[1]), increment=True)
+        assert torch.equal(got, ref)
+    finally:
+        scn.set_incremental_mode("exact")
+    # an executor traced for exact frames says how to get residual ones
+    scn.set_auto_compile(True)
+    other = NaiveUNet(m=16, levels=3, seed=9).cuda()
+    with torch.no_grad():
+        other(_inp(*frames[0]), increment=False)
+        with pytest.raises(RuntimeError, match="set_incremental_mode"):
+            other(_inp(*frames[1]), increment="residual")

@@ -264,3 +264,44 @@ def test_workload5_sweep_equals_a_full_forward_every_tenth_frame(orc):
     parity.check("workload 5, last frame of the sweep, 150k voxels", out.cpu().numpy(), oref, oref64)
     assert set(phases) == {"structure", "dirty", "layers", "output"}
     assert 0.5 < sum(phases.values()) < 50.0
+
+
+@pytest.mark.parametrize("old_from", ["scene", "frontier"])
+def test_target_frame_5k_new_voxels_on_a_150k_scene(orc, old_from):
+    """The frame the latency target is stated on (one full pass, then ONE frame with increment=True, as
+    in the reference's demo.py:26-38): full forward over the first 145 000 voxels of the room in sweep
+    order, then an incremental frame of exactly 5 000 new voxels plus 1 500 re-observed ones.  The
+    incremental result must equal a full recompute over all points bit for bit - through the executor
+    and through the module tree fed with CPU int64 coordinates as the reference's callers pass them -
+    and match the CPU oracle (fp32 and double precision) per element."""
+    import sparseconvnet as scn
+    from oracle import oracle_net
+    from workloads.netdefs import NaiveUNet
+
+    (p0, c0), (p1, c1) = scenes.target_frame(old_from=old_from)
+    assert len(p0) == 145000 and len(p1) == 6500
+    model = NaiveUNet(m=32, levels=7, seed=4).cuda()
+    net = scn.compile(model.sparseModel, capacity_sites=1 << 18)
+    ref_net = scn.compile(model.sparseModel, capacity_sites=1 << 18)
+    dev = lambda p, c: [torch.from_numpy(p.astype(np.int32)).cuda(), torch.from_numpy(c).cuda(), 1]
+    ref_cpu = lambda p, c: [torch.from_numpy(p[:, :3].astype(np.int64)), torch.from_numpy(c).cuda(), 1]
+    allp, allc = np.concatenate([p0, p1]), np.concatenate([c0, c1])
+    with torch.no_grad():
+        net(dev(p0, c0), increment=False)
+        assert net.n_sites == 145000
+        out = net(dev(p1, c1), increment=True, all_points=True)
+        assert net.n_sites == 150000
+        full = ref_net(dev(allp, allc), increment=False)
+        assert torch.equal(out, full), "max |incremental - full| = %.3e" % (out - full).abs().max().item()
+        # the same two calls through the reference's own entry: the module tree, CPU int64 coordinates
+        model.sparseModel(ref_cpu(p0, c0))
+        for m in model.modules():
+            if isinstance(m, scn.OutputLayer):
+                m.all_points = True
+        out_mod = model.sparseModel(ref_cpu(p1, c1), increment=True)
+    assert torch.equal(out_mod, full)
+    oref = oracle_net.forward(model.sparseModel, [allp, allc, 1])
+    with orc.double_precision():
+        oref64 = oracle_net.forward(model.sparseModel, [allp, allc, 1])
+    parity.check("target frame (5k new + 1.5k re-observed from the %s on 145k voxels)" % old_from, out.cpu().numpy(),
+                 oref, oref64)

@@ -316,3 +316,30 @@ def test_row_subset_leaves_other_rows_untouched(S, orc):
     mask = torch.ones(sc.n, dtype=torch.bool, device="cuda")
     mask[done] = False
     assert bool((out[mask] == 123.0).all())
+
+
+@pytest.mark.parametrize("Cin,Cout,n_sites", [(224, 224, 70), (128, 128, 2900), (160, 160, 700), (256, 128, 2900),
+                                              (192, 96, 10000)])
+def test_split_layers_repeat_bit_for_bit(S, orc, Cin, Cout, n_sites):
+    """Wide 3^3 layers at the coarse scales split a tile's items over G = 2, 4 or 8 blocks, which exchange
+    partial sums through memory (the block that arrives last adds them in block order).  Nothing in that
+    exchange may depend on timing: 300 launches on the same input must give the same bits every time
+    (stopping at the first difference), and they must match the oracle."""
+    pts = scenes.boxes_scene(seed=9, n=n_sites)
+    m, x, feats = setup_sites(S, pts, Cin, seed=Cin + n_sites)
+    sc = m.ssc_rulebook(SZ)
+    plan = m.ssc_plan(sc)
+    rng = np.random.default_rng(Cout)
+    W = (rng.normal(size=(27, Cin, Cout)) * (2.0 / Cin / 27) ** 0.5).astype(np.float32)
+    Wd = cu(W)
+    first = torch.empty((sc.n, Cout), device="cuda")
+    S.ssc_rows_planned(feats, first, Wd, None, sc, plan)
+    _, osc, _ = orc.grid_build(pts)
+    _, counts, pairs = orc.ssc_rules(osc)
+    ref, _ = orc.conv_forward(feats.cpu().numpy(), W, None, pairs, counts, len(osc))
+    np.testing.assert_allclose(first.cpu().numpy(), ref, rtol=RTOL, atol=ATOL)
+    out = torch.empty_like(first)
+    for i in range(300):
+        out.fill_(float(i))
+        S.ssc_rows_planned(feats, out, Wd, None, sc, plan)
+        assert torch.equal(out, first), "launch %d differs: max |diff| %.3e" % (i, (out - first).abs().max().item())
