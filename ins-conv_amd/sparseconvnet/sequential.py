@@ -16,13 +16,18 @@ import torch
 from . import incremental
 
 _AUTO = True
+_CAPACITY = 1 << 18
 
 
-def set_auto_compile(flag):
+def set_auto_compile(flag, capacity_sites=None):
     """Whether whole-network Sequentials run through the network executor (default) or layer by
-    layer.  Returns the previous setting."""
-    global _AUTO
+    layer.  `capacity_sites`: sites at the input scale that an executor traced from now on is sized
+    for at the start (default 262 144; it grows by half whenever a frame does not fit, which costs
+    that frame a reallocation).  Returns the previous setting of the switch."""
+    global _AUTO, _CAPACITY
     prev, _AUTO = _AUTO, bool(flag)
+    if capacity_sites is not None:
+        _CAPACITY = int(capacity_sites)
     return prev
 
 
@@ -75,7 +80,7 @@ class Sequential(torch.nn.Sequential):
 
                 # residual frames need the raw input of every batch norm kept; asked for when that
                 # is the kind of incremental forward in force as the first frame arrives
-                net = CompiledNet(self, capacity_sites=max(16384, 2 * int(feats.size(0))),
+                net = CompiledNet(self, capacity_sites=max(_CAPACITY, 2 * int(feats.size(0))),
                                   residual=incremental.get_mode() == "residual")
                 state = (net, None, feats.device)
             except (NotImplementedError, ValueError) as e:

@@ -189,7 +189,7 @@ def test_sequential_falls_back_to_the_layer_path(auto_compile):
         scn.SubmanifoldConvolution(3, 3, 16, 3, False)).add(
         scn.ConcatTable().add(scn.Identity()).add(scn.SubmanifoldConvolution(3, 16, 16, 3, False)).add(
             scn.NetworkInNetwork(16, 16, False))).add(
-        scn.JoinTable()).add(scn.BatchNormReLU(48)).add(scn.OutputLayer(3)).cuda()
+        scn.JoinTable()).add(scn.BatchNormReLU(48)).add(scn.OutputLayer(3)).cuda().eval()
     pts, rgb = _frames(2, seed=36)[0]
     with torch.no_grad():
         out = net(_inp(pts, rgb))

@@ -227,9 +227,7 @@ def test_residual_frame_network_vs_oracle(levels, m):
     oracle_net.forward(cpu.sparseModel, [f0[0][:, :3], f0[1], 1], save)
     ref = oracle_net.forward_residual(cpu.sparseModel, [f1[0][:, :3], f1[1], 1], save)
     assert got.shape == ref.shape == (len(f1[0]), m)
-    parity.check("residual frame, %d-level U-Net vs residual oracle" % levels, got.cpu().numpy(), ref, enforce=False)
-    scale = max(1.0, float(np.abs(ref).max()))
-    np.testing.assert_allclose(got.cpu().numpy(), ref, rtol=1e-3, atol=1e-4 * scale)
+    parity.check("residual frame, %d-level U-Net vs residual oracle" % levels, got.cpu().numpy(), ref)
     # a residual frame leaves the saved state alone: the same frame again gives the same bits,
     # and an exact incremental frame afterwards still equals a full forward over all points
     assert torch.equal(got, again)
@@ -260,9 +258,7 @@ def test_residual_frame_covering_scene_equals_full_forward():
         res = model(_inp(b, f_b), increment="residual")
         full = model(_inp(np.concatenate([a, b]), np.concatenate([f_a, f_b])), increment=False)
     ref = full[len(a):]
-    parity.check("residual frame covering the scene vs full forward", res.cpu().numpy(), ref.cpu().numpy(), enforce=False)
-    scale = max(1.0, float(ref.abs().max()))
-    np.testing.assert_allclose(res.cpu().numpy(), ref.cpu().numpy(), rtol=1e-3, atol=2e-4 * scale)
+    parity.check("residual frame covering the scene vs full forward", res.cpu().numpy(), ref.cpu().numpy())
 
 
 def test_increment_true_follows_set_mode():
