@@ -26,6 +26,11 @@ struct insc_grid {
   int32_t *d_err = nullptr;    // device flag: bit0 bad coordinate, bit1 table full
   int64_t n_upper = 0;         // host upper bound of the site count
   int64_t n_exact = -1;        // host copy of the count, -1 = stale
+  // pinned host words that the last kernel of insc_grid_insert writes: [0] site count, [1] error flags.
+  // h_fresh: they describe the grid's current state, once h_stream has been waited for.
+  int32_t *h_n = nullptr;
+  bool h_fresh = false;
+  void *h_stream = nullptr;
   // insert scratch, grown on demand
   int32_t *slot_of_point = nullptr;
   int32_t *flags = nullptr;

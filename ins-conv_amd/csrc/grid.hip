@@ -58,57 +58,102 @@ __global__ void grid_clear_kernel(Slot *table, int64_t n_slots, int32_t *d_n, in
   }
 }
 
-// pass 1: claim a slot per distinct key; the smallest row index claiming a new slot wins it
+// ---- numbering the new cells of an insert ----------------------------------------------------
+// A site's id is the rank of its first row in the inserted list, so every new cell needs the smallest
+// row that falls into it.  Protocol on a slot (key, val, pad), one claim kernel, then whatever ranks:
+//   * the row whose compare-and-swap sets the key - the slot's first claimant - leaves row + 1 in
+//     `pad` (a plain store: it is read by later kernels only) and is the cell's winner for now;
+//   * every other row of the call that finds the key there lowers `val` to VAL_PENDING + row with an
+//     atomic minimum (skipped when the value it read is already a smaller row's claim);
+//   * afterwards the cell's first row is min(pad - 1, val - VAL_PENDING), which only the rows of the
+//     second kind look at: a point list without repeats costs one atomic per new site and no second
+//     visit of its slot (one compare-and-swap plus one minimum per point, and a visit of the slot by
+//     every row to see who won, measured 55 + 8 us for 220 000 points).
+// A slot that holds an id (0 <= val < VAL_PENDING) was numbered by an earlier insert.
+// State of a row after the claim kernel, in site_of_point: its own row index (first claimant), ST_DUP
+// (other claimant, to be resolved), -2 - id (cell numbered earlier), -1 (skipped / bad / table full).
+constexpr int32_t ST_DUP = INT32_MIN + 1;
+
 __global__ void grid_claim_kernel(Slot *table, int64_t mask, const int32_t *__restrict__ coords4, int64_t P,
-                                  int32_t *__restrict__ slot_of_point, int32_t *d_err) {
+                                  int32_t *__restrict__ slot_of_point, int32_t *__restrict__ flags,
+                                  int32_t *__restrict__ site_of_point, int32_t *d_err) {
   int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (p >= P) return;
   int4 c = reinterpret_cast<const int4 *>(coords4)[p];
-  if (c.x == COORD_SKIP) {
-    slot_of_point[p] = -1;
-    return;
-  }
-  if (!coord_ok(c.x, c.y, c.z, c.w)) {
-    slot_of_point[p] = -1;
-    atomicOr(d_err, 1);
-    return;
-  }
-  uint64_t key = pack_key(c.x, c.y, c.z, c.w);
-  int64_t s = home_slot(key, mask);
-  int64_t found = -1;
-  for (int64_t probe = 0; probe <= mask && probe < MAX_PROBES; probe++) {
-    unsigned long long k = table[s].key;
-    if (k == INSC_EMPTY_KEY) k = atomicCAS(&table[s].key, INSC_EMPTY_KEY, (unsigned long long)key);
-    if (k == INSC_EMPTY_KEY || k == key) {
-      found = s;
-      break;
+  int32_t slot = -1, state = -1, flag = 0;
+  if (c.x != COORD_SKIP) {
+    if (!coord_ok(c.x, c.y, c.z, c.w)) {
+      atomicOr(d_err, 1);
+    } else {
+      const uint64_t key = pack_key(c.x, c.y, c.z, c.w);
+      int64_t s = home_slot(key, mask);
+      bool full = true;
+      for (int64_t probe = 0; probe <= mask && probe < MAX_PROBES; probe++) {
+        const int4 raw = *reinterpret_cast<const int4 *>(&table[s]);  // key (two words), val, pad
+        unsigned long long k = ((unsigned long long)(unsigned)raw.y << 32) | (unsigned)raw.x;
+        const bool seen = k == key;
+        if (seen && raw.z >= 0 && raw.z < VAL_PENDING) {  // numbered by an earlier insert
+          slot = (int32_t)s;
+          state = -2 - raw.z;
+          full = false;
+          break;
+        }
+        bool first = false;
+        if (k == INSC_EMPTY_KEY) {
+          k = atomicCAS(&table[s].key, INSC_EMPTY_KEY, (unsigned long long)key);
+          first = k == INSC_EMPTY_KEY;
+        }
+        if (first) {
+          table[s].pad = (int)p + 1;
+          slot = (int32_t)s;
+          state = (int32_t)p;
+          flag = 1;
+          full = false;
+          break;
+        }
+        if (k == key) {
+          if (!(seen && raw.z >= VAL_PENDING && raw.z <= VAL_PENDING + (int)p)) atomicMin(&table[s].val, VAL_PENDING + (int)p);
+          slot = (int32_t)s;
+          state = ST_DUP;
+          full = false;
+          break;
+        }
+        s = (s + 1) & mask;
+      }
+      if (full) atomicOr(d_err, 2);
     }
-    s = (s + 1) & mask;
   }
-  if (found < 0) {
-    slot_of_point[p] = -1;
-    atomicOr(d_err, 2);
-    return;
-  }
-  slot_of_point[p] = (int32_t)found;
-  // existing sites hold ids < VAL_PENDING and are left alone by the min
-  atomicMin(&table[found].val, VAL_PENDING + (int)p);
+  slot_of_point[p] = slot;
+  site_of_point[p] = state;
+  if (flags) flags[p] = flag;
 }
 
-// pass 2 of a large insert: flag the winning rows for the scan and leave for every row what pass 3
-// needs in site_of_point: the winner's row (>= 0), -1 for a skipped row, or -2 - id for a cell that
-// held a site before this insert.  Row 0 also saves the site count from before the insert beside
-// the scan's total, so that pass 3 can replace the counters while its other threads still read it.
-__global__ void grid_flag_kernel(const Slot *__restrict__ table, const int32_t *__restrict__ slot_of_point, int64_t P,
-                                 int32_t *__restrict__ flags, int32_t *__restrict__ site_of_point,
-                                 const int32_t *__restrict__ d_n, int32_t *__restrict__ n_before) {
+// pass 2 of a large insert, for the rows that found their key claimed by another row of the call: who
+// numbers the cell.  If it is this row (the smallest of the later claimants, and smaller than the
+// first claimant) it takes the first claimant's place.  Row 0 also saves the site count from before
+// the insert beside the scan's total, so that pass 3 can replace the counters while its other threads
+// still read it.
+__global__ void grid_resolve_kernel(const Slot *__restrict__ table, const int32_t *__restrict__ slot_of_point, int64_t P,
+                                    int32_t *__restrict__ flags, int32_t *__restrict__ site_of_point,
+                                    const int32_t *__restrict__ d_n, int32_t *__restrict__ n_before) {
   int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (p >= P) return;
   if (p == 0) *n_before = d_n[0];
-  int s = slot_of_point[p];
-  int v = s >= 0 ? table[s].val : -1;
-  flags[p] = (s >= 0 && v == VAL_PENDING + (int)p) ? 1 : 0;
-  site_of_point[p] = s < 0 ? -1 : v >= VAL_PENDING ? v - VAL_PENDING : -2 - v;
+  if (site_of_point[p] != ST_DUP) return;
+  const int4 raw = *reinterpret_cast<const int4 *>(&table[slot_of_point[p]]);
+  if (raw.z >= 0 && raw.z < VAL_PENDING) {  // (the key was there all along; the row had read a stale empty slot)
+    site_of_point[p] = -2 - raw.z;
+    return;
+  }
+  const int first = raw.w - 1, later = raw.z - VAL_PENDING;  // (later: huge when no row lowered the value)
+  if (later == (int)p && (int)p < first) {
+    flags[p] = 1;
+    site_of_point[p] = (int32_t)p;
+    flags[first] = 0;
+    site_of_point[first] = (int32_t)p;
+  } else {
+    site_of_point[p] = first < later ? first : later;
+  }
 }
 
 // pass 3: winners take id = n_before + rank, publish it in the slot and record the coordinates; every
@@ -117,13 +162,21 @@ __global__ void grid_assign_kernel(Slot *table, const int32_t *__restrict__ coor
                                    const int32_t *__restrict__ slot_of_point, const int32_t *__restrict__ excl,
                                    int64_t P, int32_t *__restrict__ d_n, const int32_t *__restrict__ total,
                                    int32_t *__restrict__ site_coords, int64_t capacity_sites, int32_t *d_err,
-                                   int32_t *__restrict__ site_of_point) {
+                                   int32_t *__restrict__ site_of_point, int32_t *__restrict__ h_n) {
   int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (p >= P) return;
   const int n_before = total[1];
   if (p == 0) {
+    // (more new sites than there is room for: the rows beyond get no site below and raise the flag, but
+    // perhaps only after this thread has read it - so it is worked out here as well)
+    const bool over = (int64_t)n_before + total[0] > capacity_sites;
+    const int n_new = over ? (int)(capacity_sites - n_before) : total[0];
     d_n[1] = n_before;
-    d_n[0] = n_before + total[0];
+    d_n[0] = n_before + n_new;
+    if (h_n) {  // the host's copy of the count and of the error flags (pinned memory)
+      h_n[0] = n_before + n_new;
+      h_n[1] = __hip_atomic_load(d_err, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) | (over ? 2 : 0);
+    }
   }
   int r = site_of_point[p];
   if (r < 0) {
@@ -143,29 +196,49 @@ __global__ void grid_assign_kernel(Slot *table, const int32_t *__restrict__ coor
   }
 }
 
-// Passes 2-4 and the counter update in one workgroup, for inserts of up to FINISH_SMALL_MAX rows
+// Passes 2-3 and the counter update in one workgroup, for inserts of up to FINISH_SMALL_MAX rows
 // (an incremental frame): thread t owns a contiguous run of rows, so the ids come out in row
-// order exactly as from the scan-based passes.
+// order exactly as from the scan-based passes.  site_of_point holds the rows' states on entry and
+// their sites on exit.
 constexpr int FINISH_SMALL_MAX = 16384;
 __global__ __launch_bounds__(1024) void grid_finish_small_kernel(Slot *table, const int32_t *__restrict__ coords4,
                                                                  const int32_t *__restrict__ slot_of_point, int P,
                                                                  int32_t *d_n, int32_t *__restrict__ site_coords,
                                                                  int64_t capacity_sites, int32_t *d_err,
-                                                                 int32_t *__restrict__ site_of_point) {
+                                                                 int32_t *site_of_point, int32_t *__restrict__ h_n) {
   __shared__ int wave_total[16];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int per = (P + 1023) / 1024, p0 = tid * per;
   const int n_before = d_n[0];
-  unsigned win = 0;
-  int cnt = 0;
+  // later claimants find out who numbers their cell (grid_resolve_kernel)
   for (int j = 0; j < per; j++) {
     const int p = p0 + j;
-    if (p < P) {
-      const int s = slot_of_point[p];
-      if (s >= 0 && table[s].val == VAL_PENDING + p) {
-        win |= 1u << j;
-        cnt++;
-      }
+    if (p >= P || site_of_point[p] != ST_DUP) continue;
+    const int4 raw = *reinterpret_cast<const int4 *>(&table[slot_of_point[p]]);
+    if (raw.z >= 0 && raw.z < VAL_PENDING) {
+      site_of_point[p] = -2 - raw.z;
+      continue;
+    }
+    const int first = raw.w - 1, later = raw.z - VAL_PENDING;
+    if (later == p && p < first) {
+      site_of_point[p] = p;
+      site_of_point[first] = p;
+    } else {
+      site_of_point[p] = first < later ? first : later;
+    }
+  }
+  __threadfence_block();
+  __syncthreads();
+  int st[16];
+  unsigned win = 0;
+  int cnt = 0;
+#pragma unroll
+  for (int j = 0; j < 16; j++) {
+    const int p = p0 + j;
+    st[j] = (j < per && p < P) ? site_of_point[p] : -1;
+    if (j < per && p < P && st[j] == p) {
+      win |= 1u << j;
+      cnt++;
     }
   }
   // exclusive scan of cnt over the workgroup
@@ -181,28 +254,40 @@ __global__ __launch_bounds__(1024) void grid_finish_small_kernel(Slot *table, co
     if (w < wave) base += wave_total[w];
     total += wave_total[w];
   }
-  for (int j = 0; j < per; j++) {
+#pragma unroll
+  for (int j = 0; j < 16; j++) {
     if (!((win >> j) & 1u)) continue;
     const int p = p0 + j, id = base++;
     if (id >= capacity_sites) {
       atomicOr(d_err, 2);
+      site_of_point[p] = -1;
       continue;
     }
     table[slot_of_point[p]].val = id;
     reinterpret_cast<int4 *>(site_coords)[id] = reinterpret_cast<const int4 *>(coords4)[p];
+    site_of_point[p] = id;
   }
   __threadfence_block();
   __syncthreads();
-  for (int j = 0; j < per; j++) {
+  // every other row takes its site from the row that numbered its cell
+#pragma unroll
+  for (int j = 0; j < 16; j++) {
     const int p = p0 + j;
-    if (p >= P) break;
-    const int s = slot_of_point[p];
-    const int v = (s >= 0) ? table[s].val : -1;
-    site_of_point[p] = (v >= 0 && v < VAL_PENDING) ? v : -1;
+    if (j >= per || p >= P || ((win >> j) & 1u)) continue;
+    if (st[j] < -1)
+      site_of_point[p] = -2 - st[j];
+    else if (st[j] >= 0)
+      site_of_point[p] = site_of_point[st[j]];
   }
+  const bool over = total > capacity_sites - n_before;
+  if (over) total = (int)(capacity_sites - n_before);
   if (tid == 0) {
     d_n[1] = n_before;
     d_n[0] = n_before + total;
+    if (h_n) {  // the host's copy of the count and of the error flags (pinned memory)
+      h_n[0] = n_before + total;
+      h_n[1] = __hip_atomic_load(d_err, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) | (over ? 2 : 0);
+    }
   }
 }
 
@@ -394,9 +479,19 @@ static int grid_alloc_table(insc_grid *g, int64_t capacity_sites) {
 
 static int grid_sync_errors(insc_grid *g, hipStream_t s, const char *who) {
   int32_t h[2];
-  INSC_HIP(hipMemcpyAsync(&h[0], g->d_n, sizeof(int32_t), hipMemcpyDeviceToHost, s));
-  INSC_HIP(hipMemcpyAsync(&h[1], g->d_err, sizeof(int32_t), hipMemcpyDeviceToHost, s));
-  INSC_HIP(hipStreamSynchronize(s));
+  if (g->h_fresh && g->h_stream == (void *)s) {
+    // the last insert left both words in pinned host memory: waiting for its stream is all it takes
+    // (two small device-to-host copies and their waits cost ~50 us per call, most of a 220 000-point insert)
+    INSC_HIP(hipStreamSynchronize(s));
+    h[0] = g->h_n[0];
+    h[1] = g->h_n[1];
+  } else {
+    int32_t both[17];  // d_n[0] .. d_err (= d_n + 16) in one copy
+    INSC_HIP(hipMemcpyAsync(both, g->d_n, sizeof(both), hipMemcpyDeviceToHost, s));
+    INSC_HIP(hipStreamSynchronize(s));
+    h[0] = both[0];
+    h[1] = both[16];
+  }
   g->n_exact = h[0];
   g->n_upper = h[0];
   if (h[1]) {
@@ -404,6 +499,7 @@ static int grid_sync_errors(insc_grid *g, hipStream_t s, const char *who) {
     // the grid stays usable
     INSC_HIP(hipMemsetAsync(g->d_err, 0, sizeof(int32_t), s));
     INSC_HIP(hipStreamSynchronize(s));
+    if (g->h_n) g->h_n[1] = 0;
   }
   if (h[1] & 1) {
     set_error("%s: a coordinate is outside 0..65535 (batch 0..32767)", who);
@@ -438,26 +534,31 @@ static int grid_insert_launch(insc_grid *g, const int32_t *d_coords4, int64_t P,
   const int64_t mask = g->n_slots - 1;
   const unsigned nb = grid_for(P, 256);
   int32_t *total = g->flags + g->scratch_rows;  // spare int after the flags
+  const bool small = P <= FINISH_SMALL_MAX;
   hipLaunchKernelGGL(grid_claim_kernel, dim3(nb), dim3(256), 0, s, g->table, mask, d_coords4, P, g->slot_of_point,
-                     g->d_err);
-  if (P <= FINISH_SMALL_MAX) {
+                     small ? nullptr : g->flags, d_site_of_point, g->d_err);
+  if (small) {
     hipLaunchKernelGGL(grid_finish_small_kernel, dim3(1), dim3(1024), 0, s, g->table, d_coords4, g->slot_of_point,
-                       (int)P, g->d_n, g->coords, g->capacity_sites, g->d_err, d_site_of_point);
+                       (int)P, g->d_n, g->coords, g->capacity_sites, g->d_err, d_site_of_point, g->h_n);
     INSC_LAUNCH_CHECK();
     g->n_upper += P;
     g->n_exact = -1;
+    g->h_fresh = g->h_n != nullptr;
+    g->h_stream = (void *)s;
     return INSC_OK;
   }
-  hipLaunchKernelGGL(grid_flag_kernel, dim3(nb), dim3(256), 0, s, g->table, g->slot_of_point, P, g->flags,
+  hipLaunchKernelGGL(grid_resolve_kernel, dim3(nb), dim3(256), 0, s, g->table, g->slot_of_point, P, g->flags,
                      d_site_of_point, g->d_n, total + 1);
   INSC_LAUNCH_CHECK();
   rc = scan_exclusive_i32(g->flags, g->flags, P, total, s);
   if (rc) return rc;
   hipLaunchKernelGGL(grid_assign_kernel, dim3(nb), dim3(256), 0, s, g->table, d_coords4, g->slot_of_point, g->flags,
-                     P, g->d_n, total, g->coords, g->capacity_sites, g->d_err, d_site_of_point);
+                     P, g->d_n, total, g->coords, g->capacity_sites, g->d_err, d_site_of_point, g->h_n);
   INSC_LAUNCH_CHECK();
   g->n_upper += P;
   g->n_exact = -1;
+  g->h_fresh = g->h_n != nullptr;
+  g->h_stream = (void *)s;
   return INSC_OK;
 }
 
@@ -703,6 +804,7 @@ int grid_clear_batch(insc_grid *const *grids, int32_t *const *minus1, const int6
     most = std::max(most, std::max(g->n_slots, b.job[i].n_minus1));
     g->n_upper = 0;
     g->n_exact = 0;
+    g->h_fresh = false;
   }
   b.zero = (uint32_t *)zero;
   b.n_zero = zero ? zero_bytes / 4 : 0;
@@ -742,23 +844,34 @@ __device__ __forceinline__ int table_val(const Slot *table, int64_t s) {
   return __hip_atomic_load(&table[s].val, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 constexpr uint32_t REC_SITE = 0x80000000u;  // rec = REC_SITE | id: the cell was numbered before this frame
+constexpr uint32_t REC_DUP = 0x40000000u;   // rec = REC_DUP | slot: the cell was claimed first by another row of the frame
 constexpr uint32_t REC_NONE = 0xFFFFFFFFu;  // no slot: bad coordinate, or the table is full
+__device__ __forceinline__ bool rec_is_slot(uint32_t r) { return r != REC_NONE && !(r & REC_SITE); }
+__device__ __forceinline__ int64_t rec_slot(uint32_t r) { return (int64_t)(r & ~REC_DUP); }
 __device__ __forceinline__ int4 frame_point(const int32_t *__restrict__ coords_in, int cols, int p, int l) {
   const int32_t *c = coords_in + (int64_t)p * cols;
   return make_int4(c[0] >> l, c[1] >> l, c[2] >> l, cols > 3 ? c[3] : 0);
 }
-// rec[l * P + p]: what row p found at scale l - REC_SITE | id, the slot it claimed, or REC_NONE
+// rec[l * P + p]: what row p found at scale l - REC_SITE | id, the slot it claimed first, REC_DUP | the slot
+// another row claimed first, or REC_NONE (protocol: see grid_claim_kernel).  With flag / rep (frames
+// ranked by a prefix sum) the first claimants also enter themselves as winners there: flag 1, rep -1.
 __global__ __launch_bounds__(256) void frame_claim_kernel(FrameInsertArgs a, const int32_t *__restrict__ coords_in,
                                                           int cols, int P, int32_t *__restrict__ bad, int32_t frame,
-                                                          uint32_t *__restrict__ rec, int shared_from) {
+                                                          uint32_t *__restrict__ rec, int shared_from,
+                                                          int32_t *__restrict__ flag, int32_t *__restrict__ rep) {
   const int l = blockIdx.y;
   const FrameLevelDev &L = a.lv[l];
   const int p = blockIdx.x * 256 + threadIdx.x;
   if (p >= P) return;
+  const int64_t idx = (int64_t)l * P + p;
   const int32_t *c0 = coords_in + (int64_t)p * cols;
   if (!coord_ok(c0[0], c0[1], c0[2], cols > 3 ? c0[3] : 0)) {
     if (l == 0) bad[0] = frame;
-    rec[(int64_t)l * P + p] = REC_NONE;
+    rec[idx] = REC_NONE;
+    if (flag) {
+      flag[idx] = 0;
+      rep[idx] = -1;
+    }
     return;
   }
   const int4 c = frame_point(coords_in, cols, p, l);
@@ -770,12 +883,18 @@ __global__ __launch_bounds__(256) void frame_claim_kernel(FrameInsertArgs a, con
       unsigned long long k = ((unsigned long long)(unsigned)raw.y << 32) | (unsigned)raw.x;
       if (k == key && raw.z >= 0 && raw.z < VAL_PENDING) return REC_SITE | (uint32_t)raw.z;  // numbered before this frame
       const bool seen = k == key;  // the slot already held this key when it was read
-      if (k == INSC_EMPTY_KEY) k = atomicCAS(&L.table[s].key, INSC_EMPTY_KEY, (unsigned long long)key);
-      if (k == INSC_EMPTY_KEY || k == key) {
+      if (k == INSC_EMPTY_KEY) {
+        k = atomicCAS(&L.table[s].key, INSC_EMPTY_KEY, (unsigned long long)key);
+        if (k == INSC_EMPTY_KEY) {  // first claimant
+          L.table[s].pad = p + 1;
+          return (uint32_t)s;
+        }
+      }
+      if (k == key) {
         // (the claim of a smaller row that this row has seen stands: the value only ever goes down, so a
         // stale read errs on the side of one more atomic)
         if (!(seen && raw.z >= VAL_PENDING && raw.z <= VAL_PENDING + p)) atomicMin(&L.table[s].val, VAL_PENDING + p);
-        return (uint32_t)s;
+        return REC_DUP | (uint32_t)s;
       }
       s = (s + 1) & L.mask;
     }
@@ -788,8 +907,10 @@ __global__ __launch_bounds__(256) void frame_claim_kernel(FrameInsertArgs a, con
     // From the third scale on, neighbouring rows mostly fall into the same cell (at the coarsest scale of
     // a full frame thousands of rows per cell), and atomics on one address are served one at a time: the
     // rows of a wavefront that share a cell send one claim, that of their first lane - the smallest row,
-    // rows ascending with the lanes - and all take its answer.
+    // rows ascending with the lanes - and all take its answer (the others as later claimants: whoever
+    // numbers the cell, it is not one of them).
     bool todo = true;
+    const int lane = (int)(threadIdx.x & 63);
     while (todo) {  // (lanes leave as their cell is served; every turn serves the first waiting lane's cell)
       const uint64_t waiting = __ballot(true);
       const int leader = (int)__builtin_ctzll(waiting);
@@ -797,23 +918,28 @@ __global__ __launch_bounds__(256) void frame_claim_kernel(FrameInsertArgs a, con
       const uint32_t khi = (uint32_t)__shfl((int)(uint32_t)(key >> 32), leader, 64);
       const bool same = key == (((uint64_t)khi << 32) | klo);
       uint32_t mine = REC_NONE;
-      if ((int)(threadIdx.x & 63) == leader) mine = claim();
+      if (lane == leader) mine = claim();
       const uint32_t got = (uint32_t)__shfl((int)mine, leader, 64);
       if (same) {
-        r = got;
+        r = (lane == leader || !rec_is_slot(got)) ? got : (got | REC_DUP);
         todo = false;
       }
     }
   }
   if (r == REC_NONE) atomicOr(L.d_err, 2);
-  rec[(int64_t)l * P + p] = r;
+  rec[idx] = r;
+  if (flag) {
+    flag[idx] = (rec_is_slot(r) && !(r & REC_DUP)) ? 1 : 0;
+    rep[idx] = -1;
+  }
 }
 
-// site[l * P + p] = site of row p at scale l
+// site[l * P + p] = site of row p at scale l (while the kernel runs: the row's state, as site_of_point
+// in grid_finish_small_kernel)
 __global__ __launch_bounds__(1024) void frame_finish_kernel(FrameInsertArgs a, const int32_t *__restrict__ coords_in,
                                                             int cols, int P, const int32_t *__restrict__ bad,
                                                             int32_t frame, int32_t *__restrict__ sop,
-                                                            int32_t *__restrict__ site, const uint32_t *__restrict__ rec,
+                                                            int32_t *site, const uint32_t *__restrict__ rec,
                                                             int32_t *h_counts) {
   __shared__ int wave_total[16];
   const int l = blockIdx.x;
@@ -831,9 +957,9 @@ __global__ __launch_bounds__(1024) void frame_finish_kernel(FrameInsertArgs a, c
 #pragma unroll
     for (int j = 0; j < 16; j++) {
       if (j >= per || p0 + j >= P) continue;
-      if (rr[j] != REC_NONE && !(rr[j] & REC_SITE)) {
-        __hip_atomic_store(&L.table[rr[j]].val, VAL_UNSET, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_store(&L.table[rr[j]].key, INSC_EMPTY_KEY, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (rec_is_slot(rr[j])) {
+        __hip_atomic_store(&L.table[rec_slot(rr[j])].val, VAL_UNSET, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(&L.table[rec_slot(rr[j])].key, INSC_EMPTY_KEY, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
       site[p0 + j] = -1;
       if (l == 0) sop[p0 + j] = -1;
@@ -848,15 +974,45 @@ __global__ __launch_bounds__(1024) void frame_finish_kernel(FrameInsertArgs a, c
     }
     return;
   }
-  // winners, ranked in row order
-  int tv[16];
+  // states: own row (first claimant), ST_DUP, -2 - id (numbered before this frame), -1
 #pragma unroll
-  for (int j = 0; j < 16; j++) tv[j] = (rr[j] != REC_NONE && !(rr[j] & REC_SITE)) ? table_val(L.table, (int64_t)rr[j]) : -1;
+  for (int j = 0; j < 16; j++) {
+    const int p = p0 + j;
+    if (j >= per || p >= P) continue;
+    const uint32_t r = rr[j];
+    site[p] = r == REC_NONE ? -1 : (r & REC_SITE) ? -2 - (int)(r & ~REC_SITE) : (r & REC_DUP) ? ST_DUP : p;
+  }
+  __threadfence_block();
+  __syncthreads();
+  // later claimants find out who numbers their cell
+#pragma unroll
+  for (int j = 0; j < 16; j++) {
+    const int p = p0 + j;
+    if (j >= per || p >= P || !rec_is_slot(rr[j]) || !(rr[j] & REC_DUP)) continue;
+    const int4 raw = *reinterpret_cast<const int4 *>(&L.table[rec_slot(rr[j])]);
+    if (raw.z >= 0 && raw.z < VAL_PENDING) {  // (the key was there all along; the row had read a stale empty slot)
+      site[p] = -2 - raw.z;
+      continue;
+    }
+    const int first = raw.w - 1, later = raw.z - VAL_PENDING;
+    if (later == p && p < first) {
+      site[p] = p;
+      site[first] = p;
+    } else {
+      site[p] = first < later ? first : later;
+    }
+  }
+  __threadfence_block();
+  __syncthreads();
+  // winners, ranked in row order
+  int st[16];
   unsigned win = 0;
   int cnt = 0;
 #pragma unroll
   for (int j = 0; j < 16; j++) {
-    if (tv[j] == VAL_PENDING + p0 + j) {
+    const int p = p0 + j;
+    st[j] = (j < per && p < P) ? site[p] : -1;
+    if (j < per && p < P && st[j] == p) {
       win |= 1u << j;
       cnt++;
     }
@@ -877,28 +1033,30 @@ __global__ __launch_bounds__(1024) void frame_finish_kernel(FrameInsertArgs a, c
 #pragma unroll
   for (int j = 0; j < 16; j++) {
     if (!((win >> j) & 1u)) continue;
-    const int id = base++;
+    const int p = p0 + j, id = base++;
     if (id >= L.capacity) {
       atomicOr(L.d_err, 2);
+      site[p] = -1;
+      if (l == 0) sop[p] = -1;
       continue;
     }
-    const int4 c = frame_point(coords_in, cols, p0 + j, l);
-    __hip_atomic_store(&L.table[rr[j]].val, id, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const int4 c = frame_point(coords_in, cols, p, l);
+    L.table[rec_slot(rr[j])].val = id;
     reinterpret_cast<int4 *>(L.coords)[id] = c;
     if (L.offset) L.offset[id] = (c.x & 1) * 4 + (c.y & 1) * 2 + (c.z & 1);
+    site[p] = id;
+    if (l == 0) sop[p] = id;
   }
+  __threadfence_block();
   __syncthreads();
-  // every row learns its site
-#pragma unroll
-  for (int j = 0; j < 16; j++) tv[j] = (rr[j] != REC_NONE && !(rr[j] & REC_SITE)) ? table_val(L.table, (int64_t)rr[j]) : -1;
+  // every other row takes its site from the row that numbered its cell
 #pragma unroll
   for (int j = 0; j < 16; j++) {
     const int p = p0 + j;
-    if (j >= per || p >= P) continue;
-    const int v = rr[j] == REC_NONE ? -1 : (rr[j] & REC_SITE) ? (int)(rr[j] & ~REC_SITE) : tv[j];
-    const int st = (v >= 0 && v < VAL_PENDING) ? v : -1;
-    site[p] = st;
-    if (l == 0) sop[p] = st;
+    if (j >= per || p >= P || ((win >> j) & 1u)) continue;
+    const int v = st[j] < -1 ? -2 - st[j] : st[j] >= 0 ? site[st[j]] : -1;
+    site[p] = v;
+    if (l == 0) sop[p] = v;
   }
   if (total > L.capacity - n_before) total = (int)(L.capacity - n_before);  // (the error flag is up)
   if (tid == 0) {
@@ -931,7 +1089,7 @@ __global__ void frame_link_kernel(FrameInsertArgs a, int P, const int32_t *__res
 // cell; if not, which row is), scan, assign (a winner publishes its id and the site's coordinates;
 // every row works out its site from the prefix sums alone, a loser through its winner's row, so no
 // row has to wait for another one's write).
-__global__ __launch_bounds__(256) void frame_flag_kernel(FrameInsertArgs a, int P, const uint32_t *__restrict__ rec,
+__global__ __launch_bounds__(256) void frame_flag_kernel(FrameInsertArgs a, int P, uint32_t *__restrict__ rec,
                                                          int32_t *__restrict__ flag, int32_t *__restrict__ rep,
                                                          int32_t *__restrict__ n_before) {
   const int l = blockIdx.y;
@@ -942,18 +1100,23 @@ __global__ __launch_bounds__(256) void frame_flag_kernel(FrameInsertArgs a, int 
     if (l == 0) flag[(int64_t)a.n_levels * P] = 0;  // (one entry past the end: the scan then leaves the grand total there)
   }
   if (p >= P) return;
-  const int64_t idx = (int64_t)l * P + p;
+  const int64_t lp = (int64_t)l * P, idx = lp + p;
   const uint32_t r = rec[idx];
-  int f = 0, w = -1;
-  if (r != REC_NONE && !(r & REC_SITE)) {
-    const int v = table_val(L.table, (int64_t)r);
-    if (v == VAL_PENDING + p)
-      f = 1;
-    else if (v >= VAL_PENDING && v != VAL_UNSET)
-      w = v - VAL_PENDING;
+  // (first claimants entered themselves as winners in the claim kernel; only later claimants look at their slot)
+  if (!rec_is_slot(r) || !(r & REC_DUP)) return;
+  const int4 raw = *reinterpret_cast<const int4 *>(&L.table[rec_slot(r)]);
+  if (raw.z >= 0 && raw.z < VAL_PENDING) {  // (the key was there all along; the row had read a stale empty slot)
+    rec[idx] = REC_SITE | (uint32_t)raw.z;
+    return;
   }
-  flag[idx] = f;
-  rep[idx] = w;
+  const int first = raw.w - 1, later = raw.z - VAL_PENDING;
+  if (later == p && p < first) {
+    flag[idx] = 1;
+    flag[lp + first] = 0;
+    rep[lp + first] = p;
+  } else {
+    rep[idx] = first < later ? first : later;
+  }
 }
 
 __global__ __launch_bounds__(256) void frame_assign_kernel(FrameInsertArgs a, const int32_t *__restrict__ coords_in,
@@ -992,9 +1155,9 @@ __global__ __launch_bounds__(256) void frame_assign_kernel(FrameInsertArgs a, co
   int st = -1;
   if (dropped) {
     // the frame is dropped: its claims leave the table, no row gets a site
-    if (r != REC_NONE && !(r & REC_SITE)) {
-      __hip_atomic_store(&L.table[r].val, VAL_UNSET, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      __hip_atomic_store(&L.table[r].key, INSC_EMPTY_KEY, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (rec_is_slot(r)) {
+      __hip_atomic_store(&L.table[rec_slot(r)].val, VAL_UNSET, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(&L.table[rec_slot(r)].key, INSC_EMPTY_KEY, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
   } else if (r != REC_NONE) {
     if (r & REC_SITE) {
@@ -1009,7 +1172,7 @@ __global__ __launch_bounds__(256) void frame_assign_kernel(FrameInsertArgs a, co
           st = id;
           if (win) {
             const int4 c = frame_point(coords_in, cols, p, l);
-            __hip_atomic_store(&L.table[r].val, id, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            L.table[rec_slot(r)].val = id;
             reinterpret_cast<int4 *>(L.coords)[id] = c;
             if (L.offset) L.offset[id] = (c.x & 1) * 4 + (c.y & 1) * 2 + (c.z & 1);
           }
@@ -1040,6 +1203,10 @@ int frame_insert_levels(const FrameInsertLevel *lv, int n_levels, const int32_t 
                 (long long)P, (long long)g->capacity_sites, l);
       return INSC_ERR_CAPACITY;
     }
+    if (g->n_slots > (1ll << 30)) {  // (a row's record keeps the slot in 30 bits)
+      set_error("frame_insert_levels: the table of scale %d has more than 2^30 slots", l);
+      return INSC_ERR_ARG;
+    }
     a.lv[l] = FrameLevelDev{g->table, g->n_slots - 1, g->capacity_sites, g->coords, g->d_n, g->d_err,
                             lv[l].parent, lv[l].offset, lv[l].child};
   }
@@ -1053,12 +1220,13 @@ int frame_insert_levels(const FrameInsertLevel *lv, int n_levels, const int32_t 
   // (frames of many points: from the third scale on the rows of a wavefront share their claims; for a few
   // thousand points the turns this takes cost more than the atomics they save)
   const int shared_from = large ? 2 : 16;
+  int32_t *rep = large ? (int32_t *)(rec + PL) : nullptr, *flag = large ? rep + PL : nullptr;
   hipLaunchKernelGGL(frame_claim_kernel, dim3(grid_for(P, 256), (unsigned)n_levels), dim3(256), 0, s, a, d_coords, cols,
-                     (int)P, d_bad, frame, rec, shared_from);
+                     (int)P, d_bad, frame, rec, shared_from, flag, rep);
   if (large) {
-    int32_t *rep = (int32_t *)(rec + PL), *flag = rep + PL, *n_before = flag + PL + 1;
-    hipLaunchKernelGGL(frame_flag_kernel, dim3(grid_for(P, 256), (unsigned)n_levels), dim3(256), 0, s, a, (int)P,
-                       (const uint32_t *)rec, flag, rep, n_before);
+    int32_t *n_before = flag + PL + 1;
+    hipLaunchKernelGGL(frame_flag_kernel, dim3(grid_for(P, 256), (unsigned)n_levels), dim3(256), 0, s, a, (int)P, rec, flag,
+                       rep, n_before);
     INSC_LAUNCH_CHECK();
     if ((rc = scan_exclusive_i32(flag, flag, (int64_t)PL + 1, nullptr, s))) return rc;
     hipLaunchKernelGGL(frame_assign_kernel, dim3(grid_for(P, 256), (unsigned)n_levels), dim3(256), 0, s, a, d_coords, cols,
@@ -1075,6 +1243,7 @@ int frame_insert_levels(const FrameInsertLevel *lv, int n_levels, const int32_t 
   for (int l = 0; l < n_levels; l++) {
     lv[l].grid->n_upper += P;
     lv[l].grid->n_exact = -1;
+    lv[l].grid->h_fresh = false;
   }
   return INSC_OK;
 }
@@ -1240,6 +1409,8 @@ int insc_grid_create(int64_t capacity_sites, insc_grid **out) {
   INSC_HIP(hipMalloc((void **)&g->coords, sizeof(int32_t) * 4 * (size_t)capacity_sites));
   INSC_HIP(hipMalloc((void **)&g->d_n, 256));
   g->d_err = g->d_n + 16;
+  INSC_HIP(hipHostMalloc((void **)&g->h_n, 64, hipHostMallocDefault));
+  g->h_n[0] = g->h_n[1] = 0;
   *out = g;
   return insc_grid_clear(g, nullptr);
 }
@@ -1250,6 +1421,7 @@ int insc_grid_destroy(insc_grid *g) {
   if (g->table) (void)hipFree(g->table);
   if (g->coords) (void)hipFree(g->coords);
   if (g->d_n) (void)hipFree(g->d_n);
+  if (g->h_n) (void)hipHostFree(g->h_n);
   if (g->slot_of_point) (void)hipFree(g->slot_of_point);
   if (g->flags) (void)hipFree(g->flags);
   delete g;
@@ -1263,6 +1435,7 @@ int insc_grid_clear(insc_grid *g, void *stream) {
   INSC_LAUNCH_CHECK();
   g->n_upper = 0;
   g->n_exact = 0;
+  g->h_fresh = false;
   return INSC_OK;
 }
 
@@ -1272,6 +1445,7 @@ int insc_grid_reserve(insc_grid *g, int64_t capacity_sites, void *stream) {
   if (capacity_sites <= g->capacity_sites) return INSC_OK;
   hipStream_t s = (hipStream_t)stream;
   INSC_HIP(hipStreamSynchronize(s));
+  g->h_fresh = false;
   int32_t *coords = nullptr;
   INSC_HIP(hipMalloc((void **)&coords, sizeof(int32_t) * 4 * (size_t)capacity_sites));
   INSC_HIP(hipMemcpyAsync(coords, g->coords, sizeof(int32_t) * 4 * (size_t)g->capacity_sites,
@@ -1355,12 +1529,14 @@ int insc_grid_insert_noalloc(insc_grid *g, const int32_t *d_coords4, int64_t P, 
                  "insc_grid_reserve first (or insc_grid_size to tighten the bound after inserts with repeats)",
                  (long long)g->n_upper, (long long)P, (long long)g->capacity_sites);
     hipLaunchKernelGGL(grid_claim_kernel, dim3(grid_for(P, 256)), dim3(256), 0, s, g->table, g->n_slots - 1, d_coords4,
-                       P, slot_of_point, g->d_err);
+                       P, slot_of_point, (int32_t *)nullptr, d_site_of_point, g->d_err);
     hipLaunchKernelGGL(grid_finish_small_kernel, dim3(1), dim3(1024), 0, s, g->table, d_coords4, slot_of_point, (int)P,
-                       g->d_n, g->coords, g->capacity_sites, g->d_err, d_site_of_point);
+                       g->d_n, g->coords, g->capacity_sites, g->d_err, d_site_of_point, g->h_n);
     INSC_LAUNCH_CHECK();
     g->n_upper += P;
     g->n_exact = -1;
+    g->h_fresh = g->h_n != nullptr;
+    g->h_stream = (void *)s;
   }
   if (h_n_sites) {
     int rc = grid_sync_errors(g, s, "insc_grid_insert_noalloc");
