@@ -87,6 +87,40 @@ __global__ __launch_bounds__(SCAN_THREADS) void scan_final(const int32_t *__rest
   }
 }
 
+// scan_final for up to SCAN_FUSED_MAX_BLOCKS blocks: every block adds up the sums of the blocks before it by
+// itself (at most 16 loads per thread) instead of reading them from a scan that a launch of its own made;
+// the last block leaves the grand total.
+constexpr int SCAN_FUSED_MAX_BLOCKS = 4096;
+__global__ __launch_bounds__(SCAN_THREADS) void scan_final_fused(const int32_t *__restrict__ in, int32_t *__restrict__ out,
+                                                                 int64_t n, const int32_t *__restrict__ bsums,
+                                                                 int32_t *__restrict__ total) {
+  __shared__ int lds[4];
+  __shared__ int pre_w[4];
+  int pre = 0;
+  for (int i = threadIdx.x; i < (int)blockIdx.x; i += SCAN_THREADS) pre += bsums[i];
+#pragma unroll
+  for (int d = 32; d > 0; d >>= 1) pre += __shfl_xor(pre, d, 64);
+  if ((threadIdx.x & 63) == 0) pre_w[threadIdx.x >> 6] = pre;
+  int64_t base = (int64_t)blockIdx.x * SCAN_TILE + (int64_t)threadIdx.x * SCAN_ITEMS;
+  int v[SCAN_ITEMS];
+  int s = 0;
+#pragma unroll
+  for (int i = 0; i < SCAN_ITEMS; i++) {
+    v[i] = (base + i < n) ? in[base + i] : 0;
+    s += v[i];
+  }
+  int tot;
+  int ex = block_excl_scan(s, &tot, lds);  // (its barriers also publish pre_w)
+  const int before = pre_w[0] + pre_w[1] + pre_w[2] + pre_w[3];
+  ex += before;
+#pragma unroll
+  for (int i = 0; i < SCAN_ITEMS; i++) {
+    if (base + i < n) out[base + i] = ex;
+    ex += v[i];
+  }
+  if (total && blockIdx.x == gridDim.x - 1 && threadIdx.x == 0) *total = before + tot;
+}
+
 __global__ void scan_zero_total(int32_t *total) { *total = 0; }
 
 // Short inputs (the digit counts of a radix pass, the rows of a coarse scale): one workgroup of 1024
@@ -150,8 +184,12 @@ int scan_exclusive_i32(const int32_t *in, int32_t *out, int64_t n, int32_t *tota
   if (rc) return rc;
   int32_t *bsums = (int32_t *)ws;
   hipLaunchKernelGGL(scan_block_sums, dim3((unsigned)nb), dim3(SCAN_THREADS), 0, s, in, n, bsums);
-  hipLaunchKernelGGL(scan_bsums, dim3(1), dim3(SCAN_THREADS), 0, s, bsums, nb, total);
-  hipLaunchKernelGGL(scan_final, dim3((unsigned)nb), dim3(SCAN_THREADS), 0, s, in, out, n, bsums);
+  if (nb <= SCAN_FUSED_MAX_BLOCKS) {
+    hipLaunchKernelGGL(scan_final_fused, dim3((unsigned)nb), dim3(SCAN_THREADS), 0, s, in, out, n, bsums, total);
+  } else {
+    hipLaunchKernelGGL(scan_bsums, dim3(1), dim3(SCAN_THREADS), 0, s, bsums, nb, total);
+    hipLaunchKernelGGL(scan_final, dim3((unsigned)nb), dim3(SCAN_THREADS), 0, s, in, out, n, bsums);
+  }
   INSC_LAUNCH_CHECK();
   return INSC_OK;
 }

@@ -30,7 +30,7 @@ def dev(a, dtype=None):
     return t.cuda()
 
 
-@pytest.mark.parametrize("n", [0, 1, 63, 1023, 1025, 2048, 2049, 32768, 32769, 100003, 3000000])
+@pytest.mark.parametrize("n", [0, 1, 63, 1023, 1025, 2048, 2049, 32768, 32769, 100003, 3000000, 8388608, 8400001])
 def test_scan(S, n):
     from sparseconvnet._lib import lib, ptr, stream_ptr
 
@@ -43,7 +43,7 @@ def test_scan(S, n):
     exp = np.concatenate([[0], np.cumsum(a)[:-1]]) if n else np.zeros(0)
     assert (d_out.cpu().numpy() == exp).all()
     assert int(tot.item()) == int(a.sum())
-    if n:  # in place, as the library's own callers use it (short inputs take one workgroup, long ones three launches)
+    if n:  # in place, as the library's own callers use it (short inputs take one workgroup, longer ones two launches, beyond 8.4 M values three)
         lib.insc_scan_exclusive_i32(ptr(d_in), ptr(d_in), I64(n), None, stream_ptr())
         assert (d_in.cpu().numpy() == exp).all()
 
