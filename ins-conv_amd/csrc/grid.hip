@@ -104,7 +104,8 @@ __global__ void grid_claim_kernel(Slot *table, int64_t mask, const int32_t *__re
           first = k == INSC_EMPTY_KEY;
         }
         if (first) {
-          table[s].pad = (int)p + 1;
+          // (written through, so that later claimants on other XCDs may see it and spare their atomic)
+          __hip_atomic_store(&table[s].pad, (int)p + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           slot = (int32_t)s;
           state = (int32_t)p;
           flag = 1;
@@ -112,7 +113,11 @@ __global__ void grid_claim_kernel(Slot *table, int64_t mask, const int32_t *__re
           break;
         }
         if (k == key) {
-          if (!(seen && raw.z >= VAL_PENDING && raw.z <= VAL_PENDING + (int)p)) atomicMin(&table[s].val, VAL_PENDING + (int)p);
+          // no atomic for a row that has seen a smaller row in the slot - as the first claimant (pad) or
+          // as a later one (val): it cannot be the cell's first row.  (The values only ever go down during
+          // a call, so a stale read errs on the side of one more atomic.)
+          const bool beaten = seen && ((raw.w > 0 && raw.w - 1 < (int)p) || (raw.z >= VAL_PENDING && raw.z <= VAL_PENDING + (int)p));
+          if (!beaten) atomicMin(&table[s].val, VAL_PENDING + (int)p);
           slot = (int32_t)s;
           state = ST_DUP;
           full = false;
@@ -884,11 +889,12 @@ __device__ __forceinline__ int4 frame_point(const int32_t *__restrict__ coords_i
 __global__ __launch_bounds__(256) void frame_claim_kernel(FrameInsertArgs a, const int32_t *__restrict__ coords_in,
                                                           int cols, int P, int32_t *__restrict__ bad, int32_t frame,
                                                           uint32_t *__restrict__ rec, int shared_from,
-                                                          int32_t *__restrict__ flag, int32_t *__restrict__ rep) {
+                                                          int32_t *__restrict__ flag, int32_t *__restrict__ rep,
+                                                          int p_begin, int p_end) {
   const int l = blockIdx.y;
   const FrameLevelDev &L = a.lv[l];
-  const int p = blockIdx.x * 256 + threadIdx.x;
-  if (p >= P) return;
+  const int p = p_begin + blockIdx.x * 256 + threadIdx.x;  // (this launch serves rows p_begin .. p_end - 1)
+  if (p >= p_end) return;
   const int64_t idx = (int64_t)l * P + p;
   const int32_t *c0 = coords_in + (int64_t)p * cols;
   if (!coord_ok(c0[0], c0[1], c0[2], cols > 3 ? c0[3] : 0)) {
@@ -912,14 +918,16 @@ __global__ __launch_bounds__(256) void frame_claim_kernel(FrameInsertArgs a, con
       if (k == INSC_EMPTY_KEY) {
         k = atomicCAS(&L.table[s].key, INSC_EMPTY_KEY, (unsigned long long)key);
         if (k == INSC_EMPTY_KEY) {  // first claimant
-          L.table[s].pad = p + 1;
+          __hip_atomic_store(&L.table[s].pad, p + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           return (uint32_t)s;
         }
       }
       if (k == key) {
-        // (the claim of a smaller row that this row has seen stands: the value only ever goes down, so a
-        // stale read errs on the side of one more atomic)
-        if (!(seen && raw.z >= VAL_PENDING && raw.z <= VAL_PENDING + p)) atomicMin(&L.table[s].val, VAL_PENDING + p);
+        // (a smaller row that this row has seen in the slot - first claimant in pad, later one in val -
+        // stands: the values only ever go down during a frame, so a stale read errs on the side of one
+        // more atomic; a dropped frame takes its pads out again)
+        const bool beaten = seen && ((raw.w > 0 && raw.w - 1 < p) || (raw.z >= VAL_PENDING && raw.z <= VAL_PENDING + p));
+        if (!beaten) atomicMin(&L.table[s].val, VAL_PENDING + p);
         return REC_DUP | (uint32_t)s;
       }
       s = (s + 1) & L.mask;
@@ -930,27 +938,25 @@ __global__ __launch_bounds__(256) void frame_claim_kernel(FrameInsertArgs a, con
   if (l < shared_from) {
     r = claim();
   } else {
-    // From the third scale on, neighbouring rows mostly fall into the same cell (at the coarsest scale of
-    // a full frame thousands of rows per cell), and atomics on one address are served one at a time: the
-    // rows of a wavefront that share a cell send one claim, that of their first lane - the smallest row,
-    // rows ascending with the lanes - and all take its answer (the others as later claimants: whoever
-    // numbers the cell, it is not one of them).
-    bool todo = true;
+    // Above the input scale the rows of a wavefront often fall into the same cell (at the coarsest scale
+    // of a full frame thousands of rows per cell), and atomics on one address are served one at a time.
+    // Of the lanes that share a cell only the first - the smallest row, rows ascending with the lanes -
+    // sends a claim, and the others take its answer, as later claimants: whoever numbers the cell, it is
+    // not one of them.  Finding the first lane of every cell takes 64 broadcasts and no memory access,
+    // and the first lanes then claim side by side.
     const int lane = (int)(threadIdx.x & 63);
-    while (todo) {  // (lanes leave as their cell is served; every turn serves the first waiting lane's cell)
-      const uint64_t waiting = __ballot(true);
-      const int leader = (int)__builtin_ctzll(waiting);
-      const uint32_t klo = (uint32_t)__shfl((int)(uint32_t)key, leader, 64);
-      const uint32_t khi = (uint32_t)__shfl((int)(uint32_t)(key >> 32), leader, 64);
-      const bool same = key == (((uint64_t)khi << 32) | klo);
-      uint32_t mine = REC_NONE;
-      if (lane == leader) mine = claim();
-      const uint32_t got = (uint32_t)__shfl((int)mine, leader, 64);
-      if (same) {
-        r = (lane == leader || !rec_is_slot(got)) ? got : (got | REC_DUP);
-        todo = false;
-      }
+    const uint32_t klo = (uint32_t)key, khi = (uint32_t)(key >> 32);
+    int leader = lane;
+    const uint64_t live = __ballot(true);
+    for (int i = 0; i < 64; i++) {
+      if (!((live >> i) & 1ull)) continue;  // (uniform)
+      const uint32_t ilo = (uint32_t)__builtin_amdgcn_readlane((int)klo, i), ihi = (uint32_t)__builtin_amdgcn_readlane((int)khi, i);
+      if (i < leader && ilo == klo && ihi == khi) leader = i;
     }
+    uint32_t mine = REC_NONE;
+    if (lane == leader) mine = claim();
+    const uint32_t got = (uint32_t)__shfl((int)mine, leader, 64);
+    r = (lane == leader || !rec_is_slot(got)) ? got : (got | REC_DUP);
   }
   if (r == REC_NONE) atomicOr(L.d_err, 2);
   rec[idx] = r;
@@ -985,6 +991,7 @@ __global__ __launch_bounds__(1024) void frame_finish_kernel(FrameInsertArgs a, c
       if (j >= per || p0 + j >= P) continue;
       if (rec_is_slot(rr[j])) {
         __hip_atomic_store(&L.table[rec_slot(rr[j])].val, VAL_UNSET, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(&L.table[rec_slot(rr[j])].pad, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __hip_atomic_store(&L.table[rec_slot(rr[j])].key, INSC_EMPTY_KEY, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
       site[p0 + j] = -1;
@@ -1183,6 +1190,7 @@ __global__ __launch_bounds__(256) void frame_assign_kernel(FrameInsertArgs a, co
     // the frame is dropped: its claims leave the table, no row gets a site
     if (rec_is_slot(r)) {
       __hip_atomic_store(&L.table[rec_slot(r)].val, VAL_UNSET, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(&L.table[rec_slot(r)].pad, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       __hip_atomic_store(&L.table[rec_slot(r)].key, INSC_EMPTY_KEY, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
   } else if (r != REC_NONE) {
@@ -1243,12 +1251,22 @@ int frame_insert_levels(const FrameInsertLevel *lv, int n_levels, const int32_t 
   if (rc) return rc;
   int32_t *site = (int32_t *)ws;
   uint32_t *rec = (uint32_t *)(site + PL);
-  // (frames of many points: from the third scale on the rows of a wavefront share their claims; for a few
-  // thousand points the turns this takes cost more than the atomics they save)
-  const int shared_from = large ? 2 : 16;
+  // (above the input scale the rows of a wavefront that fall into one cell share a claim)
+  const int shared_from = 1;
   int32_t *rep = large ? (int32_t *)(rec + PL) : nullptr, *flag = large ? rep + PL : nullptr;
-  hipLaunchKernelGGL(frame_claim_kernel, dim3(grid_for(P, 256), (unsigned)n_levels), dim3(256), 0, s, a, d_coords, cols,
-                     (int)P, d_bad, frame, rec, shared_from, flag, rep);
+  // The claims are bound by the rate of atomics on scattered addresses (some 6 per nanosecond on this
+  // part, whatever their width or scope), and with all rows in flight at once every row of a cell sends
+  // one: 7 x 165 000 for a full frame of a 7-scale network, though its coarse scales hold a few thousand
+  // cells.  A cell's first row is its smallest, so the first sixteenth of the rows go ahead in a launch
+  // of their own: they claim nearly every cell of the coarse scales, and the rows of the second launch,
+  // which find a smaller row there, send nothing.  165 000 points at 7 scales: 132 us in one launch,
+  // 18 + 64 us in two (a sixty-fourth of the rows first: 13 + 79 us; a quarter: 43 + 49 us).
+  const int64_t head = large ? std::max<int64_t>(P / 16, 1024) : P;
+  for (int part = 0; part < (head < P ? 2 : 1); part++) {
+    const int64_t b = part ? head : 0, e = (part || head >= P) ? P : head;
+    hipLaunchKernelGGL(frame_claim_kernel, dim3(grid_for(e - b, 256), (unsigned)n_levels), dim3(256), 0, s, a, d_coords,
+                       cols, (int)P, d_bad, frame, rec, shared_from, flag, rep, (int)b, (int)e);
+  }
   if (large) {
     int32_t *n_before = flag + PL + 1;
     hipLaunchKernelGGL(frame_flag_kernel, dim3(grid_for(P, 256), (unsigned)n_levels), dim3(256), 0, s, a, (int)P, rec, flag,
