@@ -530,7 +530,10 @@ static int run_op(insc_net *net, const Op &op, bool incremental, hipStream_t s) 
   const Level &Lo = net->levels[To.level];
   // (a set known to hold every row needs no flags: the layer runs as in a full frame)
   const DirtyNode *d = incremental && !net->dirty_full[(size_t)To.dirty] ? &net->dirty[To.dirty] : nullptr;
-  const int32_t *d_n = Lo.grid->d_n;
+  // (the host has had the exact site counts since the structure phase - apply_counts - so the layers take
+  // their row count by value: a kernel that starts by loading it from device memory has one more
+  // dependent memory round trip ahead of its first useful load)
+  const int32_t *d_n = nullptr;
   const int64_t n_up = Lo.n_upper;
   // a convolution that also forms the sum of its residual block writes what the OP_ADD would
   const Op *add = op.fused_add >= 0 ? &net->ops[op.fused_add] : nullptr;
