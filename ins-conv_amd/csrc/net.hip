@@ -1178,12 +1178,6 @@ int insc_net_forward(insc_net *net, const int32_t *d_coords, int coord_cols, con
   }
   if ((rc = points_reserve(net, net->n_points + P, s))) return rc;
 
-  if (inc && net->mask_arena_bytes) {
-    hipLaunchKernelGGL(fill_bytes_kernel, dim3(1024), dim3(256), 0, s, (uint4 *)net->mask_arena,
-                       net->mask_arena_bytes / 16);
-    INSC_LAUNCH_CHECK();
-  }
-
   if (net->profiling) INSC_HIP(hipEventRecord(net->ev[0], s));
   int32_t *sop = net->site_of_point + net->n_points;
   net->frame_sop = sop;
@@ -1202,6 +1196,15 @@ int insc_net_forward(insc_net *net, const int32_t *d_coords, int coord_cols, con
         return rc;
       INSC_HIP(hipEventRecord(net->ev_counts, s));
     }
+  }
+  // the dirty masks, tile flags and list counters of the last frame go back to zero (behind the insert:
+  // nothing before the input accumulation reads them, and the host gets its site counts that much earlier)
+  if (inc && net->mask_arena_bytes) {
+    hipLaunchKernelGGL(fill_bytes_kernel, dim3(1024), dim3(256), 0, s, (uint4 *)net->mask_arena,
+                       net->mask_arena_bytes / 16);
+    INSC_LAUNCH_CHECK();
+  }
+  if (P > 0) {
     // ---- neighbour maps and processing orders of the new sites, all scales per launch ------
     const insc_grid *grids[16];
     int32_t *nbrs[16], *orders[16], *poss[16], *bo_orders[16], *bo_poss[16];
