@@ -696,7 +696,10 @@ __global__ __launch_bounds__((S == 1 ? CONV_WAVES : S) * 64) void conv_mfma_kern
 // The sums are formed exactly as in conv_mfma_kernel<1, 27, MAP_NBR, 1> (offsets ascending,
 // same MFMA sequence), so both kernels give the same bits.
 // ---------------------------------------------------------------------------------------
-constexpr int WL_WAVES = 12;
+#ifndef INSC_WL_WAVES
+#define INSC_WL_WAVES 12
+#endif
+constexpr int WL_WAVES = INSC_WL_WAVES;
 #ifndef INSC_WL_DEPTH
 #define INSC_WL_DEPTH 4
 #endif
