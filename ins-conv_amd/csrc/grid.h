@@ -11,8 +11,6 @@ struct __attribute__((aligned(16))) Slot {
 };
 
 constexpr int VAL_UNSET = 0x7FFFFFFF;
-// At load <= 0.5 probe runs are a handful of slots; the cap only bounds a corrupted table.
-constexpr int64_t MAX_PROBES = 1 << 16;
 constexpr int VAL_PENDING = 0x40000000;  // VAL_PENDING + p : claimed during this insert by row p
 
 }  // namespace insc
@@ -35,6 +33,7 @@ struct insc_grid {
   int32_t *slot_of_point = nullptr;
   int32_t *flags = nullptr;
   int64_t scratch_rows = 0;
+  int32_t *part = nullptr;  // partition counters and offsets of the large insert (PART_INTS words, zero between calls)
   int device = 0;
 };
 

@@ -3,7 +3,19 @@
 // Home slot: the eight voxels (x, y, z0..z0+7) of one z-run share one aligned group of eight
 // slots (128 bytes, one L2 line), voxel z at position z&7.  The three z-neighbours of a
 // 3x3x3 query therefore read the same line, and the lanes of a wavefront that handle
-// consecutive filter offsets probe it together.  Collisions move on linearly.
+// consecutive filter offsets probe it together.
+//
+// Probe order: a key stays inside the aligned run of PART_SLOTS slots that holds its home slot (the whole
+// table if it is smaller) - its partition - which lets a large insert build the table partition by
+// partition in LDS (part_* kernels below).  From a taken slot it moves on by an odd number of groups (taken
+// from hash bits the home slot does not use) and one position inside the group; once it has seen as many
+// slots as the partition has groups it walks the partition slot by slot from the home slot, so that every
+// slot is reached (never seen in practice: at load <= 0.5 that takes a hundred-odd taken slots in a row).
+// Moving on to the neighbouring slot instead - plain linear probing - does badly with these homes: the
+// groups of a scene fill up whole, so a key whose home group is shared sits eight or more slots away
+// (200 000 voxels of a room in 2^20 slots: 4 % of the keys at 8 or more probes, 1 % at 16 or more, which
+// is what nearly every wavefront then waits for; this way 9 % of the keys take a second probe and the
+// longest walk is 8).
 //
 // Numbering: a site's id is its rank among first occurrences in the inserted list, offset by
 // the count before the call - deterministic and append-only.
@@ -23,21 +35,49 @@ __device__ __forceinline__ uint64_t mix64(uint64_t h) {
   return h;
 }
 
-__device__ __forceinline__ int64_t home_slot(uint64_t key, int64_t mask) {
-  // drop z's low three bits from the hashed part, put them back as the position in the group
-  uint64_t zlow = (key >> 32) & 7ull;
-  uint64_t h = mix64(key & ~(7ull << 32));
-  return (int64_t)(((h << 3) | zlow) & (uint64_t)mask);
+constexpr int PART_SHIFT = 11;
+constexpr int64_t PART_SLOTS = 1ll << PART_SHIFT;
+
+struct Walk {
+  int64_t part;            // first slot of the key's partition
+  int wm;                  // slots of a partition - 1
+  int home, loc, step, i;  // slots inside the partition: home, current; groups to move on by; probes so far
+};
+__device__ __forceinline__ Walk walk_begin(uint64_t key, int64_t mask) {
+  // z's low three bits stay out of the hashed part and come back as the position in the group
+  const uint64_t zlow = (key >> 32) & 7ull;
+  const uint64_t h = mix64(key & ~(7ull << 32));
+  const int64_t home = (int64_t)(((h << 3) | zlow) & (uint64_t)mask);
+  Walk w;
+  w.wm = (int)(mask < PART_SLOTS - 1 ? mask : PART_SLOTS - 1);
+  w.part = home & ~(int64_t)w.wm;
+  w.home = w.loc = (int)(home & w.wm);
+  w.step = (int)(h >> 44) | 1;
+  w.i = 0;
+  return w;
+}
+__device__ __forceinline__ int64_t walk_slot(const Walk &w) { return w.part + w.loc; }
+// the next slot to look at; false: the whole partition has been seen
+__device__ __forceinline__ bool walk_next(Walk &w) {
+  const int groups = (w.wm + 1) >> 3;
+  w.i++;
+  if (w.i < groups) {
+    w.loc = ((((w.loc >> 3) + w.step) & (groups - 1)) << 3) | ((w.loc + 1) & 7);
+    return true;
+  }
+  if (w.i > groups + w.wm) return false;
+  w.loc = (w.home + (w.i - groups)) & w.wm;
+  return true;
 }
 
 __device__ __forceinline__ int grid_find(const Slot *__restrict__ table, int64_t mask, uint64_t key) {
-  int64_t s = home_slot(key, mask);
-  for (int64_t probe = 0; probe <= mask && probe < MAX_PROBES; probe++) {
+  Walk w = walk_begin(key, mask);
+  do {
+    const int64_t s = walk_slot(w);
     unsigned long long k = table[s].key;
     if (k == key) return table[s].val;
     if (k == INSC_EMPTY_KEY) return -1;
-    s = (s + 1) & mask;
-  }
+  } while (walk_next(w));
   return -1;
 }
 
@@ -86,9 +126,10 @@ __global__ void grid_claim_kernel(Slot *table, int64_t mask, const int32_t *__re
       atomicOr(d_err, 1);
     } else {
       const uint64_t key = pack_key(c.x, c.y, c.z, c.w);
-      int64_t s = home_slot(key, mask);
+      Walk w = walk_begin(key, mask);
       bool full = true;
-      for (int64_t probe = 0; probe <= mask && probe < MAX_PROBES; probe++) {
+      do {
+        const int64_t s = walk_slot(w);
         const int4 raw = *reinterpret_cast<const int4 *>(&table[s]);  // key (two words), val, pad
         unsigned long long k = ((unsigned long long)(unsigned)raw.y << 32) | (unsigned)raw.x;
         const bool seen = k == key;
@@ -123,8 +164,7 @@ __global__ void grid_claim_kernel(Slot *table, int64_t mask, const int32_t *__re
           full = false;
           break;
         }
-        s = (s + 1) & mask;
-      }
+      } while (walk_next(w));
       if (full) atomicOr(d_err, 2);
     }
   }
@@ -296,45 +336,291 @@ __global__ __launch_bounds__(1024) void grid_finish_small_kernel(Slot *table, co
   }
 }
 
-// Point query, wavefront-cooperative: eight lanes per query.  The lanes of a group read the eight slots of
-// one aligned group of the table - 128 bytes, one line, one request - starting with the group that holds
-// the key's home slot; they ballot "holds the key" and "is empty" over the slots at or after the home slot
-// (a key sits before the first empty slot at or after its home: slots are never emptied under a key) and
-// move on to the next group while they have seen neither.  Measured against one thread per query walking
-// the slots one by one, on 220 000 queries into 200 000 sites: 13.3 against 17.0 us, hits or misses, at
-// load 0.19 and 0.38 alike.
+// ---- large inserts: the table built partition by partition in LDS -----------------------------
+// The claim kernel above sends one atomic per point to a slot somewhere in the table; the lines of the
+// table travel between the L2s of the chip's dies for it (measured on 220 000 points into 2^20 slots:
+// 29 MB fetched and 24 MB written for 3.5 MB of points, 43 us).  A large insert sorts its rows by home
+// partition first (count, scatter: coalesced passes with LDS histograms) and then one workgroup per
+// partition plays the same protocol on a copy of its PART_SLOTS slots in LDS: winners (the smallest
+// row of every new cell), the prefix sum over the rows' winner flags that ranks them, and a second
+// build that stores the numbered slots - the only time the table itself is touched.
+constexpr int PART_MAX = 4096;   // partitions of the largest table that takes this path
+constexpr int PART_PAD = 16;     // ints between two partitions' counters (their atomics spread over the L2 channels)
+constexpr int PART_ROWS = 4;     // rows per thread of count / scatter
+constexpr int PART_INTS = 2 * PART_MAX * PART_PAD + PART_MAX + 64;  // cnt | cursor | base
+
+__device__ __forceinline__ int part_of_row(const int32_t *__restrict__ coords4, int64_t p, int64_t mask, int32_t *d_err,
+                                           bool report, uint64_t *key_out = nullptr) {
+  const int4 c = reinterpret_cast<const int4 *>(coords4)[p];
+  if (c.x == COORD_SKIP) return -1;
+  if (!coord_ok(c.x, c.y, c.z, c.w)) {
+    if (report) atomicOr(d_err, 1);
+    return -1;
+  }
+  const uint64_t key = pack_key(c.x, c.y, c.z, c.w);
+  if (key_out) *key_out = key;
+  return (int)(walk_begin(key, mask).part >> PART_SHIFT);
+}
+__device__ __forceinline__ int4 unpack_key(uint64_t key) {
+  return make_int4((int)(key & 0xFFFF), (int)((key >> 16) & 0xFFFF), (int)((key >> 32) & 0xFFFF), (int)(key >> 48));
+}
+
+// rows per partition
+__global__ __launch_bounds__(1024) void part_count_kernel(const int32_t *__restrict__ coords4, int64_t P, int64_t mask,
+                                                          int n_parts, int32_t *cnt, int32_t *d_err) {
+  extern __shared__ int32_t hist[];
+  const int tid = threadIdx.x;
+  for (int i = tid; i < n_parts; i += 1024) hist[i] = 0;
+  __syncthreads();
+#pragma unroll
+  for (int j = 0; j < PART_ROWS; j++) {
+    const int64_t p = ((int64_t)blockIdx.x * PART_ROWS + j) * 1024 + tid;
+    if (p >= P) break;
+    const int q = part_of_row(coords4, p, mask, d_err, true);
+    if (q >= 0) atomicAdd(&hist[q], 1);
+  }
+  __syncthreads();
+  for (int i = tid; i < n_parts; i += 1024)
+    if (hist[i]) atomicAdd(&cnt[i * PART_PAD], hist[i]);
+}
+
+// rows and their keys sorted by partition (any order inside one), so that the kernels that follow read them
+// in order instead of gathering coordinates (with all workgroups gathering at once, the slowest took 13 us
+// over it); the rows that go nowhere get their answer here.  Every
+// workgroup turns the counts into offsets for itself (a prefix sum over at most PART_MAX values; a
+// single workgroup doing it for all would have to publish them through a fence that writes the L2 back,
+// measured 15 us), the first one stores them for the kernels that follow.
+__global__ __launch_bounds__(1024) void part_scatter_kernel(const int32_t *__restrict__ coords4, int64_t P, int64_t mask,
+                                                            int n_parts, const int32_t *__restrict__ cnt, int32_t *cursor,
+                                                            int32_t *__restrict__ base, int32_t *__restrict__ part_rows,
+                                                            uint64_t *__restrict__ part_keys,
+                                                            int32_t *__restrict__ site_of_point, int32_t *__restrict__ flags) {
+  extern __shared__ int32_t lds[];
+  int32_t *hist = lds, *off = lds + n_parts;
+  __shared__ int wave_total[16];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  for (int i = tid; i < n_parts; i += 1024) hist[i] = 0;
+  // exclusive prefix sum of the counts: thread t takes partitions 4t .. 4t+3
+  int v[4], sum = 0;
+#pragma unroll
+  for (int j = 0; j < 4; j++) {
+    const int i = tid * 4 + j;
+    v[j] = i < n_parts ? cnt[i * PART_PAD] : 0;
+    sum += v[j];
+  }
+  int incl = sum;
+  for (int d = 1; d < 64; d <<= 1) {
+    const int u = __shfl_up(incl, d, 64);
+    if (lane >= d) incl += u;
+  }
+  if (lane == 63) wave_total[wave] = incl;
+  __syncthreads();
+  int run = incl - sum;
+  for (int w = 0; w < wave; w++) run += wave_total[w];
+#pragma unroll
+  for (int j = 0; j < 4; j++) {
+    const int i = tid * 4 + j;
+    if (i < n_parts) {
+      off[i] = run;
+      if (blockIdx.x == 0) base[i] = run;
+      run += v[j];
+    }
+  }
+  if (blockIdx.x == 0 && tid == 1023) base[n_parts] = run;  // (the last thread's total: all rows that go somewhere)
+  int q[PART_ROWS], r[PART_ROWS];
+  uint64_t key[PART_ROWS];
+#pragma unroll
+  for (int j = 0; j < PART_ROWS; j++) {
+    const int64_t p = ((int64_t)blockIdx.x * PART_ROWS + j) * 1024 + tid;
+    q[j] = -2;
+    if (p >= P) continue;
+    q[j] = part_of_row(coords4, p, mask, nullptr, false, &key[j]);
+    if (q[j] >= 0) {
+      r[j] = atomicAdd(&hist[q[j]], 1);
+    } else {
+      site_of_point[p] = -1;
+      flags[p] = 0;
+    }
+  }
+  __syncthreads();
+  for (int i = tid; i < n_parts; i += 1024)
+    if (hist[i]) off[i] += atomicAdd(&cursor[i * PART_PAD], hist[i]);
+  __syncthreads();
+#pragma unroll
+  for (int j = 0; j < PART_ROWS; j++) {
+    const int64_t p = ((int64_t)blockIdx.x * PART_ROWS + j) * 1024 + tid;
+    if (q[j] >= 0) {
+      const int at = off[q[j]] + r[j];
+      part_rows[at] = (int32_t)p;
+      part_keys[at] = key[j];
+    }
+  }
+}
+
+// slot of `key` in the LDS copy of its partition, claiming the first empty slot of its walk; -1: full
+__device__ __forceinline__ int part_slot(unsigned long long *keys, unsigned long long key, int64_t mask) {
+  Walk w = walk_begin(key, mask);
+  do {
+    unsigned long long k = keys[w.loc];
+    if (k == INSC_EMPTY_KEY) {
+      k = atomicCAS(&keys[w.loc], INSC_EMPTY_KEY, key);
+      if (k == INSC_EMPTY_KEY) return w.loc;
+    }
+    if (k == key) return w.loc;
+  } while (walk_next(w));
+  return -1;
+}
+
+// One workgroup per partition plays the insert on a copy of the partition's slots in LDS - as they are
+// in the table (load), or empty; a slot that holds a key without an id (left by a call that ran out of
+// room) counts as holding the key, to be numbered by this call.  Per row, in partition order: state =
+// the smallest row of the row's cell (flags 1 for that row itself), -2 - id for a cell numbered earlier,
+// -1 if the partition is full; where = the cell's slot in the table.  Leaves the partition's counters zero.
+#ifndef PART_THREADS_V
+#define PART_THREADS_V 512
+#endif
+constexpr int PART_THREADS = PART_THREADS_V;
+#ifdef PART_DEBUG
+__device__ long long part_dbg[4096 * 8];
+#define PDBG(k) if (tid == 0) part_dbg[q * 8 + (k)] = wall_clock64()
+#else
+#define PDBG(k)
+#endif
+#ifndef PART_KEEP_V
+#define PART_KEEP_V 2
+#endif
+constexpr int PART_KEEP = PART_KEEP_V;  // rows per thread kept in registers between the two passes (more are looked up again)
+__global__ __launch_bounds__(PART_THREADS) void part_winners_kernel(
+    const Slot *__restrict__ table, int64_t mask, int load, const int32_t *__restrict__ base,
+    const int32_t *__restrict__ part_rows, const uint64_t *__restrict__ part_keys, const int32_t *__restrict__ d_n,
+    int32_t *__restrict__ flags, int32_t *__restrict__ state, int32_t *__restrict__ where, int32_t *cnt, int32_t *cursor,
+    int32_t *__restrict__ n_before, int32_t *d_err) {
+  __shared__ unsigned long long keys[PART_SLOTS];
+  __shared__ int vals[PART_SLOTS];
+  const int q = blockIdx.x, tid = threadIdx.x;
+  const int W = (int)(mask < PART_SLOTS - 1 ? mask + 1 : PART_SLOTS);
+  PDBG(0);
+  const int b0 = base[q], b1 = base[q + 1];
+  if (tid == 0) {
+    if (q == 0) *n_before = d_n[0];
+    cnt[q * PART_PAD] = 0;
+    cursor[q * PART_PAD] = 0;
+  }
+  int pr[PART_KEEP], sr[PART_KEEP];
+  uint64_t kr[PART_KEEP];
+#pragma unroll
+  for (int j = 0; j < PART_KEEP; j++) {
+    const int i = b0 + j * PART_THREADS + tid;
+    pr[j] = i < b1 ? part_rows[i] : -1;
+    kr[j] = i < b1 ? part_keys[i] : 0;
+  }
+  const Slot *slab = table + (int64_t)q * W;
+  for (int i = tid; i < W; i += PART_THREADS) {
+    unsigned long long k = INSC_EMPTY_KEY;
+    int v = VAL_UNSET;
+    if (load) {
+      const int4 raw = *reinterpret_cast<const int4 *>(&slab[i]);
+      k = ((unsigned long long)(unsigned)raw.y << 32) | (unsigned)raw.x;
+      if (raw.z >= 0 && raw.z < VAL_PENDING) v = raw.z;
+    }
+    keys[i] = k;
+    vals[i] = v;
+  }
+#ifdef PART_DEBUG
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#endif
+  PDBG(1);
+  __syncthreads();
+  PDBG(2);
+  auto claim = [&](int p, const uint64_t key) -> int {
+    const int s = part_slot(keys, key, mask);
+    if (s < 0)
+      atomicOr(d_err, 2);
+    else if (!load || vals[s] >= VAL_PENDING)  // (ids were there before the loop and stay)
+      atomicMin(&vals[s], VAL_PENDING + p);
+    return s;
+  };
+  auto answer = [&](int i, int p, int s) {
+    int st = -1;
+    if (s >= 0) {
+      const int v = vals[s];
+      st = v < VAL_PENDING ? -2 - v : v - VAL_PENDING;
+    }
+    state[i] = st;
+    where[i] = s < 0 ? -1 : (int)((int64_t)q * W + s);
+    flags[p] = st == p ? 1 : 0;
+  };
+#pragma unroll
+  for (int j = 0; j < PART_KEEP; j++)
+    if (pr[j] >= 0) sr[j] = claim(pr[j], kr[j]);
+  PDBG(3);
+  for (int i = b0 + PART_KEEP * PART_THREADS + tid; i < b1; i += PART_THREADS) claim(part_rows[i], part_keys[i]);
+  __syncthreads();
+  PDBG(4);
+#pragma unroll
+  for (int j = 0; j < PART_KEEP; j++)
+    if (pr[j] >= 0) answer(b0 + j * PART_THREADS + tid, pr[j], sr[j]);
+  for (int i = b0 + PART_KEEP * PART_THREADS + tid; i < b1; i += PART_THREADS) {
+    const uint64_t key = part_keys[i];
+    answer(i, part_rows[i], part_slot(keys, key, mask));  // (finds what the first pass left)
+  }
+  PDBG(5);
+}
+
+// numbered: every row takes id = n_before + rank of its cell's winner; the winners store their slots
+// (16 bytes each, the only writes to the table) and their coordinates; the first thread moves the
+// counters on (as grid_assign_kernel).  One thread per row, in partition order.
+__global__ __launch_bounds__(256) void part_assign_kernel(Slot *table, const int32_t *__restrict__ base, int n_parts,
+                                                          const int32_t *__restrict__ part_rows,
+                                                          const uint64_t *__restrict__ part_keys,
+                                                          const int32_t *__restrict__ state,
+                                                          const int32_t *__restrict__ where,
+                                                          const int32_t *__restrict__ excl, int32_t *__restrict__ d_n,
+                                                          const int32_t *__restrict__ total,
+                                                          int32_t *__restrict__ site_coords, int64_t capacity_sites,
+                                                          int32_t *d_err, int32_t *__restrict__ site_of_point,
+                                                          int32_t *__restrict__ h_n) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int n_before = total[1];
+  if (i == 0) {
+    const bool over = (int64_t)n_before + total[0] > capacity_sites;
+    const int n_new = over ? (int)(capacity_sites - n_before) : total[0];
+    d_n[1] = n_before;
+    d_n[0] = n_before + n_new;
+    if (h_n) {
+      h_n[0] = n_before + n_new;
+      h_n[1] = __hip_atomic_load(d_err, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) | (over ? 2 : 0);
+    }
+  }
+  if (i >= base[n_parts]) return;
+  const int p = part_rows[i], r = state[i];
+  if (r < 0) {
+    site_of_point[p] = r < -1 ? -2 - r : -1;
+    return;
+  }
+  const int id = n_before + excl[r];
+  if (id >= capacity_sites) {
+    site_of_point[p] = -1;
+    if (r == p) atomicOr(d_err, 2);
+    return;
+  }
+  site_of_point[p] = id;
+  if (r != p) return;
+  const uint64_t key = part_keys[i];
+  *reinterpret_cast<int4 *>(&table[where[i]]) = make_int4((int)(uint32_t)key, (int)(uint32_t)(key >> 32), id, 0);
+  reinterpret_cast<int4 *>(site_coords)[id] = unpack_key(key);
+}
+
+// Point query, one thread per query.  (Eight lanes per query reading a whole group of the table at once paid
+// while keys sat up to dozens of slots from home in the same and the following lines; with walks of one
+// or two probes, each in a line of its own, there is nothing to share.)
 __global__ __launch_bounds__(256) void grid_query_kernel(const Slot *__restrict__ table, int64_t mask,
                                                          const int32_t *__restrict__ coords4, int64_t Q,
                                                          int32_t *__restrict__ out) {
-  const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  const int64_t q = t >> 3;
-  const int sub = (int)(t & 7), g0 = (int)(threadIdx.x & 63) & ~7;  // lane inside the group; the group's first lane
-  const bool live = q < Q;
-  const int4 c = live ? reinterpret_cast<const int4 *>(coords4)[q] : make_int4(0, 0, 0, 0);
-  const bool ok = live && coord_ok(c.x, c.y, c.z, c.w);
-  const uint64_t key = ok ? pack_key(c.x, c.y, c.z, c.w) : 0;
-  const int64_t home = ok ? home_slot(key, mask) : 0;
-  int64_t s = home & ~(int64_t)7;  // first slot of the table group being looked at
-  int from = (int)(home & 7);      // slots of that group before this one do not count (first group only)
-  int r = -1;
-  bool done = !ok;  // (the lanes of a group agree on `done`; groups that are done ride along in the ballots)
-  for (int64_t probe = 0; probe <= mask && probe < MAX_PROBES; probe += 8) {
-    if (__ballot(!done) == 0) break;
-    const int4 raw = *reinterpret_cast<const int4 *>(&table[s + sub]);  // key (two words), val, pad
-    const unsigned long long k = ((unsigned long long)(unsigned)raw.y << 32) | (unsigned)raw.x;
-    const bool counts = !done && sub >= from;
-    const unsigned hit = (unsigned)((__ballot(counts && k == key) >> g0) & 0xFF);
-    const unsigned empty = (unsigned)((__ballot(counts && k == INSC_EMPTY_KEY) >> g0) & 0xFF);
-    const int hi = hit ? __builtin_ctz(hit) : 8, ei = empty ? __builtin_ctz(empty) : 8;
-    const int v = __shfl(raw.z, g0 + (hi & 7), 64);
-    if (!done) {
-      if (hi < ei) r = v;
-      done = hi < 8 || ei < 8;
-    }
-    s = (s + 8) & mask;
-    from = 0;
-  }
-  if (live && sub == 0) out[q] = r;
+  const int64_t q = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (q >= Q) return;
+  const int4 c = reinterpret_cast<const int4 *>(coords4)[q];
+  out[q] = coord_ok(c.x, c.y, c.z, c.w) ? grid_find(table, mask, pack_key(c.x, c.y, c.z, c.w)) : -1;
 }
 
 // re-insert site i with value i (used after a resize; keys are unique so no min is needed)
@@ -344,15 +630,15 @@ __global__ void grid_rehash_kernel(Slot *table, int64_t mask, const int32_t *__r
   if (i >= *d_n) return;
   int4 c = reinterpret_cast<const int4 *>(site_coords)[i];
   uint64_t key = pack_key(c.x, c.y, c.z, c.w);
-  int64_t s = home_slot(key, mask);
-  for (int64_t probe = 0; probe <= mask && probe < MAX_PROBES; probe++) {
+  Walk w = walk_begin(key, mask);
+  do {
+    const int64_t s = walk_slot(w);
     unsigned long long k = atomicCAS(&table[s].key, INSC_EMPTY_KEY, (unsigned long long)key);
     if (k == INSC_EMPTY_KEY) {
       table[s].val = (int)i;
       return;
     }
-    s = (s + 1) & mask;
-  }
+  } while (walk_next(w));
   atomicOr(d_err, 2);
 }
 
@@ -554,8 +840,9 @@ static int grid_ensure_scratch(insc_grid *g, int64_t P, hipStream_t s) {
     if (g->slot_of_point) INSC_HIP(hipFree(g->slot_of_point));
     if (g->flags) INSC_HIP(hipFree(g->flags));
     g->slot_of_point = g->flags = nullptr;
-    int64_t rows = P + P / 2;
-    INSC_HIP(hipMalloc((void **)&g->slot_of_point, sizeof(int32_t) * (size_t)rows));
+    int64_t rows = (P + P / 2 + 1) & ~1ll;
+    // (with the large insert's row states, slots and keys: five arrays of `rows` words)
+    INSC_HIP(hipMalloc((void **)&g->slot_of_point, sizeof(int32_t) * 5 * (size_t)rows));
     INSC_HIP(hipMalloc((void **)&g->flags, sizeof(int32_t) * (size_t)(rows + 64)));
     g->scratch_rows = rows;
   }
@@ -571,6 +858,34 @@ static int grid_insert_launch(insc_grid *g, const int32_t *d_coords4, int64_t P,
   const unsigned nb = grid_for(P, 256);
   int32_t *total = g->flags + g->scratch_rows;  // spare int after the flags
   const bool small = P <= FINISH_SMALL_MAX;
+  const int64_t n_parts = g->n_slots >> PART_SHIFT;
+  // built in LDS, partition by partition - into an empty grid always; into one that holds sites when the
+  // rows are many enough to pay for two passes over the table
+  if (!small && g->part && n_parts >= 1 && n_parts <= PART_MAX && (g->n_upper == 0 || P * 8 >= g->n_slots)) {
+    int32_t *cnt = g->part, *cursor = cnt + PART_MAX * PART_PAD, *base = cursor + PART_MAX * PART_PAD;
+    int32_t *part_rows = g->slot_of_point, *state = part_rows + g->scratch_rows, *where = state + g->scratch_rows;
+    uint64_t *part_keys = reinterpret_cast<uint64_t *>(where + g->scratch_rows);
+    const int load = g->n_upper > 0 ? 1 : 0;
+    const unsigned blocks = (unsigned)((P + 1024 * PART_ROWS - 1) / (1024 * PART_ROWS));
+    const size_t lds = sizeof(int32_t) * (size_t)n_parts;
+    hipLaunchKernelGGL(part_count_kernel, dim3(blocks), dim3(1024), lds, s, d_coords4, P, mask, (int)n_parts, cnt, g->d_err);
+    hipLaunchKernelGGL(part_scatter_kernel, dim3(blocks), dim3(1024), 2 * lds, s, d_coords4, P, mask, (int)n_parts, cnt,
+                       cursor, base, part_rows, part_keys, d_site_of_point, g->flags);
+    hipLaunchKernelGGL(part_winners_kernel, dim3((unsigned)n_parts), dim3(PART_THREADS), 0, s, g->table, mask, load,
+                       base, part_rows, part_keys, g->d_n, g->flags, state, where, cnt, cursor, total + 1, g->d_err);
+    INSC_LAUNCH_CHECK();
+    rc = scan_exclusive_i32(g->flags, g->flags, P, total, s);
+    if (rc) return rc;
+    hipLaunchKernelGGL(part_assign_kernel, dim3(nb), dim3(256), 0, s, g->table, base, (int)n_parts, part_rows, part_keys,
+                       state, where, g->flags, g->d_n, total, g->coords, g->capacity_sites, g->d_err, d_site_of_point,
+                       g->h_n);
+    INSC_LAUNCH_CHECK();
+    g->n_upper += P;
+    g->n_exact = -1;
+    g->h_fresh = g->h_n != nullptr;
+    g->h_stream = (void *)s;
+    return INSC_OK;
+  }
   hipLaunchKernelGGL(grid_claim_kernel, dim3(nb), dim3(256), 0, s, g->table, mask, d_coords4, P, g->slot_of_point,
                      small ? nullptr : g->flags, d_site_of_point, g->d_err);
   if (small) {
@@ -914,8 +1229,9 @@ __global__ __launch_bounds__(256) void frame_claim_kernel(FrameInsertArgs a, con
   const int4 c = frame_point(coords_in, cols, p, l);
   const uint64_t key = pack_key(c.x, c.y, c.z, c.w);
   auto claim = [&]() -> uint32_t {
-    int64_t s = home_slot(key, L.mask);
-    for (int64_t probe = 0; probe <= L.mask && probe < MAX_PROBES; probe++) {
+    Walk w = walk_begin(key, L.mask);
+    do {
+      const int64_t s = walk_slot(w);
       const int4 raw = *reinterpret_cast<const int4 *>(&L.table[s]);  // key (two words), val, pad
       unsigned long long k = ((unsigned long long)(unsigned)raw.y << 32) | (unsigned)raw.x;
       if (k == key && raw.z >= 0 && raw.z < VAL_PENDING) return REC_SITE | (uint32_t)raw.z;  // numbered before this frame
@@ -935,8 +1251,7 @@ __global__ __launch_bounds__(256) void frame_claim_kernel(FrameInsertArgs a, con
         if (!beaten) atomicMin(&L.table[s].val, VAL_PENDING + p);
         return REC_DUP | (uint32_t)s;
       }
-      s = (s + 1) & L.mask;
-    }
+    } while (walk_next(w));
     return REC_NONE;
   };
   uint32_t r = REC_NONE;
@@ -1441,6 +1756,9 @@ int order_append_new_sites_both_batch(const insc_grid *const *grids, const int32
 using namespace insc;
 
 extern "C" {
+#ifdef PART_DEBUG
+int insc_debug_part(long long *h) { return (int)hipMemcpyFromSymbol(h, HIP_SYMBOL(part_dbg), sizeof(long long) * 4096 * 8); }
+#endif
 
 int insc_grid_create(int64_t capacity_sites, insc_grid **out) {
   INSC_REQUIRE(out, INSC_ERR_ARG, "insc_grid_create: out is null");
@@ -1460,6 +1778,8 @@ int insc_grid_create(int64_t capacity_sites, insc_grid **out) {
   g->d_err = g->d_n + 16;
   INSC_HIP(hipHostMalloc((void **)&g->h_n, 64, hipHostMallocDefault));
   g->h_n[0] = g->h_n[1] = 0;
+  INSC_HIP(hipMalloc((void **)&g->part, sizeof(int32_t) * PART_INTS));
+  INSC_HIP(hipMemset(g->part, 0, sizeof(int32_t) * PART_INTS));
   *out = g;
   return insc_grid_clear(g, nullptr);
 }
@@ -1473,6 +1793,7 @@ int insc_grid_destroy(insc_grid *g) {
   if (g->h_n) (void)hipHostFree(g->h_n);
   if (g->slot_of_point) (void)hipFree(g->slot_of_point);
   if (g->flags) (void)hipFree(g->flags);
+  if (g->part) (void)hipFree(g->part);
   delete g;
   return INSC_OK;
 }
@@ -1599,7 +1920,7 @@ int insc_grid_query(const insc_grid *g, const int32_t *d_coords4, int64_t Q, int
   INSC_REQUIRE(g, INSC_ERR_ARG, "insc_grid_query: grid is null");
   INSC_REQUIRE(Q >= 0 && (Q == 0 || (d_coords4 && d_site)), INSC_ERR_ARG, "insc_grid_query: bad arguments");
   if (Q == 0) return INSC_OK;
-  hipLaunchKernelGGL(grid_query_kernel, dim3(grid_for(Q * 8, 256, 1ll << 30)), dim3(256), 0, (hipStream_t)stream, g->table,
+  hipLaunchKernelGGL(grid_query_kernel, dim3(grid_for(Q, 256)), dim3(256), 0, (hipStream_t)stream, g->table,
                      g->n_slots - 1, d_coords4, Q, d_site);
   INSC_LAUNCH_CHECK();
   return INSC_OK;

@@ -121,6 +121,45 @@ def test_grid_query_append_and_grow(S, orc):
     assert (out.cpu().numpy() == orc.grid_query(o_sc, q)).all()
 
 
+@pytest.mark.parametrize("case", ["hot_cells", "scene", "batched_wide"])
+def test_large_insert_built_by_partitions(S, orc, case):
+    """Inserts of more than 16 384 rows sort their rows by table partition and build each partition in LDS -
+    into an empty grid, and into one that holds sites when the rows are at least an eighth of the slots.
+    Ids, per-row sites and the table itself (queries) against the oracle; rows with the skip mark get -1."""
+    from sparseconvnet._lib import lib, ptr, stream_ptr
+
+    rng = np.random.default_rng(21)
+    if case == "hot_cells":  # 1 728 cells hit by 300 000 rows: a few partitions take nearly every row
+        a = np.concatenate([rng.integers(0, 12, (300000, 3)), np.zeros((300000, 1), np.int64)], 1).astype(np.int32)
+        b = np.concatenate([rng.integers(6, 40, (70000, 3)), np.zeros((70000, 1), np.int64)], 1).astype(np.int32)
+    elif case == "scene":
+        pts = scenes.boxes_scene(seed=5, n=230000).astype(np.int32)
+        a, b = pts[:150000], np.concatenate([pts[100000:140000], pts[150000:]], 0)
+    else:
+        a = np.concatenate([rng.integers(0, 65536, (200000, 3)), rng.integers(0, 32768, (200000, 1))], 1).astype(np.int32)
+        b = np.concatenate([a[rng.integers(0, len(a), 30000)], a[:40000] ^ 1], 0).astype(np.int32)
+    skip = np.zeros(len(a), bool)
+    skip[rng.integers(0, len(a), 50)] = True
+    a_in = a.copy()
+    a_in[skip, 0] = np.iinfo(np.int32).min
+    m, sc, sop = _insert(S, a_in, capacity=262144)
+    o_sop, o_sc, _ = orc.grid_build(np.concatenate([a[~skip], b], 0))
+    n_a = int((~skip).sum())
+    got = sop.cpu().numpy()
+    assert (got[skip] == -1).all()
+    assert (got[~skip] == o_sop[:n_a]).all()
+    assert sc.n == int(o_sop[:n_a].max()) + 1
+    sop_b = m.insert(sc, dev(b))  # the grid holds sites now: the partitions start from the table's slots
+    assert sc.n == len(o_sc)
+    assert (sop_b.cpu().numpy() == o_sop[n_a:]).all()
+    assert (sc.coords_view().cpu().numpy() == o_sc).all()
+    q = np.concatenate([a[::7], b[::5], (a[:20000] + np.array([1, 0, 0, 0], np.int32)) & 65535], 0).astype(np.int32)
+    q[:, 3] &= 32767
+    out = torch.empty(len(q), dtype=torch.int32, device="cuda")
+    lib.insc_grid_query(sc.grid, ptr(dev(q)), I64(len(q)), ptr(out), stream_ptr())
+    assert (out.cpu().numpy() == orc.grid_query(o_sc, q)).all()
+
+
 def test_grid_rejects_bad_coordinate(S):
     from sparseconvnet._lib import InscError
 
