@@ -336,17 +336,19 @@ __global__ __launch_bounds__(1024) void grid_finish_small_kernel(Slot *table, co
   }
 }
 
-// ---- large inserts: the table built partition by partition in LDS -----------------------------
-// The claim kernel above sends one atomic per point to a slot somewhere in the table; the lines of the
-// table travel between the L2s of the chip's dies for it (measured on 220 000 points into 2^20 slots:
-// 29 MB fetched and 24 MB written for 3.5 MB of points, 43 us).  A large insert sorts its rows by home
-// partition first (count, scatter: coalesced passes with LDS histograms) and then one workgroup per
-// partition plays the same protocol on a copy of its PART_SLOTS slots in LDS: winners (the smallest
-// row of every new cell), the prefix sum over the rows' winner flags that ranks them, and a second
-// build that stores the numbered slots - the only time the table itself is touched.
+// ---- large inserts into an empty grid: the table built partition by partition in LDS ---------
+// The claim kernel above sends one atomic per point to a slot somewhere in the table, and the lines of
+// the table travel between the L2s of the chip's dies for it.  A large insert into an empty grid sorts
+// its rows by home partition first (count, scatter: coalesced passes with LDS histograms) and then one
+// workgroup per partition plays the same protocol on its PART_SLOTS slots in LDS: winners (the smallest
+// row of every new cell), the prefix sum over the rows' winner flags that ranks them, and one pass that
+// stores the numbered slots - the only time the table itself is touched.  Measured on 220 000 points
+// into 2^20 slots: 54 MB of memory traffic and 41 us, against 74 MB and 44 us for the claim kernel's way.
+// A grid that holds sites takes the claim kernel: its partitions would have to be read from the table
+// first (measured with 80 000 rows onto 150 000 sites: 31 against 25 us).
 constexpr int PART_MAX = 4096;   // partitions of the largest table that takes this path
 constexpr int PART_PAD = 16;     // ints between two partitions' counters (their atomics spread over the L2 channels)
-constexpr int PART_ROWS = 4;     // rows per thread of count / scatter
+constexpr int PART_ROWS = 2;     // rows per thread of count / scatter
 constexpr int PART_INTS = 2 * PART_MAX * PART_PAD + PART_MAX + 64;  // cnt | cursor | base
 
 __device__ __forceinline__ int part_of_row(const int32_t *__restrict__ coords4, int64_t p, int64_t mask, int32_t *d_err,
@@ -471,27 +473,13 @@ __device__ __forceinline__ int part_slot(unsigned long long *keys, unsigned long
   return -1;
 }
 
-// One workgroup per partition plays the insert on a copy of the partition's slots in LDS - as they are
-// in the table (load), or empty; a slot that holds a key without an id (left by a call that ran out of
-// room) counts as holding the key, to be numbered by this call.  Per row, in partition order: state =
-// the smallest row of the row's cell (flags 1 for that row itself), -2 - id for a cell numbered earlier,
+// One workgroup per partition plays the insert on the partition's slots in LDS, all empty at the start.
+// Per row, in partition order: state = the smallest row of the row's cell (flags 1 for that row itself),
 // -1 if the partition is full; where = the cell's slot in the table.  Leaves the partition's counters zero.
-#ifndef PART_THREADS_V
-#define PART_THREADS_V 512
-#endif
-constexpr int PART_THREADS = PART_THREADS_V;
-#ifdef PART_DEBUG
-__device__ long long part_dbg[4096 * 8];
-#define PDBG(k) if (tid == 0) part_dbg[q * 8 + (k)] = wall_clock64()
-#else
-#define PDBG(k)
-#endif
-#ifndef PART_KEEP_V
-#define PART_KEEP_V 2
-#endif
-constexpr int PART_KEEP = PART_KEEP_V;  // rows per thread kept in registers between the two passes (more are looked up again)
+constexpr int PART_THREADS = 512;
+constexpr int PART_KEEP = 2;  // rows per thread kept in registers between the two passes (more are looked up again)
 __global__ __launch_bounds__(PART_THREADS) void part_winners_kernel(
-    const Slot *__restrict__ table, int64_t mask, int load, const int32_t *__restrict__ base,
+    int64_t mask, const int32_t *__restrict__ base,
     const int32_t *__restrict__ part_rows, const uint64_t *__restrict__ part_keys, const int32_t *__restrict__ d_n,
     int32_t *__restrict__ flags, int32_t *__restrict__ state, int32_t *__restrict__ where, int32_t *cnt, int32_t *cursor,
     int32_t *__restrict__ n_before, int32_t *d_err) {
@@ -499,7 +487,6 @@ __global__ __launch_bounds__(PART_THREADS) void part_winners_kernel(
   __shared__ int vals[PART_SLOTS];
   const int q = blockIdx.x, tid = threadIdx.x;
   const int W = (int)(mask < PART_SLOTS - 1 ? mask + 1 : PART_SLOTS);
-  PDBG(0);
   const int b0 = base[q], b1 = base[q + 1];
   if (tid == 0) {
     if (q == 0) *n_before = d_n[0];
@@ -514,38 +501,21 @@ __global__ __launch_bounds__(PART_THREADS) void part_winners_kernel(
     pr[j] = i < b1 ? part_rows[i] : -1;
     kr[j] = i < b1 ? part_keys[i] : 0;
   }
-  const Slot *slab = table + (int64_t)q * W;
   for (int i = tid; i < W; i += PART_THREADS) {
-    unsigned long long k = INSC_EMPTY_KEY;
-    int v = VAL_UNSET;
-    if (load) {
-      const int4 raw = *reinterpret_cast<const int4 *>(&slab[i]);
-      k = ((unsigned long long)(unsigned)raw.y << 32) | (unsigned)raw.x;
-      if (raw.z >= 0 && raw.z < VAL_PENDING) v = raw.z;
-    }
-    keys[i] = k;
-    vals[i] = v;
+    keys[i] = INSC_EMPTY_KEY;
+    vals[i] = VAL_UNSET;
   }
-#ifdef PART_DEBUG
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-#endif
-  PDBG(1);
   __syncthreads();
-  PDBG(2);
   auto claim = [&](int p, const uint64_t key) -> int {
     const int s = part_slot(keys, key, mask);
     if (s < 0)
       atomicOr(d_err, 2);
-    else if (!load || vals[s] >= VAL_PENDING)  // (ids were there before the loop and stay)
+    else
       atomicMin(&vals[s], VAL_PENDING + p);
     return s;
   };
   auto answer = [&](int i, int p, int s) {
-    int st = -1;
-    if (s >= 0) {
-      const int v = vals[s];
-      st = v < VAL_PENDING ? -2 - v : v - VAL_PENDING;
-    }
+    const int st = s >= 0 ? vals[s] - VAL_PENDING : -1;
     state[i] = st;
     where[i] = s < 0 ? -1 : (int)((int64_t)q * W + s);
     flags[p] = st == p ? 1 : 0;
@@ -553,10 +523,8 @@ __global__ __launch_bounds__(PART_THREADS) void part_winners_kernel(
 #pragma unroll
   for (int j = 0; j < PART_KEEP; j++)
     if (pr[j] >= 0) sr[j] = claim(pr[j], kr[j]);
-  PDBG(3);
   for (int i = b0 + PART_KEEP * PART_THREADS + tid; i < b1; i += PART_THREADS) claim(part_rows[i], part_keys[i]);
   __syncthreads();
-  PDBG(4);
 #pragma unroll
   for (int j = 0; j < PART_KEEP; j++)
     if (pr[j] >= 0) answer(b0 + j * PART_THREADS + tid, pr[j], sr[j]);
@@ -564,7 +532,6 @@ __global__ __launch_bounds__(PART_THREADS) void part_winners_kernel(
     const uint64_t key = part_keys[i];
     answer(i, part_rows[i], part_slot(keys, key, mask));  // (finds what the first pass left)
   }
-  PDBG(5);
 }
 
 // numbered: every row takes id = n_before + rank of its cell's winner; the winners store their slots
@@ -595,7 +562,7 @@ __global__ __launch_bounds__(256) void part_assign_kernel(Slot *table, const int
   if (i >= base[n_parts]) return;
   const int p = part_rows[i], r = state[i];
   if (r < 0) {
-    site_of_point[p] = r < -1 ? -2 - r : -1;
+    site_of_point[p] = -1;  // (the partition was full)
     return;
   }
   const int id = n_before + excl[r];
@@ -859,20 +826,17 @@ static int grid_insert_launch(insc_grid *g, const int32_t *d_coords4, int64_t P,
   int32_t *total = g->flags + g->scratch_rows;  // spare int after the flags
   const bool small = P <= FINISH_SMALL_MAX;
   const int64_t n_parts = g->n_slots >> PART_SHIFT;
-  // built in LDS, partition by partition - into an empty grid always; into one that holds sites when the
-  // rows are many enough to pay for two passes over the table
-  if (!small && g->part && n_parts >= 1 && n_parts <= PART_MAX && (g->n_upper == 0 || P * 8 >= g->n_slots)) {
+  if (!small && g->n_upper == 0 && g->part && n_parts >= 1 && n_parts <= PART_MAX) {  // empty: built in LDS
     int32_t *cnt = g->part, *cursor = cnt + PART_MAX * PART_PAD, *base = cursor + PART_MAX * PART_PAD;
     int32_t *part_rows = g->slot_of_point, *state = part_rows + g->scratch_rows, *where = state + g->scratch_rows;
     uint64_t *part_keys = reinterpret_cast<uint64_t *>(where + g->scratch_rows);
-    const int load = g->n_upper > 0 ? 1 : 0;
     const unsigned blocks = (unsigned)((P + 1024 * PART_ROWS - 1) / (1024 * PART_ROWS));
     const size_t lds = sizeof(int32_t) * (size_t)n_parts;
     hipLaunchKernelGGL(part_count_kernel, dim3(blocks), dim3(1024), lds, s, d_coords4, P, mask, (int)n_parts, cnt, g->d_err);
     hipLaunchKernelGGL(part_scatter_kernel, dim3(blocks), dim3(1024), 2 * lds, s, d_coords4, P, mask, (int)n_parts, cnt,
                        cursor, base, part_rows, part_keys, d_site_of_point, g->flags);
-    hipLaunchKernelGGL(part_winners_kernel, dim3((unsigned)n_parts), dim3(PART_THREADS), 0, s, g->table, mask, load,
-                       base, part_rows, part_keys, g->d_n, g->flags, state, where, cnt, cursor, total + 1, g->d_err);
+    hipLaunchKernelGGL(part_winners_kernel, dim3((unsigned)n_parts), dim3(PART_THREADS), 0, s, mask, base,
+                       part_rows, part_keys, g->d_n, g->flags, state, where, cnt, cursor, total + 1, g->d_err);
     INSC_LAUNCH_CHECK();
     rc = scan_exclusive_i32(g->flags, g->flags, P, total, s);
     if (rc) return rc;
@@ -1756,9 +1720,6 @@ int order_append_new_sites_both_batch(const insc_grid *const *grids, const int32
 using namespace insc;
 
 extern "C" {
-#ifdef PART_DEBUG
-int insc_debug_part(long long *h) { return (int)hipMemcpyFromSymbol(h, HIP_SYMBOL(part_dbg), sizeof(long long) * 4096 * 8); }
-#endif
 
 int insc_grid_create(int64_t capacity_sites, insc_grid **out) {
   INSC_REQUIRE(out, INSC_ERR_ARG, "insc_grid_create: out is null");

@@ -123,9 +123,10 @@ def test_grid_query_append_and_grow(S, orc):
 
 @pytest.mark.parametrize("case", ["hot_cells", "scene", "batched_wide"])
 def test_large_insert_built_by_partitions(S, orc, case):
-    """Inserts of more than 16 384 rows sort their rows by table partition and build each partition in LDS -
-    into an empty grid, and into one that holds sites when the rows are at least an eighth of the slots.
-    Ids, per-row sites and the table itself (queries) against the oracle; rows with the skip mark get -1."""
+    """An insert of more than 16 384 rows into an empty grid sorts its rows by table partition and builds each
+    partition in LDS; the large insert that follows, into the grid that then holds sites, claims its slots
+    in the table itself.  Ids, per-row sites and the table (queries) against the oracle; rows with the skip
+    mark get -1."""
     from sparseconvnet._lib import lib, ptr, stream_ptr
 
     rng = np.random.default_rng(21)
@@ -149,7 +150,7 @@ def test_large_insert_built_by_partitions(S, orc, case):
     assert (got[skip] == -1).all()
     assert (got[~skip] == o_sop[:n_a]).all()
     assert sc.n == int(o_sop[:n_a].max()) + 1
-    sop_b = m.insert(sc, dev(b))  # the grid holds sites now: the partitions start from the table's slots
+    sop_b = m.insert(sc, dev(b))  # the grid holds sites now
     assert sc.n == len(o_sc)
     assert (sop_b.cpu().numpy() == o_sop[n_a:]).all()
     assert (sc.coords_view().cpu().numpy() == o_sc).all()
