@@ -470,6 +470,29 @@ def time_sweep(call, frames, first):
     return per_frame, dt
 
 
+def sweep_phases(call, net, frames, first):
+    """The timed frames once more with the executor's phase events on (five event records per frame):
+    median milliseconds per phase - structure (grids, maps, orders, tile plans of the frame's new sites,
+    input features), dirty (the sets of rows to recompute), layers, output (rows of the frame's points)."""
+    import numpy as np
+    import torch
+
+    rows = []
+    with torch.no_grad():
+        call(frames[0], False)
+        for f in range(1, first):
+            call(frames[f], True)
+        net.profile(True)
+        for f in range(first, len(frames)):
+            call(frames[f], True)
+            torch.cuda.synchronize()
+            ph = net.profile(True)
+            if ph:
+                rows.append(ph)
+        net.profile(False)
+    return {k: round(float(np.median([r[k] for r in rows])), 3) for k in rows[0]} if rows else None
+
+
 def to_host_long(pts, rgb, device):
     """A frame as the reference's callers hand it over (ioLayers.py:52-69): coordinates as a CPU
     LongTensor [P,3], features on the GPU, batch size 1."""
@@ -913,6 +936,7 @@ def main():
         # flop accounting of the last timed frame against the fp32 MFMA peak (the frame is bound by
         # matrix-core issue at the coarse scales, not by HBM)
         extra["frame"] = frame_work_summary(net, per_frame[-1])
+        extra["frame_phases_ms"] = sweep_phases(lambda x, inc: model.linear(net(x, increment=inc)), net, frames, first)
         if not args.no_extras:
             # (a) the same frames through the reference's own call path: model(x, increment) on the module
             # tree with CPU int64 coordinates (model.py:23-26, ioLayers.py:52-69); the whole-network

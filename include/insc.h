@@ -161,6 +161,18 @@ int insc_order_build_scales(const insc_grid *const *grids, const int32_t *const 
                             const int64_t *n, int n_scales, int32_t *const *d_order, int32_t *const *d_pos,
                             int32_t *const *d_bo_order, int32_t *const *d_bo_pos, void *stream);
 
+/* The sites added by the grid's most recent insert - [count before it, count) - appended to the grid's
+ * processing order in ONE launch (one workgroup, a radix sort in shared memory): d_order[first..count) =
+ * those sites sorted among themselves by (64^3 block, neighbour pattern), equal keys in id order;
+ * d_pos (nullable) the inverse over the same range.  With d_offset (position inside the parent cell,
+ * from insc_rulebook_down2) also d_bo_order / d_bo_pos: the same sites grouped by that position, each
+ * group in the sequence of d_order.  d_nbr: the grid's 27-neighbour map, up to date for the new sites.
+ * More than 8192 new sites keep their id order (every order gives the same results; insc_order_build
+ * sorts any number).  n_new_upper: a host-side upper bound of the number of new sites (0: nothing to
+ * do); the counts themselves are read on the device.  No counterpart in the reference. */
+int insc_order_append(const insc_grid *g, const int32_t *d_nbr, const int32_t *d_offset, int32_t *d_order,
+                      int32_t *d_pos, int32_t *d_bo_order, int32_t *d_bo_pos, int64_t n_new_upper, void *stream);
+
 /* ---------------------------------------------------------------------------------------
  * Feature kernels.
  * ------------------------------------------------------------------------------------- */

@@ -901,13 +901,27 @@ __device__ __forceinline__ uint64_t spread3_10(uint64_t v) {  // 10 bits -> ever
   v = (v | (v << 2)) & 0x9249249ull;
   return v;
 }
+// LDS of the two appends: the keys of the new sites, their indices in two buffers that a radix pass reads
+// and writes in turn, the digit counters of a pass ([digit][wavefront], 17 words per digit so that the
+// lanes of a wavefront - same wavefront, different digits - fall into different banks) twice (the other
+// set is zeroed for the pass that follows), and a few words for sums across the wavefronts.
+// LDS of the two appends: the keys of the new sites in two buffers that a merge round reads and writes in turn
+struct OrderLds {
+  uint64_t key[2][SORT_NEW_MAX];
+};
+// Sorted by (key, arrival) - one 64-bit word per site, sort key in the upper 51 bits, index among the new
+// sites in the lower 13, so no two words are equal - by one workgroup (all of it on one compute unit: what
+// it costs is the number of instructions, ~14 us for 3000 sites): every wavefront sorts runs of 64
+// words in registers (a bitonic network over the lanes), then rounds of merges double the runs: a word's
+// place in the merged run is its place in its own run plus the number of smaller words in the sibling run,
+// found by a binary search of a fixed number of steps, the searches of a thread's words side by side.
+// log2(n / 64) rounds with one barrier each.  (A bitonic network over all keys took 78 passes for 4096 of
+// them, 40-48 us for the 2-3k new sites of a frame; a radix sort eight bits a pass, 3 us per pass.)
 __device__ __forceinline__ void order_append_sorted_body(const int first, const int n,
                                                          const int32_t *__restrict__ coords,
                                                          const int32_t *__restrict__ nbr, int32_t *__restrict__ order,
-                                                         int32_t *__restrict__ pos, uint64_t *key) {
-  // key: SORT_NEW_MAX 64-bit words of LDS, one per new site: sort key in the upper 51 bits, index of
-  // the site among the new ones in the lower 13
-  const int tid = threadIdx.x;
+                                                         int32_t *__restrict__ pos, OrderLds &L) {
+  const int tid = threadIdx.x, lane = tid & 63;
   if (n <= 0) return;
   if (n > SORT_NEW_MAX) {
     for (int i = tid; i < n; i += 1024) {
@@ -916,10 +930,9 @@ __device__ __forceinline__ void order_append_sorted_body(const int first, const 
     }
     return;
   }
-  int N = 2;
-  while (N < n) N <<= 1;
+  const int N = (n + 63) & ~63;  // whole runs of 64; the words past n have all key bits set and end up last
   for (int i = tid; i < N; i += 1024) {
-    uint64_t k = ~0ull;
+    uint64_t k = ~8191ull | (uint64_t)i;
     if (i < n) {
       const int v = first + i;
       const int4 c = reinterpret_cast<const int4 *>(coords)[v];
@@ -930,36 +943,58 @@ __device__ __forceinline__ void order_append_sorted_body(const int first, const 
                             (spread3_10((uint64_t)((c.z >> 6) & 255)) << 2);
       k = (((mort << 27) | (uint64_t)m) << 13) | (uint64_t)i;
     }
-    key[i] = k;
-  }
-  __syncthreads();
-  // Bitonic sort.  A pass of stride j <= 64 stays inside the 128 keys that the 64 pairs of one
-  // wavefront cover, so runs of such passes are ordered by the wavefront itself (LDS accesses of a
-  // wavefront complete in order); only passes of a larger stride, and the change from one kind to
-  // the other, need the whole workgroup to meet.
-  for (int k = 2; k <= N; k <<= 1) {
-    for (int j = k >> 1; j > 0; j >>= 1) {
-      for (int p = tid; p < (N >> 1); p += 1024) {
-        const int i = ((p & ~(j - 1)) << 1) | (p & (j - 1)), x = i | j;
-        const uint64_t a = key[i], b = key[x];
-        if ((a > b) == ((i & k) == 0)) {
-          key[i] = b;
-          key[x] = a;
-        }
-      }
-      const int jn = j > 1 ? (j >> 1) : k;  // stride of the pass that follows (k: first pass of the next stage)
-      if (j > 64 || jn > 64) {
-        __syncthreads();
-      } else {
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    // the run of 64 that this word belongs to is held by one wavefront (i and lane agree mod 64): sorted here
+#pragma unroll
+    for (int kk = 2; kk <= 64; kk <<= 1) {
+#pragma unroll
+      for (int j = kk >> 1; j > 0; j >>= 1) {
+        const uint64_t y = __shfl_xor(k, j, 64);
+        const bool keep_small = ((lane & j) == 0) == ((lane & kk) == 0);
+        k = keep_small ? (k < y ? k : y) : (k < y ? y : k);
       }
     }
+    L.key[0][i] = k;
   }
   __syncthreads();
+  int src = 0;
+  for (int len = 64, lg = 6; len < N; len <<= 1, lg++) {
+    const uint64_t *a = L.key[src];
+    uint64_t *d = L.key[src ^ 1];
+    uint64_t w[8];
+    int sib[8], sib_n[8], lo[8];
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+      const int p = e * 1024 + tid;
+      if (e * 1024 >= N) continue;  // (uniform)
+      const int run = p >> lg;
+      w[e] = p < N ? a[p] : 0;
+      sib[e] = (run ^ 1) << lg;
+      sib_n[e] = p < N ? min(max(N - sib[e], 0), len) : 0;
+      lo[e] = 0;
+    }
+    // words of the sibling run that come before w: the smaller ones
+    for (int step = len; step >= 1; step >>= 1) {
+#pragma unroll
+      for (int e = 0; e < 8; e++) {
+        if (e * 1024 >= N) continue;
+        const int probe = lo[e] + step;
+        if (probe <= sib_n[e]) {
+          if (a[sib[e] + probe - 1] < w[e]) lo[e] = probe;
+        }
+      }
+    }
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+      const int p = e * 1024 + tid;
+      if (e * 1024 >= N || p >= N) continue;
+      const int run = p >> lg;
+      d[((run >> 1) << (lg + 1)) + (p & (len - 1)) + lo[e]] = w[e];
+    }
+    __syncthreads();
+    src ^= 1;
+  }
   for (int i = tid; i < n; i += 1024) {
-    const int v = first + (int)(key[i] & 8191);
+    const int v = first + (int)(L.key[src][i] & 8191);
     order[first + i] = v;
     if (pos) pos[v] = first + i;
   }
@@ -1056,13 +1091,13 @@ struct OrderBothBatch {
   OrderBothJob job[16];
 };
 __global__ __launch_bounds__(1024) void order_append_both_batch_kernel(OrderBothBatch b) {
-  __shared__ uint64_t key[SORT_NEW_MAX];
+  __shared__ OrderLds L;
   const OrderBothJob &j = b.job[blockIdx.x];
   const int first = j.all ? 0 : j.d_n[1], n = j.d_n[0] - first;
-  order_append_sorted_body(first, n, j.coords, j.nbr, j.order, j.pos, key);
+  order_append_sorted_body(first, n, j.coords, j.nbr, j.order, j.pos, L);
   if (!j.offset) return;
   __syncthreads();  // the order written above is read below (by other threads than wrote it), and the LDS is reused
-  order_append_grouped_body(first, n, j.offset, j.order, j.bo_order, j.bo_pos, key);
+  order_append_grouped_body(first, n, j.offset, j.order, j.bo_order, j.bo_pos, L.key[0]);
 }
 
 int64_t order_sorted_max() { return SORT_NEW_MAX; }
@@ -1875,6 +1910,17 @@ int insc_grid_insert_noalloc(insc_grid *g, const int32_t *d_coords4, int64_t P, 
     *h_n_sites = g->n_exact;
   }
   return INSC_OK;
+}
+
+int insc_order_append(const insc_grid *g, const int32_t *d_nbr, const int32_t *d_offset, int32_t *d_order, int32_t *d_pos,
+                      int32_t *d_bo_order, int32_t *d_bo_pos, int64_t n_new_upper, void *stream) {
+  INSC_REQUIRE(g && d_nbr && d_order, INSC_ERR_ARG, "insc_order_append: null argument");
+  INSC_REQUIRE(!d_offset || (d_bo_order && d_bo_pos), INSC_ERR_ARG,
+               "insc_order_append: with d_offset, d_bo_order and d_bo_pos are needed as well");
+  const insc_grid *gs[1] = {g};
+  const int32_t *nbr[1] = {d_nbr}, *off[1] = {d_offset};
+  int32_t *order[1] = {d_order}, *pos[1] = {d_pos}, *bo[1] = {d_bo_order}, *bop[1] = {d_bo_pos};
+  return order_append_new_sites_both_batch(gs, nbr, off, order, pos, bo, bop, 1, n_new_upper, (hipStream_t)stream);
 }
 
 int insc_grid_query(const insc_grid *g, const int32_t *d_coords4, int64_t Q, int32_t *d_site, void *stream) {

@@ -32,6 +32,7 @@ _SIGS = {
     "insc_order_build": [vp, vp, c_i64, c_i64, vp, vp],
     "insc_order_by_offset": [vp, vp, c_i64, vp, vp],
     "insc_order_build_scales": [vp, vp, vp, vp, c_int, vp, vp, vp, vp, vp],
+    "insc_order_append": [vp, vp, vp, vp, vp, vp, vp, c_i64, vp],
     "insc_conv_nbr": [vp, c_i64, c_i64, vp, c_i64, vp, vp, vp, vp, c_int, vp, vp, c_i64, c_int, c_int,
                       ctypes.POINTER(ctypes.c_double), vp],
     "insc_conv_pack_weights": [vp, c_int, c_int, c_int, vp, vp],

@@ -210,6 +210,51 @@ def test_ssc_rulebook_incremental_patch(S, orc):
     assert (np.sort(sc.order.t[:sc.n].cpu().numpy()) == np.arange(sc.n)).all()
 
 
+def _spread3(v):
+    out = np.zeros_like(v)
+    for b in range(8):
+        out |= ((v >> np.uint64(b)) & np.uint64(1)) << np.uint64(3 * b)
+    return out
+
+
+@pytest.mark.parametrize("n_old,n_new", [(7000, 1), (7000, 63), (7000, 700), (40000, 3300), (9000, 8192), (9000, 8193)])
+def test_order_append_sorts_the_new_sites(S, n_old, n_new):
+    """insc_order_append against numpy: the sites of the last insert in the order of (64^3 block, neighbour
+    pattern), equal keys by id; the inverse; the same sites grouped by their position inside the parent
+    cell, each group in that order.  One site, fewer than a wavefront, a frame's worth, the most the
+    workgroup sorts, and one more (which keep their id order)."""
+    from sparseconvnet._lib import lib, ptr, stream_ptr
+
+    rng = np.random.default_rng(n_new)
+    pts = scenes.boxes_scene(seed=13, n=n_old + n_new).astype(np.int32)
+    pts[:, :3] += rng.integers(0, 3, 3).astype(np.int32) * 64  # several 64^3 blocks
+    m, sc, _ = _insert(S, pts[:n_old], capacity=n_old + n_new)
+    m.ssc_rulebook((4096,) * 3)
+    m.insert(sc, dev(pts[n_old:]))
+    assert sc.n == n_old + n_new
+    nbr = sc.nbr.ensure(sc.capacity(), keep=sc.nbr_n)
+    lib.insc_rulebook_ssc3(sc.grid, I64(n_old), I64(n_new), ptr(nbr), 1, stream_ptr())
+    offset = dev(rng.integers(0, 8, sc.n).astype(np.int32))
+    order, pos, bo, bop = (torch.full((sc.n,), -5, dtype=torch.int32, device="cuda") for _ in range(4))
+    lib.insc_order_append(sc.grid, ptr(nbr), ptr(offset), ptr(order), ptr(pos), ptr(bo), ptr(bop), I64(n_new),
+                          stream_ptr())
+    c = sc.coords_view().cpu().numpy()[n_old:].astype(np.uint64)
+    has = nbr[:sc.n].view(-1, 27)[n_old:].cpu().numpy() >= 0
+    pattern = (has.astype(np.uint64) << np.arange(27, dtype=np.uint64)).sum(1)
+    mort = _spread3((c[:, 0] >> np.uint64(6)) & np.uint64(255)) | (_spread3((c[:, 1] >> np.uint64(6)) & np.uint64(255)) << np.uint64(1)) \
+        | (_spread3((c[:, 2] >> np.uint64(6)) & np.uint64(255)) << np.uint64(2))
+    key = (mort << np.uint64(27)) | pattern
+    exp = n_old + (np.argsort(key, kind="stable") if n_new <= 8192 else np.arange(n_new))
+    got = order.cpu().numpy()
+    assert (got[:n_old] == -5).all()  # older sites are not touched
+    assert (got[n_old:] == exp).all()
+    assert (pos.cpu().numpy()[exp] == n_old + np.arange(n_new)).all()
+    off = offset.cpu().numpy()
+    exp_bo = exp[np.argsort(off[exp] & 7, kind="stable")] if n_new <= 8192 else exp
+    assert (bo.cpu().numpy()[n_old:] == exp_bo).all()
+    assert (bop.cpu().numpy()[exp_bo] == n_old + np.arange(n_new)).all()
+
+
 def test_down2_rulebook_matches_oracle(S, orc):
     pts = scenes.boxes_scene(seed=2, n=20000)
     m, sc, _ = _insert(S, pts)
