@@ -358,7 +358,7 @@ def kernel_table(device, reps=20, strict=True):
     add("device-to-device copy (torch; reference point, not a kernel of the path)", t, NF * C * 8, "%d x %d" % (NF, C))
     t = timed(lambda: lib.insc_grid_insert(grid, ptr(c4), I64(P), ptr(sop), ctypes.byref(n_sites), st),
               pre=lambda: lib.insc_grid_clear(grid, st))
-    add("hash grid insert (claim, scan, assign, resolve; incl. count read-back)", t, P * 32, "%d points -> %d sites" % (P, n_sites.value), key="insert")
+    add("hash grid insert (into an empty grid: rows sorted by table partition, partitions built in LDS, scan, assign; incl. count read-back)", t, P * 32, "%d points -> %d sites" % (P, n_sites.value), key="insert")
     t = timed(lambda: lib.insc_grid_query(grid, ptr(c4), I64(P), ptr(sop), st))
     add("hash grid query", t, P * 28, "%d queries" % P, key="query")
     t = timed(lambda: lib.insc_rulebook_ssc3(grid, I64(0), I64(N), ptr(nbr), 0, st))
