@@ -777,15 +777,19 @@ __global__ __launch_bounds__(WL_WAVES * 64) void conv_wlds_kernel(
   // draw(): the next tile of this block that has work, or ntiles.
   // With fewer than three tiles per wavefront the draws ahead of the tile pipeline (up to three tiles
   // in hand per wavefront) would leave late wavefronts with nothing: then the turns are dealt instead,
-  // wavefront w takes w, w + WL_WAVES, ...
+  // back and forth: wavefront w takes w, 2 WL_WAVES - 1 - w, 2 WL_WAVES + w, ...  (What a block lasts is the
+  // matrix core of its busiest SIMD, which three wavefronts share - w, w + 4, w + 8; with the turns going
+  // round the same way, w + WL_WAVES next, the SIMD that starts with the three most expensive tiles also
+  // gets the first of the second round.)
   const bool dealt = my_tiles < 3 * WL_WAVES;
-  int my_turn = wave;
+  int my_turn = wave, my_round = 0;
   auto draw = [&]() -> int64_t {
     for (;;) {
       int turn;
       if (dealt) {
         turn = my_turn;
-        my_turn += WL_WAVES;
+        my_round++;
+        my_turn = my_round * WL_WAVES + ((my_round & 1) ? WL_WAVES - 1 - wave : wave);
       } else {
         int v = 0;
         if (lane == 0) v = atomicAdd(&next_turn, 1);
