@@ -163,7 +163,8 @@ int insc_order_build_scales(const insc_grid *const *grids, const int32_t *const 
 
 /* The sites added by the grid's most recent insert - [count before it, count) - appended to the grid's
  * processing order in ONE launch (one workgroup, a radix sort in shared memory): d_order[first..count) =
- * those sites sorted among themselves by (64^3 block, neighbour pattern), equal keys in id order;
+ * those sites sorted among themselves by the key of insc_order_build (what that call gives for the same
+ * range), equal keys in id order;
  * d_pos (nullable) the inverse over the same range.  With d_offset (position inside the parent cell,
  * from insc_rulebook_down2) also d_bo_order / d_bo_pos: the same sites grouped by that position, each
  * group in the sequence of d_order.  d_nbr: the grid's 27-neighbour map, up to date for the new sites.

@@ -110,6 +110,21 @@ int grid_clear_batch(insc_grid *const *grids, int32_t *const *minus1, const int6
                      int64_t zero_bytes, hipStream_t s);
 // most sites the two sorted appends put in order (more keep their arrival order)
 int64_t order_sorted_max();
+// Sort key of a site in the processing orders, from its coordinates and the 27-bit pattern m of the
+// neighbours it has (see insc_order_build): batch parity, Morton code of the 64^3 block (4 bits per axis:
+// blocks 1024 voxels apart share a group, harmless), pattern.
+constexpr int ORDER_KEY_BITS = 40;
+__device__ __forceinline__ uint64_t order_spread3(uint64_t v) {  // 4 bits -> every third bit
+  v &= 0xf;
+  v = (v | (v << 4)) & 0xc3ull;
+  v = (v | (v << 2)) & 0x249ull;
+  return v;
+}
+__device__ __forceinline__ uint64_t order_key(int4 c, uint32_t m) {
+  const uint64_t mort = order_spread3((uint64_t)(c.x >> 6)) | (order_spread3((uint64_t)(c.y >> 6)) << 1) |
+                        (order_spread3((uint64_t)(c.z >> 6)) << 2);
+  return ((uint64_t)(c.w & 1) << 39) | (mort << 27) | (uint64_t)m;
+}
 // device pointer to the site count before the most recent insert
 static inline const int32_t *grid_n_prev_ptr(const insc_grid *g) { return g->d_n + 1; }
 

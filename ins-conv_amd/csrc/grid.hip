@@ -893,14 +893,6 @@ int grid_insert_nosync(insc_grid *g, const int32_t *d_coords4, int64_t P, int32_
 // Key = Morton code of the 64^3 block | neighbour pattern (the key of insc_order_build).
 // More new sites than SORT_NEW_MAX keep their arrival order (any order gives the same results).
 constexpr int SORT_NEW_MAX = 8192;
-__device__ __forceinline__ uint64_t spread3_10(uint64_t v) {  // 10 bits -> every third bit
-  v &= 0x3ff;
-  v = (v | (v << 16)) & 0x30000ffull;
-  v = (v | (v << 8)) & 0x300f00full;
-  v = (v | (v << 4)) & 0x30c30c3ull;
-  v = (v | (v << 2)) & 0x9249249ull;
-  return v;
-}
 // LDS of the two appends: the keys of the new sites, their indices in two buffers that a radix pass reads
 // and writes in turn, the digit counters of a pass ([digit][wavefront], 17 words per digit so that the
 // lanes of a wavefront - same wavefront, different digits - fall into different banks) twice (the other
@@ -938,10 +930,7 @@ __device__ __forceinline__ void order_append_sorted_body(const int first, const 
       const int4 c = reinterpret_cast<const int4 *>(coords)[v];
       uint32_t m = 0;
       for (int j = 0; j < 27; j++) m |= (nbr[(int64_t)v * 27 + j] >= 0 ? 1u : 0u) << j;
-      // (8 bits of block coordinate per axis: blocks 16384 voxels apart share a group, harmless)
-      const uint64_t mort = spread3_10((uint64_t)((c.x >> 6) & 255)) | (spread3_10((uint64_t)((c.y >> 6) & 255)) << 1) |
-                            (spread3_10((uint64_t)((c.z >> 6) & 255)) << 2);
-      k = (((mort << 27) | (uint64_t)m) << 13) | (uint64_t)i;
+      k = (order_key(c, m) << 13) | (uint64_t)i;
     }
     // the run of 64 that this word belongs to is held by one wavefront (i and lane agree mod 64): sorted here
 #pragma unroll

@@ -31,14 +31,6 @@ __global__ void pairs_write_kernel(const int32_t *__restrict__ nbr, int64_t N, i
   }
 }
 
-__device__ __forceinline__ uint64_t spread3(uint64_t v) {  // 12 bits -> every third bit
-  v &= 0xfff;
-  v = (v | (v << 16)) & 0x0000ff0000ffull;
-  v = (v | (v << 8)) & 0x00f00f00f00full;
-  v = (v | (v << 4)) & 0x0c30c30c30c3ull;
-  v = (v | (v << 2)) & 0x249249249249ull;
-  return v;
-}
 
 // sort key, 40 bits (five 8-bit radix passes): batch parity | Morton code of the 64^3 block, four
 // bits per axis | neighbour pattern (27 bits).  Sites with the same pattern inside a block end up
@@ -46,7 +38,6 @@ __device__ __forceinline__ uint64_t spread3(uint64_t v) {  // 12 bits -> every t
 // tiles (the gather locality they cost matters less than the matrix-core work they save).  The
 // order is a heuristic only: blocks 1024 voxels apart and batches of equal parity share groups,
 // which costs some locality and nothing else.
-constexpr int ORDER_KEY_BITS = 40;
 __global__ void order_key_kernel(const int32_t *__restrict__ coords, const int32_t *__restrict__ nbr, int64_t first,
                                  int64_t n, uint64_t *__restrict__ keys, int32_t *__restrict__ vals) {
   int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -55,9 +46,7 @@ __global__ void order_key_kernel(const int32_t *__restrict__ coords, const int32
   int4 c = reinterpret_cast<const int4 *>(coords)[i];
   uint32_t m = 0;
   for (int k = 0; k < 27; k++) m |= (nbr[i * 27 + k] >= 0 ? 1u : 0u) << k;
-  const uint64_t mort = spread3((uint64_t)((c.x >> 6) & 15)) | (spread3((uint64_t)((c.y >> 6) & 15)) << 1) |
-                        (spread3((uint64_t)((c.z >> 6) & 15)) << 2);
-  keys[t] = ((uint64_t)(c.w & 1) << 39) | (mort << 27) | (uint64_t)m;
+  keys[t] = order_key(c, m);
   vals[t] = (int)i;
 }
 
@@ -87,9 +76,7 @@ __global__ void order_key_batch_kernel(OrderBuildBatchDev b) {
   const int4 c = reinterpret_cast<const int4 *>(j.coords)[t];
   uint32_t m = 0;
   for (int k = 0; k < 27; k++) m |= (j.nbr[t * 27 + k] >= 0 ? 1u : 0u) << k;
-  const uint64_t mort = spread3((uint64_t)((c.x >> 6) & 15)) | (spread3((uint64_t)((c.y >> 6) & 15)) << 1) |
-                        (spread3((uint64_t)((c.z >> 6) & 15)) << 2);
-  j.keys[t] = ((uint64_t)(c.w & 1) << 39) | (mort << 27) | (uint64_t)m;
+  j.keys[t] = order_key(c, m);
   j.vals[t] = (int)t;
 }
 __global__ void offset_key_batch_kernel(OrderBuildBatchDev b) {

@@ -228,6 +228,7 @@ def test_order_append_sorts_the_new_sites(S, n_old, n_new):
     rng = np.random.default_rng(n_new)
     pts = scenes.boxes_scene(seed=13, n=n_old + n_new).astype(np.int32)
     pts[:, :3] += rng.integers(0, 3, 3).astype(np.int32) * 64  # several 64^3 blocks
+    pts[:, 3] = rng.integers(0, 2, len(pts))  # two batch entries
     m, sc, _ = _insert(S, pts[:n_old], capacity=n_old + n_new)
     m.ssc_rulebook((4096,) * 3)
     m.insert(sc, dev(pts[n_old:]))
@@ -241,13 +242,17 @@ def test_order_append_sorts_the_new_sites(S, n_old, n_new):
     c = sc.coords_view().cpu().numpy()[n_old:].astype(np.uint64)
     has = nbr[:sc.n].view(-1, 27)[n_old:].cpu().numpy() >= 0
     pattern = (has.astype(np.uint64) << np.arange(27, dtype=np.uint64)).sum(1)
-    mort = _spread3((c[:, 0] >> np.uint64(6)) & np.uint64(255)) | (_spread3((c[:, 1] >> np.uint64(6)) & np.uint64(255)) << np.uint64(1)) \
-        | (_spread3((c[:, 2] >> np.uint64(6)) & np.uint64(255)) << np.uint64(2))
-    key = (mort << np.uint64(27)) | pattern
+    mort = _spread3((c[:, 0] >> np.uint64(6)) & np.uint64(15)) | (_spread3((c[:, 1] >> np.uint64(6)) & np.uint64(15)) << np.uint64(1)) \
+        | (_spread3((c[:, 2] >> np.uint64(6)) & np.uint64(15)) << np.uint64(2))
+    key = ((c[:, 3] & np.uint64(1)) << np.uint64(39)) | (mort << np.uint64(27)) | pattern
     exp = n_old + (np.argsort(key, kind="stable") if n_new <= 8192 else np.arange(n_new))
     got = order.cpu().numpy()
     assert (got[:n_old] == -5).all()  # older sites are not touched
     assert (got[n_old:] == exp).all()
+    if n_new <= 8192:  # the device-wide radix sort of insc_order_build orders them the same way
+        order2 = torch.full((sc.n,), -5, dtype=torch.int32, device="cuda")
+        lib.insc_order_build(sc.grid, ptr(nbr), I64(n_old), I64(n_new), ptr(order2), stream_ptr())
+        assert (order2.cpu().numpy() == got).all()
     assert (pos.cpu().numpy()[exp] == n_old + np.arange(n_new)).all()
     off = offset.cpu().numpy()
     exp_bo = exp[np.argsort(off[exp] & 7, kind="stable")] if n_new <= 8192 else exp
