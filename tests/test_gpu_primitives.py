@@ -161,6 +161,37 @@ def test_large_insert_built_by_partitions(S, orc, case):
     assert (out.cpu().numpy() == orc.grid_query(o_sc, q)).all()
 
 
+@pytest.mark.parametrize("shape", ["cube", "plane", "column"])
+def test_grid_at_half_load_with_crowded_groups(S, orc, shape):
+    """Scenes that crowd the table's groups of eight slots, at the highest load the grid allows (0.5): a solid
+    cube (every z-run fills its group), a flat plane (every key wants position z & 7 = 5 of its group) and
+    columns along z; inserted in one call and in two, then looked up (hits and misses)."""
+    from sparseconvnet._lib import lib, ptr, stream_ptr
+
+    rng = np.random.default_rng(3)
+    if shape == "cube":
+        g = np.stack(np.meshgrid(np.arange(64), np.arange(64), np.arange(64), indexing="ij"), -1).reshape(-1, 3) + 100
+    elif shape == "plane":
+        g = np.stack(np.meshgrid(np.arange(512), np.arange(512), [5], indexing="ij"), -1).reshape(-1, 3)
+    else:
+        g = np.stack(np.meshgrid(np.arange(16), np.arange(16), np.arange(1024), indexing="ij"), -1).reshape(-1, 3)
+    pts = np.concatenate([g, np.zeros((len(g), 1), np.int64)], 1).astype(np.int32)[rng.permutation(len(g))]
+    assert len(pts) == 262144
+    o_sop, o_sc, _ = orc.grid_build(pts)
+    for cut in (len(pts), 200000):
+        m, sc, sop = _insert(S, pts[:cut], capacity=262144)  # 2^19 slots
+        got = sop.cpu().numpy()
+        if cut < len(pts):
+            got = np.concatenate([got, m.insert(sc, dev(pts[cut:])).cpu().numpy()])
+        assert sc.n == len(o_sc)
+        assert (got == o_sop).all()
+        assert (sc.coords_view().cpu().numpy() == o_sc).all()
+        q = np.concatenate([pts[::3], pts[:30000] + np.array([0, 0, 1100, 0], np.int32)], 0).astype(np.int32)
+        out = torch.empty(len(q), dtype=torch.int32, device="cuda")
+        lib.insc_grid_query(sc.grid, ptr(dev(q)), I64(len(q)), ptr(out), stream_ptr())
+        assert (out.cpu().numpy() == orc.grid_query(o_sc, q)).all()
+
+
 def test_grid_rejects_bad_coordinate(S):
     from sparseconvnet._lib import InscError
 
