@@ -1957,8 +1957,10 @@ static std::atomic<int64_t> g_pers_min_units{INT64_MAX};
 static std::atomic<int64_t> g_shared_min_units{896};
 // Below that, with at least this many (tile, output block) units - half as many again for layers of more
 // than 64 input channels, whose units are longer - the kernel that gives every unit a wavefront of its own
-// (64 -> 64: 55 us against 57 us at 2452 units = 39k sites, 54 against 48 at 2044).
-static std::atomic<int64_t> g_own_min_units{2400};
+// (64 -> 64 at 39k sites = 2452 units: 50 us against 56 us; 2084 units: 48 against 50; 1840: 41 against 44;
+// 1716: 41.1 against 41.5; 1472: 41 against 39 - the split kernel's launch is whole rounds of 1024 blocks, four to
+// a compute unit, this kernel's is the SIMD with the most units).
+static std::atomic<int64_t> g_own_min_units{1750};
 // Narrow 3^3 layers (Cin, Cout <= 32) with at least this many 32-row tiles run on the persistent
 // kernel that keeps the whole filter in LDS; smaller ones on the one-wavefront-per-tile kernel.
 // Same bits either way.
